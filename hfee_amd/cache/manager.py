@@ -1,0 +1,244 @@
+"""The cache manager: pages, block tables and fixed-size state slots.
+
+The reference gives every sequence one dense array per layer, all allocated up
+front and never returned (/root/reference/internal/llm/forward.go:10-26), and only
+its token count says how much of it is valid (forward.go:28-34, 121-123).  Here the
+same memory is cut into pages of `page_size` tokens.  A request holds, for every
+cache group, a block table (page ids by position // page_size) and one state slot.
+
+Groups: layers whose caches have the same needs share a group and a page id
+addresses the same place in each of the group's layers.  A "full" group keeps every
+key; a "window" group keeps the last `window` keys, and pages that the window has
+passed go back to the pool at commit time.  Pages come back when a request is
+released and are handed out again at once (last freed, first reused).
+
+This file is bookkeeping only (no tensors); storage.py holds the device memory.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+
+class OutOfPages(RuntimeError):
+    """A reservation needs more pages than the pool has free."""
+
+
+class CacheError(RuntimeError):
+    """The manager was used against its contract (unknown request, double release...)."""
+
+
+@dataclass(frozen=True)
+class CacheGroupSpec:
+    kind: str                 # "full" or "window"
+    kv_heads: int
+    head_dim: int
+    cache_layers: tuple       # ids of the cache layers in this group
+    window: int = 0           # keys kept per token for kind == "window"
+
+    def __post_init__(self):
+        if self.kind not in ("full", "window"):
+            raise CacheError(f"unknown cache group kind {self.kind!r}")
+        if self.kind == "window" and self.window <= 0:
+            raise CacheError("a window group needs a positive window")
+
+
+class PagePool:
+    """The pages of one group.  LIFO free list; every page is free or owned by
+    exactly one request."""
+
+    def __init__(self, num_pages: int):
+        if num_pages < 1:
+            raise CacheError("a page pool needs at least one page")
+        self.num_pages = num_pages
+        self._free = list(range(num_pages - 1, -1, -1))   # pop() hands out 0 first
+        self._owner: list = [None] * num_pages
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def take(self, owner) -> int:
+        if not self._free:
+            raise OutOfPages("no free page")
+        page = self._free.pop()
+        assert self._owner[page] is None, "a free page had an owner"
+        self._owner[page] = owner
+        return page
+
+    def give_back(self, page: int, owner) -> None:
+        if not 0 <= page < self.num_pages:
+            raise CacheError(f"page {page} does not exist")
+        if self._owner[page] is None:
+            raise CacheError(f"page {page} is freed twice")
+        if self._owner[page] != owner:
+            raise CacheError(f"page {page} belongs to {self._owner[page]!r}, not {owner!r}")
+        self._owner[page] = None
+        self._free.append(page)
+
+    def owner_of(self, page: int):
+        return self._owner[page]
+
+
+@dataclass
+class RequestCache:
+    request_id: object
+    slot: int
+    length: int = 0                                   # committed tokens
+    tables: list = field(default_factory=list)        # per group: page id per block, -1 once released
+    first_live_block: list = field(default_factory=list)   # per group
+
+
+class CacheManager:
+    def __init__(self, groups, page_size: int, pages_per_group, max_requests: int):
+        if page_size < 16 or page_size & (page_size - 1):
+            raise CacheError(f"page_size must be a power of two >= 16, got {page_size}")
+        self.groups = tuple(groups)
+        if isinstance(pages_per_group, int):
+            pages_per_group = [pages_per_group] * len(self.groups)
+        if len(pages_per_group) != len(self.groups):
+            raise CacheError("one page count per cache group is needed")
+        self.page_size = page_size
+        self.pools = [PagePool(n) for n in pages_per_group]
+        self.max_requests = max_requests
+        self._free_slots = list(range(max_requests - 1, -1, -1))
+        self.requests: dict = {}
+
+    # ------------------------------------------------------------ requests
+    def admit(self, request_id) -> RequestCache:
+        if request_id in self.requests:
+            raise CacheError(f"request {request_id!r} is already live")
+        if not self._free_slots:
+            raise CacheError(f"all {self.max_requests} state slots are in use")
+        rc = RequestCache(request_id, self._free_slots.pop(),
+                          tables=[[] for _ in self.groups], first_live_block=[0] * len(self.groups))
+        self.requests[request_id] = rc
+        return rc
+
+    def get(self, request_id) -> RequestCache:
+        try:
+            return self.requests[request_id]
+        except KeyError:
+            raise CacheError(f"request {request_id!r} is not live") from None
+
+    def release(self, request_id) -> None:
+        rc = self.get(request_id)
+        for g, table in enumerate(rc.tables):
+            for page in table:
+                if page >= 0:
+                    self.pools[g].give_back(page, request_id)
+        del self.requests[request_id]
+        self._free_slots.append(rc.slot)
+
+    @property
+    def num_free_slots(self) -> int:
+        return len(self._free_slots)
+
+    # --------------------------------------------------------------- pages
+    def _blocks_for(self, length: int) -> int:
+        return (length + self.page_size - 1) // self.page_size
+
+    def pages_needed(self, request_id, n_new: int) -> list:
+        """Pages each group would have to take so that positions
+        length .. length + n_new - 1 have a place."""
+        rc = self.get(request_id)
+        want = self._blocks_for(rc.length + n_new)
+        return [max(0, want - len(t)) for t in rc.tables]
+
+    def pages_for_tokens(self, n_tokens: int) -> list:
+        """Pages per group that a fresh request of n_tokens holds at most at one time
+        when it is run in one portion."""
+        return [self._blocks_for(n_tokens)] * len(self.groups)
+
+    def can_reserve(self, request_id, n_new: int) -> bool:
+        return all(need <= pool.num_free for need, pool in zip(self.pages_needed(request_id, n_new), self.pools))
+
+    def free_pages(self) -> list:
+        return [p.num_free for p in self.pools]
+
+    def reserve(self, request_id, n_new: int) -> None:
+        """Takes the pages for the next n_new tokens in every group, or none at all
+        (OutOfPages)."""
+        if n_new < 0:
+            raise CacheError("cannot reserve a negative number of tokens")
+        rc = self.get(request_id)
+        need = self.pages_needed(request_id, n_new)
+        for n, pool, g in zip(need, self.pools, range(len(self.pools))):
+            if n > pool.num_free:
+                raise OutOfPages(f"request {request_id!r} needs {n} more pages in cache group {g}, "
+                                 f"{pool.num_free} are free")
+        for g, n in enumerate(need):
+            for _ in range(n):
+                rc.tables[g].append(self.pools[g].take(request_id))
+
+    def commit(self, request_id, n_new: int) -> None:
+        """The step has written n_new tokens: advance the length and return the
+        pages that a window has passed."""
+        rc = self.get(request_id)
+        if any(self._blocks_for(rc.length + n_new) > len(t) for t in rc.tables):
+            raise CacheError(f"request {request_id!r}: commit of {n_new} tokens beyond the reserved pages")
+        rc.length += n_new
+        for g, spec in enumerate(self.groups):
+            if spec.kind != "window":
+                continue
+            # the next query sits at position >= length and reads keys >= length - window + 1
+            first_needed = max(0, rc.length - spec.window + 1)
+            dead_until = first_needed // self.page_size        # blocks < dead_until are never read again
+            table = rc.tables[g]
+            for b in range(rc.first_live_block[g], min(dead_until, len(table))):
+                if table[b] >= 0:
+                    self.pools[g].give_back(table[b], request_id)
+                    table[b] = -1
+            rc.first_live_block[g] = max(rc.first_live_block[g], min(dead_until, len(table)))
+
+    def truncate(self, request_id, length: int) -> None:
+        """Forget tokens at and after `length` (full groups give back whole pages
+        beyond it; the rows left in a kept page are overwritten later, as the
+        reference's Truncate leaves stale rows, forward.go:31-34).  Window groups
+        cannot go back past what they have released."""
+        rc = self.get(request_id)
+        if not 0 <= length <= rc.length:
+            raise CacheError(f"cannot truncate request {request_id!r} from {rc.length} to {length}")
+        keep = self._blocks_for(length)
+        for g, spec in enumerate(self.groups):
+            table = rc.tables[g]
+            if spec.kind == "window" and length > 0 and any(
+                    table[b] < 0 for b in range(max(0, (length - spec.window) // self.page_size), min(keep, len(table)))):
+                raise CacheError("a window group has already released pages this truncation needs")
+            while len(table) > keep:
+                page = table.pop()
+                if page >= 0:
+                    self.pools[g].give_back(page, request_id)
+            rc.first_live_block[g] = min(rc.first_live_block[g], len(table))
+        rc.length = length
+
+    def block_table(self, request_id, group: int) -> list:
+        return self.get(request_id).tables[group]
+
+    # ---------------------------------------------------------- invariants
+    def check(self) -> None:
+        """No page lost, held twice or freed twice; every table entry is owned by its request."""
+        for g, pool in enumerate(self.pools):
+            held = []
+            for rid, rc in self.requests.items():
+                for page in rc.tables[g]:
+                    if page >= 0:
+                        if pool.owner_of(page) != rid:
+                            raise CacheError(f"group {g}: page {page} in the table of {rid!r} is owned by "
+                                             f"{pool.owner_of(page)!r}")
+                        held.append(page)
+            if len(held) != len(set(held)):
+                raise CacheError(f"group {g}: a page is held twice")
+            free = list(pool._free)
+            if len(free) != len(set(free)):
+                raise CacheError(f"group {g}: a page is on the free list twice")
+            if set(free) & set(held):
+                raise CacheError(f"group {g}: a page is both free and held")
+            if len(free) + len(held) != pool.num_pages:
+                raise CacheError(f"group {g}: {pool.num_pages - len(free) - len(held)} page(s) lost")
+            for page in free:
+                if pool.owner_of(page) is not None:
+                    raise CacheError(f"group {g}: free page {page} has an owner")
+        slots = [rc.slot for rc in self.requests.values()]
+        if len(slots) != len(set(slots)) or set(slots) & set(self._free_slots) \
+                or len(slots) + len(self._free_slots) != self.max_requests:
+            raise CacheError("state slots are inconsistent")

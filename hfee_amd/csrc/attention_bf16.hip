@@ -1,0 +1,361 @@
+// Paged causal attention on the matrix cores, bfloat16 in, float32 softmax and
+// accumulation.  Compiled once per head size (HFEE_HEAD_DIM, a multiple of 16).
+//
+// The formulas are the reference's (/root/reference/internal/llm/forward.go:144-178):
+// head h reads KV head h / (H/K); scores are dot * scale over the keys
+// 0..pos (the range is the mask; a window narrows it), softmax, weighted sum of
+// the values.  The softmax runs online over tiles of 32 keys.
+//
+// One wave owns 32 query slots.  Per key tile it computes S^T = K Q^T with
+// v_mfma_f32_32x32x16_bf16 (the key rows come straight from the page as the A
+// operand, 16 bytes per lane), keeps each query's running maximum and sum in the
+// lane that holds that query's column, and feeds P^T back as the B operand of
+// O^T += V^T P^T without leaving registers: the A operand of that product is the
+// transposed value page, whose 4-key runs are contiguous.  The k index of a matrix
+// instruction is only a label shared by its two operands, so the keys that a lane
+// happens to hold after the first product (8b + 4G + i) need no shuffle.
+//
+//   prefill: a slot is a position of one segment's portion, all for one head;
+//   decode:  a slot is one of the heads that share a KV head, all at one position;
+//            the keys may be split over several waves whose partial results a
+//            second kernel joins.
+#include "common.h"
+
+#ifndef HFEE_HEAD_DIM
+#error "compile with -DHFEE_HEAD_DIM=<multiple of 16>"
+#endif
+
+using namespace hfee;
+
+HFEE_DEFINE_LAST_ERROR
+
+namespace {
+
+constexpr int HD = HFEE_HEAD_DIM;
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 in 16..256");
+constexpr int NC = HD / 16;            // 16-wide chunks of the head for Q K^T
+constexpr int NDT = (HD + 31) / 32;    // 32-wide tiles of the head for P V
+constexpr float LOG2E = 1.4426950408889634f;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+union Op {          // one matrix-instruction operand: eight bfloat16
+  u32x4 u;
+  u32x2 h[2];
+  bf16x8 v;
+  bf16_t e[8];
+};
+
+struct Tile {
+  // running state of 32 query slots; this lane's slot is lane % 32
+  float m;              // running maximum of the scaled scores (log2 domain)
+  float l;              // running sum
+  f32x16 o[NDT];        // O^T: register r of tile t is dim 32t + 8*(r/4) + 4*(lane/32) + r%4
+};
+
+// Adds the keys k0 .. k0+31 of one sequence to the running state.
+// q_op: this slot's query, pre-loaded as NC operands.  pos: this slot's position
+// (keys lo..pos are visible; -1 for an unused slot).  kv_first..kv_last: the keys
+// whose pages may be touched at all (a window group has given back the pages
+// before kv_first; nothing exists after kv_last).
+__device__ __forceinline__ void attend_tile(Tile& st, const Op* q_op, const bf16_t* __restrict__ cache,
+                                            const CacheLayout& lay, const int* __restrict__ bt, int kvh,
+                                            int k0, int kv_first, int kv_last, int pos, int lo,
+                                            float scale_log2) {
+  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+
+  // ---- S^T = K Q^T ------------------------------------------------------------
+  f32x16 s;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s[r] = 0.f;
+  {
+    const int key = k0 + r32;
+    const bool ok = key <= kv_last && key >= kv_first;
+    const bf16_t* krow = ok ? cache + lay.key_offset(bt[key >> lay.page_shift], kvh, key & (lay.page_size - 1), 0)
+                            : cache;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      Op k;
+      k.u = u32x4{0u, 0u, 0u, 0u};
+      if (ok) k.u = *reinterpret_cast<const u32x4*>(krow + c * 16 + G * 8);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k.v, q_op[c].v, s, 0, 0, 0);
+    }
+  }
+
+  // ---- mask, running maximum and sum ------------------------------------------
+  float tile_max = -INFINITY;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int key = k0 + 8 * (r >> 2) + 4 * G + (r & 3);
+    const bool visible = key <= pos && key >= lo;
+    s[r] = visible ? s[r] * scale_log2 : -INFINITY;
+    tile_max = fmaxf(tile_max, s[r]);
+  }
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+  const float m_new = fmaxf(st.m, tile_max);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = exp2f(st.m - m_use);          // st.m == -inf gives 0
+  float psum = 0.f;
+  Op p[2];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float e = exp2f(s[r] - m_use);
+    psum += e;
+    p[r >> 3].e[r & 7] = float_to_bf16(e);
+  }
+  psum += __shfl_xor(psum, 32, 64);
+  st.l = st.l * alpha + psum;
+  st.m = m_new;
+#pragma unroll
+  for (int t = 0; t < NDT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
+
+  // ---- O^T += V^T P^T ----------------------------------------------------------
+  // step u covers keys k0+16u .. k0+16u+15; this lane's operand slots 0..3 are keys
+  // 16u + 4G + 0..3 and slots 4..7 are keys 16u + 8 + 4G + 0..3 (as P holds them).
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int kb = k0 + 16 * u;
+    const bool ok = kb <= kv_last && kb + 15 >= kv_first;
+    const int page = ok ? bt[kb >> lay.page_shift] : 0;
+    const int slot = (kb & (lay.page_size - 1)) + 4 * G;
+#pragma unroll
+    for (int t = 0; t < NDT; ++t) {
+      const int d = 32 * t + r32;
+      Op v;
+      v.u = u32x4{0u, 0u, 0u, 0u};
+      if (ok && d < HD) {
+        const bf16_t* vrow = cache + lay.value_offset(page, kvh, slot, d);
+        v.h[0] = *reinterpret_cast<const u32x2*>(vrow);
+        v.h[1] = *reinterpret_cast<const u32x2*>(vrow + 8);
+      }
+      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v.v, p[u].v, st.o[t], 0, 0, 0);
+    }
+  }
+}
+
+__device__ __forceinline__ void load_query(Op* q_op, const bf16_t* __restrict__ qrow, bool ok) {
+  const int G = (threadIdx.x & 63) >> 5;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    q_op[c].u = u32x4{0u, 0u, 0u, 0u};
+    if (ok) q_op[c].u = *reinterpret_cast<const u32x4*>(qrow + c * 16 + G * 8);
+  }
+}
+
+__device__ __forceinline__ void init_tile(Tile& st) {
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int t = 0; t < NDT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st.o[t][r] = 0.f;
+}
+
+// ------------------------------------------------------------------- prefill ---
+// work: per workgroup 4 ints: first row of the tile in the batch, number of rows
+// in the tile (<= 32), position of the first row, block-table row (segment).
+__global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, int64_t ld_out,
+                                                     const bf16_t* __restrict__ q, int64_t ldq,
+                                                     const bf16_t* __restrict__ cache, CacheLayout lay,
+                                                     const int* __restrict__ work,
+                                                     const int* __restrict__ block_tables, int bt_stride,
+                                                     int num_heads, float scale_log2, int window) {
+  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+  const int* wk = work + 4 * blockIdx.x;
+  const int row0 = wk[0], rows = wk[1], pos0 = wk[2], seg = wk[3];
+  const int h = blockIdx.y;
+  const int kvh = h / (num_heads / lay.kv_heads);
+  const int* bt = block_tables + (int64_t)seg * bt_stride;
+
+  const bool slot_ok = r32 < rows;
+  const int pos = slot_ok ? pos0 + r32 : -1;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  Op q_op[NC];
+  load_query(q_op, q + (int64_t)(row0 + (slot_ok ? r32 : 0)) * ldq + h * HD, slot_ok);
+
+  Tile st;
+  init_tile(st);
+  const int kv_last = pos0 + rows - 1;
+  const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
+  for (int k0 = kv_first & ~31; k0 <= kv_last; k0 += 32)
+    attend_tile(st, q_op, cache, lay, bt, kvh, k0, kv_first, kv_last, pos, lo, scale_log2);
+
+  if (slot_ok) {
+    const float inv = 1.0f / st.l;
+    bf16_t* orow = out + (int64_t)(row0 + r32) * ld_out + h * HD;
+#pragma unroll
+    for (int t = 0; t < NDT; ++t)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int d = 32 * t + 8 * b + 4 * G;
+        if (d < HD) {
+          bf16_t v4[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v4[i] = float_to_bf16(st.o[t][4 * b + i] * inv);
+          *reinterpret_cast<u32x2*>(orow + d) = *reinterpret_cast<const u32x2*>(v4);
+        }
+      }
+  }
+}
+
+// -------------------------------------------------------------------- decode ---
+// One workgroup (one wave) per (decode segment, KV head, split).  The slots are
+// the heads of the group, 32 at a time.  partial: per (segment, head, split)
+// HD + 2 floats: the unnormalised output, the maximum, the sum.
+__global__ __launch_bounds__(64) void decode_kernel(bf16_t* __restrict__ out, int64_t ld_out,
+                                                    const bf16_t* __restrict__ q, int64_t ldq,
+                                                    const bf16_t* __restrict__ cache, CacheLayout lay,
+                                                    const int* __restrict__ seg_rows,
+                                                    const int* __restrict__ seg_positions,
+                                                    const int* __restrict__ seg_tables,
+                                                    const int* __restrict__ block_tables, int bt_stride,
+                                                    int num_heads, float scale_log2, int window,
+                                                    float* __restrict__ partial, int num_splits) {
+  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+  const int sidx = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int group = num_heads / lay.kv_heads;
+  const int row = seg_rows[sidx], pos = seg_positions[sidx];
+  const int* bt = block_tables + (int64_t)seg_tables[sidx] * bt_stride;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+
+  // key tiles of this split: a contiguous share of the tiles lo/32 .. pos/32
+  const int tile_first = lo >> 5, tile_count = (pos >> 5) - tile_first + 1;
+  const int per = (tile_count + num_splits - 1) / num_splits;
+  const int t_begin = tile_first + split * per;
+  const int t_end = min(tile_first + tile_count, t_begin + per);
+
+  for (int g0 = 0; g0 < group; g0 += 32) {
+    const bool slot_ok = g0 + r32 < group;
+    const int h = kvh * group + g0 + (slot_ok ? r32 : 0);
+    Op q_op[NC];
+    load_query(q_op, q + (int64_t)row * ldq + h * HD, slot_ok);
+    Tile st;
+    init_tile(st);
+    for (int t = t_begin; t < t_end; ++t)
+      attend_tile(st, q_op, cache, lay, bt, kvh, t * 32, lo, pos, slot_ok ? pos : -1, lo, scale_log2);
+    if (!slot_ok) continue;
+    if (num_splits == 1) {
+      const float inv = 1.0f / st.l;
+      bf16_t* orow = out + (int64_t)row * ld_out + h * HD;
+#pragma unroll
+      for (int t = 0; t < NDT; ++t)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int d = 32 * t + 8 * b + 4 * G;
+          if (d < HD) {
+            bf16_t v4[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v4[i] = float_to_bf16(st.o[t][4 * b + i] * inv);
+            *reinterpret_cast<u32x2*>(orow + d) = *reinterpret_cast<const u32x2*>(v4);
+          }
+        }
+    } else {
+      float* pr = partial + ((int64_t)(sidx * num_heads + h) * num_splits + split) * (HD + 2);
+#pragma unroll
+      for (int t = 0; t < NDT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int d = 32 * t + 8 * (r >> 2) + 4 * G + (r & 3);
+          if (d < HD) pr[d] = st.o[t][r];
+        }
+      if (G == 0) {
+        pr[HD] = st.m;
+        pr[HD + 1] = st.l;
+      }
+    }
+  }
+}
+
+// Joins the splits of one (segment, head) in ascending split order.
+__global__ __launch_bounds__(64) void combine_kernel(bf16_t* __restrict__ out, int64_t ld_out,
+                                                     const int* __restrict__ seg_rows,
+                                                     const float* __restrict__ partial, int num_heads,
+                                                     int num_splits) {
+  const int sidx = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* pr = partial + (int64_t)(sidx * num_heads + h) * num_splits * (HD + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) m = fmaxf(m, pr[s * (HD + 2) + HD]);
+  const float m_use = m == -INFINITY ? 0.f : m;
+  float l = 0.f;
+  for (int s = 0; s < num_splits; ++s) l += pr[s * (HD + 2) + HD + 1] * exp2f(pr[s * (HD + 2) + HD] - m_use);
+  const float inv = 1.0f / l;
+  bf16_t* orow = out + (int64_t)seg_rows[sidx] * ld_out + h * HD;
+  for (int d = lane; d < HD; d += 64) {
+    float o = 0.f;
+    for (int s = 0; s < num_splits; ++s) o += pr[s * (HD + 2) + d] * exp2f(pr[s * (HD + 2) + HD] - m_use);
+    orow[d] = float_to_bf16(o * inv);
+  }
+}
+
+}  // namespace
+
+HFEE_API int hfee_attention_bf16_head_dim() { return HD; }
+
+static int check_common(const char* name, int64_t ld_out, int64_t ldq, int num_heads, int kv_heads,
+                        int page_size, int window, const void* out, const void* q, CacheLayout* lay) {
+  HFEE_REQUIRE(num_heads > 0 && kv_heads > 0 && num_heads % kv_heads == 0,
+               "%s: %d heads are not a multiple of %d kv heads", name, num_heads, kv_heads);
+  HFEE_REQUIRE(num_heads <= 65535, "%s: too many heads", name);
+  HFEE_REQUIRE(window >= 0, "%s: negative window", name);
+  HFEE_REQUIRE(ldq >= (int64_t)num_heads * HD && ld_out >= (int64_t)num_heads * HD, "%s: q/out row too short", name);
+  HFEE_REQUIRE(ldq % 8 == 0 && (uintptr_t)q % 16 == 0, "%s: q rows must be 16-byte aligned", name);
+  HFEE_REQUIRE(ld_out % 4 == 0 && (uintptr_t)out % 8 == 0, "%s: out rows must be 8-byte aligned", name);
+  return make_cache_layout(lay, kv_heads, HD, page_size);
+}
+
+// work: num_tiles x 4 int32 (first row, rows <= 32, first position, block-table row).
+HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* q, int64_t ldq,
+                                         const void* cache, const int* work, int num_tiles,
+                                         const int* block_tables, int bt_stride, int num_heads, int kv_heads,
+                                         int page_size, float scale, int window, hipStream_t stream) {
+  HFEE_REQUIRE(num_tiles >= 0, "attention_bf16_prefill: bad tile count");
+  if (num_tiles == 0) return 0;
+  CacheLayout lay;
+  if (check_common("attention_bf16_prefill", ld_out, ldq, num_heads, kv_heads, page_size, window, out, q, &lay))
+    return 1;
+  dim3 grid(num_tiles, num_heads);
+  prefill_kernel<<<grid, 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
+                                          work, block_tables, bt_stride, num_heads, scale * LOG2E, window);
+  HFEE_CHECK_LAUNCH("attention_bf16_prefill");
+  return 0;
+}
+
+// seg_rows / seg_positions / seg_tables: per decode segment its row in the batch,
+// its position and its block-table row.  partial: at least
+// num_segments * num_heads * num_splits * (head_dim + 2) floats when num_splits > 1.
+HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
+                                        const int* seg_rows, const int* seg_positions, const int* seg_tables,
+                                        int num_segments, const int* block_tables, int bt_stride,
+                                        int num_heads, int kv_heads, int page_size, float scale, int window,
+                                        float* partial, int64_t partial_floats, int num_splits,
+                                        hipStream_t stream) {
+  HFEE_REQUIRE(num_segments >= 0, "attention_bf16_decode: bad segment count");
+  if (num_segments == 0) return 0;
+  CacheLayout lay;
+  if (check_common("attention_bf16_decode", ld_out, ldq, num_heads, kv_heads, page_size, window, out, q, &lay))
+    return 1;
+  HFEE_REQUIRE(num_splits >= 1 && num_splits <= 65535, "attention_bf16_decode: bad split count %d", num_splits);
+  HFEE_REQUIRE(kv_heads <= 65535, "attention_bf16_decode: too many kv heads");
+  if (num_splits > 1) {
+    const int64_t need = (int64_t)num_segments * num_heads * num_splits * (HD + 2);
+    HFEE_REQUIRE(partial != nullptr && partial_floats >= need,
+                 "attention_bf16_decode: the partial buffer holds %lld floats, %lld needed",
+                 (long long)partial_floats, (long long)need);
+  }
+  dim3 grid(num_segments, kv_heads, num_splits);
+  decode_kernel<<<grid, 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
+                                         seg_rows, seg_positions, seg_tables, block_tables, bt_stride, num_heads,
+                                         scale * LOG2E, window, partial, num_splits);
+  HFEE_CHECK_LAUNCH("attention_bf16_decode");
+  if (num_splits > 1) {
+    dim3 cgrid(num_segments, num_heads);
+    combine_kernel<<<cgrid, 64, 0, stream>>>((bf16_t*)out, ld_out, seg_rows, partial, num_heads, num_splits);
+    HFEE_CHECK_LAUNCH("attention_bf16_decode(combine)");
+  }
+  return 0;
+}

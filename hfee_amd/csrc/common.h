@@ -1,0 +1,144 @@
+// Shared device helpers and the host-side error channel of the kernel library.
+// Target: gfx950 (CDNA4), wave64.  Every entry point is extern "C", takes raw
+// device pointers, sizes and a stream, checks its arguments on the host and
+// returns 0, or a nonzero code after recording a message that
+// hfee_last_error() returns.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#define HFEE_API extern "C" __attribute__((visibility("default")))
+
+typedef uint16_t bf16_t;   // storage type of bfloat16 values
+
+namespace hfee {
+
+constexpr int kWave = 64;
+
+// ---- host-side error channel -------------------------------------------------
+inline char* error_buffer() {
+  static thread_local char buffer[512];
+  return buffer;
+}
+
+inline int fail(const char* fmt, ...) {   // records the message, returns 1
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+// Exactly one translation unit of each shared library expands this.
+#define HFEE_DEFINE_LAST_ERROR \
+  HFEE_API const char* hfee_last_error() { return hfee::error_buffer(); }
+
+#define HFEE_REQUIRE(cond, ...)                     \
+  do {                                              \
+    if (!(cond)) return hfee::fail(__VA_ARGS__);    \
+  } while (0)
+
+#define HFEE_CHECK_LAUNCH(name)                                              \
+  do {                                                                       \
+    hipError_t e_ = hipGetLastError();                                       \
+    if (e_ != hipSuccess) return hfee::fail("%s: launch failed: %s", name,   \
+                                            hipGetErrorString(e_));          \
+  } while (0)
+
+// ---- bfloat16 <-> float --------------------------------------------------------
+__device__ __forceinline__ float bf16_to_float(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                          // round to nearest even
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float to_float(T v);
+template <> __device__ __forceinline__ float to_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_float<bf16_t>(bf16_t v) { return bf16_to_float(v); }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return float_to_bf16(v); }
+
+// ---- reductions with a fixed order -------------------------------------------
+// Every lane ends with the same value; the tree's shape does not depend on data.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds 16 floats of LDS.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nwaves = (blockDim.x + 63) >> 6;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nwaves = (blockDim.x + 63) >> 6;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = scratch[0];
+  for (int w = 1; w < nwaves; ++w) total = fmaxf(total, scratch[w]);
+  return total;
+}
+
+// ---- the paged cache's layout -------------------------------------------------
+// One cache layer is [num_pages][2][kv_heads][page_size * head_dim] elements:
+// keys of a (page, head) as [slot][head_dim], values transposed as [head_dim][slot],
+// so that eight consecutive keys of one value column are 16 contiguous bytes in bf16.
+struct CacheLayout {
+  int64_t page_stride;   // elements between pages: 2 * kv_heads * page_size * head_dim
+  int kv_heads;
+  int head_dim;
+  int page_size;
+  int page_shift;        // log2(page_size)
+
+  __host__ __device__ __forceinline__ int64_t key_offset(int page, int kvh, int slot, int d) const {
+    return (int64_t)page * page_stride + (int64_t)kvh * page_size * head_dim + (int64_t)slot * head_dim + d;
+  }
+  __host__ __device__ __forceinline__ int64_t value_offset(int page, int kvh, int slot, int d) const {
+    return (int64_t)page * page_stride + (int64_t)(kv_heads + kvh) * page_size * head_dim +
+           (int64_t)d * page_size + slot;
+  }
+};
+
+inline int make_cache_layout(CacheLayout* out, int kv_heads, int head_dim, int page_size) {
+  if (page_size < 16 || (page_size & (page_size - 1)) != 0)
+    return fail("page_size must be a power of two >= 16, got %d", page_size);
+  if (kv_heads < 1 || head_dim < 1) return fail("bad cache shape: kv_heads %d head_dim %d", kv_heads, head_dim);
+  out->kv_heads = kv_heads;
+  out->head_dim = head_dim;
+  out->page_size = page_size;
+  out->page_stride = (int64_t)2 * kv_heads * page_size * head_dim;
+  int s = 0;
+  while ((1 << s) < page_size) ++s;
+  out->page_shift = s;
+  return 0;
+}
+
+}  // namespace hfee

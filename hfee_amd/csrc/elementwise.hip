@@ -1,0 +1,226 @@
+// Embedding gather, RMSNorm, rotary encoding with the write into the paged
+// cache, SiLU gating and the residual add.  All of them are bound by memory
+// traffic; sums, angles and the residual stream are float32.
+//
+// Formulas (file:line in /root/reference):
+//   embedding   internal/llm/forward.go:75-77
+//   RMSNorm     internal/ggml/ops.go:124-134  (x * scale * weight, eps inside the root)
+//   rotation    internal/llm/forward.go:180-196, cache write forward.go:99-101
+//   SiLU gate   internal/ggml/ops.go:159-165  (g / (1 + exp(-g)) * up)
+//   residual    internal/ggml/ops.go:152-157
+#include "common.h"
+
+using namespace hfee;
+
+HFEE_DEFINE_LAST_ERROR
+
+enum { DT_F32 = 0, DT_BF16 = 1 };
+
+// ------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
+                             const int* __restrict__ ids, int d) {
+  const int row = blockIdx.x;
+  const int64_t src = (int64_t)ids[row] * d;
+  for (int j = threadIdx.x; j < d; j += blockDim.x) out[(int64_t)row * d + j] = to_float<T>(table[src + j]);
+}
+
+HFEE_API int hfee_embed(float* out, const void* table, int table_dtype, const int* ids,
+                        int n, int d, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && d > 0, "embed: bad sizes n=%d d=%d", n, d);
+  if (n == 0) return 0;
+  if (table_dtype == DT_F32)
+    embed_kernel<float><<<n, 256, 0, stream>>>(out, (const float*)table, ids, d);
+  else if (table_dtype == DT_BF16)
+    embed_kernel<bf16_t><<<n, 256, 0, stream>>>(out, (const bf16_t*)table, ids, d);
+  else
+    return fail("embed: unknown dtype %d", table_dtype);
+  HFEE_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// -------------------------------------------------------------------- RMSNorm
+// One block per output row.  rows == nullptr: row r of x; else row rows[r] of x.
+template <typename TOut, typename TW>
+__global__ void rmsnorm_kernel(TOut* __restrict__ out, const float* __restrict__ x,
+                               const TW* __restrict__ w, const int* __restrict__ rows,
+                               float eps, int d) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const float* xr = x + (int64_t)(rows ? rows[r] : r) * d;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < d; j += blockDim.x) {
+    const float v = xr[j];
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+  TOut* o = out + (int64_t)r * d;
+  for (int j = threadIdx.x; j < d; j += blockDim.x)
+    o[j] = from_float<TOut>(xr[j] * scale * to_float<TW>(w[j]));
+}
+
+HFEE_API int hfee_rmsnorm(void* out, int out_dtype, const float* x, const void* w, int w_dtype,
+                          const int* rows, float eps, int n, int d, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && d > 0, "rmsnorm: bad sizes n=%d d=%d", n, d);
+  HFEE_REQUIRE(eps >= 0.f, "rmsnorm: eps must not be negative");
+  if (n == 0) return 0;
+  const int threads = d >= 2048 ? 512 : 256;
+#define LAUNCH(TO, TW) rmsnorm_kernel<TO, TW><<<n, threads, 0, stream>>>((TO*)out, x, (const TW*)w, rows, eps, d)
+  if (out_dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
+  else if (out_dtype == DT_F32 && w_dtype == DT_BF16) LAUNCH(float, bf16_t);
+  else if (out_dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16_t, float);
+  else if (out_dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
+  else return fail("rmsnorm: unknown dtypes out=%d w=%d", out_dtype, w_dtype);
+#undef LAUNCH
+  HFEE_CHECK_LAUNCH("rmsnorm");
+  return 0;
+}
+
+// ------------------------------------------------------------------ SiLU gate
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, int64_t ld_out, const T* __restrict__ gate,
+                              const T* __restrict__ up, int64_t ld_in, int width) {
+  const int row = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= width) return;
+  const float g = to_float<T>(gate[(int64_t)row * ld_in + j]);
+  const float u = to_float<T>(up[(int64_t)row * ld_in + j]);
+  out[(int64_t)row * ld_out + j] = from_float<T>(g / (1.0f + expf(-g)) * u);
+}
+
+HFEE_API int hfee_swiglu(void* out, int64_t ld_out, const void* gate, const void* up, int64_t ld_in,
+                         int dtype, int n, int width, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && width > 0 && ld_out >= width && ld_in >= width, "swiglu: bad sizes");
+  HFEE_REQUIRE(n <= 65535 * 16, "swiglu: too many rows (%d)", n);
+  if (n == 0) return 0;
+  // grid.y is limited to 65535: fold rows beyond that into several launches
+  for (int row0 = 0; row0 < n; row0 += 65535) {
+    const int rows = n - row0 < 65535 ? n - row0 : 65535;
+    dim3 grid((width + 255) / 256, rows);
+    if (dtype == DT_F32)
+      swiglu_kernel<float><<<grid, 256, 0, stream>>>((float*)out + row0 * ld_out, ld_out,
+                                                     (const float*)gate + row0 * ld_in,
+                                                     (const float*)up + row0 * ld_in, ld_in, width);
+    else if (dtype == DT_BF16)
+      swiglu_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out + row0 * ld_out, ld_out,
+                                                      (const bf16_t*)gate + row0 * ld_in,
+                                                      (const bf16_t*)up + row0 * ld_in, ld_in, width);
+    else
+      return fail("swiglu: unknown dtype %d", dtype);
+  }
+  HFEE_CHECK_LAUNCH("swiglu");
+  return 0;
+}
+
+// --------------------------------------------------------------- residual add
+template <typename T>
+__global__ void add_kernel(float* __restrict__ x, const T* __restrict__ y, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) x[i] += to_float<T>(y[i]);
+}
+
+HFEE_API int hfee_residual_add(float* x, const void* y, int y_dtype, int64_t total, hipStream_t stream) {
+  HFEE_REQUIRE(total >= 0, "residual_add: bad size");
+  if (total == 0) return 0;
+  const int64_t blocks = (total + 255) / 256;
+  HFEE_REQUIRE(blocks < (1ll << 31), "residual_add: too many elements");
+  if (y_dtype == DT_F32) add_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(x, (const float*)y, total);
+  else if (y_dtype == DT_BF16) add_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>(x, (const bf16_t*)y, total);
+  else return fail("residual_add: unknown dtype %d", y_dtype);
+  HFEE_CHECK_LAUNCH("residual_add");
+  return 0;
+}
+
+// ------------------------------------------------- rotation + write to the cache
+// One block per token.  q is rotated in place; k is rotated and written to the
+// token's slot of its page, v is written transposed.  cos/sin: [positions][half]
+// float32, made on the host in float64 from the exact angle position * inv_freq.
+// pairing 0: (i, i + half); pairing 1: (2i, 2i + 1).  Dimensions at and beyond
+// 2 * half are not rotated.  Any of q, k/v may be null (nothing to do for it).
+template <typename T>
+__global__ void rope_cache_kernel(T* __restrict__ q, int64_t ldq, const T* __restrict__ k, int64_t ldk,
+                                  const T* __restrict__ v, int64_t ldv,
+                                  const int* __restrict__ positions, const int* __restrict__ token_segment,
+                                  const int* __restrict__ block_tables, int bt_stride,
+                                  const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                                  int half, int pairing, T* __restrict__ cache, CacheLayout lay,
+                                  int num_heads) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int hd = lay.head_dim;
+  const float* cs = cos_table ? cos_table + (int64_t)pos * half : nullptr;
+  const float* sn = sin_table ? sin_table + (int64_t)pos * half : nullptr;
+
+  if (q != nullptr && cs != nullptr) {
+    T* qt = q + (int64_t)t * ldq;
+    for (int w = threadIdx.x; w < num_heads * half; w += blockDim.x) {
+      const int h = w / half, i = w - h * half;
+      const int a = pairing == 0 ? i : 2 * i;
+      const int b = pairing == 0 ? i + half : 2 * i + 1;
+      const float x0 = to_float<T>(qt[h * hd + a]), x1 = to_float<T>(qt[h * hd + b]);
+      const float c = cs[i], s = sn[i];
+      qt[h * hd + a] = from_float<T>(x0 * c - x1 * s);
+      qt[h * hd + b] = from_float<T>(x0 * s + x1 * c);
+    }
+  }
+  if (k == nullptr || cache == nullptr) return;
+
+  const int page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
+  const int slot = pos & (lay.page_size - 1);
+  const T* kt = k + (int64_t)t * ldk;
+  const T* vt = v + (int64_t)t * ldv;
+  const int rot = cs != nullptr ? 2 * half : 0;
+  for (int w = threadIdx.x; w < lay.kv_heads * hd; w += blockDim.x) {
+    const int h = w / hd, dd = w - h * hd;
+    float val;
+    if (dd < rot) {
+      int i, partner;
+      bool first;
+      if (pairing == 0) { first = dd < half; i = first ? dd : dd - half; partner = first ? dd + half : dd - half; }
+      else { first = (dd & 1) == 0; i = dd >> 1; partner = first ? dd + 1 : dd - 1; }
+      const float me = to_float<T>(kt[h * hd + dd]), other = to_float<T>(kt[h * hd + partner]);
+      const float c = cs[i], s = sn[i];
+      val = first ? (me * c - other * s) : (other * s + me * c);
+    } else {
+      val = to_float<T>(kt[h * hd + dd]);
+    }
+    cache[lay.key_offset(page, h, slot, dd)] = from_float<T>(val);
+    cache[lay.value_offset(page, h, slot, dd)] = vt[h * hd + dd];
+  }
+}
+
+HFEE_API int hfee_rope_cache_write(void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
+                                   int dtype, const int* positions, const int* token_segment,
+                                   const int* block_tables, int bt_stride,
+                                   const float* cos_table, const float* sin_table, int half, int pairing,
+                                   int table_positions, int max_position,
+                                   void* cache, int num_heads, int kv_heads, int head_dim, int page_size,
+                                   int n, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0, "rope_cache_write: bad token count");
+  if (n == 0) return 0;
+  HFEE_REQUIRE(pairing == 0 || pairing == 1, "rope_cache_write: pairing must be 0 (half) or 1 (interleaved)");
+  HFEE_REQUIRE(half >= 0 && 2 * half <= head_dim, "rope_cache_write: rotary width %d exceeds head_dim %d",
+               2 * half, head_dim);
+  HFEE_REQUIRE(cos_table == nullptr || max_position < table_positions,
+               "rope_cache_write: position %d is beyond the rotation table (%d positions)",
+               max_position, table_positions);
+  HFEE_REQUIRE((k == nullptr) == (v == nullptr), "rope_cache_write: k and v come together");
+  CacheLayout lay;
+  if (make_cache_layout(&lay, kv_heads, head_dim, page_size)) return 1;
+  HFEE_REQUIRE(q == nullptr || ldq >= (int64_t)num_heads * head_dim, "rope_cache_write: q row too short");
+  HFEE_REQUIRE(k == nullptr || (ldk >= (int64_t)kv_heads * head_dim && ldv >= (int64_t)kv_heads * head_dim),
+               "rope_cache_write: k/v row too short");
+  if (dtype == DT_F32)
+    rope_cache_kernel<float><<<n, 256, 0, stream>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
+        positions, token_segment, block_tables, bt_stride, cos_table, sin_table, half, pairing,
+        (float*)cache, lay, num_heads);
+  else if (dtype == DT_BF16)
+    rope_cache_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv,
+        positions, token_segment, block_tables, bt_stride, cos_table, sin_table, half, pairing,
+        (bf16_t*)cache, lay, num_heads);
+  else
+    return fail("rope_cache_write: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("rope_cache_write");
+  return 0;
+}

@@ -1,0 +1,277 @@
+// bfloat16 matrix products on the matrix cores: C[M,N] = A[M,K] * W[N,K]^T with
+// float32 accumulation.  The role of /root/reference/internal/ggml/ops.go:54-91
+// (every weight row is read once for all rows of the batch).
+//
+// Two kernels:
+//  * tiled   (M > 64, prefill): 128x128x32 tiles staged through LDS, four waves,
+//            each wave a 64x64 block of v_mfma_f32_32x32x16_bf16 tiles.  Bound by
+//            the matrix cores.
+//  * skinny  (M <= 64, decode): bound by reading W once from HBM.  A workgroup owns
+//            16 weight rows; its eight waves split K and stream their slices of W
+//            straight from global memory into v_mfma_f32_16x16x32_bf16 operands
+//            (no LDS on the way); the batch rows are the other operand.  Partial
+//            sums meet in LDS in a fixed order.
+// Output modes: bfloat16 store, float32 store, float32 accumulate (the residual
+// add of /root/reference/internal/llm/forward.go:106-107 fused into the epilogue).
+#include "common.h"
+
+using namespace hfee;
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+enum { OUT_BF16 = 0, OUT_F32 = 1, OUT_ADD_F32 = 2 };
+
+union Chunk {           // eight bfloat16 values = 16 bytes
+  u32x4 u;
+  bf16x8 v;
+  bf16_t e[8];
+};
+
+// Eight consecutive elements of a row starting at column k (zeros beyond K or when
+// the row is out of range).  VEC: the row start is 16-byte aligned and K % 8 == 0.
+template <bool VEC>
+__device__ __forceinline__ Chunk load_chunk(const bf16_t* __restrict__ row, bool row_ok, int k, int K) {
+  Chunk c;
+  c.u = u32x4{0u, 0u, 0u, 0u};
+  if (!row_ok) return c;
+  if (VEC) {
+    if (k < K) c.u = *reinterpret_cast<const u32x4*>(row + k);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (k + j < K) c.e[j] = row[k + j];
+  }
+  return c;
+}
+
+template <int MODE>
+__device__ __forceinline__ void store_out(void* C, int64_t ldc, int m, int n, float v) {
+  if (MODE == OUT_BF16) ((bf16_t*)C)[(int64_t)m * ldc + n] = float_to_bf16(v);
+  else if (MODE == OUT_F32) ((float*)C)[(int64_t)m * ldc + n] = v;
+  else ((float*)C)[(int64_t)m * ldc + n] += v;
+}
+
+// ------------------------------------------------------------------- tiled ---
+constexpr int TBM = 128, TBN = 128, TBK = 32, TPITCH = 40;   // LDS row pitch in elements (80 bytes)
+
+template <int MODE, bool VEC>
+__global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(void* __restrict__ C, int64_t ldc,
+                                                              const bf16_t* __restrict__ A, int64_t lda,
+                                                              const bf16_t* __restrict__ W, int64_t ldw,
+                                                              int M, int N, int K) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][TBM * TPITCH];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][TBN * TPITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * TBM, n0 = blockIdx.x * TBN;
+
+  // staging: thread -> (row, 16-byte chunk) of the 128 x 32 tile, two rows apart by 64
+  const int srow = tid >> 2, schunk = (tid & 3) * 8;
+  const bf16_t* a_row[2];
+  const bf16_t* w_row[2];
+  bool a_ok[2], w_ok[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int am = m0 + srow + 64 * p, wn_ = n0 + srow + 64 * p;
+    a_ok[p] = am < M;
+    w_ok[p] = wn_ < N;
+    a_row[p] = A + (int64_t)(a_ok[p] ? am : 0) * lda;
+    w_row[p] = W + (int64_t)(w_ok[p] ? wn_ : 0) * ldw;
+  }
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  Chunk ra[2], rw[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    ra[p] = load_chunk<VEC>(a_row[p], a_ok[p], schunk, K);
+    rw[p] = load_chunk<VEC>(w_row[p], w_ok[p], schunk, K);
+  }
+  const int ktiles = (K + TBK - 1) / TBK;
+  int buf = 0;
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    *reinterpret_cast<u32x4*>(&As[0][(srow + 64 * p) * TPITCH + schunk]) = ra[p].u;
+    *reinterpret_cast<u32x4*>(&Ws[0][(srow + 64 * p) * TPITCH + schunk]) = rw[p].u;
+  }
+  __syncthreads();
+
+  const int lrow = lane & 31, lk = (lane >> 5) * 8;
+  for (int kt = 0; kt < ktiles; ++kt) {
+    if (kt + 1 < ktiles) {
+      const int k = (kt + 1) * TBK + schunk;
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        ra[p] = load_chunk<VEC>(a_row[p], a_ok[p], k, K);
+        rw[p] = load_chunk<VEC>(w_row[p], w_ok[p], k, K);
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16x8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *reinterpret_cast<const bf16x8*>(&As[buf][(wm * 64 + i * 32 + lrow) * TPITCH + ks * 16 + lk]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][(wn * 64 + j * 32 + lrow) * TPITCH + ks * 16 + lk]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < ktiles) {
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        *reinterpret_cast<u32x4*>(&As[buf ^ 1][(srow + 64 * p) * TPITCH + schunk]) = ra[p].u;
+        *reinterpret_cast<u32x4*>(&Ws[buf ^ 1][(srow + 64 * p) * TPITCH + schunk]) = rw[p].u;
+      }
+    }
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  // D layout of the 32x32 tile: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn * 64 + j * 32 + lrow;
+      if (n >= N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < M) store_out<MODE>(C, ldc, m, n, acc[i][j][r]);
+      }
+    }
+}
+
+// ------------------------------------------------------------------ skinny ---
+constexpr int SK_WAVES = 8, SK_ROWS = 16, SK_UNROLL = 4;
+
+// MT: number of 16-row groups of the batch (M <= 16 * MT).
+template <int MODE, bool VEC, int MT>
+__global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(
+    void* __restrict__ C, int64_t ldc, const bf16_t* __restrict__ A, int64_t lda,
+    const bf16_t* __restrict__ W, int64_t ldw, int M, int N, int K) {
+  __shared__ float partial[SK_WAVES][MT][64][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * SK_ROWS;
+  const bool w_ok = n0 + r16 < N;
+  const bf16_t* w_row = W + (int64_t)(w_ok ? n0 + r16 : 0) * ldw;
+  const bf16_t* x_row[MT];
+  bool x_ok[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    x_ok[t] = t * 16 + r16 < M;
+    x_row[t] = A + (int64_t)(x_ok[t] ? t * 16 + r16 : 0) * lda;
+  }
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int KBLOCK = 32 * SK_UNROLL;
+  for (int kb = wave * KBLOCK; kb < K; kb += SK_WAVES * KBLOCK) {
+    Chunk w[SK_UNROLL];
+#pragma unroll
+    for (int s = 0; s < SK_UNROLL; ++s) w[s] = load_chunk<VEC>(w_row, w_ok, kb + s * 32 + g * 8, K);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      Chunk x[SK_UNROLL];
+#pragma unroll
+      for (int s = 0; s < SK_UNROLL; ++s) x[s] = load_chunk<VEC>(x_row[t], x_ok[t], kb + s * 32 + g * 8, K);
+#pragma unroll
+      for (int s = 0; s < SK_UNROLL; ++s)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[s].v, x[s].v, acc[t], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) partial[wave][t][lane][i] = acc[t][i];
+  __syncthreads();
+  // D layout of the 16x16 tile: register i of lane l is weight row 4*(l/16) + i, batch row l%16
+  for (int idx = threadIdx.x; idx < MT * 64; idx += SK_WAVES * 64) {
+    const int t = idx >> 6, l = idx & 63;
+    const int m = t * 16 + (l & 15);
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * (l >> 4) + i;
+      if (n >= N) continue;
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < SK_WAVES; ++w) s += partial[w][t][l][i];
+      store_out<MODE>(C, ldc, m, n, s);
+    }
+  }
+}
+
+template <int MODE, bool VEC>
+int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
+           int M, int N, int K, int force_kernel, hipStream_t stream) {
+  const bool skinny = force_kernel == 1 || (force_kernel == 0 && M <= 64);
+  if (skinny) {
+    const int mt = (M + 15) / 16;
+    dim3 grid((N + SK_ROWS - 1) / SK_ROWS);
+    for (int m0 = 0; m0 < M; m0 += 64) {   // M > 64 only when the kernel was forced
+      const int rows = M - m0 < 64 ? M - m0 : 64;
+      const int g = (rows + 15) / 16;
+      void* c = MODE == OUT_BF16 ? (void*)((bf16_t*)C + (int64_t)m0 * ldc) : (void*)((float*)C + (int64_t)m0 * ldc);
+      const bf16_t* a = A + (int64_t)m0 * lda;
+      if (g == 1) gemm_bf16_skinny_kernel<MODE, VEC, 1><<<grid, SK_WAVES * 64, 0, stream>>>(c, ldc, a, lda, W, ldw, rows, N, K);
+      else if (g == 2) gemm_bf16_skinny_kernel<MODE, VEC, 2><<<grid, SK_WAVES * 64, 0, stream>>>(c, ldc, a, lda, W, ldw, rows, N, K);
+      else if (g == 3) gemm_bf16_skinny_kernel<MODE, VEC, 3><<<grid, SK_WAVES * 64, 0, stream>>>(c, ldc, a, lda, W, ldw, rows, N, K);
+      else gemm_bf16_skinny_kernel<MODE, VEC, 4><<<grid, SK_WAVES * 64, 0, stream>>>(c, ldc, a, lda, W, ldw, rows, N, K);
+    }
+    (void)mt;
+  } else {
+    dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM);
+    if (grid.y > 65535) return fail("gemm_bf16: too many rows (%d)", M);
+    gemm_bf16_tiled_kernel<MODE, VEC><<<grid, 256, 0, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
+  }
+  return 0;
+}
+
+}  // namespace
+
+// out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate.
+// force_kernel: 0 choose by M, 1 skinny, 2 tiled (for tests of each kernel alone).
+HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
+                            int64_t ldw, int M, int N, int K, int force_kernel, hipStream_t stream) {
+  HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
+  HFEE_REQUIRE(ldc >= N && lda >= K && ldw >= K, "gemm_bf16: a leading dimension is shorter than its row");
+  HFEE_REQUIRE(out_mode >= 0 && out_mode <= 2, "gemm_bf16: unknown output mode %d", out_mode);
+  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 2, "gemm_bf16: unknown kernel choice %d", force_kernel);
+  if (M == 0) return 0;
+  const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) &&
+                   ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  int rc;
+#define GO(MODE)                                                                                  \
+  rc = vec ? launch<MODE, true>(C, ldc, a, lda, w, ldw, M, N, K, force_kernel, stream)             \
+           : launch<MODE, false>(C, ldc, a, lda, w, ldw, M, N, K, force_kernel, stream)
+  if (out_mode == OUT_BF16) GO(OUT_BF16);
+  else if (out_mode == OUT_F32) GO(OUT_F32);
+  else GO(OUT_ADD_F32);
+#undef GO
+  if (rc) return rc;
+  HFEE_CHECK_LAUNCH("gemm_bf16");
+  return 0;
+}

@@ -1,0 +1,325 @@
+// Picking the next token on the device: greedy, or temperature sampling with
+// repeat penalty, top-k, top-p and min-p.
+//
+// The rules and their order are the reference's
+// (/root/reference/internal/llm/sampler.go:54-130): repeat penalty on each distinct
+// recent id (logit > 0: divide, else multiply); temperature <= 0: the first maximum;
+// else the top_k largest logits, prob = exp((logit - max) / temperature) normalised,
+// top_p keeps the shortest prefix (in descending order) whose cumulative probability
+// reaches it, min_p cuts what falls below min_p * prob[0], and the draw is
+// proportional to what is kept.
+//
+// Nothing is sorted.  A prefix of the descending order is the set {key > t} plus the
+// first r ties at t (ties taken in ascending id), so each rule becomes a search for
+// its threshold: a radix select on counts for top_k, a bit-by-bit bisection on
+// probability mass for top_p.  All sums run in a fixed order (thread-owned contiguous
+// chunks, then a fixed tree), so a row's result is the same in every batch.
+//
+// The random number is counter based: splitmix64 of (seed, draw index), one stream
+// per request, independent of what else is sampled in the same call.
+#include "common.h"
+
+using namespace hfee;
+
+namespace {
+
+constexpr int THREADS = 1024;
+
+struct SampleParams {          // one per row; 12 x 4 bytes, filled by the host
+  float temperature;
+  int top_k;
+  float top_p;
+  float min_p;
+  float repeat_penalty;
+  int history_offset;          // into the flat history array
+  int history_length;          // ids to penalise (already cut to repeat_last_n)
+  uint32_t seed_lo, seed_hi;
+  uint32_t draw_lo, draw_hi;   // index of this draw in the request's stream
+  int logits_row;
+};
+
+__device__ __forceinline__ uint32_t order_key(float v) {   // larger float <=> larger key
+  const uint32_t b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+__device__ __forceinline__ double uniform_from(uint64_t seed, uint64_t draw) {
+  uint64_t z = seed + (draw + 1) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z ^= z >> 31;
+  return (double)(z >> 11) * (1.0 / 9007199254740992.0);
+}
+
+// Exclusive prefix sums over the block in thread order; *total gets the sum.
+template <typename T>
+__device__ __forceinline__ T block_exclusive_scan(T v, T* wave_totals, T* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  T incl = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const T up = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += up;
+  }
+  __syncthreads();
+  if (lane == 63) wave_totals[wave] = incl;
+  __syncthreads();
+  T before = 0, all = 0;
+  for (int w = 0; w < THREADS / 64; ++w) {
+    const T wt = wave_totals[w];
+    if (w < wave) before += wt;
+    all += wt;
+  }
+  *total = all;
+  return before + incl - v;
+}
+
+struct MaxIdx {
+  float v;
+  int i;
+};
+
+__device__ __forceinline__ MaxIdx better(MaxIdx a, MaxIdx b) {   // greater value, then smaller id
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+  return a;
+}
+
+__device__ MaxIdx block_argmax(const float* __restrict__ lg, int V, MaxIdx* scratch) {
+  MaxIdx best{-INFINITY, 0x7fffffff};
+  for (int j = threadIdx.x; j < V; j += blockDim.x) {
+    const float v = lg[j];
+    if (v > best.v) best = MaxIdx{v, j};   // ascending j per thread: strict '>' keeps the first
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    MaxIdx o{__shfl_xor(best.v, off, 64), __shfl_xor(best.i, off, 64)};
+    best = better(best, o);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = best;
+  __syncthreads();
+  MaxIdx r = scratch[0];
+  for (int w = 1; w < (int)(blockDim.x + 63) / 64; ++w) r = better(r, scratch[w]);
+  if (r.i == 0x7fffffff) r.i = 0;   // every logit is NaN or -inf
+  return r;
+}
+
+__global__ __launch_bounds__(THREADS) void argmax_kernel(int* __restrict__ out, const float* __restrict__ logits,
+                                                         int64_t ld, int V) {
+  __shared__ MaxIdx scratch[16];
+  const MaxIdx r = block_argmax(logits + (int64_t)blockIdx.x * ld, V, scratch);
+  if (threadIdx.x == 0) out[blockIdx.x] = r.i;
+}
+
+__global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, float* __restrict__ logits,
+                                                         int64_t ld, int V, const SampleParams* __restrict__ params,
+                                                         const int* __restrict__ history,
+                                                         float* __restrict__ scratch, int64_t ld_scratch) {
+  extern __shared__ uint32_t bits[];            // (V + 31) / 32 words, used by the repeat penalty
+  __shared__ MaxIdx mscratch[16];
+  __shared__ float fscratch[16];
+  __shared__ int iscratch[16];
+  __shared__ int hist[256];
+  __shared__ uint32_t sh_prefix;
+  __shared__ int sh_need;
+
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const SampleParams p = params[row];
+  float* lg = logits + (int64_t)p.logits_row * ld;
+  float* q = scratch + (int64_t)row * ld_scratch;
+
+  // ---- repeat penalty (sampler.go:57-74)
+  if (p.repeat_penalty != 1.0f && p.history_length > 0) {
+    const int words = (V + 31) / 32;
+    for (int w = tid; w < words; w += THREADS) bits[w] = 0u;
+    __syncthreads();
+    for (int i = tid; i < p.history_length; i += THREADS) {
+      const int id = history[p.history_offset + i];
+      if (id >= 0 && id < V) atomicOr(&bits[id >> 5], 1u << (id & 31));
+    }
+    __syncthreads();
+    for (int j = tid; j < V; j += THREADS) {
+      if (bits[j >> 5] & (1u << (j & 31))) {
+        const float v = lg[j];
+        lg[j] = v > 0.f ? v / p.repeat_penalty : v * p.repeat_penalty;
+      }
+    }
+    __threadfence_block();
+    __syncthreads();
+  }
+
+  // ---- greedy (sampler.go:76-84)
+  const MaxIdx top = block_argmax(lg, V, mscratch);
+  if (p.temperature <= 0.f) {
+    if (tid == 0) out[row] = top.i;
+    return;
+  }
+
+  // ---- top_k: key of the k-th largest and how many of its ties belong (sampler.go:132-151)
+  uint32_t t_k = 0u;
+  int r_k = 0x7fffffff;
+  if (p.top_k > 0 && p.top_k < V) {
+    if (tid == 0) { sh_prefix = 0u; sh_need = p.top_k; }
+    uint32_t mask = 0u;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      for (int b = tid; b < 256; b += THREADS) hist[b] = 0;
+      __syncthreads();
+      const uint32_t prefix = sh_prefix;
+      for (int j = tid; j < V; j += THREADS) {
+        const uint32_t key = order_key(lg[j]);
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        int need = sh_need, b = 255;
+        for (; b > 0; --b) {
+          if (hist[b] >= need) break;
+          need -= hist[b];
+        }
+        sh_need = need;
+        sh_prefix = prefix | ((uint32_t)b << shift);
+      }
+      mask |= 255u << shift;
+      __syncthreads();
+    }
+    t_k = sh_prefix;
+    r_k = sh_need;
+  }
+
+  // ---- probabilities of the top_k set, in q (sampler.go:88-96); thread-owned chunks
+  const int chunk = (V + THREADS - 1) / THREADS;
+  const int j0 = min(V, tid * chunk), j1 = min(V, j0 + chunk);
+  int my_ties = 0;
+  for (int j = j0; j < j1; ++j) my_ties += order_key(lg[j]) == t_k;
+  int all_ties;
+  int tie_rank = block_exclusive_scan<int>(my_ties, iscratch, &all_ties);
+  float my_mass = 0.f;
+  for (int j = j0; j < j1; ++j) {
+    const float v = lg[j];
+    const uint32_t key = order_key(v);
+    bool in = key > t_k;
+    if (key == t_k) in = tie_rank++ < r_k;
+    const float e = in ? expf((v - top.v) / p.temperature) : 0.f;
+    q[j] = e;
+    my_mass += e;
+  }
+  __threadfence_block();
+  float Z;
+  block_exclusive_scan<float>(my_mass, fscratch, &Z);
+
+  // ---- top_p: threshold key and how many of its ties belong (sampler.go:98-108)
+  uint32_t t_p = 0u;
+  int r_p = 0x7fffffff;
+  if (p.top_p > 0.f && p.top_p < 1.f) {
+    const float target = p.top_p * Z;
+    uint32_t t = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t cand = t | (1u << bit);
+      float mass = 0.f;
+      for (int j = j0; j < j1; ++j) mass += order_key(lg[j]) >= cand ? q[j] : 0.f;
+      float total;
+      block_exclusive_scan<float>(mass, fscratch, &total);
+      if (total >= target) t = cand;
+    }
+    t_p = t;
+    float above = 0.f, tie_p = 0.f;
+    for (int j = j0; j < j1; ++j) {
+      const uint32_t key = order_key(lg[j]);
+      if (key > t_p) above += q[j];
+      else if (key == t_p && q[j] > 0.f) tie_p = q[j];
+    }
+    float mass_above;
+    block_exclusive_scan<float>(above, fscratch, &mass_above);
+    tie_p = block_max(tie_p, fscratch);
+    r_p = tie_p > 0.f ? max(1, (int)ceilf((target - mass_above) / tie_p)) : 1;
+  }
+
+  // ---- min_p and the kept set (sampler.go:109-116), then the draw (sampler.go:118-129)
+  int my_pties = 0;
+  for (int j = j0; j < j1; ++j) my_pties += (order_key(lg[j]) == t_p && q[j] > 0.f);
+  int all_pties;
+  int ptie_rank = block_exclusive_scan<int>(my_pties, iscratch, &all_pties);
+  float my_keep = 0.f;
+  int my_last = -1;
+  for (int j = j0; j < j1; ++j) {
+    const uint32_t key = order_key(lg[j]);
+    float w = q[j];
+    if (w > 0.f) {
+      bool in = key > t_p;
+      if (key == t_p) in = ptie_rank++ < r_p;
+      if (p.min_p > 0.f && w < p.min_p && j != top.i) in = false;
+      if (!in) w = 0.f;
+    }
+    q[j] = w;
+    if (w > 0.f) my_last = j;
+    my_keep += w;
+  }
+  __threadfence_block();
+  float total;
+  const float before = block_exclusive_scan<float>(my_keep, fscratch, &total);
+  const uint64_t seed = ((uint64_t)p.seed_hi << 32) | p.seed_lo;
+  const uint64_t draw = ((uint64_t)p.draw_hi << 32) | p.draw_lo;
+  const float r = (float)(uniform_from(seed, draw) * (double)total);
+
+    __shared__ int sh_choice;
+  if (tid == 0) sh_choice = 0x7fffffff;
+  __syncthreads();
+  if (my_keep > 0.f && (before < r || r <= 0.f)) {
+    // every chunk that starts below r walks; the smallest id whose running sum
+    // reaches r wins, whatever rounding does to the chunk sums
+    float run = before;
+    for (int j = j0; j < j1; ++j) {
+      if (q[j] <= 0.f) continue;
+      run += q[j];
+      if (run >= r) { atomicMin(&sh_choice, j); break; }
+    }
+  }
+  __syncthreads();
+  if (sh_choice == 0x7fffffff) {
+    // rounding left r above every running sum: the last kept id (sampler.go:129)
+    int last = my_last;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off, 64));
+    if ((tid & 63) == 0) iscratch[tid >> 6] = last;
+    __syncthreads();
+    if (tid == 0) {
+      int l = -1;
+      for (int w = 0; w < THREADS / 64; ++w) l = max(l, iscratch[w]);
+      sh_choice = l < 0 ? top.i : l;
+    }
+    __syncthreads();
+  }
+  if (tid == 0) out[row] = sh_choice;
+}
+
+}  // namespace
+
+HFEE_API int hfee_argmax(int* out, const float* logits, int64_t ld, int rows, int V, hipStream_t stream) {
+  HFEE_REQUIRE(rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d", rows, V);
+  if (rows == 0) return 0;
+  argmax_kernel<<<rows, THREADS, 0, stream>>>(out, logits, ld, V);
+  HFEE_CHECK_LAUNCH("argmax");
+  return 0;
+}
+
+// params: rows x 12 32-bit words (SampleParams).  logits may be changed in place by
+// the repeat penalty, as the reference changes them.  scratch: rows x ld_scratch floats.
+HFEE_API int hfee_sample(int* out, float* logits, int64_t ld, int rows, int V, const void* params,
+                         const int* history, float* scratch, int64_t ld_scratch, hipStream_t stream) {
+  HFEE_REQUIRE(rows >= 0 && V > 0 && ld >= V && ld_scratch >= V, "sample: bad sizes rows=%d V=%d", rows, V);
+  if (rows == 0) return 0;
+  const size_t lds = (size_t)((V + 31) / 32) * 4;
+  HFEE_REQUIRE(lds <= 96 * 1024, "sample: a vocabulary of %d ids does not fit the penalty's bit set", V);
+  static bool raised = false;
+  if (lds > 32 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)sample_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       96 * 1024);
+    HFEE_REQUIRE(e == hipSuccess, "sample: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  sample_kernel<<<rows, THREADS, lds, stream>>>(out, logits, ld, V, (const SampleParams*)params, history,
+                                                scratch, ld_scratch);
+  HFEE_CHECK_LAUNCH("sample");
+  return 0;
+}

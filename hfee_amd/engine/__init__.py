@@ -1,0 +1,2 @@
+from .model import Model, EngineInfo, load_model, random_model, declared_tensors
+from .step import Engine, StepEntry, StepPlan, StepError

@@ -1,0 +1,228 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+It is the reference's Model.Forward (/root/reference/internal/llm/forward.go:41-142):
+every entry brings any number >= 1 of consecutive new tokens of one sequence,
+starting at that sequence's cached length; portions of prompts sit beside single
+decoded tokens; all rows run through the layers together; keys and values go to the
+cache; the final norm and the head run only for the rows whose logits are wanted.
+Unlike the reference, logits can be asked for at any of an entry's tokens, not only
+its last, and the cache is paged.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager, CacheStorage, OutOfPages
+from ..parts.base import Segment, StepContext, Workspace
+from .model import EngineInfo, Model
+
+
+@dataclass
+class StepEntry:
+    request_id: object
+    tokens: list
+    want: list = field(default_factory=list)    # indices into `tokens` whose logits are wanted
+
+
+class StepError(ValueError):
+    """The batch breaks the step function's contract."""
+
+
+class StepPlan:
+    """Host side of a step: the segments and every int32 array that goes to the device."""
+
+    def __init__(self, segments):
+        self.segments = segments
+        self.arrays: dict = {}
+        self.host: dict = {}
+
+    def add(self, key: str, array: np.ndarray):
+        if key in self.arrays:
+            raise StepError(f"step metadata {key!r} is planned twice")
+        self.arrays[key] = np.ascontiguousarray(array, dtype=np.int32)
+
+
+class Engine:
+    """Model + cache + workspace on one GPU, and step()."""
+
+    def __init__(self, model: Model, *, num_pages=None, cache_tokens=None, page_size: int = 16,
+                 max_requests: int = 64, max_batch_tokens: int = 2048, num_positions: int | None = None,
+                 device="cuda:0"):
+        if not model.bound:
+            raise ValueError("the model has no weights bound")
+        if not torch.cuda.is_available():
+            raise RuntimeError("hfee_amd runs on a GPU only; no GPU is visible")
+        self.model, self.dtype, self.device = model, model.dtype, torch.device(device)
+        self.page_size = page_size
+        self.max_requests = max_requests
+        self.max_batch_tokens = max_batch_tokens
+        self.num_positions = min(num_positions or model.spec.max_positions, model.spec.max_positions)
+        self.vocab = model.spec.vocab
+        self.groups = model.cache_groups()
+        if num_pages is None:
+            if cache_tokens is None:
+                cache_tokens = self.num_positions * max_requests
+            num_pages = (cache_tokens + page_size - 1) // page_size
+        self.num_pages = num_pages
+        self.cache = CacheManager(self.groups, page_size, num_pages, max_requests)
+        self.storage = CacheStorage(self.groups, page_size, num_pages, max_requests, self.dtype, self.device)
+        self.workspace = Workspace(max_batch_tokens, self.device)
+        info = EngineInfo(self.num_positions, self.device, self.dtype, page_size, max_requests, self.storage)
+        for m in model.mixers():
+            for name, shape, dt in m.state_specs():
+                self.storage.add_state(name, shape, dt)
+        model.prepare(info)
+        self._meta_capacity = 0
+        self._meta_ring, self._meta_device = [], None
+        self.steps_run = 0
+
+    # ------------------------------------------------------------ requests
+    def admit(self, request_id):
+        rc = self.cache.admit(request_id)
+        self.storage.clear_slot(rc.slot)
+        return rc
+
+    def release(self, request_id):
+        self.cache.release(request_id)
+
+    def is_live(self, request_id) -> bool:
+        return request_id in self.cache.requests
+
+    def cached_length(self, request_id) -> int:
+        return self.cache.get(request_id).length
+
+    # ---------------------------------------------------------------- step
+    def _check(self, entries):
+        if not entries:
+            raise StepError("an empty step")
+        seen = set()
+        total = 0
+        for e in entries:
+            if e.request_id in seen:
+                raise StepError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            if len(e.tokens) < 1:
+                raise StepError(f"request {e.request_id!r} brings no tokens")
+            rc = self.cache.get(e.request_id)
+            if rc.length + len(e.tokens) > self.num_positions:
+                raise StepError(f"request {e.request_id!r} would reach position "
+                                f"{rc.length + len(e.tokens) - 1}, the context holds {self.num_positions}")
+            for t in e.tokens:
+                if not 0 <= t < self.vocab:
+                    raise StepError(f"token id {t} is outside the vocabulary of {self.vocab}")
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise StepError(f"request {e.request_id!r} wants logits at {w} of {len(e.tokens)} tokens")
+            total += len(e.tokens)
+        if total > self.max_batch_tokens:
+            raise StepError(f"{total} tokens in one step, the engine was made for {self.max_batch_tokens}")
+
+    def _reserve(self, entries):
+        need = [0] * len(self.groups)
+        for e in entries:
+            for g, k in enumerate(self.cache.pages_needed(e.request_id, len(e.tokens))):
+                need[g] += k
+        free = self.cache.free_pages()
+        for g in range(len(self.groups)):
+            if need[g] > free[g]:
+                raise OutOfPages(f"the step needs {need[g]} pages in cache group {g}, {free[g]} are free")
+        for e in entries:
+            self.cache.reserve(e.request_id, len(e.tokens))
+
+    def _upload(self, plan: StepPlan) -> dict:
+        """All planned arrays in one pinned buffer, one copy to the device."""
+        offsets, total = {}, 0
+        for key, a in plan.arrays.items():
+            offsets[key] = total
+            total += (a.size + 3) // 4 * 4
+        total = max(total, 4)
+        if total > self._meta_capacity:
+            cap = max(total * 2, 4096)
+            # a ring of pinned buffers: the copy of step k may still be in flight
+            # while the host fills the buffer of step k+1
+            self._meta_ring = [(torch.empty(cap, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+                               for _ in range(4)]
+            self._meta_device = torch.empty(cap, dtype=torch.int32, device=self.device)
+            self._meta_capacity = cap
+        pinned, event = self._meta_ring[self.steps_run % len(self._meta_ring)]
+        event.synchronize()
+        host = pinned.numpy()
+        for key, a in plan.arrays.items():
+            host[offsets[key]:offsets[key] + a.size] = a.reshape(-1)
+        self._meta_device[:total].copy_(pinned[:total], non_blocking=True)
+        event.record()
+        out = {}
+        for key, a in plan.arrays.items():
+            out[key] = self._meta_device[offsets[key]:offsets[key] + a.size].view(a.shape)
+        return out
+
+    def step(self, entries) -> torch.Tensor:
+        """Runs the entries as one batch; returns float32 logits [wanted, vocab] in the
+        order of the entries and of each entry's `want` (None if nothing is wanted).
+        The tensor is a view of the workspace: the next step overwrites it."""
+        entries = list(entries)
+        self._check(entries)
+        self._reserve(entries)
+
+        segments, tokens, positions, token_segment, logit_rows = [], [], [], [], []
+        row = 0
+        for s, e in enumerate(entries):
+            rc = self.cache.get(e.request_id)
+            segments.append(Segment(e.request_id, rc.slot, rc.length, len(e.tokens), row))
+            tokens += list(e.tokens)
+            positions += range(rc.length, rc.length + len(e.tokens))
+            token_segment += [s] * len(e.tokens)
+            logit_rows += [row + w for w in e.want]
+            row += len(e.tokens)
+        n = row
+
+        plan = StepPlan(segments)
+        plan.add("token_ids", np.asarray(tokens))
+        plan.add("positions", np.asarray(positions))
+        plan.add("token_segment", np.asarray(token_segment))
+        plan.add("segment_slots", np.asarray([s.slot for s in segments]))
+        plan.add("segment_starts", np.asarray([s.start for s in segments]))
+        plan.add("segment_lengths", np.asarray([s.length for s in segments]))
+        plan.add("segment_rows", np.asarray([s.row0 for s in segments]))
+        plan.add("logit_rows", np.asarray(logit_rows))
+        for g in range(len(self.groups)):
+            tables = [self.cache.block_table(s.request_id, g) for s in segments]
+            width = max(1, max(len(t) for t in tables))
+            bt = np.zeros((len(segments), width), dtype=np.int32)
+            for i, t in enumerate(tables):
+                bt[i, :len(t)] = [max(p, 0) for p in t]   # pages a window has given back are never read
+            plan.add(f"block_tables.{g}", bt)
+        seen = set()
+        for entry in self.model.schedule:
+            mixer = self.model.blocks[entry.layer].mixer
+            if id(mixer) not in seen:
+                seen.add(id(mixer))
+                mixer.plan(plan)
+
+        dev = self._upload(plan)
+        ctx = StepContext(
+            n=n, dtype=self.dtype, device=self.device, segments=segments,
+            token_ids=dev["token_ids"], positions=dev["positions"], token_segment=dev["token_segment"],
+            segment_slots=dev["segment_slots"], segment_starts=dev["segment_starts"],
+            segment_lengths=dev["segment_lengths"], segment_rows=dev["segment_rows"],
+            block_tables=[dev[f"block_tables.{g}"] for g in range(len(self.groups))],
+            max_position=max(positions), storage=self.storage, workspace=self.workspace,
+            page_size=self.page_size, extra=dev, host=plan.host)
+
+        x = self.workspace.rows("residual", n, self.model.spec.hidden, torch.float32)
+        self.model.embedding.forward(ctx, x)
+        for entry in self.model.schedule:
+            self.model.blocks[entry.layer].forward(ctx, x, entry)
+        w = len(logit_rows)
+        logits = None
+        if w:
+            logits = self.workspace.rows("logits", w, self.vocab, torch.float32)
+            self.model.head.forward(ctx, logits, x, dev["logit_rows"])
+
+        for e in entries:
+            self.cache.commit(e.request_id, len(e.tokens))
+        self.steps_run += 1
+        return logits

@@ -1,0 +1,97 @@
+"""Loading the compiled kernel libraries and declaring their entry points.
+
+There is no fallback: if a library cannot be built or loaded, KernelLibraryError
+is raised and nothing runs.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import c_void_p, c_int, c_int64, c_float, c_uint64, c_char_p
+
+from . import build
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+class KernelError(RuntimeError):
+    """An entry point refused its arguments or its launch failed."""
+
+
+P, I, L, F, U64 = c_void_p, c_int, c_int64, c_float, c_uint64
+
+_CORE_SIGNATURES = {
+    "hfee_embed": [P, P, I, P, I, I, P],
+    "hfee_rmsnorm": [P, I, P, P, I, P, F, I, I, P],
+    "hfee_swiglu": [P, L, P, P, L, I, I, I, P],
+    "hfee_residual_add": [P, P, I, L, P],
+    "hfee_rope_cache_write": [P, L, P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, P, I, I, I, I, I, P],
+    "hfee_gemm_f32": [P, L, P, L, P, L, I, I, I, I, P],
+    "hfee_attention_ref": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
+    "hfee_gemm_bf16": [P, I, L, P, L, P, L, I, I, I, I, P],
+    "hfee_argmax": [P, P, L, I, I, P],
+    "hfee_sample": [P, P, L, I, I, P, P, P, L, P],
+}
+
+_ATTENTION_SIGNATURES = {
+    "hfee_attention_bf16_head_dim": [],
+    "hfee_attention_bf16_prefill": [P, L, P, L, P, P, I, P, I, I, I, I, F, I, P],
+    "hfee_attention_bf16_decode": [P, L, P, L, P, P, P, P, I, P, I, I, I, I, F, I, P, L, I, P],
+}
+
+_lock = threading.Lock()
+_loaded: dict[str, "Library"] = {}
+
+
+class Library:
+    def __init__(self, name: str, path: str, signatures: dict):
+        self.name, self.path = name, path
+        try:
+            self._dll = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelLibraryError(f"cannot load kernel library {path}: {e}") from None
+        self._dll.hfee_last_error.restype = c_char_p
+        self._dll.hfee_last_error.argtypes = []
+        for fn, argtypes in signatures.items():
+            try:
+                f = getattr(self._dll, fn)
+            except AttributeError:
+                raise KernelLibraryError(f"kernel library {path} has no entry point {fn}") from None
+            f.argtypes = argtypes
+            f.restype = c_int
+
+    def call(self, fn: str, *args):
+        rc = getattr(self._dll, fn)(*args)
+        if rc != 0:
+            msg = self._dll.hfee_last_error()
+            raise KernelError((msg or b"unknown error").decode("utf-8", "replace"))
+
+    def raw(self, fn: str):
+        return getattr(self._dll, fn)
+
+
+def load(name: str) -> Library:
+    """The named library, built first if no up-to-date build exists."""
+    with _lock:
+        lib = _loaded.get(name)
+        if lib is None:
+            try:
+                path = build.build_library(name)
+            except build.BuildError as e:
+                raise KernelLibraryError(f"the HIP kernel library '{name}' is not available: {e}") from None
+            sigs = _CORE_SIGNATURES if name == "core" else _ATTENTION_SIGNATURES
+            lib = _loaded[name] = Library(name, path, sigs)
+        return lib
+
+
+def core() -> Library:
+    return load("core")
+
+
+def attention_bf16(head_dim: int) -> Library:
+    if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
+        raise KernelError(f"the bfloat16 attention kernels take head sizes 16..256 in steps of 16, "
+                          f"not {head_dim}")
+    return load(f"attention_bf16_hd{head_dim}")

@@ -1,0 +1,270 @@
+"""The operations the parts call.  Each wrapper checks shapes, dtypes and
+contiguity on the host, then launches the HIP kernel on the current stream.
+Tensors are torch tensors on the GPU; torch only provides the memory and the
+stream here, every computation is the library's.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import lib
+from .lib import KernelError
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {t.dtype}") from None
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _check(cond, msg):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("the kernels take GPU tensors; there is no CPU path")
+
+
+def _rows2d(t: torch.Tensor, what: str):
+    """A 2-D tensor whose rows are contiguous: (rows, cols, leading dimension)."""
+    _check(t.dim() == 2 and t.stride(1) == 1, f"{what}: expected a 2-D tensor with contiguous rows")
+    return t.shape[0], t.shape[1], t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _i32(t, what, n=None):
+    _check(t.dtype == torch.int32 and t.is_contiguous(), f"{what}: expected a contiguous int32 tensor")
+    if n is not None:
+        _check(t.numel() >= n, f"{what}: {t.numel()} entries, {n} needed")
+
+
+# ------------------------------------------------------------------ simple ops
+
+def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor):
+    """out[i, :] = table[ids[i], :] as float32."""
+    _gpu(out, table, ids)
+    n, d, _ = _rows2d(out, "embed out")
+    _check(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous float32")
+    _check(table.dim() == 2 and table.is_contiguous() and table.shape[1] == d, "embed: table shape")
+    _i32(ids, "embed ids", n)
+    lib.core().call("hfee_embed", _ptr(out), _ptr(table), _dt(table), _ptr(ids), n, d, _stream())
+
+
+def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None):
+    """out[r] = x[rows[r] or r] / sqrt(mean(x^2) + eps) * weight; x float32."""
+    _gpu(out, x, weight, rows)
+    n, d, _ = _rows2d(out, "rmsnorm out")
+    _check(out.is_contiguous() and x.is_contiguous() and x.dtype == torch.float32, "rmsnorm: contiguous float32 x")
+    _check(x.dim() == 2 and x.shape[1] == d, "rmsnorm: width mismatch")
+    _check(weight.numel() == d and weight.is_contiguous(), "rmsnorm: weight width mismatch")
+    if rows is None:
+        _check(x.shape[0] >= n, "rmsnorm: fewer input rows than output rows")
+    else:
+        _i32(rows, "rmsnorm rows", n)
+    lib.core().call("hfee_rmsnorm", _ptr(out), _dt(out), _ptr(x), _ptr(weight), _dt(weight), _ptr(rows),
+                    float(eps), n, d, _stream())
+
+
+def swiglu(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
+    """out = gate / (1 + exp(-gate)) * up; gate and up share a leading dimension."""
+    _gpu(out, gate, up)
+    n, w, ldo = _rows2d(out, "swiglu out")
+    ng, wg, ldg = _rows2d(gate, "swiglu gate")
+    nu, wu, ldu = _rows2d(up, "swiglu up")
+    _check((ng, wg) == (n, w) and (nu, wu) == (n, w) and ldg == ldu, "swiglu: shape mismatch")
+    _check(out.dtype == gate.dtype == up.dtype, "swiglu: dtype mismatch")
+    lib.core().call("hfee_swiglu", _ptr(out), ldo, _ptr(gate), _ptr(up), ldg, _dt(out), n, w, _stream())
+
+
+def residual_add(x: torch.Tensor, y: torch.Tensor):
+    """x (float32) += y."""
+    _gpu(x, y)
+    _check(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous(), "residual_add: contiguity")
+    _check(x.shape == y.shape, "residual_add: shape mismatch")
+    lib.core().call("hfee_residual_add", _ptr(x), _ptr(y), _dt(y), x.numel(), _stream())
+
+
+# ---------------------------------------------------------------- matrix product
+
+def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate: bool = False, kernel: int = 0):
+    """out (+)= x @ weight.T, weight stored [out_features, in_features].
+
+    float32 x and weight: the true 32-bit product, out float32.
+    bfloat16 x and weight: matrix cores with float32 accumulation; out bfloat16, or
+    float32 (required when accumulating: the residual stream).
+    kernel: 0 automatic, 1 skinny, 2 tiled (bfloat16 only)."""
+    _gpu(out, x, weight)
+    M, K, lda = _rows2d(x, "linear x")
+    N, Kw, ldw = _rows2d(weight, "linear weight")
+    Mo, No, ldc = _rows2d(out, "linear out")
+    _check(Kw == K and Mo == M and No == N, f"linear: shapes x{list(x.shape)} w{list(weight.shape)} out{list(out.shape)}")
+    _check(x.dtype == weight.dtype, "linear: x and weight dtypes differ")
+    if x.dtype == torch.float32:
+        _check(out.dtype == torch.float32, "linear: float32 product needs a float32 out")
+        lib.core().call("hfee_gemm_f32", _ptr(out), ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K,
+                        1 if accumulate else 0, _stream())
+    elif x.dtype == torch.bfloat16:
+        if accumulate:
+            _check(out.dtype == torch.float32, "linear: accumulation needs a float32 out")
+            mode = 2
+        else:
+            mode = 0 if out.dtype == torch.bfloat16 else 1
+            _check(out.dtype in (torch.bfloat16, torch.float32), "linear: out dtype")
+        lib.core().call("hfee_gemm_bf16", _ptr(out), mode, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K,
+                        kernel, _stream())
+    else:
+        raise KernelError(f"linear: unsupported dtype {x.dtype}")
+
+
+# --------------------------------------------------------- rotation and the cache
+
+def rope_cache_write(q, k, v, positions, token_segment, block_tables, cos, sin, pairing: int,
+                     cache_layer, num_heads: int, kv_heads: int, head_dim: int, page_size: int,
+                     max_position: int):
+    """Rotates q in place, writes rotated k and v into the pages of `cache_layer`.
+    q, k, v: 2-D views [n, heads * head_dim] (any leading dimension), or None.
+    cos/sin: [positions, half] float32 or None (no rotation).  cache_layer:
+    [pages, 2, kv_heads, page_size * head_dim] or None (no write)."""
+    _gpu(q, k, v, positions, cos, sin, cache_layer)
+    some = q if q is not None else k
+    _check(some is not None, "rope_cache_write: nothing to do")
+    n = some.shape[0]
+    ldq = ldk = ldv = 0
+    if q is not None:
+        nq, wq, ldq = _rows2d(q, "rope q")
+        _check(nq == n and wq == num_heads * head_dim, "rope: q shape")
+    if k is not None:
+        _check(v is not None and cache_layer is not None, "rope: k, v and the cache come together")
+        nk, wk, ldk = _rows2d(k, "rope k")
+        nv, wv, ldv = _rows2d(v, "rope v")
+        _check(nk == n and nv == n and wk == wv == kv_heads * head_dim, "rope: k/v shape")
+        _check(k.dtype == v.dtype == cache_layer.dtype and (q is None or q.dtype == k.dtype), "rope: dtype mismatch")
+        _check(cache_layer.is_contiguous() and cache_layer.dim() == 4 and
+               tuple(cache_layer.shape[1:]) == (2, kv_heads, page_size * head_dim), "rope: cache layer shape")
+        _i32(token_segment, "rope token_segment", n)
+        _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+               "rope: block tables")
+    _i32(positions, "rope positions", n)
+    half = 0
+    table_positions = 0
+    if cos is not None:
+        _check(cos.shape == sin.shape and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous()
+               and cos.dtype == sin.dtype == torch.float32, "rope: cos/sin tables")
+        table_positions, half = cos.shape
+    lib.core().call("hfee_rope_cache_write", _ptr(q), ldq, _ptr(k), ldk, _ptr(v), ldv, _dt(some),
+                    _ptr(positions), _ptr(token_segment if k is not None else None),
+                    _ptr(block_tables if k is not None else None),
+                    block_tables.stride(0) if k is not None else 0,
+                    _ptr(cos), _ptr(sin), half, pairing, table_positions, max_position,
+                    _ptr(cache_layer if k is not None else None), num_heads, kv_heads, head_dim, page_size,
+                    n, _stream())
+
+
+def attention_plain(out, q, cache_layer, positions, token_segment, block_tables, num_heads: int,
+                    kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0):
+    """One wave per (token, head): the 32-bit path's attention and the slow twin of
+    the matrix-core kernels.  Token t reads keys max(0, pos-window+1)..pos of its
+    segment's pages."""
+    _gpu(out, q, cache_layer, positions, token_segment, block_tables)
+    n, w, ldq = _rows2d(q, "attention q")
+    no, wo, ldo = _rows2d(out, "attention out")
+    _check(no == n and wo == w == num_heads * head_dim, "attention: q/out shape")
+    _check(q.dtype == out.dtype == cache_layer.dtype, "attention: dtype mismatch")
+    _check(cache_layer.is_contiguous() and tuple(cache_layer.shape[1:]) == (2, kv_heads, page_size * head_dim),
+           "attention: cache layer shape")
+    _i32(positions, "attention positions", n)
+    _i32(token_segment, "attention token_segment", n)
+    _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+           "attention: block tables")
+    lib.core().call("hfee_attention_ref", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _dt(q),
+                    _ptr(positions), _ptr(token_segment), _ptr(block_tables), block_tables.stride(0),
+                    num_heads, kv_heads, head_dim, page_size, float(scale), int(window), n, _stream())
+
+
+# ------------------------------------------------------------------- sampling
+
+def argmax(out: torch.Tensor, logits: torch.Tensor):
+    """out[r] = id of the first maximum of logits[r]."""
+    _gpu(out, logits)
+    rows, V, ld = _rows2d(logits, "argmax logits")
+    _check(logits.dtype == torch.float32, "argmax: float32 logits")
+    _i32(out, "argmax out", rows)
+    lib.core().call("hfee_argmax", _ptr(out), _ptr(logits), ld, rows, V, _stream())
+
+
+def sample(out: torch.Tensor, logits: torch.Tensor, params: torch.Tensor, history: torch.Tensor,
+           scratch: torch.Tensor):
+    """out[r] = sampled id for row r; params is [rows, 12] int32 (see sampling/params.py)."""
+    _gpu(out, logits, params, history, scratch)
+    _, V, ld = _rows2d(logits, "sample logits")
+    rows = params.shape[0]
+    _check(logits.dtype == torch.float32 and scratch.dtype == torch.float32, "sample: float32 logits and scratch")
+    _check(params.dtype == torch.int32 and params.is_contiguous() and params.dim() == 2 and params.shape[1] == 12,
+           "sample: params must be [rows, 12] int32")
+    rs, Vs, lds = _rows2d(scratch, "sample scratch")
+    _check(rs >= rows and Vs >= V, "sample: scratch too small")
+    _i32(out, "sample out", rows)
+    _check(history.dtype == torch.int32 and history.is_contiguous(), "sample: history must be int32")
+    lib.core().call("hfee_sample", _ptr(out), _ptr(logits), ld, rows, V, _ptr(params), _ptr(history),
+                    _ptr(scratch), lds, _stream())
+
+
+# ------------------------------------------------- matrix-core attention (bfloat16)
+
+def _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size):
+    _gpu(out, q, cache_layer, block_tables)
+    n, w, ldq = _rows2d(q, "attention q")
+    no, wo, ldo = _rows2d(out, "attention out")
+    _check(no == n and wo == w == num_heads * head_dim, "attention: q/out shape")
+    _check(q.dtype == out.dtype == cache_layer.dtype == torch.bfloat16, "attention: bfloat16 tensors expected")
+    _check(cache_layer.is_contiguous() and tuple(cache_layer.shape[1:]) == (2, kv_heads, page_size * head_dim),
+           "attention: cache layer shape")
+    _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+           "attention: block tables")
+    return n, ldq, ldo
+
+
+def attention_bf16_prefill(out, q, cache_layer, tiles, block_tables, num_heads: int, kv_heads: int,
+                           head_dim: int, page_size: int, scale: float, window: int = 0):
+    """tiles: [num_tiles, 4] int32 (first row, rows <= 32, first position, block-table row)."""
+    n, ldq, ldo = _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size)
+    _check(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
+           "attention: tiles must be [num_tiles, 4] int32")
+    lib.attention_bf16(head_dim).call(
+        "hfee_attention_bf16_prefill", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(tiles),
+        tiles.shape[0], _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, page_size,
+        float(scale), int(window), _stream())
+
+
+def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tables, block_tables,
+                          num_heads: int, kv_heads: int, head_dim: int, page_size: int, scale: float,
+                          window: int, partial, num_splits: int):
+    """One query token per listed segment; keys split over num_splits waves."""
+    n, ldq, ldo = _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size)
+    count = seg_rows.numel()
+    _i32(seg_rows, "attention seg_rows")
+    _i32(seg_positions, "attention seg_positions", count)
+    _i32(seg_tables, "attention seg_tables", count)
+    if num_splits > 1:
+        _check(partial is not None and partial.dtype == torch.float32 and partial.is_contiguous(),
+               "attention: float32 partial buffer expected")
+    lib.attention_bf16(head_dim).call(
+        "hfee_attention_bf16_decode", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(seg_rows),
+        _ptr(seg_positions), _ptr(seg_tables), count, _ptr(block_tables), block_tables.stride(0),
+        num_heads, kv_heads, page_size, float(scale), int(window), _ptr(partial),
+        0 if partial is None else partial.numel(), int(num_splits), _stream())

@@ -1,0 +1,135 @@
+"""Attention over the paged cache, with grouped KV heads and an optional window.
+
+The reference's layer (/root/reference/internal/llm/forward.go:83-107): project to
+q, k, v; rotate q and k at the token's position; write k (rotated) and v to the
+cache; each token attends to the keys of its own sequence up to its position, head
+h reading KV head h // (heads / kv_heads), scores scaled by `scale`; project back
+and add to the residual stream.
+
+The three projections run as one product over the concatenated weight.  In
+bfloat16, portions of prompts go through the tiled matrix-core kernel (tiles of 32
+positions), single decoded tokens through the split-key kernel; in float32 every
+token goes through the plain kernel.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..config.specs import MixerSpec
+from ..kernels import ops
+from ..weights.spec import TensorSpec
+from .base import Mixer, lookup, register_mixer
+
+_TILE = 32            # query rows per workgroup of the prefill kernel
+_DECODE_WAVES = 1024  # waves the decode kernel aims for when it splits the keys
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.hidden = spec.get("hidden")
+        self.num_heads = spec.get("num_heads")
+        self.kv_heads = spec.get("num_kv_heads", self.num_heads)
+        self.head_dim = spec.get("head_dim")
+        self.scale = float(spec.get("scale", self.head_dim ** -0.5))
+        self.window = int(spec.get("window", 0) or 0)
+        if self.num_heads % self.kv_heads:
+            raise ValueError(f"{self.num_heads} heads are not a multiple of {self.kv_heads} kv heads")
+        if dtype == torch.bfloat16 and (self.head_dim % 16 or not 16 <= self.head_dim <= 256):
+            raise ValueError(f"the bfloat16 attention kernels take head sizes 16..256 in steps of 16, "
+                             f"not {self.head_dim}")
+        if self.head_dim > 256:
+            raise ValueError(f"head sizes above 256 are not built, got {self.head_dim}")
+        self.prefix, self.dtype = prefix, dtype
+        self.position = lookup("position", spec.position.kind)(spec.position) if spec.position else None
+        self.q_width = self.num_heads * self.head_dim
+        self.kv_width = self.kv_heads * self.head_dim
+        self.w_qkv = self.w_o = None
+
+    # ---- weights
+    def tensor_specs(self):
+        p = self.prefix
+        return [TensorSpec(p + "q_proj.weight", (self.q_width, self.hidden)),
+                TensorSpec(p + "k_proj.weight", (self.kv_width, self.hidden)),
+                TensorSpec(p + "v_proj.weight", (self.kv_width, self.hidden)),
+                TensorSpec(p + "o_proj.weight", (self.hidden, self.q_width))]
+
+    def bind(self, tensors):
+        p = self.prefix
+        self.w_qkv = torch.cat([tensors.pop(p + "q_proj.weight"), tensors.pop(p + "k_proj.weight"),
+                                tensors.pop(p + "v_proj.weight")], dim=0).contiguous()
+        self.w_o = tensors.pop(p + "o_proj.weight").contiguous()
+
+    # ---- cache
+    def cache_spec(self):
+        return ("window" if self.window > 0 else "full", self.kv_heads, self.head_dim, self.window)
+
+    def prepare(self, info):
+        if self.position is not None:
+            self.position.prepare(info.num_positions, info.device)
+
+    def plan(self, plan):
+        if self.dtype != torch.bfloat16 or "attention.tiles" in plan.arrays:
+            return
+        tiles, d_rows, d_pos, d_tab = [], [], [], []
+        for s, seg in enumerate(plan.segments):
+            if seg.length == 1:
+                d_rows.append(seg.row0)
+                d_pos.append(seg.start)
+                d_tab.append(s)
+            else:
+                for off in range(0, seg.length, _TILE):
+                    tiles.append((seg.row0 + off, min(_TILE, seg.length - off), seg.start + off, s))
+        plan.add("attention.tiles", np.asarray(tiles, dtype=np.int32).reshape(-1, 4))
+        plan.add("attention.decode_rows", np.asarray(d_rows, dtype=np.int32))
+        plan.add("attention.decode_positions", np.asarray(d_pos, dtype=np.int32))
+        plan.add("attention.decode_tables", np.asarray(d_tab, dtype=np.int32))
+        plan.host["attention.decode_max_position"] = max(d_pos) if d_pos else 0
+
+    # ---- the layer
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+        H, K, hd = self.num_heads, self.kv_heads, self.head_dim
+        n = ctx.n
+        group = ctx.storage.group_of(cache_layer)
+        cache = ctx.storage.layer(cache_layer)
+        tables = ctx.block_tables[group]
+        if writes_cache:
+            qkv = ctx.rows("attention.qkv", self.q_width + 2 * self.kv_width)
+            ops.linear(qkv, h, self.w_qkv)
+            q = qkv[:, :self.q_width]
+            k = qkv[:, self.q_width:self.q_width + self.kv_width]
+            v = qkv[:, self.q_width + self.kv_width:]
+        else:   # this run of the layer reads keys and values that another run wrote
+            q = ctx.rows("attention.qkv", self.q_width + 2 * self.kv_width)[:, :self.q_width]
+            ops.linear(q, h, self.w_qkv[:self.q_width])
+            k = v = None
+        pos = self.position
+        ops.rope_cache_write(q, k, v, ctx.positions, ctx.token_segment, tables,
+                             pos.cos if pos else None, pos.sin if pos else None, pos.pairing if pos else 0,
+                             cache if writes_cache else None, H, K, hd, ctx.page_size, ctx.max_position)
+        att = ctx.rows("attention.out", self.q_width)
+        if self.dtype == torch.float32:
+            ops.attention_plain(att, q, cache, ctx.positions, ctx.token_segment, tables, H, K, hd,
+                                ctx.page_size, self.scale, self.window)
+        else:
+            tiles = ctx.extra["attention.tiles"]
+            if tiles.shape[0]:
+                ops.attention_bf16_prefill(att, q, cache, tiles, tables, H, K, hd, ctx.page_size,
+                                           self.scale, self.window)
+            rows = ctx.extra["attention.decode_rows"]
+            if rows.numel():
+                nseg = rows.numel()
+                span = ctx.host["attention.decode_max_position"] + 1
+                if self.window > 0:
+                    span = min(span, self.window + _TILE)
+                key_tiles = (span + _TILE - 1) // _TILE
+                splits = max(1, min(key_tiles, _DECODE_WAVES // max(1, nseg * K)))
+                splits = ctx.host.get("attention.decode_splits", splits)
+                partial = None
+                if splits > 1:
+                    partial = ctx.workspace.flat("attention.partial", nseg * H * splits * (hd + 2), torch.float32)
+                ops.attention_bf16_decode(att, q, cache, rows, ctx.extra["attention.decode_positions"],
+                                          ctx.extra["attention.decode_tables"], tables, H, K, hd,
+                                          ctx.page_size, self.scale, self.window, partial, splits)
+        ops.linear(x, att, self.w_o, accumulate=True)

@@ -1,0 +1,167 @@
+"""What every part has in common: how it names its tensors, how it is registered,
+and what a step hands it.
+
+A part gets all its sizes and constants through its spec; it never learns which
+model it is in.  Five kinds, each with a registry from the spec's `kind` string to
+a class:
+
+  norm            forward(ctx, out, x, rows=None)
+  position        prepare(num_positions, device); applied by the mixer that owns it
+  mixer           forward_add(ctx, x, h, cache_layer, writes_cache): x += mix(h)
+  feed_forward    forward_add(ctx, x, h):                            x += ffn(h)
+  block           forward(ctx, x, entry): one layer's arrangement of the above
+
+`x` is the residual stream, float32 [n, hidden]; `h` is a normed copy in the
+engine's dtype.  Every part also has tensor_specs() -> [TensorSpec] and
+bind(tensors) (take your tensors out of the dict by full name).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Optional
+
+import torch
+
+from ..weights.spec import TensorSpec
+
+_REGISTRIES: dict[str, dict] = {"norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}}
+
+
+def _register(family: str, kind: str, cls):
+    _REGISTRIES[family][kind] = cls
+    return cls
+
+
+def register_norm(kind: str, cls=None):
+    return _register("norm", kind, cls) if cls else (lambda c: _register("norm", kind, c))
+
+
+def register_position(kind: str, cls=None):
+    return _register("position", kind, cls) if cls else (lambda c: _register("position", kind, c))
+
+
+def register_mixer(kind: str, cls=None):
+    return _register("mixer", kind, cls) if cls else (lambda c: _register("mixer", kind, c))
+
+
+def register_feed_forward(kind: str, cls=None):
+    return _register("feed_forward", kind, cls) if cls else (lambda c: _register("feed_forward", kind, c))
+
+
+def register_block(kind: str, cls=None):
+    return _register("block", kind, cls) if cls else (lambda c: _register("block", kind, c))
+
+
+def lookup(family: str, kind: str):
+    try:
+        return _REGISTRIES[family][kind]
+    except KeyError:
+        known = ", ".join(sorted(_REGISTRIES[family])) or "none"
+        raise KeyError(f"no {family} part is registered under {kind!r} (known: {known})") from None
+
+
+class Part:
+    """Base of all parts."""
+
+    def tensor_specs(self) -> list:
+        return []
+
+    def bind(self, tensors: dict) -> None:
+        pass
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a sequence."""
+
+    def cache_spec(self):
+        """None, or (kind, kv_heads, head_dim, window): the growing memory one
+        cache layer of this mixer needs ("full" or "window")."""
+        return None
+
+    def state_specs(self) -> list:
+        """Per-request states of fixed size: [(name, shape, dtype)]."""
+        return []
+
+    def prepare(self, engine_info) -> None:
+        """Called once before the first step (tables, state tensors...)."""
+
+    def plan(self, plan) -> None:
+        """Called once per step before the metadata goes to the device; may add
+        int32 arrays with plan.add(key, array) (shared by parts that use one key)."""
+
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward_add(self, ctx, x, h) -> None:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(self, ctx, out, x, rows=None) -> None:
+        raise NotImplementedError
+
+
+@dataclass
+class Segment:
+    """One request's share of a step (host side)."""
+    request_id: object
+    slot: int        # state slot
+    start: int       # tokens already in the cache
+    length: int      # new tokens in this step
+    row0: int        # first row of the segment in the flattened batch
+
+
+class Workspace:
+    """Scratch buffers by name, allocated once for `capacity` rows and reused by
+    every step (the reference allocates its scratch per call,
+    /root/reference/internal/llm/forward.go:66-73)."""
+
+    def __init__(self, capacity: int, device):
+        self.capacity = capacity
+        self.device = device
+        self._buffers: dict = {}
+
+    def rows(self, name: str, n: int, width: int, dtype: torch.dtype) -> torch.Tensor:
+        """A [n, width] view of the buffer `name` ([capacity, width])."""
+        if n > self.capacity:
+            raise ValueError(f"a step of {n} tokens exceeds the workspace of {self.capacity}")
+        key = (name, width, dtype)
+        buf = self._buffers.get(key)
+        if buf is None:
+            buf = self._buffers[key] = torch.empty((self.capacity, width), dtype=dtype, device=self.device)
+        return buf[:n]
+
+    def flat(self, name: str, count: int, dtype: torch.dtype) -> torch.Tensor:
+        key = (name, "flat", dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < count:
+            buf = self._buffers[key] = torch.empty((count,), dtype=dtype, device=self.device)
+        return buf[:count]
+
+
+@dataclass
+class StepContext:
+    """What a step hands to the parts.  Device tensors are int32."""
+    n: int
+    dtype: torch.dtype
+    device: object
+    segments: list                      # of Segment (host)
+    token_ids: torch.Tensor             # [n]
+    positions: torch.Tensor             # [n] absolute position of each token
+    token_segment: torch.Tensor         # [n] index of the token's segment
+    segment_slots: torch.Tensor         # [segments] state slot of each segment
+    segment_starts: torch.Tensor        # [segments] tokens cached before this step
+    segment_lengths: torch.Tensor       # [segments]
+    segment_rows: torch.Tensor          # [segments] first row in the batch
+    block_tables: list                  # per cache group: [segments, blocks] page ids
+    max_position: int                   # largest position in the step (host)
+    storage: object                     # CacheStorage
+    workspace: Workspace
+    page_size: int
+    extra: dict = field(default_factory=dict)   # arrays that parts planned: key -> device tensor
+    host: dict = field(default_factory=dict)    # host-side values that parts planned
+
+    def rows(self, name: str, width: int, dtype: Optional[torch.dtype] = None, n: Optional[int] = None):
+        return self.workspace.rows(name, self.n if n is None else n, width, dtype or self.dtype)

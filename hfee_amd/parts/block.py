@@ -1,0 +1,42 @@
+"""How a layer's parts are arranged around the residual stream.
+
+"prenorm" is the reference's block (/root/reference/internal/llm/forward.go:79-115):
+x += mixer(norm(x)); x += feed_forward(norm(x)).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.specs import LayerSpec
+from .base import Part, lookup, register_block
+
+
+@register_block("prenorm")
+class PreNormBlock(Part):
+    def __init__(self, spec: LayerSpec, dtype: torch.dtype):
+        self.spec, self.dtype = spec, dtype
+        self.mixer_norm = lookup("norm", spec.mixer_norm.kind)(
+            spec.mixer_norm, spec.name_of("mixer_norm", "mixer_norm.") + "weight")
+        self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, spec.name_of("mixer", "mixer."), dtype)
+        self.feed_forward_norm = lookup("norm", spec.feed_forward_norm.kind)(
+            spec.feed_forward_norm, spec.name_of("feed_forward_norm", "feed_forward_norm.") + "weight")
+        self.feed_forward = lookup("feed_forward", spec.feed_forward.kind)(
+            spec.feed_forward, spec.name_of("feed_forward", "feed_forward."), dtype)
+        self.hidden = spec.hidden
+
+    def parts(self):
+        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+
+    def tensor_specs(self):
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors):
+        for p in self.parts():
+            p.bind(tensors)
+
+    def forward(self, ctx, x, entry):
+        h = ctx.rows("block.normed", self.hidden)
+        self.mixer_norm.forward(ctx, h, x)
+        self.mixer.forward_add(ctx, x, h, entry.cache, entry.writes_cache)
+        self.feed_forward_norm.forward(ctx, h, x)
+        self.feed_forward.forward_add(ctx, x, h)

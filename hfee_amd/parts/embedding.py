@@ -1,0 +1,54 @@
+"""Token embedding and the output head.
+
+Embedding: a row gather into the float32 residual stream, no scaling
+(/root/reference/internal/llm/forward.go:75-77).  Head: final norm and the
+vocabulary product only for the rows whose logits are wanted
+(/root/reference/internal/llm/forward.go:117-141); it shares the embedding table
+when the model has no separate head (/root/reference/internal/llm/model.go:118-121).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.spec import TensorSpec
+from .base import Part
+
+
+class Embedding(Part):
+    def __init__(self, name: str, vocab: int, hidden: int):
+        self.name, self.vocab, self.hidden = name, vocab, hidden
+        self.table = None
+
+    def tensor_specs(self):
+        return [TensorSpec(self.name, (self.vocab, self.hidden))]
+
+    def bind(self, tensors):
+        self.table = tensors[self.name].contiguous()
+
+    def forward(self, ctx, x):
+        ops.embed(x, self.table, ctx.token_ids)
+
+
+class Head(Part):
+    def __init__(self, norm, name, vocab: int, hidden: int, embedding: Embedding, dtype: torch.dtype):
+        self.norm, self.name, self.vocab, self.hidden = norm, name, vocab, hidden
+        self.embedding, self.dtype = embedding, dtype
+        self.weight = None
+
+    def tensor_specs(self):
+        specs = self.norm.tensor_specs()
+        if self.name is not None:
+            specs.append(TensorSpec(self.name, (self.vocab, self.hidden)))
+        return specs
+
+    def bind(self, tensors):
+        self.norm.bind(tensors)
+        self.weight = tensors[self.name].contiguous() if self.name is not None else self.embedding.table
+
+    def forward(self, ctx, logits, x, rows):
+        """logits[i] = head(norm(x[rows[i]])); logits float32 [len(rows), vocab]."""
+        w = logits.shape[0]
+        normed = ctx.rows("head.normed", self.hidden, n=w)
+        self.norm.forward(ctx, normed, x, rows)
+        ops.linear(logits, normed, self.weight)

@@ -1,0 +1,24 @@
+"""RMSNorm (/root/reference/internal/ggml/ops.go:124-134): y = x / sqrt(mean(x^2) + eps) * w,
+the sum in float32, x the float32 residual stream, y in the engine's dtype."""
+from __future__ import annotations
+
+from ..config.specs import NormSpec
+from ..kernels import ops
+from ..weights.spec import TensorSpec
+from .base import Norm, register_norm
+
+
+@register_norm("rmsnorm")
+class RMSNorm(Norm):
+    def __init__(self, spec: NormSpec, name: str):
+        self.width, self.eps, self.name = spec.width, spec.eps, name
+        self.weight = None
+
+    def tensor_specs(self):
+        return [TensorSpec(self.name, (self.width,), role="vector", init=("one_plus_normal",))]
+
+    def bind(self, tensors):
+        self.weight = tensors[self.name]
+
+    def forward(self, ctx, out, x, rows=None):
+        ops.rmsnorm(out, x, self.weight, self.eps, rows)

@@ -1,0 +1,122 @@
+"""Trace replay: feeds given token ids through the engine step by step and writes
+the logits that are asked for.  Nothing is sampled.  It drives the same model,
+step function, cache and kernels that generation uses.
+
+The closest thing in the reference is State.Forward, which appends tokens and
+returns the last logits (/root/reference/internal/llm/forward.go:36-39).
+
+Input: one JSON object per line,
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+Output: for a step in which something is wanted, <out>/<step>.f32 holds the logits
+at the wanted places as little-endian float32 [wanted, vocab], in the order of the
+entries and of `want`.  After every step a line `done <step>` is printed.
+"""
+from __future__ import annotations
+
+import json
+import os
+import sys
+
+import numpy as np
+
+
+def _split(entries, limit):
+    """Cuts a step that is larger than the workspace into consecutive steps."""
+    from .engine import StepEntry
+    steps, current, room = [], [], limit
+    for e in entries:
+        tokens, want, offset = list(e.tokens), sorted(set(e.want)), 0
+        while offset < len(tokens):
+            take = min(room, len(tokens) - offset)
+            current.append(StepEntry(e.request_id, tokens[offset:offset + take],
+                                     [w - offset for w in want if offset <= w < offset + take]))
+            offset += take
+            room -= take
+            if room == 0:
+                steps.append(current)
+                current, room = [], limit
+    if current:
+        steps.append(current)
+    return steps
+
+
+class Replayer:
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16,
+                 max_requests: int = 8, device: str = "cuda:0"):
+        from .engine import Engine, load_model
+        model, _ = load_model(model_dir, dtype, device)
+        page = page_size
+        tokens = max(max_tokens, 64)
+        self.batch_limit = min(tokens, 8192)
+        self.engine = Engine(model, num_pages=(tokens + page - 1) // page, page_size=page,
+                             max_requests=max_requests, max_batch_tokens=self.batch_limit,
+                             num_positions=min(tokens, model.spec.max_positions), device=device)
+
+    def step(self, entries, end=()):
+        """entries: [(id, tokens, want)]; returns float32 numpy [wanted, vocab] or None.
+        `want` order within an entry is kept."""
+        from .engine import StepEntry
+        ents = []
+        for rid, tokens, want in entries:
+            if not self.engine.is_live(rid):
+                self.engine.admit(rid)
+            ents.append(StepEntry(rid, list(tokens), list(want)))
+        total = sum(len(e.tokens) for e in ents)
+        if total <= self.batch_limit:
+            logits = self.engine.step(ents)
+            out = None if logits is None else logits.cpu().numpy()
+        else:
+            # rows come back entry by entry, ascending within an entry; put them in `want` order
+            parts = {}
+            for sub in _split(ents, self.batch_limit):
+                logits = self.engine.step(sub)
+                if logits is None:
+                    continue
+                rows = logits.cpu().numpy()
+                i = 0
+                for e in sub:
+                    for _ in e.want:
+                        parts.setdefault(e.request_id, []).append(rows[i].copy())
+                        i += 1
+            out_rows = []
+            for e in ents:
+                order = sorted(set(e.want))
+                got = dict(zip(order, parts.get(e.request_id, [])))
+                out_rows += [got[w] for w in e.want]
+            out = np.stack(out_rows) if out_rows else None
+        for rid in end:
+            if self.engine.is_live(rid):
+                self.engine.release(rid)
+        return out
+
+
+def main(argv=None) -> int:
+    import argparse
+    ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="most tokens that live requests hold at any time (the cache pool is made for it)")
+    ap.add_argument("--page-size", type=int, default=16)
+    args = ap.parse_args(argv)
+    os.makedirs(args.out, exist_ok=True)
+    rep = Replayer(args.model, args.dtype, args.max_tokens, page_size=args.page_size)
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        rec = json.loads(line)
+        entries = [(e["id"], e["tokens"], e.get("want", [])) for e in rec.get("entries", [])]
+        step = rec["step"]
+        out = rep.step(entries, rec.get("end", [])) if entries else None
+        if not entries:
+            for rid in rec.get("end", []):
+                if rep.engine.is_live(rid):
+                    rep.engine.release(rid)
+        if out is not None:
+            tmp = os.path.join(args.out, f".{step}.f32.tmp")
+            out.astype("<f4").tofile(tmp)
+            os.replace(tmp, os.path.join(args.out, f"{step}.f32"))
+        print(f"done {step}", flush=True)
+    return 0

@@ -1,0 +1,252 @@
+"""A plain, slow implementation of the Llama dense decoder: whole sequences, no
+cache, no batching, one function per part, written from the reference's formulas.
+It shares no code with hfee_amd (it reads config.json and the safetensors file
+through the `json` and `safetensors` libraries itself).
+
+All arithmetic is float64 by default: the reference computes in float32 with
+float64 in the spots named below, so float64 throughout differs from it by
+float32 rounding only and serves both the 32-bit and the bfloat16 comparison.
+"""
+from __future__ import annotations
+
+import json
+import math
+import os
+
+import torch
+
+F64 = torch.float64
+
+
+# ---------------------------------------------------------------- parts -----
+
+def plain_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """/root/reference/internal/ggml/ops.go:124-134: ss = sum x^2 (float64);
+    scale = 1/sqrt(ss/len + eps); y = x * scale * weight.  eps is inside the
+    square root, added to the mean."""
+    x = x.to(F64)
+    ss = (x * x).sum(dim=-1, keepdim=True)
+    scale = 1.0 / torch.sqrt(ss / x.shape[-1] + float(eps))
+    return x * scale * weight.to(F64)
+
+
+def plain_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """/root/reference/internal/ggml/ops.go:54-71: out[t, r] = W[r, :] . x[t, :],
+    W stored [out, in]."""
+    return x.to(F64) @ w.to(F64).t()
+
+
+def plain_rope_frequencies(head_dim: int, theta: float, scaling=None) -> torch.Tensor:
+    """/root/reference/internal/llm/model.go:150-158: inv_freq[i] = 1/theta^(2i/dim),
+    divided by a per-dimension factor when the file brings one.  The llama3 rule
+    that makes those factors from config.json's rope_scaling: wavelengths shorter
+    than N0/high keep their frequency, longer than N0/low are divided by `factor`,
+    between the two the result slides linearly in N0/wavelength."""
+    half = head_dim // 2
+    inv = [1.0 / math.pow(theta, (2 * i) / head_dim) for i in range(half)]
+    if scaling is not None:
+        factor = float(scaling["factor"])
+        lo = float(scaling["low_freq_factor"])
+        hi = float(scaling["high_freq_factor"])
+        n0 = float(scaling["original_max_position_embeddings"])
+        out = []
+        for f in inv:
+            wavelen = 2 * math.pi / f
+            if wavelen < n0 / hi:
+                out.append(f)
+            elif wavelen > n0 / lo:
+                out.append(f / factor)
+            else:
+                s = (n0 / wavelen - lo) / (hi - lo)
+                out.append((1 - s) * f / factor + s * f)
+        inv = out
+    return torch.tensor(inv, dtype=F64)
+
+
+def plain_rope(x: torch.Tensor, positions, inv_freq: torch.Tensor, pairing: str = "half") -> torch.Tensor:
+    """/root/reference/internal/llm/forward.go:180-196.  x: [T, heads, head_dim].
+    For i < half: angle = pos * inv_freq[i]; pair (a, b) = (i, i+half) ("half") or
+    (2i, 2i+1) ("interleaved"); x[a] <- x[a] cos - x[b] sin; x[b] <- x[a] sin + x[b] cos."""
+    x = x.to(F64).clone()
+    T, _, hd = x.shape
+    half = inv_freq.numel()
+    pos = torch.as_tensor(positions, dtype=F64).reshape(T, 1)
+    ang = pos * inv_freq.reshape(1, half)          # [T, half]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    if pairing == "half":
+        a = torch.arange(half)
+        b = a + half
+    elif pairing == "interleaved":
+        a = 2 * torch.arange(half)
+        b = a + 1
+    else:
+        raise ValueError(pairing)
+    x0, x1 = x[:, :, a].clone(), x[:, :, b].clone()
+    x[:, :, a] = x0 * cos - x1 * sin
+    x[:, :, b] = x0 * sin + x1 * cos
+    return x
+
+
+def plain_softmax(s: torch.Tensor) -> torch.Tensor:
+    """/root/reference/internal/ggml/ops.go:136-150: subtract the maximum,
+    exponentiate, divide by the sum."""
+    s = s.to(F64)
+    e = torch.exp(s - s.max())
+    return e / e.sum()
+
+
+def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None = None,
+                    window: int = 0, positions=None) -> torch.Tensor:
+    """/root/reference/internal/llm/forward.go:144-178.  q: [T, H, hd], k, v:
+    [T, K, hd] (k already rotated).  Head h reads KV head h // (H/K); token i
+    scores keys 0..i (no mask values: the range is the mask), score = dot * scale,
+    softmax, weighted sum of v.  `window` > 0 narrows the range to the last
+    `window` keys (the reference has no window; 0 is its behaviour)."""
+    T, H, hd = q.shape
+    K = k.shape[1]
+    group = H // K
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    q, k, v = q.to(F64), k.to(F64), v.to(F64)
+    out = torch.zeros(T, H, hd, dtype=F64)
+    for i in range(T):
+        lo = 0 if window <= 0 else max(0, i - window + 1)
+        for h in range(H):
+            kvh = h // group
+            scores = (k[lo:i + 1, kvh, :] @ q[i, h, :]) * scale
+            p = plain_softmax(scores)
+            out[i, h, :] = p @ v[lo:i + 1, kvh, :]
+    return out
+
+
+def plain_swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """/root/reference/internal/ggml/ops.go:159-165: g / (1 + exp(-g)) * up."""
+    g = gate.to(F64)
+    return g / (1 + torch.exp(-g)) * up.to(F64)
+
+
+# ---------------------------------------------------------------- model -----
+
+class PlainLlama:
+    """Reads a model folder; forward(tokens) -> logits [T, vocab] (float64)."""
+
+    def __init__(self, model_dir: str):
+        from safetensors import safe_open
+        with open(os.path.join(model_dir, "config.json"), "r", encoding="utf-8") as f:
+            c = json.load(f)
+        self.c = c
+        self.d = c["hidden_size"]
+        self.L = c["num_hidden_layers"]
+        self.H = c["num_attention_heads"]
+        self.K = c.get("num_key_value_heads") or self.H
+        self.hd = c.get("head_dim") or self.d // self.H
+        self.eps = c.get("rms_norm_eps", 1e-5)
+        self.tied = bool(c.get("tie_word_embeddings", False))
+        scaling = c.get("rope_scaling")
+        if scaling is not None and scaling.get("rope_type", scaling.get("type")) != "llama3":
+            scaling = None
+        self.inv_freq = plain_rope_frequencies(self.hd, c.get("rope_theta", 10000.0), scaling)
+        self.w = {}
+        with safe_open(os.path.join(model_dir, "model.safetensors"), framework="pt") as f:
+            for name in f.keys():
+                self.w[name] = f.get_tensor(name).to(F64)
+
+    def forward(self, tokens, upto_layer: int | None = None) -> torch.Tensor:
+        """/root/reference/internal/llm/forward.go:51-142 for one sequence from
+        position 0, logits at every position."""
+        w = self.w
+        T = len(tokens)
+        pos = list(range(T))
+        x = w["model.embed_tokens.weight"][torch.as_tensor(tokens, dtype=torch.long)]   # forward.go:75-77
+        layers = self.L if upto_layer is None else upto_layer
+        for l in range(layers):
+            p = f"model.layers.{l}."
+            xb = plain_rmsnorm(x, w[p + "input_layernorm.weight"], self.eps)           # forward.go:82
+            q = plain_matmul(xb, w[p + "self_attn.q_proj.weight"]).reshape(T, self.H, self.hd)
+            k = plain_matmul(xb, w[p + "self_attn.k_proj.weight"]).reshape(T, self.K, self.hd)
+            v = plain_matmul(xb, w[p + "self_attn.v_proj.weight"]).reshape(T, self.K, self.hd)
+            q = plain_rope(q, pos, self.inv_freq)                                      # forward.go:96-97
+            k = plain_rope(k, pos, self.inv_freq)
+            att = plain_attention(q, k, v).reshape(T, self.H * self.hd)                # forward.go:104
+            x = x + plain_matmul(att, w[p + "self_attn.o_proj.weight"])                # forward.go:106-107
+            xb = plain_rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps)  # forward.go:109
+            h = plain_swiglu(plain_matmul(xb, w[p + "mlp.gate_proj.weight"]),
+                             plain_matmul(xb, w[p + "mlp.up_proj.weight"]))            # forward.go:110-112
+            x = x + plain_matmul(h, w[p + "mlp.down_proj.weight"])                     # forward.go:113-114
+        if upto_layer is not None:
+            return x
+        x = plain_rmsnorm(x, w["model.norm.weight"], self.eps)                         # forward.go:124-128
+        head = w["model.embed_tokens.weight"] if self.tied else w["lm_head.weight"]    # model.go:118-121
+        return plain_matmul(x, head)                                                   # forward.go:132-141
+
+    def greedy(self, prompt, n_new: int) -> list:
+        """Greedy continuation: first maximum wins (/root/reference/internal/llm/sampler.go:76-84)."""
+        toks = list(prompt)
+        out = []
+        for _ in range(n_new):
+            logits = self.forward(toks)[-1]
+            nxt = plain_argmax(logits)
+            out.append(nxt)
+            toks.append(nxt)
+        return out
+
+
+# -------------------------------------------------------------- sampler -----
+
+def plain_argmax(logits) -> int:
+    """/root/reference/internal/llm/sampler.go:76-84: strict '>' keeps the first maximum."""
+    best = 0
+    vals = logits.tolist()
+    for i, v in enumerate(vals):
+        if v > vals[best]:
+            best = i
+    return best
+
+
+def plain_repeat_penalty(logits: torch.Tensor, history, penalty: float, last_n: int) -> torch.Tensor:
+    """/root/reference/internal/llm/sampler.go:57-74: each distinct id in the last
+    `last_n` ids (all if last_n < 0): logit > 0 -> / penalty, else * penalty."""
+    logits = logits.clone()
+    if penalty == 1 or last_n == 0:
+        return logits
+    recent = list(history)
+    if last_n > 0 and len(recent) > last_n:
+        recent = recent[-last_n:]
+    for i in set(recent):
+        if i >= logits.numel():
+            continue
+        logits[i] = logits[i] / penalty if logits[i] > 0 else logits[i] * penalty
+    return logits
+
+
+def plain_sampling_distribution(logits: torch.Tensor, temperature: float, top_k: int = 0,
+                                top_p: float = 1.0, min_p: float = 0.0) -> torch.Tensor:
+    """/root/reference/internal/llm/sampler.go:86-129 up to the draw: the
+    probability of every id (zeros outside the kept set).  Candidates are the
+    top_k largest in descending order; prob = exp((logit - max)/T) normalised;
+    top_p keeps the shortest prefix whose cumulative probability reaches it;
+    min_p cuts at the first candidate below min_p * prob[0]; the draw is
+    proportional to the kept probabilities."""
+    V = logits.numel()
+    k = V if top_k <= 0 or top_k > V else top_k
+    l32 = logits.to(torch.float32)
+    order = torch.argsort(l32, descending=True, stable=True)[:k]
+    cl = l32[order]
+    probs = torch.exp(((cl - cl[0]) / torch.tensor(temperature, dtype=torch.float32)).to(F64))
+    probs = probs / probs.sum()
+    keep = k
+    if 0 < top_p < 1:
+        cum = torch.cumsum(probs, 0)
+        # compare against the float32 value of top_p widened, as the reference does
+        hit = (cum >= float(torch.tensor(top_p, dtype=torch.float32))).nonzero()
+        if hit.numel():
+            keep = int(hit[0]) + 1
+    if min_p > 0:
+        thr = float(torch.tensor(min_p, dtype=torch.float32)) * probs[0]
+        for i in range(1, keep):
+            if probs[i] < thr:
+                keep = i
+                break
+    dist = torch.zeros(V, dtype=F64)
+    dist[order[:keep]] = probs[:keep] / probs[:keep].sum()
+    return dist

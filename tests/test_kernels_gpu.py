@@ -1,0 +1,242 @@
+"""Each HIP kernel alone against a plain torch reference of the same operation, at
+sizes other than the engine's (tails, widths that are no power of two)."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def close(a, b, tol):
+    """|a - b| <= tol * (1 + |b|), the reference's form (/root/reference/internal/ggml/q8_test.go:24-26)."""
+    a, b = a.double().cpu(), b.double().cpu()
+    bad = (a - b).abs() > tol * (1 + b.abs())
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} differ; worst {float((a - b).abs().max()):.3e}"
+
+
+@pytest.mark.parametrize("n,d", [(1, 7), (5, 64), (3, 1027), (17, 4096)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm(n, d, out_dtype):
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(n * 1000 + d)
+    x = torch.randn(n, d, generator=g) * 3
+    w = 1 + 0.1 * torch.randn(d, generator=g)
+    eps = 1e-5
+    ref = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps) * w.double()
+    out = torch.empty(n, d, dtype=out_dtype, device=DEV)
+    ops.rmsnorm(out, x.to(DEV), w.to(DEV), eps)
+    close(out, ref, 1e-5 if out_dtype == torch.float32 else 1e-2)
+    # gathered rows, bfloat16 weight
+    rows = torch.tensor([n - 1, 0], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, d, dtype=out_dtype, device=DEV)
+    wb = w.to(torch.bfloat16)
+    ops.rmsnorm(out2, x.to(DEV), wb.to(DEV), eps, rows)
+    ref2 = (x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps) * wb.double())[[n - 1, 0]]
+    close(out2, ref2, 1e-5 if out_dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (7, 33, 100), (64, 64, 16), (65, 130, 1027), (3, 172, 64), (200, 96, 172)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_gemm_f32(M, N, K, accumulate):
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(M + 7 * N + 13 * K)
+    x, w = torch.randn(M, K, generator=g), torch.randn(N, K, generator=g)
+    c0 = torch.randn(M, N, generator=g)
+    ref = x.double() @ w.double().t() + (c0.double() if accumulate else 0)
+    out = c0.clone().to(DEV)
+    ops.linear(out, x.to(DEV), w.to(DEV), accumulate=accumulate)
+    mag = (x.abs().double() @ w.abs().double().t())        # error relative to the terms' size
+    err = (out.double().cpu() - ref).abs()
+    assert (err <= 1e-6 * (1 + mag)).all(), float((err / (1 + mag)).max())
+
+
+def test_gemm_f32_rows_do_not_depend_on_the_batch():
+    """Bit-equal results for a row whether it runs alone or among others."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(5)
+    x, w = torch.randn(77, 300, generator=g).to(DEV), torch.randn(130, 300, generator=g).to(DEV)
+    full = torch.empty(77, 130, device=DEV)
+    ops.linear(full, x, w)
+    for r in (0, 63, 64, 76):
+        one = torch.empty(1, 130, device=DEV)
+        ops.linear(one, x[r:r + 1].contiguous(), w)
+        assert torch.equal(one[0], full[r])
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 16, 32), (1, 4096, 4096), (8, 100, 256), (16, 33, 1000), (17, 64, 128),
+                                   (64, 172, 96), (5, 96, 172), (33, 320, 96), (3, 50, 20)])
+@pytest.mark.parametrize("kernel", [1, 2])
+@pytest.mark.parametrize("mode", ["bf16", "f32", "add"])
+def test_gemm_bf16(M, N, K, kernel, mode):
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(M + 7 * N + 13 * K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    ref = x.double() @ w.double().t()
+    if mode == "bf16":
+        out = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.linear(out, x.to(DEV), w.to(DEV), kernel=kernel)
+        tol = 1e-2
+    elif mode == "f32":
+        out = torch.zeros(M, N, dtype=torch.float32, device=DEV)
+        ops.linear(out, x.to(DEV), w.to(DEV), kernel=kernel)
+        tol = 1e-5
+    else:
+        c0 = torch.randn(M, N, generator=g)
+        out = c0.clone().to(DEV)
+        ops.linear(out, x.to(DEV), w.to(DEV), accumulate=True, kernel=kernel)
+        ref = ref + c0.double()
+        tol = 1e-5
+    mag = x.abs().double() @ w.abs().double().t()
+    err = (out.double().cpu() - ref).abs()
+    assert (err <= tol * (1 + mag)).all(), float((err / (1 + mag)).max())
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 32), (300, 200, 520), (2048, 512, 1024), (129, 257, 72)])
+def test_gemm_bf16_tiled_large(M, N, K):
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    ref = x.double() @ w.double().t()
+    out = torch.zeros(M, N, dtype=torch.float32, device=DEV)
+    ops.linear(out, x.to(DEV), w.to(DEV))
+    mag = x.abs().double() @ w.abs().double().t()
+    err = (out.double().cpu() - ref).abs()
+    assert (err <= 1e-5 * (1 + mag)).all(), float((err / (1 + mag)).max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_and_add(dtype):
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(3)
+    gu = (torch.randn(9, 2 * 173, generator=g) * 4).to(dtype)
+    out = torch.empty(9, 173, dtype=dtype, device=DEV)
+    gud = gu.to(DEV)
+    ops.swiglu(out, gud[:, :173], gud[:, 173:])
+    ref = torch.nn.functional.silu(gu[:, :173].double()) * gu[:, 173:].double()
+    close(out, ref, 1e-6 if dtype == torch.float32 else 1e-2)
+    x = torch.randn(9, 173, generator=g)
+    xd = x.clone().to(DEV)
+    ops.residual_add(xd, out)
+    close(xd, x.double() + out.double().cpu(), 1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(4)
+    table = torch.randn(321, 97, generator=g).to(dtype)
+    ids = torch.tensor([0, 320, 5, 5, 17], dtype=torch.int32)
+    out = torch.empty(5, 97, dtype=torch.float32, device=DEV)
+    ops.embed(out, table.to(DEV), ids.to(DEV))
+    assert torch.equal(out.cpu(), table[ids.long()].float())
+
+
+def _paged(kv, page_size, pages_order):
+    """kv: [T, K, hd] -> cache layer tensor with the pages in the given order, and the table."""
+    T, K, hd = kv[0].shape
+    nblocks = (T + page_size - 1) // page_size
+    num_pages = max(pages_order) + 1
+    layer = torch.zeros(num_pages, 2, K, page_size * hd, dtype=kv[0].dtype)
+    layer += 7.0   # stale contents that must never show
+    for b in range(nblocks):
+        p = pages_order[b]
+        for s in range(min(page_size, T - b * page_size)):
+            t = b * page_size + s
+            for h in range(K):
+                layer[p, 0, h].view(page_size, hd)[s] = kv[0][t, h]
+                layer[p, 1, h].view(hd, page_size)[:, s] = kv[1][t, h]
+    return layer, torch.tensor([pages_order[:nblocks]], dtype=torch.int32)
+
+
+@pytest.mark.parametrize("H,K,hd,T,window", [(4, 2, 16, 37, 0), (3, 1, 32, 100, 0), (6, 3, 48, 70, 0),
+                                             (2, 2, 64, 33, 0), (4, 1, 128, 130, 0), (4, 2, 16, 90, 20),
+                                             (5, 5, 80, 40, 0), (1, 1, 256, 35, 0)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_kernels(H, K, hd, T, window, dtype):
+    """Plain kernel (both dtypes) and the matrix-core kernels (bfloat16) against
+    the reference formula, on pages in scrambled order."""
+    from plain_llama import plain_attention
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(H * 100 + hd + T)
+    q = torch.randn(T, H, hd, generator=g).to(dtype)
+    k = torch.randn(T, K, hd, generator=g).to(dtype)
+    v = torch.randn(T, K, hd, generator=g).to(dtype)
+    scale = 1 / math.sqrt(hd)
+    ref = plain_attention(q, k, v, scale, window=window).reshape(T, H * hd)
+    ps = 16
+    nblocks = (T + ps - 1) // ps
+    order = torch.randperm(nblocks + 5, generator=g)[:nblocks].tolist()
+    layer, table = _paged((k, v), ps, order)
+    layer, table = layer.to(DEV), table.to(DEV)
+    positions = torch.arange(T, dtype=torch.int32, device=DEV)
+    seg = torch.zeros(T, dtype=torch.int32, device=DEV)
+    qd = q.reshape(T, H * hd).to(DEV)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+    ops.attention_plain(out, qd, layer, positions, seg, table, H, K, hd, ps, scale, window)
+    close(out, ref, tol)
+    if dtype == torch.bfloat16:
+        tiles = torch.tensor([(o, min(32, T - o), o, 0) for o in range(0, T, 32)], dtype=torch.int32, device=DEV)
+        out2 = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+        ops.attention_bf16_prefill(out2, qd, layer, tiles, table, H, K, hd, ps, scale, window)
+        close(out2, ref, tol)
+        # decode kernel: the last rows as single queries, with and without split keys
+        for splits in (1, 3):
+            rows = torch.tensor([T - 1, T // 2, 0], dtype=torch.int32, device=DEV)
+            out3 = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+            partial = torch.zeros(3 * H * splits * (hd + 2), dtype=torch.float32, device=DEV)
+            ops.attention_bf16_decode(out3, qd, layer, rows, rows.clone(), torch.zeros(3, dtype=torch.int32, device=DEV),
+                                      table, H, K, hd, ps, scale, window, partial, splits)
+            close(out3[[T - 1, T // 2, 0]], ref[[T - 1, T // 2, 0]], tol)
+
+
+@pytest.mark.parametrize("pairing", ["half", "interleaved"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_cache_write(pairing, dtype):
+    from plain_llama import plain_rope, plain_rope_frequencies
+    from hfee_amd.kernels import ops
+    from hfee_amd.parts.rotary import Rotary
+    from hfee_amd.config.specs import PositionSpec, params
+    H, K, hd, T, ps = 3, 2, 32, 21, 16
+    rot = Rotary(PositionSpec("rope", params(head_dim=hd, rotary_dim=hd, theta=10000.0, scaling=None, pairing=pairing)))
+    rot.prepare(64, DEV)
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(T, H * hd, generator=g).to(dtype)
+    k = torch.randn(T, K * hd, generator=g).to(dtype)
+    v = torch.randn(T, K * hd, generator=g).to(dtype)
+    pos = torch.arange(5, 5 + T, dtype=torch.int32)
+    inv = plain_rope_frequencies(hd, 10000.0)
+    q_ref = plain_rope(q.reshape(T, H, hd), pos.tolist(), inv, pairing).reshape(T, H * hd)
+    k_ref = plain_rope(k.reshape(T, K, hd), pos.tolist(), inv, pairing)
+    layer = torch.zeros(4, 2, K, ps * hd, dtype=dtype, device=DEV)
+    table = torch.tensor([[2, 0, 3, 1]], dtype=torch.int32, device=DEV)
+    qd = q.to(DEV)
+    ops.rope_cache_write(qd, k.to(DEV), v.to(DEV), pos.to(DEV), torch.zeros(T, dtype=torch.int32, device=DEV),
+                         table, rot.cos, rot.sin, rot.pairing, layer, H, K, hd, ps, int(pos.max()))
+    tol = 1e-6 if dtype == torch.float32 else 1e-2
+    close(qd, q_ref, tol)
+    lay = layer.cpu()
+    for t in range(T):
+        p = int(pos[t])
+        page, slot = [2, 0, 3, 1][p // ps], p % ps
+        for h in range(K):
+            close(lay[page, 0, h].view(ps, hd)[slot], k_ref[t, h], tol)
+            assert torch.equal(lay[page, 1, h].view(hd, ps)[:, slot], v[t].view(K, hd)[h])
+
+
+def test_argmax_first_maximum_wins():
+    from hfee_amd.kernels import ops
+    logits = torch.zeros(3, 5000)
+    logits[0, 4000] = 2.0
+    logits[0, 17] = 2.0          # equal maxima: the first one
+    logits[1] = -1.0
+    logits[1, 4999] = -0.5
+    logits[2, 0] = 1.0
+    out = torch.zeros(3, dtype=torch.int32, device=DEV)
+    ops.argmax(out, logits.to(DEV))
+    assert out.tolist() == [17, 4999, 0]
