@@ -1,0 +1,272 @@
+"""The scheduler: continuous batching over the step function.
+
+Every step feeds one token from each request that is decoding, then portions of
+the prompts still being read, under a token budget, through one step()
+(/root/reference/internal/llm/runner.go:231-280).  What the reference decides, it
+decides the same way here:
+
+  * a prompt that does not leave room for one new token in the context is refused
+    before it queues (runner.go:95-97);
+  * decoding requests come first, then prompt portions, in admission order; a
+    portion is min(what is left of the prompt, what is left of the budget), and
+    logits are asked for only when the portion ends the prompt (runner.go:238-259);
+  * after the logits: sample; an end-of-sequence id finishes the request with
+    "stop" and is neither kept nor emitted; num_predict is checked after the token
+    is emitted, so 0 still yields one token; a full context finishes with "length"
+    at the top of a step (runner.go:248-251, 283-314).
+
+The reference reserves a whole context per slot up front, so pages never run out
+there.  Here they can, and this is what happens:
+
+  1. a waiting request is admitted only if a state slot is free and the free pages
+     cover its first portion on top of what the running requests need this step;
+  2. a prompt portion is shortened to what the free pages hold (or waits a step);
+  3. if a decoding request cannot get the page its next token needs, the request
+     admitted last is preempted: its pages go back, and it returns to the front of
+     the waiting line with prompt + generated tokens as its new prompt (its sampler
+     stream goes on where it was, so the tokens it produces are the same);
+  4. a request that is alone and still cannot get a page finishes with "length".
+The request admitted first is never preempted, so every step makes progress.
+"""
+from __future__ import annotations
+
+import time
+from collections import deque
+from dataclasses import dataclass, field
+
+from ..cache import OutOfPages
+from ..sampling import SampleRow, SamplingParams
+from .step import StepEntry
+
+
+@dataclass
+class Stats:
+    """/root/reference/internal/llm/runner.go:15-21"""
+    prompt_tokens: int = 0
+    prompt_duration: float = 0.0
+    eval_tokens: int = 0
+    eval_duration: float = 0.0
+    done_reason: str = ""
+    preemptions: int = 0
+
+
+@dataclass
+class Request:
+    request_id: object
+    prompt: list
+    params: SamplingParams
+    seed: int = 0
+    feed: list = field(default_factory=list)        # tokens to run next
+    generated: list = field(default_factory=list)
+    history: list = field(default_factory=list)     # prompt + generated (repeat penalty)
+    draws: int = 0
+    decoding: bool = False                          # the prompt has been read
+    stats: Stats = field(default_factory=Stats)
+    started: float = 0.0
+    eval_started: float = 0.0
+    admitted_order: int = -1
+    cancelled: bool = False
+    on_token: object = None
+
+
+@dataclass
+class Finished:
+    request: Request
+    reason: str
+    error: str | None = None
+
+
+class PromptTooLong(ValueError):
+    pass
+
+
+class Scheduler:
+    def __init__(self, engine, sampler, *, max_num_seqs: int, max_batch_tokens: int, num_ctx: int,
+                 eos_token_ids=(), clock=time.perf_counter):
+        self.engine, self.sampler = engine, sampler
+        self.cache = engine.cache
+        self.max_num_seqs = max_num_seqs
+        self.max_batch_tokens = max_batch_tokens
+        self.num_ctx = num_ctx
+        self.eos = set(eos_token_ids)
+        self.clock = clock
+        self.waiting: deque = deque()
+        self.running: list = []          # in admission order
+        self._order = 0
+        self.last_batch: list = []       # (request_id, tokens in the step) of the latest step, for tests
+
+    # ----------------------------------------------------------------- intake
+    def add(self, request: Request) -> None:
+        if len(request.prompt) < 1:
+            raise ValueError("an empty prompt")
+        if len(request.prompt) >= self.num_ctx:
+            raise PromptTooLong(f"prompt is {len(request.prompt)} tokens but the context window is {self.num_ctx}")
+        request.feed = list(request.prompt)
+        request.history = list(request.prompt)
+        request.stats.prompt_tokens = len(request.prompt)
+        if request.seed is None or request.seed < 0:
+            request.seed = request.params.resolved_seed()
+        self.waiting.append(request)
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def cancel(self, request_id) -> None:
+        for r in list(self.waiting) + self.running:
+            if r.request_id == request_id:
+                r.cancelled = True
+
+    # ------------------------------------------------------------------ pages
+    def _room(self, request: Request) -> int:
+        """How many more tokens of `request` the free pages can hold."""
+        rc = self.cache.get(request.request_id)
+        ps = self.cache.page_size
+        room = None
+        for table, pool in zip(rc.tables, self.cache.pools):
+            r = len(table) * ps - rc.length + pool.num_free * ps
+            room = r if room is None else min(room, r)
+        return max(room or 0, 0)
+
+    def _preempt(self, victim: Request) -> None:
+        self.engine.release(victim.request_id)
+        self.running.remove(victim)
+        victim.feed = list(victim.prompt) + list(victim.generated)
+        victim.decoding = False
+        victim.stats.preemptions += 1
+        self.waiting.appendleft(victim)
+
+    def _finish(self, request: Request, reason: str, finished: list, error: str | None = None) -> None:
+        now = self.clock()
+        request.stats.done_reason = reason
+        if request.eval_started:
+            request.stats.eval_duration = now - request.eval_started
+        if self.engine.is_live(request.request_id):
+            self.engine.release(request.request_id)
+        if request in self.running:
+            self.running.remove(request)
+        finished.append(Finished(request, reason, error))
+
+    # ------------------------------------------------------------------- step
+    def step(self) -> list:
+        """One pass: admit, batch, run, sample.  Returns the requests that finished."""
+        finished: list = []
+
+        # cancelled or out of context (runner.go:244-251)
+        for r in list(self.running):
+            if r.cancelled:
+                self._finish(r, "cancelled", finished)
+            elif self.cache.get(r.request_id).length >= self.num_ctx:
+                self._finish(r, "length", finished)
+        for r in [w for w in self.waiting if w.cancelled]:
+            self.waiting.remove(r)
+            self._finish(r, "cancelled", finished)
+
+        budget = self.max_batch_tokens
+        batch: list = []     # (request, tokens, wants_logits)
+
+        # decoding requests first, oldest first; preempt from the young end if pages run out
+        for r in [x for x in self.running if x.decoding]:
+            if r not in self.running:
+                continue          # preempted while an older request was served
+            if budget == 0:
+                break
+            while self._room(r) < 1:
+                victim = self.running[-1]
+                if victim is r:
+                    others = [x for x in self.running if x is not r]
+                    if not others:
+                        break
+                    victim = others[-1]
+                batch = [b for b in batch if b[0] is not victim]
+                self._preempt(victim)
+            if self._room(r) < 1:
+                self._finish(r, "length", finished, "the cache cannot hold this request even alone")
+                continue
+            self.cache.reserve(r.request_id, 1)
+            batch.append((r, r.feed[:1], True))
+            budget -= 1
+        budget = self.max_batch_tokens - sum(len(t) for _, t, _ in batch)
+
+        # admit waiting requests while there is a slot, a place and pages for a first portion
+        while self.waiting and len(self.running) < self.max_num_seqs and self.cache.num_free_slots > 0 and budget > 0:
+            r = self.waiting[0]
+            first = min(len(r.feed), budget)
+            free_tokens = min(p.num_free for p in self.cache.pools) * self.cache.page_size if self.cache.pools else first
+            if free_tokens < min(first, self.cache.page_size) and self.running:
+                break                      # wait until pages come back
+            if free_tokens < 1:
+                self.waiting.popleft()
+                self._finish(r, "length", finished, "the cache has no free page for this request")
+                continue
+            self.waiting.popleft()
+            self.engine.admit(r.request_id)
+            r.admitted_order = self._order
+            self._order += 1
+            if not r.started:
+                r.started = self.clock()
+            self.running.append(r)
+            # its portion is taken below with the other prompts
+            n = min(len(r.feed), budget, self._room(r))
+            if n >= 1:
+                self.cache.reserve(r.request_id, n)
+                batch.append((r, r.feed[:n], n == len(r.feed)))
+                budget -= n
+
+        # prompt portions of requests admitted earlier
+        in_batch = {id(b[0]) for b in batch}
+        for r in self.running:
+            if r.decoding or id(r) in in_batch or budget == 0:
+                continue
+            n = min(len(r.feed), budget, self._room(r))
+            if n < 1:
+                continue
+            self.cache.reserve(r.request_id, n)
+            batch.append((r, r.feed[:n], n == len(r.feed)))
+            budget -= n
+
+        if not batch:
+            if self.running and not finished:
+                # nothing fits: give the oldest request room by preempting the youngest
+                if len(self.running) > 1:
+                    self._preempt(self.running[-1])
+                else:
+                    self._finish(self.running[0], "length", finished,
+                                 "the cache cannot hold this request even alone")
+            self.last_batch = []
+            return finished
+
+        entries = [StepEntry(r.request_id, toks, [len(toks) - 1] if want else []) for r, toks, want in batch]
+        self.last_batch = [(r.request_id, len(toks)) for r, toks, _ in batch]
+        logits = self.engine.step(entries)
+
+        rows, owners = [], []
+        for r, toks, want in batch:
+            r.feed = r.feed[len(toks):]
+            if want:
+                owners.append(r)
+                rows.append(SampleRow(r.params, r.seed, r.draws, r.history, len(rows)))
+        ids = self.sampler.sample(logits, rows) if rows else []
+        now = self.clock()
+        for r, token in zip(owners, ids):
+            if not r.decoding:
+                r.decoding = True
+                if not r.eval_started:
+                    r.stats.prompt_duration = now - r.started
+                    r.eval_started = now
+            r.draws += 1
+            if token in self.eos and not r.params.ignore_eos:
+                self._finish(r, "stop", finished)
+                continue
+            r.generated.append(token)
+            r.history.append(token)
+            r.stats.eval_tokens = len(r.generated)
+            stop_now = False
+            if r.on_token is not None:
+                stop_now = bool(r.on_token(r, token))
+            if stop_now:
+                self._finish(r, "stop", finished)
+            elif r.params.num_predict >= 0 and len(r.generated) >= r.params.num_predict:
+                self._finish(r, "length", finished)
+            else:
+                r.feed = [token]
+        return finished

@@ -1,0 +1,92 @@
+"""The sampler: packs each row's options for the device kernel and reads the
+chosen ids back.
+
+One random stream per request (/root/reference/internal/llm/sampler.go:41-47,
+/root/reference/internal/llm/runner.go:223): the uniform number of a request's k-th
+draw is splitmix64(seed, k), so a request's tokens do not depend on what else is
+sampled in the same call.  `uniform()` is the host twin of the kernel's generator.
+"""
+from __future__ import annotations
+
+import struct
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from ..kernels import ops
+from .params import SamplingParams
+
+_MASK = (1 << 64) - 1
+
+
+def uniform(seed: int, draw: int) -> float:
+    """The number in [0, 1) that the kernel uses for draw number `draw` of stream `seed`."""
+    z = (seed + (draw + 1) * 0x9E3779B97F4A7C15) & _MASK
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    z ^= z >> 31
+    return (z >> 11) * (1.0 / 9007199254740992.0)
+
+
+@dataclass
+class SampleRow:
+    params: SamplingParams
+    seed: int             # resolved (non-negative) seed of the request
+    draw: int             # how many tokens the request has sampled so far
+    history: list         # prompt + generated ids (for the repeat penalty)
+    logits_row: int       # row of the logits tensor
+
+
+def _f2i(x: float) -> int:
+    return struct.unpack("<i", struct.pack("<f", float(x)))[0]
+
+
+def pack_rows(rows) -> tuple:
+    """rows -> ([n, 12] int32 parameter array, flat int32 history)."""
+    params = np.zeros((len(rows), 12), dtype=np.int32)
+    hist = []
+    for i, r in enumerate(rows):
+        p = r.params
+        recent = []
+        if p.repeat_penalty != 1 and p.repeat_last_n != 0:
+            recent = list(r.history)
+            if p.repeat_last_n > 0 and len(recent) > p.repeat_last_n:
+                recent = recent[-p.repeat_last_n:]
+        seed, draw = r.seed & _MASK, r.draw & _MASK
+        words = [_f2i(p.temperature), int(p.top_k), _f2i(p.top_p), _f2i(p.min_p), _f2i(p.repeat_penalty),
+                 len(hist), len(recent)]
+        params[i, :7] = words
+        params[i, 7:11] = np.array([seed & 0xffffffff, seed >> 32, draw & 0xffffffff, draw >> 32],
+                                   dtype=np.uint32).view(np.int32)
+        params[i, 11] = r.logits_row
+        hist += recent
+    return params, np.asarray(hist if hist else [0], dtype=np.int32)
+
+
+class Sampler:
+    def __init__(self, vocab: int, device, max_rows: int):
+        self.vocab, self.device, self.max_rows = vocab, device, max_rows
+        self._out = torch.empty(max_rows, dtype=torch.int32, device=device)
+        self._scratch = None
+
+    def sample(self, logits: torch.Tensor, rows) -> list:
+        """logits: float32 [*, vocab] on the device (changed in place by the repeat
+        penalty, as the reference changes them).  Returns one id per row."""
+        n = len(rows)
+        if n == 0:
+            return []
+        if n > self.max_rows:
+            raise ValueError(f"{n} rows to sample, the sampler was made for {self.max_rows}")
+        plain_greedy = all(r.params.temperature <= 0 and (r.params.repeat_penalty == 1 or r.params.repeat_last_n == 0)
+                           for r in rows)
+        if plain_greedy and [r.logits_row for r in rows] == list(range(logits.shape[0])):
+            ops.argmax(self._out, logits)
+            return self._out[:n].tolist()
+        params, hist = pack_rows(rows)
+        if self._scratch is None:
+            self._scratch = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
+        dparams = torch.from_numpy(params).to(self.device)
+        dhist = torch.from_numpy(hist).to(self.device)
+        ops.sample(self._out, logits, dparams, dhist, self._scratch)
+        return self._out[:n].tolist()

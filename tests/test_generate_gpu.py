@@ -1,0 +1,86 @@
+"""Generation through the entry point: greedy and seeded sampling, scheduler on the GPU."""
+import pytest
+import torch
+
+import trace_util as tu
+from conftest import TINY
+
+pytestmark = pytest.mark.gpu
+
+
+def test_greedy_generation_matches_the_plain_implementation(model_folders):
+    """Tiny A's workload: prompts of 5, 17, 32 and 1 tokens, 16 greedy tokens each."""
+    from plain_llama import PlainLlama
+    from hfee_amd import LLM, SamplingParams
+    folder = model_folders[("A", "float32")]
+    plain = PlainLlama(folder)
+    prompts = list(tu.make_requests(256, [5, 17, 32, 1], seed=1).values())
+    llm = LLM(folder, dtype="float32", num_ctx=128, num_parallel=4, max_batch_tokens=24)
+    outs = llm.generate(prompts, SamplingParams.greedy(num_predict=16))
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == plain.greedy(p, 16)
+        assert o.done_reason == "length" and o.stats.eval_tokens == 16 and o.stats.prompt_tokens == len(p)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_seeded_sampling_does_not_depend_on_the_batch(model_folders, dtype):
+    """Tiny B's workload: prompts of 40, 3 and 100 tokens, portions of 16, 24 tokens at
+    temperature 0.8 with a fixed seed: together and alone give the same tokens."""
+    from hfee_amd import LLM, SamplingParams
+    folder = model_folders[("B", dtype)]
+    prompts = list(tu.make_requests(320, [40, 3, 100], seed=2).values())
+    params = [SamplingParams(temperature=0.8, seed=100 + i, num_predict=24) for i in range(3)]
+    llm = LLM(folder, dtype=dtype, num_ctx=256, num_parallel=3, max_batch_tokens=16)
+    together = llm.generate(prompts, params)
+    for p, sp, o in zip(prompts, params, together):
+        alone = llm.generate([p], sp)[0]
+        assert len(o.token_ids) == 24
+        if dtype == "float32":
+            assert alone.token_ids == o.token_ids
+        else:       # rounding differs between batch shapes in bfloat16: most tokens still agree
+            same = sum(a == b for a, b in zip(alone.token_ids, o.token_ids))
+            assert alone.token_ids[0] == o.token_ids[0] and same >= 1
+
+
+def test_scarce_pages_preempt_and_still_give_the_same_tokens(model_folders):
+    from hfee_amd import LLM, SamplingParams
+    folder = model_folders[("A", "float32")]
+    prompts = list(tu.make_requests(256, [30, 28, 26, 31], seed=4).values())
+    sp = SamplingParams.greedy(num_predict=40)
+    roomy = LLM(folder, dtype="float32", num_ctx=128, num_parallel=4)
+    want = [o.token_ids for o in roomy.generate(prompts, sp)]
+    tight = LLM(folder, dtype="float32", num_ctx=128, num_parallel=4, num_pages=10)   # 160 tokens for 4 x 70
+    outs = tight.generate(prompts, sp)
+    assert [o.token_ids for o in outs] == want
+    assert sum(o.stats.preemptions for o in outs) > 0
+    tight.engine.cache.check()
+    assert not tight.engine.cache.requests
+
+
+def test_stop_on_eos_and_context_limit(model_folders, tmp_path):
+    import json, os, shutil
+    from plain_llama import PlainLlama
+    from hfee_amd import LLM, SamplingParams
+    src = model_folders[("A", "float32")]
+    plain = PlainLlama(src)
+    prompt = tu.make_requests(256, [12], seed=6)["r0"]
+    cont = plain.greedy(prompt, 8)
+    # make the 4th generated token the end-of-sequence id
+    dst = tmp_path / "eos"
+    shutil.copytree(src, dst)
+    cj = json.load(open(dst / "config.json"))
+    eos = cont[3]
+    cj["eos_token_id"] = eos
+    json.dump(cj, open(dst / "config.json", "w"))
+    llm = LLM(str(dst), dtype="float32", num_ctx=128, num_parallel=2)
+    o = llm.generate([prompt], SamplingParams.greedy(num_predict=8))[0]
+    first = cont.index(eos)
+    assert o.token_ids == cont[:first] and o.done_reason == "stop"
+    o = llm.generate([prompt], SamplingParams.greedy(num_predict=8, ignore_eos=True))[0]
+    assert o.token_ids == cont and o.done_reason == "length"
+    # the context window ends a request with "length"
+    small = LLM(src, dtype="float32", num_ctx=20, num_parallel=1)
+    o = small.generate([prompt], SamplingParams.greedy())[0]
+    assert o.done_reason == "length" and len(prompt) + len(o.token_ids) == 21
+    with pytest.raises(ValueError, match="context window"):
+        small.generate([list(range(20))], SamplingParams.greedy())

