@@ -1,0 +1,154 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+
+The default run: a Llama-3.1-8B-shaped model (32 layers, width 4096, 32 heads on 8
+KV heads of 128, feed-forward 14336, vocabulary 128256, llama3 rope scaling) with
+random N(0, 0.02) weights in bfloat16, context window 8192, 8 requests with
+1,024-token prompts of seeded uniform random ids.  A step is one decode step of
+the scheduler (one new token for every request).  W untimed steps, then exactly K
+timed steps between two synchronisations.  One JSON line is printed: decoded
+tokens per second, the step's achieved fraction of the HBM roofline (every weight
+read once plus the cache of the live requests), a 2,048-token prefill with its
+fraction of the bf16 matrix peak, and decode at batch 1 and 64.
+"""
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK = 8.0e12          # bytes/s, MI355X HBM3E
+BF16_PEAK = 2.5e15         # dense MFMA flop/s
+BASE_8B = dict(num_hidden_layers=32, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+               head_dim=128, intermediate_size=14336, vocab_size=128256, max_position_embeddings=131072,
+               rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+               rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                             "high_freq_factor": 4.0, "original_max_position_embeddings": 8192})
+CONTEXT = 8192
+PROMPT = 1024
+PREFILL = 2048
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=BASE_8B["num_hidden_layers"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    import hfee_amd  # noqa: F401
+    from hfee_amd.config import config_from_dict
+    from hfee_amd.engine import Engine, Request, Scheduler, random_model
+    from hfee_amd.sampling import Sampler, SamplingParams
+
+    cj = dict(BASE_8B, architectures=["LlamaForCausalLM"], num_hidden_layers=args.layers)
+    cfg = config_from_dict(cj)
+    t0 = time.perf_counter()
+    model = random_model(cfg, seed=0, dtype="bfloat16", device="cuda:0", std=0.02)
+    torch.cuda.synchronize()
+    print(f"[bench] random weights made in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
+
+    L, d, H, K, hd = cfg.num_hidden_layers, cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    F, V = cfg.intermediate_size, cfg.vocab_size
+    layer_params = d * (H + 2 * K) * hd + H * hd * d + 3 * d * F
+    weight_bytes = 2 * (L * layer_params + V * d)              # every matrix a decode step reads, once
+    kv_bytes_per_token = L * 2 * K * hd * 2
+    max_batch = max(64, args.batch)
+    steps_total = args.steps + args.warmup
+
+    page_size = 16
+    tokens_cached = max_batch * (PROMPT + steps_total + page_size) + PREFILL + page_size
+    engine = Engine(model, cache_tokens=tokens_cached, page_size=page_size, max_requests=max_batch,
+                    max_batch_tokens=PREFILL, num_positions=CONTEXT)
+    sampler = Sampler(V, engine.device, max_rows=max_batch)
+    gen = torch.Generator().manual_seed(0)
+
+    def decode_run(batch: int, steps: int, warmup: int):
+        sched = Scheduler(engine, sampler, max_num_seqs=batch, max_batch_tokens=PREFILL, num_ctx=CONTEXT)
+        params = SamplingParams.greedy(num_predict=-1, ignore_eos=True)
+        for i in range(batch):
+            prompt = torch.randint(0, V, (PROMPT,), generator=gen).tolist()
+            sched.add(Request(("bench", batch, i), prompt, params, seed=i))
+        while any(not r.decoding for r in list(sched.running) + list(sched.waiting)):
+            sched.step()
+        for _ in range(warmup):
+            sched.step()
+        lengths = [engine.cached_length(r.request_id) for r in sched.running]
+        before = sum(len(r.generated) for r in sched.running)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            sched.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        made = sum(len(r.generated) for r in sched.running) - before
+        assert made == batch * steps, f"{made} tokens decoded in {steps} steps of batch {batch}"
+        mean_ctx = sum(lengths) / batch + steps / 2
+        for r in list(sched.running):
+            sched.cancel(r.request_id)
+        sched.step()
+        return dt, mean_ctx
+
+    def prefill_run():
+        best = None
+        for i in range(3):
+            prompt = torch.randint(0, V, (PREFILL,), generator=gen).tolist()
+            from hfee_amd.engine import StepEntry
+            rid = ("prefill", i)
+            engine.admit(rid)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            logits = engine.step([StepEntry(rid, prompt, [PREFILL - 1])])
+            del logits
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            engine.release(rid)
+            best = dt if best is None else min(best, dt)
+        return best
+
+    dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
+    ms_per_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
+    achieved = step_bytes / (dt / args.steps)
+    line = {
+        "metric": "decode tok/s @ batch 1/8/64; prefill tok/s @ 2,048 tokens (Llama-3.1-8B bf16)",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (seeded uniform random token ids, random N(0,0.02) weights)",
+        "config": {"model": "Llama-3.1-8B-shaped", "layers": L, "layers_of_config": BASE_8B["num_hidden_layers"],
+                   "hidden": d, "heads": H, "kv_heads": K, "head_dim": hd, "intermediate": F, "vocab": V,
+                   "global_batch": args.batch, "seq_len": CONTEXT, "prompt_tokens": PROMPT,
+                   "mean_context_in_timed_steps": round(mean_ctx, 1), "page_size": page_size,
+                   "max_batch_tokens": PREFILL, "parallelism": "single GPU"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+    }
+    if not args.no_points:
+        pt = prefill_run()
+        gemm_flops = 2.0 * PREFILL * (L * layer_params) + 2.0 * V * d
+        attn_flops = L * 4.0 * hd * H * PREFILL * (PREFILL + 1) / 2
+        flops = gemm_flops + attn_flops
+        line["prefill"] = {"value": round(PREFILL / pt, 1), "tokens": PREFILL, "ms": round(pt * 1e3, 3),
+                           "frac": round(flops / pt / BF16_PEAK, 4)}
+        points = {}
+        for b in (1, 64):
+            steps = max(8, min(args.steps, 64))
+            dtb, _ = decode_run(b, steps, min(args.warmup, 4))
+            points[f"decode_b{b}"] = round(b * steps / dtb, 2)
+        line["points"] = points
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -50,7 +50,7 @@ class Engine:
 
     def __init__(self, model: Model, *, num_pages=None, cache_tokens=None, page_size: int = 16,
                  max_requests: int = 64, max_batch_tokens: int = 2048, num_positions: int | None = None,
-                 device="cuda:0"):
+                 device="cuda:0", use_graphs: bool = True):
         if not model.bound:
             raise ValueError("the model has no weights bound")
         if not torch.cuda.is_available():
@@ -78,6 +78,13 @@ class Engine:
         self._meta_capacity = 0
         self._meta_ring, self._meta_device = [], None
         self.steps_run = 0
+        # decode-only steps are replayed as captured HIP graphs, one per
+        # (batch size, block-table width, wanted rows): launch gaps would otherwise
+        # cost more than the kernels at small batches
+        self.use_graphs = use_graphs and all(
+            p.graph_safe for b in model.blocks for p in (b.parts() if hasattr(b, "parts") else [b]))
+        self._graphs: dict = {}
+        self.graph_replays = 0
 
     # ------------------------------------------------------------ requests
     def admit(self, request_id):
@@ -140,13 +147,14 @@ class Engine:
             total += (a.size + 3) // 4 * 4
         total = max(total, 4)
         if total > self._meta_capacity:
-            cap = max(total * 2, 4096)
+            cap = max(total * 2, self._meta_bound())
             # a ring of pinned buffers: the copy of step k may still be in flight
             # while the host fills the buffer of step k+1
             self._meta_ring = [(torch.empty(cap, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
                                for _ in range(4)]
             self._meta_device = torch.empty(cap, dtype=torch.int32, device=self.device)
             self._meta_capacity = cap
+            self._graphs.clear()      # captured graphs point into the old buffer
         pinned, event = self._meta_ring[self.steps_run % len(self._meta_ring)]
         event.synchronize()
         host = pinned.numpy()
@@ -159,10 +167,11 @@ class Engine:
             out[key] = self._meta_device[offsets[key]:offsets[key] + a.size].view(a.shape)
         return out
 
-    def step(self, entries) -> torch.Tensor:
-        """Runs the entries as one batch; returns float32 logits [wanted, vocab] in the
-        order of the entries and of each entry's `want` (None if nothing is wanted).
-        The tensor is a view of the workspace: the next step overwrites it."""
+    def begin(self, entries):
+        """Checks the entries, takes their pages, sends the step's metadata to the
+        device and returns (context, number of wanted rows, key for graph capture or
+        None).  step() is begin + the model + commit; tests of single parts call
+        begin() themselves."""
         entries = list(entries)
         self._check(entries)
         self._reserve(entries)
@@ -188,13 +197,20 @@ class Engine:
         plan.add("segment_lengths", np.asarray([s.length for s in segments]))
         plan.add("segment_rows", np.asarray([s.row0 for s in segments]))
         plan.add("logit_rows", np.asarray(logit_rows))
+        decode_only = self.use_graphs and all(s.length == 1 for s in segments)
+        widths = []
         for g in range(len(self.groups)):
             tables = [self.cache.block_table(s.request_id, g) for s in segments]
             width = max(1, max(len(t) for t in tables))
+            if decode_only:      # few distinct widths, so that few graphs are captured
+                width = min(max(8, 1 << (width - 1).bit_length()), max(width, self._max_blocks()))
+            widths.append(width)
             bt = np.zeros((len(segments), width), dtype=np.int32)
             for i, t in enumerate(tables):
                 bt[i, :len(t)] = [max(p, 0) for p in t]   # pages a window has given back are never read
             plan.add(f"block_tables.{g}", bt)
+        if decode_only:
+            plan.host["graph.max_context"] = max(widths) * self.page_size
         seen = set()
         for entry in self.model.schedule:
             mixer = self.model.blocks[entry.layer].mixer
@@ -212,17 +228,57 @@ class Engine:
             max_position=max(positions), storage=self.storage, workspace=self.workspace,
             page_size=self.page_size, extra=dev, host=plan.host)
 
+        w = len(logit_rows)
+        key = None
+        if decode_only:
+            key = (n, tuple(widths), w, tuple(sorted((k, a.shape) for k, a in plan.arrays.items())))
+        return ctx, w, key
+
+    def commit(self, entries) -> None:
+        for e in entries:
+            self.cache.commit(e.request_id, len(e.tokens))
+        self.steps_run += 1
+
+    def step(self, entries) -> torch.Tensor:
+        """Runs the entries as one batch; returns float32 logits [wanted, vocab] in the
+        order of the entries and of each entry's `want` (None if nothing is wanted).
+        The tensor is a view of the workspace: the next step overwrites it."""
+        entries = list(entries)
+        ctx, w, key = self.begin(entries)
+        n, dev = ctx.n, ctx.extra
+        if key is not None:
+            graph = self._graphs.get(key)
+            if graph is None:
+                logits = self._forward(ctx, n, w, dev)          # this step, eagerly; buffers get made
+                captured = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(captured):
+                    self._forward(ctx, n, w, dev)                # recorded, not run
+                self._graphs[key] = captured
+            else:
+                graph.replay()
+                self.graph_replays += 1
+                logits = self.workspace.rows("logits", w, self.vocab, torch.float32) if w else None
+        else:
+            logits = self._forward(ctx, n, w, dev)
+
+        self.commit(entries)
+        return logits
+
+    def _forward(self, ctx, n: int, w: int, dev: dict):
         x = self.workspace.rows("residual", n, self.model.spec.hidden, torch.float32)
         self.model.embedding.forward(ctx, x)
         for entry in self.model.schedule:
             self.model.blocks[entry.layer].forward(ctx, x, entry)
-        w = len(logit_rows)
-        logits = None
-        if w:
-            logits = self.workspace.rows("logits", w, self.vocab, torch.float32)
-            self.model.head.forward(ctx, logits, x, dev["logit_rows"])
-
-        for e in entries:
-            self.cache.commit(e.request_id, len(e.tokens))
-        self.steps_run += 1
+        if not w:
+            return None
+        logits = self.workspace.rows("logits", w, self.vocab, torch.float32)
+        self.model.head.forward(ctx, logits, x, dev["logit_rows"])
         return logits
+
+    def _max_blocks(self) -> int:
+        return (self.num_positions + self.page_size - 1) // self.page_size
+
+    def _meta_bound(self) -> int:
+        """int32 words that the metadata of the largest step can take."""
+        t, r = self.max_batch_tokens, self.max_requests
+        return 8 * t + 16 * r + len(self.groups) * r * (self._max_blocks() + 4) + 4096

@@ -27,6 +27,8 @@ _DECODE_WAVES = 1024  # waves the decode kernel aims for when it splits the keys
 
 @register_mixer("attention")
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
         self.num_heads = spec.get("num_heads")
@@ -120,12 +122,12 @@ class Attention(Mixer):
             rows = ctx.extra["attention.decode_rows"]
             if rows.numel():
                 nseg = rows.numel()
-                span = ctx.host["attention.decode_max_position"] + 1
+                # under a captured graph the split count is fixed for the whole width of the block table
+                span = ctx.host.get("graph.max_context", ctx.host["attention.decode_max_position"] + 1)
                 if self.window > 0:
                     span = min(span, self.window + _TILE)
                 key_tiles = (span + _TILE - 1) // _TILE
                 splits = max(1, min(key_tiles, _DECODE_WAVES // max(1, nseg * K)))
-                splits = ctx.host.get("attention.decode_splits", splits)
                 partial = None
                 if splits > 1:
                     partial = ctx.workspace.flat("attention.partial", nseg * H * splits * (hd + 2), torch.float32)

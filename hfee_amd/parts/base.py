@@ -63,6 +63,11 @@ def lookup(family: str, kind: str):
 class Part:
     """Base of all parts."""
 
+    # True if forward reads nothing from the host that changes between steps (only
+    # device tensors of the context), so that a decode step may be captured once as
+    # a HIP graph and replayed.  A part that leaves it False keeps its model eager.
+    graph_safe = False
+
     def tensor_specs(self) -> list:
         return []
 
@@ -122,6 +127,7 @@ class Workspace:
         self.capacity = capacity
         self.device = device
         self._buffers: dict = {}
+        self._retired: list = []     # outgrown buffers stay alive: captured graphs may still point at them
 
     def rows(self, name: str, n: int, width: int, dtype: torch.dtype) -> torch.Tensor:
         """A [n, width] view of the buffer `name` ([capacity, width])."""
@@ -137,6 +143,8 @@ class Workspace:
         key = (name, "flat", dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < count:
+            if buf is not None:
+                self._retired.append(buf)
             buf = self._buffers[key] = torch.empty((count,), dtype=dtype, device=self.device)
         return buf[:count]
 

@@ -14,6 +14,8 @@ from .base import FeedForward, register_feed_forward
 
 @register_feed_forward("gated_mlp")
 class GatedMLP(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec: FeedForwardSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
         self.intermediate = spec.get("intermediate")

@@ -10,6 +10,8 @@ from .base import Norm, register_norm
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec: NormSpec, name: str):
         self.width, self.eps, self.name = spec.width, spec.eps, name
         self.weight = None

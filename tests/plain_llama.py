@@ -151,30 +151,36 @@ class PlainLlama:
             for name in f.keys():
                 self.w[name] = f.get_tensor(name).to(F64)
 
-    def forward(self, tokens, upto_layer: int | None = None) -> torch.Tensor:
+    def forward(self, tokens, schedule=None, windows=None) -> torch.Tensor:
         """/root/reference/internal/llm/forward.go:51-142 for one sequence from
-        position 0, logits at every position."""
+        position 0, logits at every position.  schedule: [(layer, cache, writes)] in
+        running order (default: every layer once, its own cache); an entry that does
+        not write reads the keys and values that the entry which wrote `cache` made.
+        windows: {layer: keys kept} for layers with a window."""
         w = self.w
         T = len(tokens)
         pos = list(range(T))
         x = w["model.embed_tokens.weight"][torch.as_tensor(tokens, dtype=torch.long)]   # forward.go:75-77
-        layers = self.L if upto_layer is None else upto_layer
-        for l in range(layers):
+        if schedule is None:
+            schedule = [(l, l, True) for l in range(self.L)]
+        windows = windows or {}
+        caches = {}
+        for l, cache, writes in schedule:
             p = f"model.layers.{l}."
             xb = plain_rmsnorm(x, w[p + "input_layernorm.weight"], self.eps)           # forward.go:82
             q = plain_matmul(xb, w[p + "self_attn.q_proj.weight"]).reshape(T, self.H, self.hd)
-            k = plain_matmul(xb, w[p + "self_attn.k_proj.weight"]).reshape(T, self.K, self.hd)
-            v = plain_matmul(xb, w[p + "self_attn.v_proj.weight"]).reshape(T, self.K, self.hd)
             q = plain_rope(q, pos, self.inv_freq)                                      # forward.go:96-97
-            k = plain_rope(k, pos, self.inv_freq)
-            att = plain_attention(q, k, v).reshape(T, self.H * self.hd)                # forward.go:104
+            if writes:
+                k = plain_matmul(xb, w[p + "self_attn.k_proj.weight"]).reshape(T, self.K, self.hd)
+                v = plain_matmul(xb, w[p + "self_attn.v_proj.weight"]).reshape(T, self.K, self.hd)
+                caches[cache] = (plain_rope(k, pos, self.inv_freq), v)                 # forward.go:99-101
+            k, v = caches[cache]
+            att = plain_attention(q, k, v, window=windows.get(l, 0)).reshape(T, self.H * self.hd)   # forward.go:104
             x = x + plain_matmul(att, w[p + "self_attn.o_proj.weight"])                # forward.go:106-107
             xb = plain_rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps)  # forward.go:109
             h = plain_swiglu(plain_matmul(xb, w[p + "mlp.gate_proj.weight"]),
                              plain_matmul(xb, w[p + "mlp.up_proj.weight"]))            # forward.go:110-112
             x = x + plain_matmul(h, w[p + "mlp.down_proj.weight"])                     # forward.go:113-114
-        if upto_layer is not None:
-            return x
         x = plain_rmsnorm(x, w["model.norm.weight"], self.eps)                         # forward.go:124-128
         head = w["model.embed_tokens.weight"] if self.tied else w["lm_head.weight"]    # model.go:118-121
         return plain_matmul(x, head)                                                   # forward.go:132-141

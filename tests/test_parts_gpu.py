@@ -1,0 +1,399 @@
+"""Each part alone against its plain twin; the run order and the cache groups as
+data (a layer run twice, a layer reading another's cache, a windowed layer); and a
+toy mixer with state of its own, defined here, registered, built and stepped
+without touching the framework's files."""
+import math
+import os
+from dataclasses import dataclass, replace
+
+import numpy as np
+import pytest
+import torch
+
+import trace_util as tu
+from conftest import TINY, TINY_A, make_model_folder
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rel(a, b):
+    a = a.double().cpu() if isinstance(a, torch.Tensor) else torch.as_tensor(np.asarray(a)).double()
+    b = b.double().cpu() if isinstance(b, torch.Tensor) else torch.as_tensor(np.asarray(b)).double()
+    return float((a - b).abs().max() / b.abs().max())
+
+
+# ---------------------------------------------------------------- parts alone ---
+
+def _one_layer_engine(cfg_json, dtype, seed=3):
+    """An engine over a model of the given configuration; its parts are then called
+    one by one with a real step context."""
+    import hfee_amd  # noqa: F401
+    from hfee_amd.config import config_from_dict
+    from hfee_amd.engine import Engine, random_model
+    cfg = config_from_dict(cfg_json)
+    model = random_model(cfg, seed=seed, dtype=dtype, device=DEV, std=0.1)
+    return cfg, model, Engine(model, num_pages=32, page_size=16, max_requests=2, max_batch_tokens=128, use_graphs=False)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_part_alone(dtype):
+    """Sizes unlike any tiny configuration: 10 heads on 5 KV heads of 80, width 112."""
+    from plain_llama import plain_attention, plain_matmul, plain_rope, plain_rope_frequencies
+    from hfee_amd.engine import StepEntry
+    cj = dict(TINY_A, hidden_size=112, num_attention_heads=10, num_key_value_heads=5, head_dim=80,
+              num_hidden_layers=1, rope_theta=777.0)
+    cfg, model, eng = _one_layer_engine(cj, dtype)
+    att = model.blocks[0].mixer
+    T = 45
+    g = torch.Generator().manual_seed(1)
+    h = (torch.randn(T, 112, generator=g)).to(model.dtype)
+    x0 = torch.randn(T, 112, generator=g)
+    eng.admit("r")
+    entries = [StepEntry("r", [1] * T, [])]
+    ctx, _, _ = eng.begin(entries)
+    x = x0.clone().to(DEV)
+    att.forward_add(ctx, x, h.to(DEV), cache_layer=0, writes_cache=True)
+    eng.commit(entries)
+    H, K, hd = 10, 5, 80
+    wq, wk, wv = att.w_qkv.double().cpu().split([H * hd, K * hd, K * hd])
+    inv = plain_rope_frequencies(hd, 777.0)
+    q = plain_rope(plain_matmul(h, wq).reshape(T, H, hd), range(T), inv)
+    k = plain_rope(plain_matmul(h, wk).reshape(T, K, hd), range(T), inv)
+    v = plain_matmul(h, wv).reshape(T, K, hd)
+    want = x0.double() + plain_matmul(plain_attention(q, k, v).reshape(T, H * hd), att.w_o.double().cpu())
+    assert rel(x, want) < (2e-5 if dtype == "float32" else 3e-2)
+    # the same tokens one at a time on a second request give the same rows
+    eng.admit("s")
+    xs = []
+    for t in range(T):
+        entries = [StepEntry("s", [1], [])]
+        ctx, _, _ = eng.begin(entries)
+        xt = x0[t:t + 1].clone().to(DEV)
+        att.forward_add(ctx, xt, h[t:t + 1].to(DEV), 0, True)
+        eng.commit(entries)
+        xs.append(xt.cpu())
+    assert rel(torch.cat(xs), want) < (2e-5 if dtype == "float32" else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_feed_forward_norm_embedding_and_head_alone(dtype):
+    from plain_llama import plain_matmul, plain_rmsnorm, plain_swiglu
+    from hfee_amd.engine import StepEntry
+    cj = dict(TINY_A, hidden_size=72, intermediate_size=100, vocab_size=301, num_attention_heads=3,
+              num_key_value_heads=3, head_dim=16, num_hidden_layers=1, rms_norm_eps=3e-4, tie_word_embeddings=False)
+    cfg, model, eng = _one_layer_engine(cj, dtype)
+    tol = 2e-5 if dtype == "float32" else 3e-2
+    T = 19
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, 301, (T,), generator=g).tolist()
+    eng.admit("r")
+    entries = [StepEntry("r", ids, [0, T - 1])]
+    ctx, w, _ = eng.begin(entries)
+    # embedding
+    x = torch.empty(T, 72, dtype=torch.float32, device=DEV)
+    model.embedding.forward(ctx, x)
+    assert torch.equal(x.cpu(), model.embedding.table.float().cpu()[ids])
+    # norm
+    blk = model.blocks[0]
+    xin = torch.randn(T, 72, generator=g) * 2
+    h = torch.empty(T, 72, dtype=model.dtype, device=DEV)
+    blk.mixer_norm.forward(ctx, h, xin.to(DEV))
+    assert rel(h, plain_rmsnorm(xin, blk.mixer_norm.weight.cpu(), 3e-4)) < tol
+    # feed-forward
+    ff = blk.feed_forward
+    hin = torch.randn(T, 72, generator=g).to(model.dtype)
+    xr = xin.clone().to(DEV)
+    ff.forward_add(ctx, xr, hin.to(DEV))
+    wg, wu = ff.w_gate_up.double().cpu().split([100, 100])
+    want = xin.double() + plain_matmul(plain_swiglu(plain_matmul(hin, wg), plain_matmul(hin, wu)), ff.w_down.double().cpu())
+    assert rel(xr, want) < tol
+    # head: final norm and vocabulary product on the wanted rows only
+    logits = torch.empty(2, 301, dtype=torch.float32, device=DEV)
+    model.head.forward(ctx, logits, xin.to(DEV), ctx.extra["logit_rows"])
+    want = plain_matmul(plain_rmsnorm(xin[[0, T - 1]], model.head.norm.weight.cpu(), 3e-4), model.head.weight.double().cpu())
+    assert rel(logits, want) < tol
+    eng.commit(entries)
+
+
+def test_rotary_part_tables():
+    from plain_llama import plain_rope_frequencies
+    from hfee_amd.config.specs import PositionSpec, params
+    from hfee_amd.parts import Rotary
+    rot = Rotary(PositionSpec("rope", params(head_dim=64, rotary_dim=64, theta=500000.0,
+                                             scaling=("llama3", 8.0, 1.0, 4.0, 8192), pairing="half")))
+    rot.prepare(9000, DEV)
+    inv = plain_rope_frequencies(64, 500000.0, dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                                    original_max_position_embeddings=8192))
+    p = 8191
+    assert torch.allclose(rot.cos[p].double().cpu(), torch.cos(p * inv), atol=1e-7)
+    assert torch.allclose(rot.sin[p].double().cpu(), torch.sin(p * inv), atol=1e-7)
+    with pytest.raises(ValueError, match="pairing"):
+        Rotary(PositionSpec("rope", params(head_dim=8, theta=1.0, pairing="odd")))
+
+
+# ------------------------------------------------ run order and cache groups ---
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layer_twice_shared_cache_and_window(model_folders, dtype):
+    """Schedule: layer 0, layer 1 (window 24, own group), layer 0 again with a cache of
+    its own, layer 1 again reading the cache its first run wrote."""
+    from plain_llama import PlainLlama
+    import hfee_amd  # noqa: F401
+    from hfee_amd.config import config_from_folder, model_spec_of
+    from hfee_amd.config.specs import MixerSpec, ScheduleEntry
+    from hfee_amd.engine import Engine, Model, StepEntry
+    from hfee_amd.weights import load_tensors
+    folder = model_folders[("A", dtype)]
+    cfg = config_from_folder(folder)
+    spec = model_spec_of(cfg)
+    m1 = spec.layers[1].mixer
+    windowed = MixerSpec(m1.kind, tuple(sorted(dict(m1.params, window=24).items())), m1.position)
+    spec = replace(spec, layers=(spec.layers[0], replace(spec.layers[1], mixer=windowed)),
+                   schedule=(ScheduleEntry(0, 0), ScheduleEntry(1, 1), ScheduleEntry(0, 2), ScheduleEntry(1, 1, False)))
+    dt = torch.float32 if dtype == "float32" else torch.bfloat16
+    model = Model(spec, dt)
+    model.bind(load_tensors(folder, model.tensor_specs(), dt, DEV))
+    eng = Engine(model, num_pages=[16, 6], page_size=16, max_requests=2, max_batch_tokens=64)
+    assert sorted(g.kind for g in eng.groups) == ["full", "window"]
+    toks = tu.make_requests(256, [120], seed=8)["r0"]
+    want = PlainLlama(folder).forward(toks, schedule=[(0, 0, True), (1, 1, True), (0, 2, True), (1, 1, False)],
+                                      windows={1: 24})
+    tol = 3e-5 if dtype == "float32" else 5e-2
+    eng.admit("r")
+    got, i = [], 0
+    for n in [7, 16, 2, 33, 1, 1, 1, 20, 5, 34]:          # portions, some decode steps
+        got.append(eng.step([StepEntry("r", toks[i:i + n], list(range(n)))]).cpu().clone())
+        i += n
+        eng.cache.check()
+    assert i == 120
+    assert rel(torch.cat(got), want) < tol
+    # the window group never held more than its window needs: 6 pages were enough for 120 tokens
+    win = [g for g, s in enumerate(eng.groups) if s.kind == "window"][0]
+    assert sum(p >= 0 for p in eng.cache.block_table("r", win)) <= 3
+    eng.release("r")
+    eng.cache.check()
+
+
+# ----------------------------------------------------------- a toy mixer ---
+
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
+    """A mixer with per-request state of fixed size (an exponential moving average of
+    its input, then a projection), in a toy architecture that alternates it with
+    attention.  Everything toy is defined here."""
+    import hfee_amd  # noqa: F401
+    from hfee_amd.config import (ConfigError, FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
+                                 ScheduleEntry, config_from_folder, params, register_architecture)
+    from hfee_amd.config.base import KeyReader
+    from hfee_amd.engine import Engine, StepEntry, load_model
+    from hfee_amd.parts import Mixer, register_mixer
+    from hfee_amd.weights import TensorSpec, write_model_folder
+
+    @register_mixer("toy_ema")
+    class ToyEma(Mixer):
+        def __init__(self, spec, prefix, dtype):
+            self.hidden, self.decay, self.prefix, self.dtype = spec.get("hidden"), spec.get("decay"), prefix, dtype
+            self.state_name = prefix + "state"
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + "proj.weight", (self.hidden, self.hidden))]
+
+        def bind(self, tensors):
+            self.w = tensors.pop(self.prefix + "proj.weight")
+
+        def state_specs(self):
+            return [(self.state_name, (self.hidden,), torch.float32)]
+
+        def prepare(self, info):
+            self.state = info.storage.states[self.state_name]
+
+        def forward_add(self, ctx, x, h, cache_layer, writes_cache):
+            for seg in ctx.segments:                      # tokens of a request in order: state feeds on
+                s = self.state[seg.slot]
+                for r in range(seg.row0, seg.row0 + seg.length):
+                    s.mul_(self.decay).add_(h[r].float(), alpha=1 - self.decay)
+                    x[r] += (self.w.float() @ s)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str
+        hidden: int
+        layers: int
+        vocab: int
+        decay: float
+
+        @staticmethod
+        def from_dict(d, where="config.json"):
+            r = KeyReader(d, where)
+            c = ToyConfig("ToyForCausalLM", r.int("toy_hidden"), r.int("toy_layers"), r.int("toy_vocab"), r.float("toy_decay"))
+            r.finish()
+            return c
+
+        def to_dict(self):
+            return {"architectures": ["ToyForCausalLM"], "toy_hidden": self.hidden, "toy_layers": self.layers,
+                    "toy_vocab": self.vocab, "toy_decay": self.decay}
+
+    def toy_spec(c):
+        norm = NormSpec("rmsnorm", c.hidden, 1e-5)
+        ffn = FeedForwardSpec("gated_mlp", params(hidden=c.hidden, intermediate=2 * c.hidden, activation="silu"))
+        ema = MixerSpec("toy_ema", params(hidden=c.hidden, decay=c.decay))
+        att = MixerSpec("attention", params(hidden=c.hidden, num_heads=2, num_kv_heads=1, head_dim=16, scale=0.25, window=0),
+                        position=PositionSpec("rope", params(head_dim=16, rotary_dim=16, theta=100.0, scaling=None, pairing="half")))
+        layers = tuple(LayerSpec("prenorm", c.hidden, ema if i % 2 == 0 else att, ffn, norm, norm, f"toy.{i}.")
+                       for i in range(c.layers))
+        return ModelSpec("ToyForCausalLM", c.hidden, c.vocab, layers, tuple(ScheduleEntry(i, i) for i in range(c.layers)),
+                         norm, "toy.embed.weight", "toy.norm.weight", None, max_positions=512)
+
+    register_architecture("ToyForCausalLM", ToyConfig, toy_spec)
+    cfg = ToyConfig("ToyForCausalLM", 48, 3, 90, 0.75)
+    folder = write_model_folder(str(tmp_path / "toy"), cfg, seed=1, std=0.1)
+    assert config_from_folder(folder) == cfg
+    model, _ = load_model(folder, "float32")
+    eng = Engine(model, num_pages=16, page_size=16, max_requests=2, max_batch_tokens=64)
+    assert not eng.use_graphs, "a part that reads host data keeps the model eager"
+    assert len(eng.groups) == 1 and eng.groups[0].cache_layers == (1,)
+    assert set(eng.storage.states) == {"toy.0.mixer.state", "toy.2.mixer.state"}
+
+    toks = tu.make_requests(90, [40, 23], seed=3)
+    eng.admit("a")
+    whole = eng.step([StepEntry("a", toks["r0"], list(range(40)))]).cpu().clone()
+    eng.release("a")
+    # in portions, beside another request, on the slot that "a" used: the state starts from zero again
+    eng.admit("b")
+    eng.admit("c")
+    got, i, ci = [], 0, 0
+    for n in [5, 1, 1, 13, 2, 18]:
+        entries = [StepEntry("b", toks["r0"][i:i + n], list(range(n)))]
+        if ci < len(toks["r1"]):
+            entries.insert(0, StepEntry("c", toks["r1"][ci:ci + 3], []))
+            ci += 3
+        got.append(eng.step(entries).cpu().clone())
+        i += n
+    assert torch.allclose(torch.cat(got), whole, atol=1e-5, rtol=1e-5)
+
+    # the plain twin of the toy model's first layer, to show that the state is what it should be
+    w = model.blocks[0].mixer.w.double().cpu()
+    from plain_llama import plain_rmsnorm
+    emb = model.embedding.table.double().cpu()[toks["r0"]]
+    h = plain_rmsnorm(emb, model.blocks[0].mixer_norm.weight.cpu(), 1e-5)
+    s = torch.zeros(48, dtype=torch.float64)
+    for t in range(40):
+        s = 0.75 * s + 0.25 * h[t]
+    assert torch.allclose(eng.storage.states["toy.0.mixer.state"][eng.cache.get("b").slot].double().cpu(), s, atol=1e-5)
+    with pytest.raises(ConfigError, match="toy_hidden"):
+        ToyConfig.from_dict({"architectures": ["ToyForCausalLM"]})
+
+
+# -------------------------------------------------------------- the sampler ---
+
+def test_sampler_kernel_follows_the_plain_rules():
+    from plain_llama import plain_repeat_penalty, plain_sampling_distribution
+    from hfee_amd.sampling import SampleRow, Sampler, SamplingParams, uniform
+    V = 1000
+    g = torch.Generator().manual_seed(0)
+    base = torch.randn(V, generator=g) * 2
+    base[17] = base[400] = base.max() + 0.5          # tied maxima
+    sampler = Sampler(V, DEV, max_rows=64)
+    cases = [SamplingParams(temperature=0.8, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0),
+             SamplingParams(temperature=1.3, top_k=40, top_p=1.0, min_p=0.0, repeat_penalty=1.0),
+             SamplingParams(temperature=1.0, top_k=0, top_p=0.7, min_p=0.0, repeat_penalty=1.0),
+             SamplingParams(temperature=1.0, top_k=0, top_p=1.0, min_p=0.2, repeat_penalty=1.0),
+             SamplingParams(temperature=0.8, top_k=40, top_p=0.9, min_p=0.05, repeat_penalty=1.1, repeat_last_n=64),
+             SamplingParams()]
+    history = torch.randint(0, V, (100,), generator=g).tolist() + [17]
+    for p in cases:
+        pen = plain_repeat_penalty(base, history, p.repeat_penalty, p.repeat_last_n)
+        dist = plain_sampling_distribution(pen, p.temperature, p.top_k, p.top_p, p.min_p)
+        support = set(dist.nonzero().flatten().tolist())
+        counts = torch.zeros(V)
+        exact = 0
+        draws = 64 * 30
+        for c in range(30):
+            logits = base.repeat(64, 1).to(DEV)
+            rows = [SampleRow(p, seed=99, draw=c * 64 + r, history=history, logits_row=r) for r in range(64)]
+            ids = sampler.sample(logits, rows)
+            for r, i in enumerate(ids):
+                counts[i] += 1
+                # the kernel walks the kept set in ascending id with r = u * total
+                cum = torch.cumsum(dist, 0)
+                exact += int(i == int((cum >= uniform(99, c * 64 + r)).nonzero()[0]))
+        assert set(counts.nonzero().flatten().tolist()) <= support, f"{p}: sampled outside the kept set"
+        assert exact >= 0.99 * draws, f"{p}: only {exact} of {draws} draws match the inverse CDF"
+        tv = 0.5 * float((counts / draws - dist.float()).abs().sum())
+        assert tv < 0.12, f"{p}: total variation {tv}"
+    # greedy with and without penalty; one stream per request, whatever shares the call
+    greedy = SamplingParams(temperature=0.0, repeat_penalty=1.0)
+    logits = base.repeat(3, 1).to(DEV)
+    assert sampler.sample(logits, [SampleRow(greedy, 1, 0, [], r) for r in range(3)]) == [17, 17, 17]
+    pen = SamplingParams(temperature=0.0, repeat_penalty=5.0, repeat_last_n=-1)
+    assert sampler.sample(base.repeat(1, 1).to(DEV), [SampleRow(pen, 1, 0, [17], 0)]) == [400]
+    p = SamplingParams(temperature=1.0, top_k=50, top_p=1.0, repeat_penalty=1.0)
+    alone = sampler.sample(base.repeat(1, 1).to(DEV), [SampleRow(p, 7, 5, [], 0)])
+    mixed = sampler.sample(base.repeat(4, 1).to(DEV), [SampleRow(p, 3, 1, [], 0), SampleRow(greedy, 0, 0, [], 1),
+                                                       SampleRow(p, 7, 5, [], 2), SampleRow(p, 8, 5, [], 3)])
+    assert mixed[2] == alone[0] and mixed[1] == 17
+
+
+def test_kernels_refuse_what_they_cannot_do():
+    from hfee_amd.kernels import KernelError, ops
+    with pytest.raises(KernelError, match="GPU tensors"):
+        ops.rmsnorm(torch.empty(1, 4), torch.empty(1, 4), torch.empty(4), 1e-5)
+    with pytest.raises(KernelError, match="shapes"):
+        ops.linear(torch.empty(2, 3, device=DEV), torch.empty(2, 4, device=DEV), torch.empty(3, 5, device=DEV))
+    with pytest.raises(KernelError, match="head sizes"):
+        from hfee_amd.kernels import lib
+        lib.attention_bf16(40)
+    with pytest.raises(ValueError, match="head sizes"):
+        import hfee_amd  # noqa: F401
+        from hfee_amd.config import config_from_dict
+        from hfee_amd.engine import random_model
+        random_model(config_from_dict(dict(TINY_A, head_dim=40)), dtype="bfloat16", device=DEV)
+
+
+def test_attention_finds_a_far_key_among_hundreds():
+    """One key far back is made to stand out (its query and key are scaled); the
+    output must be that key's value, in both kernels of the bfloat16 path and in the
+    32-bit path, also across a page's edge and for the first key of all."""
+    from hfee_amd.kernels import ops
+    H, K, hd, T, ps = 4, 2, 64, 600, 16
+    for dtype in (torch.float32, torch.bfloat16):
+        for far in (0, 15, 16, 333, 599):
+            g = torch.Generator().manual_seed(far)
+            q = torch.randn(T, H, hd, generator=g) * 0.1
+            k = torch.randn(T, K, hd, generator=g) * 0.1
+            v = torch.randn(T, K, hd, generator=g)
+            direction = torch.randn(hd, generator=g)
+            direction /= direction.norm()
+            k[far] = 40 * direction
+            q[T - 1] = 40 * direction
+            nblocks = (T + ps - 1) // ps
+            order = torch.randperm(nblocks + 3, generator=g)[:nblocks].tolist()
+            layer = torch.zeros(nblocks + 3, 2, K, ps * hd)
+            for t in range(T):
+                p, s = order[t // ps], t % ps
+                layer[p, 0].view(K, ps, hd)[:, s] = k[t]
+                layer[p, 1].view(K, hd, ps)[:, :, s] = v[t]
+            layer = layer.to(dtype).to(DEV)
+            table = torch.tensor([order], dtype=torch.int32, device=DEV)
+            qd = q.reshape(T, H * hd).to(dtype).to(DEV)
+            positions = torch.arange(T, dtype=torch.int32, device=DEV)
+            seg = torch.zeros(T, dtype=torch.int32, device=DEV)
+            want = v[far].to(dtype).float().repeat_interleave(H // K, 0).reshape(-1)
+            outs = {}
+            out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+            ops.attention_plain(out, qd, layer, positions, seg, table, H, K, hd, ps, 1.0, 0)
+            outs["plain"] = out[T - 1]
+            if dtype == torch.bfloat16:
+                tiles = torch.tensor([(o, min(32, T - o), o, 0) for o in range(0, T, 32)], dtype=torch.int32, device=DEV)
+                out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+                ops.attention_bf16_prefill(out, qd, layer, tiles, table, H, K, hd, ps, 1.0, 0)
+                outs["prefill"] = out[T - 1]
+                rows = torch.tensor([T - 1], dtype=torch.int32, device=DEV)
+                for splits in (1, 5):
+                    out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+                    partial = torch.zeros(H * splits * (hd + 2), dtype=torch.float32, device=DEV)
+                    ops.attention_bf16_decode(out, qd, layer, rows, rows.clone(), torch.zeros(1, dtype=torch.int32, device=DEV),
+                                              table, H, K, hd, ps, 1.0, 0, partial, splits)
+                    outs[f"decode{splits}"] = out[T - 1]
+            for name, o in outs.items():
+                assert torch.allclose(o.float().cpu(), want, atol=2e-2), (dtype, far, name)

@@ -1,0 +1,184 @@
+"""The scheduler's decisions, on the CPU: a fake engine keeps the real cache manager
+and records what it is fed; the fake sampler's token depends on everything the
+request has been fed so far, so any mistake in what is run changes the output."""
+import hashlib
+
+import pytest
+
+from hfee_amd.cache import CacheGroupSpec, CacheManager
+from hfee_amd.engine.scheduler import PromptTooLong, Request, Scheduler
+from hfee_amd.sampling import SamplingParams
+
+VOCAB = 50
+EOS = 49
+
+
+class FakeEngine:
+    def __init__(self, num_pages, max_requests, page_size=16):
+        self.cache = CacheManager([CacheGroupSpec("full", 1, 16, (0,))], page_size, num_pages, max_requests)
+        self.fed = {}          # request -> tokens in its cache
+        self.batches = []      # per step: [(request, n tokens, wants logits)]
+
+    def admit(self, rid):
+        self.fed[rid] = []
+        return self.cache.admit(rid)
+
+    def release(self, rid):
+        self.cache.release(rid)
+        del self.fed[rid]
+
+    def is_live(self, rid):
+        return rid in self.cache.requests
+
+    def step(self, entries):
+        rows = []
+        assert len({e.request_id for e in entries}) == len(entries)
+        for e in entries:
+            assert len(self.fed[e.request_id]) == self.cache.get(e.request_id).length
+            self.cache.reserve(e.request_id, len(e.tokens))
+            self.fed[e.request_id] += list(e.tokens)
+            self.cache.commit(e.request_id, len(e.tokens))
+            assert e.want in ([], [len(e.tokens) - 1])
+            if e.want:
+                rows.append(tuple(self.fed[e.request_id]))
+        self.batches.append([(e.request_id, len(e.tokens), bool(e.want)) for e in entries])
+        self.cache.check()
+        return rows
+
+
+class FakeSampler:
+    def sample(self, logits, rows):
+        out = []
+        for r in rows:
+            seen = logits[r.logits_row]
+            assert list(seen) == list(r.history), "the cache does not hold the request's history"
+            h = hashlib.sha256(repr((seen, r.seed, r.draw)).encode()).digest()
+            out.append(h[0] % (VOCAB - 1))      # never EOS unless a test asks for it
+        return out
+
+
+def make(num_pages=64, seqs=4, budget=32, ctx=256, eos=()):
+    eng = FakeEngine(num_pages, seqs)
+    return eng, Scheduler(eng, FakeSampler(), max_num_seqs=seqs, max_batch_tokens=budget, num_ctx=ctx,
+                          eos_token_ids=eos, clock=lambda: 0.0)
+
+
+def run_all(sched, limit=10000):
+    done = {}
+    for _ in range(limit):
+        if not sched.has_work():
+            return done
+        for f in sched.step():
+            done[f.request.request_id] = f
+    raise AssertionError("the scheduler did not finish")
+
+
+def prompts():
+    return {i: [(7 * i + j) % (VOCAB - 1) for j in range(n)] for i, n in enumerate([5, 40, 3, 100, 17, 64])}
+
+
+def solo(prompt, rid, n_new, **kw):
+    eng, s = make(**kw)
+    s.add(Request(rid, prompt, SamplingParams.greedy(num_predict=n_new), seed=rid))
+    return run_all(s)[rid].request.generated
+
+
+def test_budget_order_and_portions():
+    eng, s = make(budget=32, seqs=3)
+    ps = prompts()
+    for i in (1, 2, 3):
+        s.add(Request(i, ps[i], SamplingParams.greedy(num_predict=6), seed=i))
+    run_all(s)
+    decoding = set()
+    for batch in eng.batches:
+        assert sum(n for _, n, _ in batch) <= 32, "token budget exceeded"
+        kinds = [rid in decoding for rid, _, _ in batch]
+        assert kinds == sorted(kinds, reverse=True), "decoding requests come first"
+        for rid, n, want in batch:
+            if rid in decoding:
+                assert n == 1 and want
+            if want:
+                decoding.add(rid)
+    # the 100-token prompt was read in portions, logits only at its end (runner.go:256-259)
+    p3 = [(n, want) for b in eng.batches for rid, n, want in b if rid == 3][:6]
+    assert sum(n for n, _ in p3 if n > 1) == 100 and [w for n, w in p3 if n > 1][-1] and not any(w for n, w in p3[:2])
+    # every decoding request is in every step until it ends: never starved
+    first = {rid: min(i for i, b in enumerate(eng.batches) if any(r == rid and w for r, _, w in b)) for rid in (1, 2, 3)}
+    for rid in (1, 2, 3):
+        steps_with = [i for i, b in enumerate(eng.batches) if any(r == rid for r, _, _ in b) and i >= first[rid]]
+        assert steps_with == list(range(first[rid], first[rid] + 6))
+
+
+def test_batched_equals_solo_with_ample_pages():
+    ps = prompts()
+    eng, s = make(num_pages=200, seqs=4, budget=48)
+    for i, p in ps.items():
+        s.add(Request(i, p, SamplingParams.greedy(num_predict=20), seed=i))
+    done = run_all(s)
+    assert max(len(b) for b in eng.batches) == 4, "at most max_num_seqs requests live"
+    for i, p in ps.items():
+        assert done[i].request.generated == solo(p, i, 20) and done[i].reason == "length"
+        assert done[i].request.stats.prompt_tokens == len(p) and done[i].request.stats.eval_tokens == 20
+    eng.cache.check()
+    assert not eng.cache.requests and eng.cache.free_pages() == [200]
+
+
+def test_scarce_pages_preempt_the_youngest_and_give_the_same_tokens():
+    ps = prompts()
+    eng, s = make(num_pages=12, seqs=4, budget=48)      # 192 tokens of cache for 229 + 6 * 30
+    for i, p in ps.items():
+        s.add(Request(i, p, SamplingParams.greedy(num_predict=30), seed=i))
+    done = run_all(s)
+    assert sum(f.request.stats.preemptions for f in done.values()) > 0
+    for i, p in ps.items():
+        assert done[i].request.generated == solo(p, i, 30), f"request {i} changed under preemption"
+    # the request admitted first is never preempted
+    assert done[0].request.stats.preemptions == 0
+    eng.cache.check()
+    assert eng.cache.free_pages() == [12]
+
+
+def test_a_request_too_large_for_the_cache_ends_with_length():
+    eng, s = make(num_pages=2, seqs=2, budget=64)
+    s.add(Request("big", list(range(40)), SamplingParams.greedy(num_predict=5), seed=1))
+    s.add(Request("small", list(range(10)), SamplingParams.greedy(num_predict=5), seed=2))
+    done = run_all(s)
+    assert done["big"].reason == "length" and done["big"].error
+    assert done["small"].reason == "length" and len(done["small"].request.generated) == 5
+    eng.cache.check()
+    assert eng.cache.free_pages() == [2]
+
+
+def test_refusals_and_finish_reasons():
+    eng, s = make(ctx=32, eos=(EOS,))
+    with pytest.raises(PromptTooLong, match="prompt is 32 tokens but the context window is 32"):
+        s.add(Request("x", list(range(32)), SamplingParams.greedy()))
+    with pytest.raises(ValueError):
+        s.add(Request("y", [], SamplingParams.greedy()))
+    # num_predict = 0 still yields one token (runner.go:309-310)
+    s.add(Request("z", [1, 2, 3], SamplingParams.greedy(num_predict=0), seed=3))
+    # no limit: the context window ends it
+    s.add(Request("w", [4, 5, 6, 7], SamplingParams.greedy(), seed=4))
+    done = run_all(s)
+    assert len(done["z"].request.generated) == 1 and done["z"].reason == "length"
+    assert done["w"].reason == "length" and 4 + len(done["w"].request.generated) == 33
+
+
+def test_eos_stops_without_keeping_the_token_and_cancel_frees():
+    class EosSampler(FakeSampler):
+        def sample(self, logits, rows):
+            return [EOS if r.draw == 3 else t for r, t in zip(rows, super().sample(logits, rows))]
+    eng = FakeEngine(32, 2)
+    s = Scheduler(eng, EosSampler(), max_num_seqs=2, max_batch_tokens=16, num_ctx=128, eos_token_ids=(EOS,),
+                  clock=lambda: 0.0)
+    s.add(Request("a", [1, 2, 3], SamplingParams.greedy(num_predict=10), seed=1))
+    s.add(Request("b", [1, 2, 3], SamplingParams.greedy(num_predict=10, ignore_eos=True), seed=1))
+    s.add(Request("c", list(range(30)), SamplingParams.greedy(num_predict=10), seed=1))
+    s.step()
+    s.cancel("c")
+    done = run_all(s)
+    assert done["a"].reason == "stop" and len(done["a"].request.generated) == 3 and EOS not in done["a"].request.generated
+    assert done["b"].reason == "length" and done["b"].request.generated[3] == EOS
+    assert done["c"].reason == "cancelled"
+    eng.cache.check()
+    assert eng.cache.free_pages() == [32] and eng.cache.num_free_slots == 2
