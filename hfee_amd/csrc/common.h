@@ -54,10 +54,8 @@ __device__ __forceinline__ float bf16_to_float(bf16_t v) {
 }
 
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);  // NaN stays NaN
-  u += 0x7fffu + ((u >> 16) & 1u);                                          // round to nearest even
-  return (bf16_t)(u >> 16);
+  // round to nearest even; gfx950 has the conversion in hardware (v_cvt_pk_bf16_f32)
+  return __builtin_bit_cast(bf16_t, (__bf16)f);
 }
 
 template <typename T> __device__ __forceinline__ float to_float(T v);

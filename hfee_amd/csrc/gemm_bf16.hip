@@ -250,6 +250,14 @@ int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, 
 
 }  // namespace
 
+HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
+                              int64_t ldw, int M, int N, int K, int epi,
+                              const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
+                              const int* positions, const int* token_segment, const int* block_tables,
+                              int bt_stride, const float* cos_table, const float* sin_table, int half,
+                              int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
+                              int page_size, hipStream_t stream);
+
 // out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate.
 // force_kernel: 0 choose by M, 1 skinny, 2 tiled (for tests of each kernel alone).
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
@@ -261,6 +269,9 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
   if (M == 0) return 0;
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) &&
                    ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+  if (vec && M <= 64 && force_kernel != 2)      // the streaming kernel with prefetch (gemm_skinny.hip)
+    return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, out_mode, nullptr, 0, 0.f, nullptr, nullptr, nullptr,
+                            nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, stream);
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   int rc;

@@ -1,0 +1,397 @@
+// The decode-time matrix product: C[M,N] = A[M,K] * W[N,K]^T for M <= 64, bound by
+// reading W once from HBM, with the neighbouring small operations folded in so that a
+// decode step of a layer is five launches instead of ten.
+//
+// A workgroup owns 16 weight rows; its eight waves split K in blocks of 128 and
+// stream their share of W straight from global memory into the A operand of
+// v_mfma_f32_16x16x32_bf16 (lane l: row l%16, eight consecutive k).  The batch rows are
+// the B operand.  Loads are issued one block ahead of the matrix instructions.
+// Partial sums meet in LDS and are added in wave order (a fixed order).
+//
+// Folded in:
+//   NORM   the RMSNorm in front of the product
+//          (/root/reference/internal/ggml/ops.go:124-134): A is the float32 residual
+//          stream; x * w is rounded to bfloat16 on the way into the operand, the sum of
+//          squares rides along, and 1/sqrt(mean + eps) scales the finished sums.
+//   EPI_ADD      C (float32) += result        (/root/reference/internal/llm/forward.go:106-107)
+//   EPI_SWIGLU   rows of W alternate gate/up: C[m, j] = silu(gate_j) * up_j
+//                                             (/root/reference/internal/ggml/ops.go:159-165)
+//   EPI_QKV      rows of W are q, k, v heads with rotation pairs adjacent (2i, 2i+1):
+//                rotate q and k at the token's position, write q to C, k and v into the
+//                token's slot of the paged cache
+//                                             (/root/reference/internal/llm/forward.go:96-101)
+#include "common.h"
+
+using namespace hfee;
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_QKV = 4 };
+
+constexpr int WAVES = 8, ROWS = 16, UNROLL = 4, KBLOCK = 32 * UNROLL;
+
+union Chunk {
+  u32x4 u;
+  bf16x8 v;
+  bf16_t e[8];
+};
+
+struct QkvArgs {
+  const int* positions;       // [M]
+  const int* token_segment;   // [M]
+  const int* block_tables;
+  int bt_stride;
+  const float* cos_table;     // [positions][half] or null
+  const float* sin_table;
+  int half;                   // rotated pairs per head
+  void* cache;                // one cache layer, or null (keys and values are not written)
+  CacheLayout lay;
+  int num_heads;
+};
+
+struct Args {
+  void* C;
+  int64_t ldc;
+  const void* A;              // bfloat16 [M, K], or float32 rows when NORM
+  int64_t lda;
+  const bf16_t* W;
+  int64_t ldw;
+  int M, N, K;
+  const void* norm_weight;    // NORM: [K]
+  int norm_weight_is_f32;
+  float eps;
+  const int* rows;            // NORM: row m of the product is row rows[m] of A (null: m)
+  QkvArgs qkv;
+};
+
+struct Block {                // one wave's operands for one K block
+  Chunk w[UNROLL];
+};
+
+template <int MT, bool NORM>
+struct XBlock;
+
+template <int MT>
+struct XBlock<MT, false> {
+  Chunk x[MT][UNROLL];
+};
+
+template <int MT>
+struct XBlock<MT, true> {     // raw float32 activations and the norm weight
+  f32x4 x[MT][UNROLL][2];
+  f32x4 nw[UNROLL][2];
+};
+
+__device__ __forceinline__ f32x4 load_f4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+
+template <int MT, bool NORM>
+__device__ __forceinline__ void load_block(Block& b, XBlock<MT, NORM>& xb, const bf16_t* __restrict__ w_row,
+                                           const void* const* x_rows, const Args& a, int k) {
+  // w_row and x_rows already point at this lane's eight-element column group
+#pragma unroll
+  for (int s = 0; s < UNROLL; ++s) b.w[s].u = *reinterpret_cast<const u32x4*>(w_row + k + 32 * s);
+  if constexpr (!NORM) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int s = 0; s < UNROLL; ++s)
+        xb.x[t][s].u = *reinterpret_cast<const u32x4*>((const bf16_t*)x_rows[t] + k + 32 * s);
+  } else {
+    const int kg = k + 8 * ((threadIdx.x & 63) >> 4);
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) {
+      if (a.norm_weight_is_f32) {
+        xb.nw[s][0] = load_f4((const float*)a.norm_weight + kg + 32 * s);
+        xb.nw[s][1] = load_f4((const float*)a.norm_weight + kg + 32 * s + 4);
+      } else {
+        Chunk c;
+        c.u = *reinterpret_cast<const u32x4*>((const bf16_t*)a.norm_weight + kg + 32 * s);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          xb.nw[s][0][j] = bf16_to_float(c.e[j]);
+          xb.nw[s][1][j] = bf16_to_float(c.e[4 + j]);
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        xb.x[t][s][0] = load_f4((const float*)x_rows[t] + k + 32 * s);
+        xb.x[t][s][1] = load_f4((const float*)x_rows[t] + k + 32 * s + 4);
+      }
+    }
+  }
+}
+
+template <int MT, bool NORM>
+__device__ __forceinline__ void compute_block(f32x4* acc, float* ss, const Block& b, const XBlock<MT, NORM>& xb) {
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) {
+      if constexpr (!NORM) {
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.w[s].v, xb.x[t][s].v, acc[t], 0, 0, 0);
+      } else {
+        Chunk c;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float v = xb.x[t][s][h][j];
+            ss[t] = fmaf(v, v, ss[t]);
+            c.e[4 * h + j] = float_to_bf16(v * xb.nw[s][h][j]);
+          }
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.w[s].v, c.v, acc[t], 0, 0, 0);
+      }
+    }
+}
+
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
+
+template <int MT, bool NORM, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
+  __shared__ float partial[WAVES][MT][64][4];
+  __shared__ float ss_part[WAVES][MT][16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * ROWS;
+  // rows beyond N or M read a valid row; what they produce is never stored
+  const bf16_t* w_row = a.W + (int64_t)min(n0 + r16, a.N - 1) * a.ldw + g * 8;
+  const void* x_rows[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    int m = min(t * 16 + r16, a.M - 1);
+    if (NORM && a.rows) m = a.rows[m];
+    x_rows[t] = NORM ? (const void*)((const float*)a.A + (int64_t)m * a.lda + g * 8)
+                     : (const void*)((const bf16_t*)a.A + (int64_t)m * a.lda + g * 8);
+  }
+
+  f32x4 acc[MT];
+  float ss[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    ss[t] = 0.f;
+  }
+
+  const int nfull = a.K / KBLOCK;
+  {
+    Block cur, nxt;
+    XBlock<MT, NORM> xcur, xnxt;
+    int kb = wave;
+    if (kb < nfull) load_block<MT, NORM>(cur, xcur, w_row, x_rows, a, kb * KBLOCK);
+    while (kb < nfull) {
+      const int kn = kb + WAVES;
+      if (kn < nfull) load_block<MT, NORM>(nxt, xnxt, w_row, x_rows, a, kn * KBLOCK);
+      compute_block<MT, NORM>(acc, ss, cur, xcur);
+      cur = nxt;
+      xcur = xnxt;
+      kb = kn;
+    }
+  }
+  // the last, partial block (K is a multiple of 8: whole chunks are in or out)
+  if (a.K % KBLOCK != 0 && wave == nfull % WAVES) {
+    const int k0 = nfull * KBLOCK;
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) {
+      const int k = k0 + 32 * s + g * 8;      // this lane's first element of the chunk
+      if (k0 + 32 * s >= a.K) break;          // uniform: the whole step is beyond K
+      const bool in = k < a.K;
+      Chunk w;
+      w.u = u32x4{0u, 0u, 0u, 0u};
+      if (in) w.u = *reinterpret_cast<const u32x4*>(w_row + k0 + 32 * s);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        Chunk c;
+        c.u = u32x4{0u, 0u, 0u, 0u};
+        if (in) {
+          if constexpr (!NORM) {
+            c.u = *reinterpret_cast<const u32x4*>((const bf16_t*)x_rows[t] + k0 + 32 * s);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float v = ((const float*)x_rows[t])[k0 + 32 * s + j];
+              const float nw = a.norm_weight_is_f32 ? ((const float*)a.norm_weight)[k + j]
+                                                    : bf16_to_float(((const bf16_t*)a.norm_weight)[k + j]);
+              ss[t] = fmaf(v, v, ss[t]);
+              c.e[j] = float_to_bf16(v * nw);
+            }
+          }
+        }
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.v, c.v, acc[t], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- partial sums meet in LDS ---------------------------------------------------
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) partial[wave][t][lane][i] = acc[t][i];
+    if (NORM) {
+      float s = ss[t];
+      s += __shfl_xor(s, 16, 64);
+      s += __shfl_xor(s, 32, 64);
+      if (g == 0) ss_part[wave][t][r16] = s;
+    }
+  }
+  __syncthreads();
+
+  // D layout of the 16x16 tile: register i of lane l is weight row 4*(l/16) + i, batch row l%16
+  for (int idx = threadIdx.x; idx < MT * 64; idx += WAVES * 64) {
+    const int t = idx >> 6, l = idx & 63;
+    const int m = t * 16 + (l & 15);
+    const int n = n0 + 4 * (l >> 4);
+    if (m >= a.M || n >= a.N) continue;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) s += partial[w][t][l][i];
+      v[i] = s;
+    }
+    if (NORM) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) s += ss_part[w][t][l & 15];
+      const float scale = 1.0f / sqrtf(s / (float)a.K + a.eps);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= scale;
+    }
+
+    if constexpr (EPI == EPI_BF16) {
+      bf16_t* c = (bf16_t*)a.C + (int64_t)m * a.ldc + n;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < a.N) c[i] = float_to_bf16(v[i]);
+    } else if constexpr (EPI == EPI_F32) {
+      float* c = (float*)a.C + (int64_t)m * a.ldc + n;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < a.N) c[i] = v[i];
+    } else if constexpr (EPI == EPI_ADD) {
+      float* c = (float*)a.C + (int64_t)m * a.ldc + n;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < a.N) c[i] += v[i];
+    } else if constexpr (EPI == EPI_SWIGLU) {
+      // rows n, n+1 = gate, up of column n/2; rows n+2, n+3 of column n/2 + 1 (N is even)
+      bf16_t* c = (bf16_t*)a.C + (int64_t)m * a.ldc + (n >> 1);
+      c[0] = float_to_bf16(silu(v[0]) * v[1]);
+      if (n + 2 < a.N) c[1] = float_to_bf16(silu(v[2]) * v[3]);
+    } else {   // EPI_QKV: head sizes are multiples of 4, so the four rows lie in one head
+      const QkvArgs& q = a.qkv;
+      const int hd = q.lay.head_dim;
+      const int head = n / hd, d = n - head * hd;
+      const int pos = q.positions[m];
+      const bool is_v = head >= q.num_heads + q.lay.kv_heads;
+      if (!is_v && q.cos_table != nullptr && d < 2 * q.half) {
+        const float* cs = q.cos_table + (int64_t)pos * q.half + (d >> 1);
+        const float* sn = q.sin_table + (int64_t)pos * q.half + (d >> 1);
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          if (d + 2 * p < 2 * q.half) {
+            const float x0 = v[2 * p], x1 = v[2 * p + 1], c = cs[p], s = sn[p];
+            v[2 * p] = x0 * c - x1 * s;
+            v[2 * p + 1] = x0 * s + x1 * c;
+          }
+        }
+      }
+      bf16_t o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = float_to_bf16(v[i]);
+      if (head < q.num_heads) {
+        *reinterpret_cast<u32x2*>((bf16_t*)a.C + (int64_t)m * a.ldc + n) = *reinterpret_cast<const u32x2*>(o);
+      } else if (q.cache != nullptr) {
+        const int page = q.block_tables[(int64_t)q.token_segment[m] * q.bt_stride + (pos >> q.lay.page_shift)];
+        const int slot = pos & (q.lay.page_size - 1);
+        bf16_t* cache = (bf16_t*)q.cache;
+        if (!is_v) {
+          *reinterpret_cast<u32x2*>(cache + q.lay.key_offset(page, head - q.num_heads, slot, d)) =
+              *reinterpret_cast<const u32x2*>(o);
+        } else {
+          const int kvh = head - q.num_heads - q.lay.kv_heads;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) cache[q.lay.value_offset(page, kvh, slot, d + i)] = o[i];
+        }
+      }
+    }
+  }
+}
+
+template <int MT, bool NORM>
+void launch_epi(const Args& a, int epi, hipStream_t stream) {
+  dim3 grid((a.N + ROWS - 1) / ROWS);
+#define GO(E) skinny_kernel<MT, NORM, E><<<grid, WAVES * 64, 0, stream>>>(a)
+  switch (epi) {
+    case EPI_BF16: GO(EPI_BF16); break;
+    case EPI_F32: GO(EPI_F32); break;
+    case EPI_ADD: GO(EPI_ADD); break;
+    case EPI_SWIGLU: GO(EPI_SWIGLU); break;
+    default: GO(EPI_QKV); break;
+  }
+#undef GO
+}
+
+}  // namespace
+
+// One entry point for every variant.  a_is_f32 != 0 selects the fused RMSNorm (M <= 16).
+// epi: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate, 4 q/k/v.
+HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
+                              int64_t ldw, int M, int N, int K, int epi,
+                              const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
+                              const int* positions, const int* token_segment, const int* block_tables,
+                              int bt_stride, const float* cos_table, const float* sin_table, int half,
+                              int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
+                              int page_size, hipStream_t stream) {
+  HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
+  if (M == 0) return 0;
+  HFEE_REQUIRE(M <= 64, "gemm_skinny: at most 64 rows, got %d", M);
+  HFEE_REQUIRE(epi >= 0 && epi <= 4, "gemm_skinny: unknown epilogue %d", epi);
+  HFEE_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0,
+               "gemm_skinny: K and the leading dimensions must be multiples of 8 and the operands 16-byte aligned");
+  HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_skinny: a leading dimension is shorter than its row");
+  const bool norm = a_is_f32 != 0;
+  if (norm) {
+    HFEE_REQUIRE(M <= 16, "gemm_skinny: the fused norm takes at most 16 rows, got %d", M);
+    HFEE_REQUIRE(norm_weight != nullptr && eps >= 0.f, "gemm_skinny: the fused norm needs its weight");
+    HFEE_REQUIRE((uintptr_t)norm_weight % 16 == 0, "gemm_skinny: the norm weight must be 16-byte aligned");
+  } else {
+    HFEE_REQUIRE(rows == nullptr, "gemm_skinny: a row gather needs the fused norm");
+  }
+  Args a{};
+  a.C = C; a.ldc = ldc; a.A = A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw;
+  a.M = M; a.N = N; a.K = K;
+  a.norm_weight = norm_weight; a.norm_weight_is_f32 = norm_weight_is_f32; a.eps = eps; a.rows = rows;
+  if (epi == EPI_SWIGLU) {
+    HFEE_REQUIRE(N % 2 == 0 && ldc >= N / 2, "gemm_skinny: the SiLU gate needs an even N and ldc >= N/2");
+  } else if (epi == EPI_QKV) {
+    HFEE_REQUIRE(head_dim > 0 && head_dim % 4 == 0 && num_heads > 0 && kv_heads > 0 &&
+                 N == (num_heads + 2 * kv_heads) * head_dim, "gemm_skinny: q/k/v rows do not match the heads");
+    HFEE_REQUIRE(ldc >= (int64_t)num_heads * head_dim && ldc % 4 == 0 && (uintptr_t)C % 8 == 0,
+                 "gemm_skinny: the q output is too narrow or not 8-byte aligned");
+    HFEE_REQUIRE(positions != nullptr, "gemm_skinny: q/k/v needs positions");
+    HFEE_REQUIRE(half >= 0 && 2 * half <= head_dim, "gemm_skinny: rotary width exceeds the head");
+    HFEE_REQUIRE(cos_table == nullptr || table_positions > 0, "gemm_skinny: empty rotation table");
+    if (make_cache_layout(&a.qkv.lay, kv_heads, head_dim, page_size)) return 1;
+    HFEE_REQUIRE(cache == nullptr || (token_segment != nullptr && block_tables != nullptr),
+                 "gemm_skinny: writing the cache needs block tables");
+    a.qkv.positions = positions; a.qkv.token_segment = token_segment; a.qkv.block_tables = block_tables;
+    a.qkv.bt_stride = bt_stride; a.qkv.cos_table = cos_table; a.qkv.sin_table = sin_table; a.qkv.half = half;
+    a.qkv.cache = cache; a.qkv.num_heads = num_heads;
+  } else {
+    HFEE_REQUIRE(ldc >= N, "gemm_skinny: ldc is shorter than a row");
+  }
+  const int mt = (M + 15) / 16;
+  if (norm) launch_epi<1, true>(a, epi, stream);
+  else if (mt == 1) launch_epi<1, false>(a, epi, stream);
+  else if (mt == 2) launch_epi<2, false>(a, epi, stream);
+  else if (mt == 3) launch_epi<3, false>(a, epi, stream);
+  else launch_epi<4, false>(a, epi, stream);
+  HFEE_CHECK_LAUNCH("gemm_skinny");
+  return 0;
+}

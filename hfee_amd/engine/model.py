@@ -77,8 +77,12 @@ class Model:
             if spec is not None and not e.writes_cache:
                 if e.cache not in needs:
                     raise ValueError(f"layer {e.layer} reads cache layer {e.cache}, which no layer writes")
-                if needs[e.cache][1:3] != spec[1:3]:
-                    raise ValueError(f"layer {e.layer} cannot read cache layer {e.cache}: head shapes differ")
+                writer = next(w for w in self.schedule if w.cache == e.cache and w.writes_cache)
+                mine = getattr(self.blocks[e.layer].mixer, "key_layout", lambda: None)()
+                theirs = getattr(self.blocks[writer.layer].mixer, "key_layout", lambda: None)()
+                if needs[e.cache][1:3] != spec[1:3] or mine != theirs:
+                    raise ValueError(f"layer {e.layer} cannot read cache layer {e.cache}: its keys are laid out "
+                                     f"differently from those that layer {writer.layer} writes")
         by_need: dict = {}
         for layer, spec in sorted(needs.items()):
             by_need.setdefault(spec, []).append(layer)

@@ -25,12 +25,13 @@ P, I, L, F, U64 = c_void_p, c_int, c_int64, c_float, c_uint64
 _CORE_SIGNATURES = {
     "hfee_embed": [P, P, I, P, I, I, P],
     "hfee_rmsnorm": [P, I, P, P, I, P, F, I, I, P],
-    "hfee_swiglu": [P, L, P, P, L, I, I, I, P],
+    "hfee_swiglu": [P, L, P, P, L, I, I, I, I, P],
     "hfee_residual_add": [P, P, I, L, P],
     "hfee_rope_cache_write": [P, L, P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, P, I, I, I, I, I, P],
     "hfee_gemm_f32": [P, L, P, L, P, L, I, I, I, I, P],
     "hfee_attention_ref": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "hfee_gemm_bf16": [P, I, L, P, L, P, L, I, I, I, I, P],
+    "hfee_gemm_skinny": [P, L, P, I, L, P, L, I, I, I, I, P, I, F, P, P, P, P, I, P, P, I, I, P, I, I, I, I, P],
     "hfee_argmax": [P, P, L, I, I, P],
     "hfee_sample": [P, P, L, I, I, P, P, P, L, P],
 }

@@ -81,14 +81,15 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
 
 
 def swiglu(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
-    """out = gate / (1 + exp(-gate)) * up; gate and up share a leading dimension."""
+    """out = gate / (1 + exp(-gate)) * up.  gate and up are views of one buffer with the
+    same row and column strides (column stride 1: two blocks; 2: alternating columns)."""
     _gpu(out, gate, up)
     n, w, ldo = _rows2d(out, "swiglu out")
-    ng, wg, ldg = _rows2d(gate, "swiglu gate")
-    nu, wu, ldu = _rows2d(up, "swiglu up")
-    _check((ng, wg) == (n, w) and (nu, wu) == (n, w) and ldg == ldu, "swiglu: shape mismatch")
+    _check(gate.dim() == 2 and up.dim() == 2 and tuple(gate.shape) == (n, w) == tuple(up.shape), "swiglu: shape mismatch")
+    _check(gate.stride() == up.stride() and gate.stride(1) >= 1, "swiglu: gate and up must share their strides")
     _check(out.dtype == gate.dtype == up.dtype, "swiglu: dtype mismatch")
-    lib.core().call("hfee_swiglu", _ptr(out), ldo, _ptr(gate), _ptr(up), ldg, _dt(out), n, w, _stream())
+    ld = gate.stride(0) if n > 1 else max(gate.stride(0), (w - 1) * gate.stride(1) + 1)
+    lib.core().call("hfee_swiglu", _ptr(out), ldo, _ptr(gate), _ptr(up), ld, gate.stride(1), _dt(out), n, w, _stream())
 
 
 def residual_add(x: torch.Tensor, y: torch.Tensor):
@@ -268,3 +269,74 @@ def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tabl
         _ptr(seg_positions), _ptr(seg_tables), count, _ptr(block_tables), block_tables.stride(0),
         num_heads, kv_heads, page_size, float(scale), int(window), _ptr(partial),
         0 if partial is None else partial.numel(), int(num_splits), _stream())
+
+
+# ------------------------------------------------------- fused decode products (M <= 64)
+
+SKINNY_MAX_ROWS = 64
+FUSED_NORM_MAX_ROWS = 16
+_EPI = {"bf16": 0, "f32": 1, "add": 2, "swiglu": 3, "qkv": 4}
+
+
+def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether the streaming kernel takes this product (bfloat16 weight, aligned shapes)."""
+    K = weight.shape[1]
+    return (weight.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and K % 8 == 0
+            and weight.stride(0) % 8 == 0 and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0.0, rows=None, m=None, qkv=None):
+    """out = epilogue(norm(x) @ weight.T) in one launch, for at most 64 rows.
+
+    x: bfloat16 [M, K]; or, with norm_weight, the float32 residual stream (at most 16
+    rows; `rows` optionally gathers them, then `m` is their number).
+    epilogue: "bf16" | "f32" | "add" (out float32 += ...) | "swiglu" (weight rows
+    alternate gate/up; out [M, N/2]) | "qkv" (rotation + cache write; see
+    parts/attention.py; qkv = dict(positions, token_segment, block_tables, cos, sin,
+    cache_layer, num_heads, kv_heads, head_dim, page_size))."""
+    _gpu(out, x, weight, norm_weight, rows)
+    N, K, ldw = _rows2d(weight, "linear_fused weight")
+    Mx, Kx, lda = _rows2d(x, "linear_fused x")
+    M = Mx if m is None else m
+    _check(Kx == K, "linear_fused: inner sizes differ")
+    _check(weight.dtype == torch.bfloat16, "linear_fused: bfloat16 weight expected")
+    fused_norm = norm_weight is not None
+    if fused_norm:
+        _check(x.dtype == torch.float32 and M <= FUSED_NORM_MAX_ROWS, "linear_fused: the fused norm takes <= 16 float32 rows")
+        _check(norm_weight.numel() == K and norm_weight.is_contiguous(), "linear_fused: norm weight width")
+        if rows is not None:
+            _i32(rows, "linear_fused rows", M)
+    else:
+        _check(x.dtype == torch.bfloat16 and rows is None, "linear_fused: bfloat16 x expected")
+    Mo, No, ldc = _rows2d(out, "linear_fused out")
+    _check(Mo >= M, "linear_fused: out has too few rows")
+    epi = _EPI[epilogue]
+    want = {"bf16": torch.bfloat16, "f32": torch.float32, "add": torch.float32, "swiglu": torch.bfloat16,
+            "qkv": torch.bfloat16}[epilogue]
+    _check(out.dtype == want, f"linear_fused: out must be {want} for {epilogue!r}")
+    q = qkv or {}
+    if epilogue == "qkv":
+        H, KV, hd, ps = q["num_heads"], q["kv_heads"], q["head_dim"], q["page_size"]
+        _check(N == (H + 2 * KV) * hd and No == H * hd, "linear_fused: q/k/v shapes")
+        cache = q.get("cache_layer")
+        if cache is not None:
+            _check(cache.is_contiguous() and tuple(cache.shape[1:]) == (2, KV, ps * hd) and cache.dtype == torch.bfloat16,
+                   "linear_fused: cache layer shape")
+            _i32(q["token_segment"], "linear_fused token_segment", M)
+            bt = q["block_tables"]
+            _check(bt.dtype == torch.int32 and bt.dim() == 2 and bt.stride(1) == 1, "linear_fused: block tables")
+        _i32(q["positions"], "linear_fused positions", M)
+        cos, sin = q.get("cos"), q.get("sin")
+        half, table_positions = (cos.shape[1], cos.shape[0]) if cos is not None else (0, 0)
+        bt = q.get("block_tables")
+        lib.core().call("hfee_gemm_skinny", _ptr(out), ldc, _ptr(x), int(fused_norm), lda, _ptr(weight), ldw, M, N, K,
+                        epi, _ptr(norm_weight), int(fused_norm and norm_weight.dtype == torch.float32), float(eps),
+                        _ptr(rows), _ptr(q["positions"]), _ptr(q.get("token_segment")), _ptr(bt),
+                        0 if bt is None else bt.stride(0), _ptr(cos), _ptr(sin), half, table_positions,
+                        _ptr(cache), H, KV, hd, ps, _stream())
+        return
+    _check(No == (N // 2 if epilogue == "swiglu" else N), "linear_fused: out width")
+    lib.core().call("hfee_gemm_skinny", _ptr(out), ldc, _ptr(x), int(fused_norm), lda, _ptr(weight), ldw, M, N, K, epi,
+                    _ptr(norm_weight), int(fused_norm and norm_weight.dtype == torch.float32), float(eps), _ptr(rows),
+                    None, None, None, 0, None, None, 0, 0, None, 0, 0, 0, 0, _stream())

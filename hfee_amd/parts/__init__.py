@@ -1,4 +1,4 @@
-from .base import (Part, Mixer, FeedForward, Norm, Segment, StepContext, Workspace, lookup,
+from .base import (Part, Mixer, FeedForward, Norm, LazyNorm, Segment, StepContext, Workspace, lookup,
                    register_norm, register_position, register_mixer, register_feed_forward, register_block)
 from . import norm, rotary, attention, mlp, embedding, block  # noqa: F401  (registers the built-in parts)
 from .norm import RMSNorm

@@ -10,6 +10,13 @@ The three projections run as one product over the concatenated weight.  In
 bfloat16, portions of prompts go through the tiled matrix-core kernel (tiles of 32
 positions), single decoded tokens through the split-key kernel; in float32 every
 token goes through the plain kernel.
+
+Rotation pairs are made adjacent when the weights are bound: for the pairing
+(i, i + half) the rows of the q and k projections are reordered inside each head to
+(2i, 2i + 1).  Scores are dot products over the head, so reordering q and k alike
+changes nothing (the reference states the same relation between its two pairings,
+/root/reference/internal/llm/forward.go:187-190), and adjacent pairs let a step of at
+most 64 tokens do norm, projections, rotation and the cache write in one launch.
 """
 from __future__ import annotations
 
@@ -19,7 +26,7 @@ import torch
 from ..config.specs import MixerSpec
 from ..kernels import ops
 from ..weights.spec import TensorSpec
-from .base import Mixer, lookup, register_mixer
+from .base import LazyNorm, Mixer, lookup, register_mixer
 
 _TILE = 32            # query rows per workgroup of the prefill kernel
 _DECODE_WAVES = 1024  # waves the decode kernel aims for when it splits the keys
@@ -28,6 +35,7 @@ _DECODE_WAVES = 1024  # waves the decode kernel aims for when it splits the keys
 @register_mixer("attention")
 class Attention(Mixer):
     graph_safe = True
+    takes_lazy_norm = True
 
     def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
@@ -57,11 +65,30 @@ class Attention(Mixer):
                 TensorSpec(p + "v_proj.weight", (self.kv_width, self.hidden)),
                 TensorSpec(p + "o_proj.weight", (self.hidden, self.q_width))]
 
+    def _pair_order(self, device):
+        """Row order inside a head that puts rotation pairs side by side."""
+        pos = self.position
+        order = torch.arange(self.head_dim, device=device)
+        if pos is not None and pos.pairing == 0:
+            half = pos.rotary_dim // 2
+            order[0:2 * half:2] = torch.arange(half, device=device)
+            order[1:2 * half:2] = torch.arange(half, device=device) + half
+        return order
+
     def bind(self, tensors):
         p = self.prefix
-        self.w_qkv = torch.cat([tensors.pop(p + "q_proj.weight"), tensors.pop(p + "k_proj.weight"),
-                                tensors.pop(p + "v_proj.weight")], dim=0).contiguous()
+        wq, wk = tensors.pop(p + "q_proj.weight"), tensors.pop(p + "k_proj.weight")
+        order = self._pair_order(wq.device)
+        wq = wq.view(self.num_heads, self.head_dim, self.hidden)[:, order].reshape(self.q_width, self.hidden)
+        wk = wk.view(self.kv_heads, self.head_dim, self.hidden)[:, order].reshape(self.kv_width, self.hidden)
+        self.w_qkv = torch.cat([wq, wk, tensors.pop(p + "v_proj.weight")], dim=0).contiguous()
         self.w_o = tensors.pop(p + "o_proj.weight").contiguous()
+        self.pairing = 1          # pairs are (2i, 2i + 1) from here on
+
+    def key_layout(self):
+        """What two layers must share to read one cache layer."""
+        pos = self.position
+        return (self.kv_heads, self.head_dim, None if pos is None else (pos.rotary_dim, pos.theta, pos.scaling))
 
     # ---- cache
     def cache_spec(self):
@@ -96,20 +123,31 @@ class Attention(Mixer):
         group = ctx.storage.group_of(cache_layer)
         cache = ctx.storage.layer(cache_layer)
         tables = ctx.block_tables[group]
-        if writes_cache:
-            qkv = ctx.rows("attention.qkv", self.q_width + 2 * self.kv_width)
-            ops.linear(qkv, h, self.w_qkv)
-            q = qkv[:, :self.q_width]
-            k = qkv[:, self.q_width:self.q_width + self.kv_width]
-            v = qkv[:, self.q_width + self.kv_width:]
-        else:   # this run of the layer reads keys and values that another run wrote
-            q = ctx.rows("attention.qkv", self.q_width + 2 * self.kv_width)[:, :self.q_width]
-            ops.linear(q, h, self.w_qkv[:self.q_width])
-            k = v = None
         pos = self.position
-        ops.rope_cache_write(q, k, v, ctx.positions, ctx.token_segment, tables,
-                             pos.cos if pos else None, pos.sin if pos else None, pos.pairing if pos else 0,
-                             cache if writes_cache else None, H, K, hd, ctx.page_size, ctx.max_position)
+        cos, sin = (pos.cos, pos.sin) if pos else (None, None)
+        fused = self.dtype == torch.bfloat16 and n <= ops.SKINNY_MAX_ROWS and self.hidden % 8 == 0
+        qkv = ctx.rows("attention.qkv", self.q_width + 2 * self.kv_width)
+        q = qkv[:, :self.q_width]
+        if fused:
+            # norm, projections, rotation and the cache write in one launch
+            norm = h.fusable() if isinstance(h, LazyNorm) and n <= ops.FUSED_NORM_MAX_ROWS else None
+            a = h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
+            ops.linear_fused(q, a, self.w_qkv, "qkv", norm_weight=norm[0] if norm else None,
+                             eps=norm[1] if norm else 0.0,
+                             qkv=dict(positions=ctx.positions, token_segment=ctx.token_segment, block_tables=tables,
+                                      cos=cos, sin=sin, cache_layer=cache if writes_cache else None,
+                                      num_heads=H, kv_heads=K, head_dim=hd, page_size=ctx.page_size))
+        else:
+            hn = h.tensor() if isinstance(h, LazyNorm) else h
+            if writes_cache:
+                ops.linear(qkv, hn, self.w_qkv)
+                k = qkv[:, self.q_width:self.q_width + self.kv_width]
+                v = qkv[:, self.q_width + self.kv_width:]
+            else:   # this run of the layer reads keys and values that another run wrote
+                ops.linear(q, hn, self.w_qkv[:self.q_width])
+                k = v = None
+            ops.rope_cache_write(q, k, v, ctx.positions, ctx.token_segment, tables, cos, sin, self.pairing,
+                                 cache if writes_cache else None, H, K, hd, ctx.page_size, ctx.max_position)
         att = ctx.rows("attention.out", self.q_width)
         if self.dtype == torch.float32:
             ops.attention_plain(att, q, cache, ctx.positions, ctx.token_segment, tables, H, K, hd,

@@ -67,6 +67,8 @@ class Part:
     # device tensors of the context), so that a decode step may be captured once as
     # a HIP graph and replayed.  A part that leaves it False keeps its model eager.
     graph_safe = False
+    # True if forward_add accepts a LazyNorm in place of the normed tensor.
+    takes_lazy_norm = False
 
     def tensor_specs(self) -> list:
         return []
@@ -106,6 +108,27 @@ class FeedForward(Part):
 class Norm(Part):
     def forward(self, ctx, out, x, rows=None) -> None:
         raise NotImplementedError
+
+
+class LazyNorm:
+    """A normed copy of the residual stream that is made only when someone asks for
+    it.  A part that sets `takes_lazy_norm = True` gets one of these instead of a
+    tensor and may fold the norm into its first product (`fusable()`), or call
+    `tensor()` for the materialised rows."""
+
+    def __init__(self, ctx, norm, x):
+        self.ctx, self.norm, self.x = ctx, norm, x
+        self._tensor = None
+
+    def fusable(self):
+        """(weight, eps) if the norm is y = x / sqrt(mean(x^2) + eps) * weight, else None."""
+        return getattr(self.norm, "fused_form", lambda: None)()
+
+    def tensor(self):
+        if self._tensor is None:
+            self._tensor = self.ctx.rows("block.normed", self.x.shape[1])
+            self.norm.forward(self.ctx, self._tensor, self.x)
+        return self._tensor
 
 
 @dataclass

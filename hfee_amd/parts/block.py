@@ -8,7 +8,7 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import LayerSpec
-from .base import Part, lookup, register_block
+from .base import LazyNorm, Part, lookup, register_block
 
 
 @register_block("prenorm")
@@ -35,8 +35,8 @@ class PreNormBlock(Part):
             p.bind(tensors)
 
     def forward(self, ctx, x, entry):
-        h = ctx.rows("block.normed", self.hidden)
-        self.mixer_norm.forward(ctx, h, x)
-        self.mixer.forward_add(ctx, x, h, entry.cache, entry.writes_cache)
-        self.feed_forward_norm.forward(ctx, h, x)
-        self.feed_forward.forward_add(ctx, x, h)
+        h = LazyNorm(ctx, self.mixer_norm, x)
+        self.mixer.forward_add(ctx, x, h if self.mixer.takes_lazy_norm else h.tensor(), entry.cache,
+                               entry.writes_cache)
+        h = LazyNorm(ctx, self.feed_forward_norm, x)
+        self.feed_forward.forward_add(ctx, x, h if self.feed_forward.takes_lazy_norm else h.tensor())

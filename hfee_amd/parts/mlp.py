@@ -1,7 +1,8 @@
 """The gated feed-forward (/root/reference/internal/llm/forward.go:110-114,
 /root/reference/internal/ggml/ops.go:159-165): down(silu(gate(h)) * up(h)), added to
-the residual stream.  gate and up run as one product over the concatenated weight
-[gate rows; up rows]."""
+the residual stream.  gate and up run as one product over a weight whose rows
+alternate gate_j, up_j, so that a step of at most 64 tokens applies the gate in the
+product's epilogue (and folds the norm in front of it into the same launch)."""
 from __future__ import annotations
 
 import torch
@@ -9,12 +10,13 @@ import torch
 from ..config.specs import FeedForwardSpec
 from ..kernels import ops
 from ..weights.spec import TensorSpec
-from .base import FeedForward, register_feed_forward
+from .base import FeedForward, LazyNorm, register_feed_forward
 
 
 @register_feed_forward("gated_mlp")
 class GatedMLP(FeedForward):
     graph_safe = True
+    takes_lazy_norm = True
 
     def __init__(self, spec: FeedForwardSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
@@ -33,14 +35,21 @@ class GatedMLP(FeedForward):
 
     def bind(self, tensors):
         p = self.prefix
-        self.w_gate_up = torch.cat([tensors.pop(p + "gate_proj.weight"), tensors.pop(p + "up_proj.weight")],
-                                   dim=0).contiguous()
+        self.w_gate_up = torch.stack([tensors.pop(p + "gate_proj.weight"), tensors.pop(p + "up_proj.weight")],
+                                     dim=1).reshape(2 * self.intermediate, self.hidden).contiguous()
         self.w_down = tensors.pop(p + "down_proj.weight").contiguous()
 
     def forward_add(self, ctx, x, h):
         F = self.intermediate
-        gate_up = ctx.rows("mlp.gate_up", 2 * F)
-        ops.linear(gate_up, h, self.w_gate_up)
         act = ctx.rows("mlp.act", F)
-        ops.swiglu(act, gate_up[:, :F], gate_up[:, F:])
+        if self.dtype == torch.bfloat16 and ctx.n <= ops.SKINNY_MAX_ROWS and self.hidden % 8 == 0:
+            norm = h.fusable() if isinstance(h, LazyNorm) and ctx.n <= ops.FUSED_NORM_MAX_ROWS else None
+            a = h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
+            ops.linear_fused(act, a, self.w_gate_up, "swiglu", norm_weight=norm[0] if norm else None,
+                             eps=norm[1] if norm else 0.0)
+        else:
+            hn = h.tensor() if isinstance(h, LazyNorm) else h
+            gate_up = ctx.rows("mlp.gate_up", 2 * F)
+            ops.linear(gate_up, hn, self.w_gate_up)
+            ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
         ops.linear(x, act, self.w_down, accumulate=True)

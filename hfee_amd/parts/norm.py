@@ -22,5 +22,8 @@ class RMSNorm(Norm):
     def bind(self, tensors):
         self.weight = tensors[self.name]
 
+    def fused_form(self):
+        return self.weight, self.eps
+
     def forward(self, ctx, out, x, rows=None):
         ops.rmsnorm(out, x, self.weight, self.eps, rows)

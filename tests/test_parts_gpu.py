@@ -58,8 +58,9 @@ def test_attention_part_alone(dtype):
     H, K, hd = 10, 5, 80
     wq, wk, wv = att.w_qkv.double().cpu().split([H * hd, K * hd, K * hd])
     inv = plain_rope_frequencies(hd, 777.0)
-    q = plain_rope(plain_matmul(h, wq).reshape(T, H, hd), range(T), inv)
-    k = plain_rope(plain_matmul(h, wk).reshape(T, K, hd), range(T), inv)
+    # the part keeps q and k rows with rotation pairs side by side (2i, 2i+1)
+    q = plain_rope(plain_matmul(h, wq).reshape(T, H, hd), range(T), inv, "interleaved")
+    k = plain_rope(plain_matmul(h, wk).reshape(T, K, hd), range(T), inv, "interleaved")
     v = plain_matmul(h, wv).reshape(T, K, hd)
     want = x0.double() + plain_matmul(plain_attention(q, k, v).reshape(T, H * hd), att.w_o.double().cpu())
     assert rel(x, want) < (2e-5 if dtype == "float32" else 3e-2)
@@ -105,7 +106,7 @@ def test_feed_forward_norm_embedding_and_head_alone(dtype):
     hin = torch.randn(T, 72, generator=g).to(model.dtype)
     xr = xin.clone().to(DEV)
     ff.forward_add(ctx, xr, hin.to(DEV))
-    wg, wu = ff.w_gate_up.double().cpu().split([100, 100])
+    wg, wu = ff.w_gate_up.double().cpu()[0::2], ff.w_gate_up.double().cpu()[1::2]     # rows alternate gate, up
     want = xin.double() + plain_matmul(plain_swiglu(plain_matmul(hin, wg), plain_matmul(hin, wu)), ff.w_down.double().cpu())
     assert rel(xr, want) < tol
     # head: final norm and vocabulary product on the wanted rows only
