@@ -67,10 +67,8 @@ __device__ __forceinline__ void attend_tile(Tile& st, const Op* q_op, const bf16
                                             float scale_log2) {
   const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
 
-  // ---- S^T = K Q^T ------------------------------------------------------------
-  f32x16 s;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) s[r] = 0.f;
+  // ---- every load of the tile is issued before the first matrix instruction --------
+  Op kop[NC];
   {
     const int key = k0 + r32;
     const bool ok = key <= kv_last && key >= kv_first;
@@ -78,12 +76,37 @@ __device__ __forceinline__ void attend_tile(Tile& st, const Op* q_op, const bf16
                             : cache;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
-      Op k;
-      k.u = u32x4{0u, 0u, 0u, 0u};
-      if (ok) k.u = *reinterpret_cast<const u32x4*>(krow + c * 16 + G * 8);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k.v, q_op[c].v, s, 0, 0, 0);
+      kop[c].u = u32x4{0u, 0u, 0u, 0u};
+      if (ok) kop[c].u = *reinterpret_cast<const u32x4*>(krow + c * 16 + G * 8);
     }
   }
+  // step u of P V covers keys k0+16u .. k0+16u+15; this lane's operand slots 0..3 are keys
+  // 16u + 4G + 0..3 and slots 4..7 are keys 16u + 8 + 4G + 0..3 (as P holds them).
+  Op vop[2][NDT];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int kb = k0 + 16 * u;
+    const bool ok = kb <= kv_last && kb + 15 >= kv_first;
+    const int page = ok ? bt[kb >> lay.page_shift] : 0;
+    const int slot = (kb & (lay.page_size - 1)) + 4 * G;
+#pragma unroll
+    for (int t = 0; t < NDT; ++t) {
+      const int d = 32 * t + r32;
+      vop[u][t].u = u32x4{0u, 0u, 0u, 0u};
+      if (ok && d < HD) {
+        const bf16_t* vrow = cache + lay.value_offset(page, kvh, slot, d);
+        vop[u][t].h[0] = *reinterpret_cast<const u32x2*>(vrow);
+        vop[u][t].h[1] = *reinterpret_cast<const u32x2*>(vrow + 8);
+      }
+    }
+  }
+
+  // ---- S^T = K Q^T ------------------------------------------------------------
+  f32x16 s;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[c].v, q_op[c].v, s, 0, 0, 0);
 
   // ---- mask, running maximum and sum ------------------------------------------
   float tile_max = -INFINITY;
@@ -115,27 +138,11 @@ __device__ __forceinline__ void attend_tile(Tile& st, const Op* q_op, const bf16
     for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
 
   // ---- O^T += V^T P^T ----------------------------------------------------------
-  // step u covers keys k0+16u .. k0+16u+15; this lane's operand slots 0..3 are keys
-  // 16u + 4G + 0..3 and slots 4..7 are keys 16u + 8 + 4G + 0..3 (as P holds them).
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int kb = k0 + 16 * u;
-    const bool ok = kb <= kv_last && kb + 15 >= kv_first;
-    const int page = ok ? bt[kb >> lay.page_shift] : 0;
-    const int slot = (kb & (lay.page_size - 1)) + 4 * G;
+  for (int u = 0; u < 2; ++u)
 #pragma unroll
-    for (int t = 0; t < NDT; ++t) {
-      const int d = 32 * t + r32;
-      Op v;
-      v.u = u32x4{0u, 0u, 0u, 0u};
-      if (ok && d < HD) {
-        const bf16_t* vrow = cache + lay.value_offset(page, kvh, slot, d);
-        v.h[0] = *reinterpret_cast<const u32x2*>(vrow);
-        v.h[1] = *reinterpret_cast<const u32x2*>(vrow + 8);
-      }
-      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v.v, p[u].v, st.o[t], 0, 0, 0);
-    }
-  }
+    for (int t = 0; t < NDT; ++t)
+      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vop[u][t].v, p[u].v, st.o[t], 0, 0, 0);
 }
 
 __device__ __forceinline__ void load_query(Op* q_op, const bf16_t* __restrict__ qrow, bool ok) {
@@ -204,21 +211,24 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
 }
 
 // -------------------------------------------------------------------- decode ---
-// One workgroup (one wave) per (decode segment, KV head, split).  The slots are
-// the heads of the group, 32 at a time.  partial: per (segment, head, split)
-// HD + 2 floats: the unnormalised output, the maximum, the sum.
-__global__ __launch_bounds__(64) void decode_kernel(bf16_t* __restrict__ out, int64_t ld_out,
-                                                    const bf16_t* __restrict__ q, int64_t ldq,
-                                                    const bf16_t* __restrict__ cache, CacheLayout lay,
-                                                    const int* __restrict__ seg_rows,
-                                                    const int* __restrict__ seg_positions,
-                                                    const int* __restrict__ seg_tables,
-                                                    const int* __restrict__ block_tables, int bt_stride,
-                                                    int num_heads, float scale_log2, int window,
-                                                    float* __restrict__ partial, int num_splits) {
-  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+// One workgroup of DECODE_WAVES waves per (decode segment, KV head, split).  The slots
+// are the heads of the group, 32 at a time.  The workgroup's key tiles are dealt to its
+// waves in turn; their running states meet in LDS and are joined in wave order.  With
+// one split the result is final; otherwise it goes to `partial` as HD + 2 floats per
+// (segment, head, split): the unnormalised output, the maximum, the sum.
+constexpr int DECODE_WAVES = 4;
+
+__global__ __launch_bounds__(DECODE_WAVES * 64) void decode_kernel(
+    bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
+    const bf16_t* __restrict__ cache, CacheLayout lay, const int* __restrict__ seg_rows,
+    const int* __restrict__ seg_positions, const int* __restrict__ seg_tables,
+    const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2, int window,
+    float* __restrict__ partial, int num_splits) {
+  extern __shared__ float lds[];   // [DECODE_WAVES][slots][HD + 2]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r32 = lane & 31, G = lane >> 5;
   const int sidx = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int group = num_heads / lay.kv_heads;
+  const int slots = min(group, 32);
   const int row = seg_rows[sidx], pos = seg_positions[sidx];
   const int* bt = block_tables + (int64_t)seg_tables[sidx] * bt_stride;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
@@ -236,59 +246,104 @@ __global__ __launch_bounds__(64) void decode_kernel(bf16_t* __restrict__ out, in
     load_query(q_op, q + (int64_t)row * ldq + h * HD, slot_ok);
     Tile st;
     init_tile(st);
-    for (int t = t_begin; t < t_end; ++t)
+    for (int t = t_begin + wave; t < t_end; t += DECODE_WAVES)
       attend_tile(st, q_op, cache, lay, bt, kvh, t * 32, lo, pos, slot_ok ? pos : -1, lo, scale_log2);
-    if (!slot_ok) continue;
-    if (num_splits == 1) {
-      const float inv = 1.0f / st.l;
-      bf16_t* orow = out + (int64_t)row * ld_out + h * HD;
-#pragma unroll
-      for (int t = 0; t < NDT; ++t)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          const int d = 32 * t + 8 * b + 4 * G;
-          if (d < HD) {
-            bf16_t v4[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) v4[i] = float_to_bf16(st.o[t][4 * b + i] * inv);
-            *reinterpret_cast<u32x2*>(orow + d) = *reinterpret_cast<const u32x2*>(v4);
-          }
-        }
-    } else {
-      float* pr = partial + ((int64_t)(sidx * num_heads + h) * num_splits + split) * (HD + 2);
+
+    // this wave's state into LDS
+    if (g0 > 0) __syncthreads();
+    if (slot_ok) {
+      float* mine = lds + (int64_t)(wave * slots + r32) * (HD + 2);
 #pragma unroll
       for (int t = 0; t < NDT; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int d = 32 * t + 8 * (r >> 2) + 4 * G + (r & 3);
-          if (d < HD) pr[d] = st.o[t][r];
+          if (d < HD) mine[d] = st.o[t][r];
         }
       if (G == 0) {
-        pr[HD] = st.m;
-        pr[HD + 1] = st.l;
+        mine[HD] = st.m;
+        mine[HD + 1] = st.l;
+      }
+    }
+    __syncthreads();
+
+    // join the waves: thread -> (slot, four consecutive dims)
+    const int valid = min(32, group - g0);
+    for (int idx = threadIdx.x; idx < valid * (HD / 4); idx += DECODE_WAVES * 64) {
+      const int sl = idx / (HD / 4), d = 4 * (idx - sl * (HD / 4));
+      float m = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < DECODE_WAVES; ++w) m = fmaxf(m, lds[(int64_t)(w * slots + sl) * (HD + 2) + HD]);
+      const float m_use = m == -INFINITY ? 0.f : m;
+      float l = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < DECODE_WAVES; ++w) {
+        const float* src = lds + (int64_t)(w * slots + sl) * (HD + 2);
+        const float f = exp2f(src[HD] - m_use);
+        l += src[HD + 1] * f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] += src[d + i] * f;
+      }
+      const int head = kvh * group + g0 + sl;
+      if (num_splits == 1) {
+        const float inv = 1.0f / l;
+        bf16_t v4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v4[i] = float_to_bf16(o[i] * inv);
+        *reinterpret_cast<u32x2*>(out + (int64_t)row * ld_out + head * HD + d) = *reinterpret_cast<const u32x2*>(v4);
+      } else {
+        float* pr = partial + ((int64_t)(sidx * num_heads + head) * num_splits + split) * (HD + 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pr[d + i] = o[i];
+        if (d == 0) {
+          pr[HD] = m;
+          pr[HD + 1] = l;
+        }
       }
     }
   }
 }
 
-// Joins the splits of one (segment, head) in ascending split order.
+// Joins the splits of one (segment, head) in ascending split order: lane s holds the
+// weight of split s, every lane then walks the splits for its own dims.
 __global__ __launch_bounds__(64) void combine_kernel(bf16_t* __restrict__ out, int64_t ld_out,
                                                      const int* __restrict__ seg_rows,
                                                      const float* __restrict__ partial, int num_heads,
                                                      int num_splits) {
   const int sidx = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* pr = partial + (int64_t)(sidx * num_heads + h) * num_splits * (HD + 2);
-  float m = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) m = fmaxf(m, pr[s * (HD + 2) + HD]);
-  const float m_use = m == -INFINITY ? 0.f : m;
-  float l = 0.f;
-  for (int s = 0; s < num_splits; ++s) l += pr[s * (HD + 2) + HD + 1] * exp2f(pr[s * (HD + 2) + HD] - m_use);
+  float m = -INFINITY, l = 0.f;
+  float o[(HD + 63) / 64];
+#pragma unroll
+  for (int j = 0; j < (HD + 63) / 64; ++j) o[j] = 0.f;
+  for (int s0 = 0; s0 < num_splits; s0 += 64) {          // 64 splits at a time
+    const int mine = s0 + lane;
+    const float ms = mine < num_splits ? pr[(int64_t)mine * (HD + 2) + HD] : -INFINITY;
+    const float ls = mine < num_splits ? pr[(int64_t)mine * (HD + 2) + HD + 1] : 0.f;
+    const float m_new = fmaxf(m, wave_max(ms));
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float rescale = exp2f(m - m_use);
+    const float f = exp2f(ms - m_use);                    // this lane's split weight
+    l = l * rescale + wave_sum(ls * f);
+#pragma unroll
+    for (int j = 0; j < (HD + 63) / 64; ++j) o[j] *= rescale;
+    const int count = min(64, num_splits - s0);
+    for (int s = 0; s < count; ++s) {
+      const float fs = __shfl(f, s, 64);
+#pragma unroll
+      for (int j = 0; j < (HD + 63) / 64; ++j) {
+        const int d = lane + 64 * j;
+        if (d < HD) o[j] += pr[(int64_t)(s0 + s) * (HD + 2) + d] * fs;
+      }
+    }
+    m = m_new;
+  }
   const float inv = 1.0f / l;
   bf16_t* orow = out + (int64_t)seg_rows[sidx] * ld_out + h * HD;
-  for (int d = lane; d < HD; d += 64) {
-    float o = 0.f;
-    for (int s = 0; s < num_splits; ++s) o += pr[s * (HD + 2) + d] * exp2f(pr[s * (HD + 2) + HD] - m_use);
-    orow[d] = float_to_bf16(o * inv);
+#pragma unroll
+  for (int j = 0; j < (HD + 63) / 64; ++j) {
+    const int d = lane + 64 * j;
+    if (d < HD) orow[d] = float_to_bf16(o[j] * inv);
   }
 }
 
@@ -348,7 +403,16 @@ HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q
                  (long long)partial_floats, (long long)need);
   }
   dim3 grid(num_segments, kv_heads, num_splits);
-  decode_kernel<<<grid, 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
+  const int group = num_heads / kv_heads;
+  const size_t lds = (size_t)DECODE_WAVES * (group < 32 ? group : 32) * (HD + 2) * sizeof(float);
+  static bool raised = false;
+  if (lds > 48 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)decode_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)(DECODE_WAVES * 32 * (HD + 2) * sizeof(float)));
+    HFEE_REQUIRE(e == hipSuccess, "attention_bf16_decode: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  decode_kernel<<<grid, DECODE_WAVES * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
                                          seg_rows, seg_positions, seg_tables, block_tables, bt_stride, num_heads,
                                          scale * LOG2E, window, partial, num_splits);
   HFEE_CHECK_LAUNCH("attention_bf16_decode");

@@ -275,6 +275,9 @@ def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tabl
 
 SKINNY_MAX_ROWS = 64
 FUSED_NORM_MAX_ROWS = 16
+# folding the norm into the product makes every workgroup convert the activations
+# itself; beyond this many weight rows a separate norm kernel is cheaper
+FUSED_NORM_MAX_N = 8192
 _EPI = {"bf16": 0, "f32": 1, "add": 2, "swiglu": 3, "qkv": 4}
 
 

@@ -130,7 +130,8 @@ class Attention(Mixer):
         q = qkv[:, :self.q_width]
         if fused:
             # norm, projections, rotation and the cache write in one launch
-            norm = h.fusable() if isinstance(h, LazyNorm) and n <= ops.FUSED_NORM_MAX_ROWS else None
+            norm = h.fusable() if (isinstance(h, LazyNorm) and n <= ops.FUSED_NORM_MAX_ROWS
+                                   and self.w_qkv.shape[0] <= ops.FUSED_NORM_MAX_N) else None
             a = h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
             ops.linear_fused(q, a, self.w_qkv, "qkv", norm_weight=norm[0] if norm else None,
                              eps=norm[1] if norm else 0.0,
