@@ -56,19 +56,22 @@ struct Tile {
   f32x16 o[NDT];        // O^T: register r of tile t is dim 32t + 8*(r/4) + 4*(lane/32) + r%4
 };
 
-// Adds the keys k0 .. k0+31 of one sequence to the running state.
-// q_op: this slot's query, pre-loaded as NC operands.  pos: this slot's position
-// (keys lo..pos are visible; -1 for an unused slot).  kv_first..kv_last: the keys
-// whose pages may be touched at all (a window group has given back the pages
-// before kv_first; nothing exists after kv_last).
-__device__ __forceinline__ void attend_tile(Tile& st, const Op* q_op, const bf16_t* __restrict__ cache,
-                                            const CacheLayout& lay, const int* __restrict__ bt, int kvh,
-                                            int k0, int kv_first, int kv_last, int pos, int lo,
-                                            float scale_log2) {
-  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+// The operands of one tile of 32 keys: the key rows for S^T = K Q^T and the value
+// columns for O^T += V^T P^T.  Step u of P V covers keys k0+16u .. k0+16u+15; a lane's
+// operand slots 0..3 are keys 16u + 4G + 0..3 and slots 4..7 keys 16u + 8 + 4G + 0..3
+// (as P holds them after the first product): the cache stores a value column's slots
+// in exactly that order, so the operand is one 16-byte load.
+struct TileOps {
+  Op k[NC];
+  Op v[2][NDT];
+};
 
-  // ---- every load of the tile is issued before the first matrix instruction --------
-  Op kop[NC];
+// Issues every load of the tile k0 .. k0+31.  kv_first..kv_last: the keys whose pages
+// may be touched at all (a window group has given back the pages before kv_first;
+// nothing exists after kv_last); the rest reads as zeros.
+__device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict__ cache, const CacheLayout& lay,
+                                          const int* __restrict__ bt, int kvh, int k0, int kv_first, int kv_last) {
+  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
   {
     const int key = k0 + r32;
     const bool ok = key <= kv_last && key >= kv_first;
@@ -76,37 +79,39 @@ __device__ __forceinline__ void attend_tile(Tile& st, const Op* q_op, const bf16
                             : cache;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
-      kop[c].u = u32x4{0u, 0u, 0u, 0u};
-      if (ok) kop[c].u = *reinterpret_cast<const u32x4*>(krow + c * 16 + G * 8);
+      ops.k[c].u = u32x4{0u, 0u, 0u, 0u};
+      if (ok) ops.k[c].u = *reinterpret_cast<const u32x4*>(krow + c * 16 + G * 8);
     }
   }
-  // step u of P V covers keys k0+16u .. k0+16u+15; this lane's operand slots 0..3 are keys
-  // 16u + 4G + 0..3 and slots 4..7 are keys 16u + 8 + 4G + 0..3 (as P holds them).
-  Op vop[2][NDT];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int kb = k0 + 16 * u;
     const bool ok = kb <= kv_last && kb + 15 >= kv_first;
     const int page = ok ? bt[kb >> lay.page_shift] : 0;
-    const int slot = (kb & (lay.page_size - 1)) + 4 * G;
+    const int first = (kb & (lay.page_size - 1)) + 8 * G;      // stored order: 4G.., 8+4G.. are adjacent
 #pragma unroll
     for (int t = 0; t < NDT; ++t) {
       const int d = 32 * t + r32;
-      vop[u][t].u = u32x4{0u, 0u, 0u, 0u};
-      if (ok && d < HD) {
-        const bf16_t* vrow = cache + lay.value_offset(page, kvh, slot, d);
-        vop[u][t].h[0] = *reinterpret_cast<const u32x2*>(vrow);
-        vop[u][t].h[1] = *reinterpret_cast<const u32x2*>(vrow + 8);
-      }
+      ops.v[u][t].u = u32x4{0u, 0u, 0u, 0u};
+      if (ok && d < HD)
+        ops.v[u][t].u = *reinterpret_cast<const u32x4*>(cache + lay.value_column(page, kvh, d) + first);
     }
   }
+}
+
+// Adds the keys k0 .. k0+31 (already loaded) to the running state.  q_op: this slot's
+// query, pre-loaded as NC operands.  pos: this slot's position (keys lo..pos are
+// visible; -1 for an unused slot).
+__device__ __forceinline__ void compute_tile(Tile& st, const Op* q_op, const TileOps& ops, int k0, int pos, int lo,
+                                             float scale_log2) {
+  const int lane = threadIdx.x & 63, G = lane >> 5;
 
   // ---- S^T = K Q^T ------------------------------------------------------------
   f32x16 s;
 #pragma unroll
   for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
-  for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[c].v, q_op[c].v, s, 0, 0, 0);
+  for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops.k[c].v, q_op[c].v, s, 0, 0, 0);
 
   // ---- mask, running maximum and sum ------------------------------------------
   float tile_max = -INFINITY;
@@ -142,7 +147,34 @@ __device__ __forceinline__ void attend_tile(Tile& st, const Op* q_op, const bf16
   for (int u = 0; u < 2; ++u)
 #pragma unroll
     for (int t = 0; t < NDT; ++t)
-      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vop[u][t].v, p[u].v, st.o[t], 0, 0, 0);
+      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops.v[u][t].v, p[u].v, st.o[t], 0, 0, 0);
+}
+
+// The tiles first, first + step, ... < end of one sequence.  AHEAD: each tile's loads
+// are issued while the tile before it is computed (two tiles' operands in registers:
+// for kernels that run one wave per SIMD anyway); otherwise tile by tile.
+template <bool AHEAD>
+__device__ __forceinline__ void attend_tiles(Tile& st, const Op* q_op, const bf16_t* __restrict__ cache,
+                                             const CacheLayout& lay, const int* __restrict__ bt, int kvh,
+                                             int first, int end, int step, int kv_first, int kv_last, int pos,
+                                             int lo, float scale_log2) {
+  if (first >= end) return;
+  if constexpr (AHEAD) {
+    TileOps cur, nxt;
+    load_tile(cur, cache, lay, bt, kvh, first * 32, kv_first, kv_last);
+    for (int t = first; t < end; t += step) {
+      const int tn = t + step;
+      if (tn < end) load_tile(nxt, cache, lay, bt, kvh, tn * 32, kv_first, kv_last);
+      compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2);
+      cur = nxt;
+    }
+  } else {
+    for (int t = first; t < end; t += step) {
+      TileOps cur;
+      load_tile(cur, cache, lay, bt, kvh, t * 32, kv_first, kv_last);
+      compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2);
+    }
+  }
 }
 
 __device__ __forceinline__ void load_query(Op* q_op, const bf16_t* __restrict__ qrow, bool ok) {
@@ -189,8 +221,8 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
   init_tile(st);
   const int kv_last = pos0 + rows - 1;
   const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
-  for (int k0 = kv_first & ~31; k0 <= kv_last; k0 += 32)
-    attend_tile(st, q_op, cache, lay, bt, kvh, k0, kv_first, kv_last, pos, lo, scale_log2);
+  attend_tiles<false>(st, q_op, cache, lay, bt, kvh, kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
+               scale_log2);
 
   if (slot_ok) {
     const float inv = 1.0f / st.l;
@@ -211,21 +243,22 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
 }
 
 // -------------------------------------------------------------------- decode ---
-// One workgroup of DECODE_WAVES waves per (decode segment, KV head, split).  The slots
+// One workgroup of up to four waves per (decode segment, KV head, split).  The slots
 // are the heads of the group, 32 at a time.  The workgroup's key tiles are dealt to its
 // waves in turn; their running states meet in LDS and are joined in wave order.  With
 // one split the result is final; otherwise it goes to `partial` as HD + 2 floats per
 // (segment, head, split): the unnormalised output, the maximum, the sum.
-constexpr int DECODE_WAVES = 4;
+constexpr int DECODE_MAX_WAVES = 4;      // each wave holds two tiles' operands: registers allow no more
 
-__global__ __launch_bounds__(DECODE_WAVES * 64) void decode_kernel(
+__global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, CacheLayout lay, const int* __restrict__ seg_rows,
     const int* __restrict__ seg_positions, const int* __restrict__ seg_tables,
     const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2, int window,
     float* __restrict__ partial, int num_splits) {
-  extern __shared__ float lds[];   // [DECODE_WAVES][slots][HD + 2]
+  extern __shared__ float lds[];   // [waves][slots][HD + 2]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r32 = lane & 31, G = lane >> 5;
+  const int waves = blockDim.x >> 6;
   const int sidx = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int group = num_heads / lay.kv_heads;
   const int slots = min(group, 32);
@@ -246,8 +279,8 @@ __global__ __launch_bounds__(DECODE_WAVES * 64) void decode_kernel(
     load_query(q_op, q + (int64_t)row * ldq + h * HD, slot_ok);
     Tile st;
     init_tile(st);
-    for (int t = t_begin + wave; t < t_end; t += DECODE_WAVES)
-      attend_tile(st, q_op, cache, lay, bt, kvh, t * 32, lo, pos, slot_ok ? pos : -1, lo, scale_log2);
+    attend_tiles<true>(st, q_op, cache, lay, bt, kvh, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
+                 scale_log2);
 
     // this wave's state into LDS
     if (g0 > 0) __syncthreads();
@@ -269,15 +302,13 @@ __global__ __launch_bounds__(DECODE_WAVES * 64) void decode_kernel(
 
     // join the waves: thread -> (slot, four consecutive dims)
     const int valid = min(32, group - g0);
-    for (int idx = threadIdx.x; idx < valid * (HD / 4); idx += DECODE_WAVES * 64) {
+    for (int idx = threadIdx.x; idx < valid * (HD / 4); idx += blockDim.x) {
       const int sl = idx / (HD / 4), d = 4 * (idx - sl * (HD / 4));
       float m = -INFINITY;
-#pragma unroll
-      for (int w = 0; w < DECODE_WAVES; ++w) m = fmaxf(m, lds[(int64_t)(w * slots + sl) * (HD + 2) + HD]);
+      for (int w = 0; w < waves; ++w) m = fmaxf(m, lds[(int64_t)(w * slots + sl) * (HD + 2) + HD]);
       const float m_use = m == -INFINITY ? 0.f : m;
       float l = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int w = 0; w < DECODE_WAVES; ++w) {
+      for (int w = 0; w < waves; ++w) {
         const float* src = lds + (int64_t)(w * slots + sl) * (HD + 2);
         const float f = exp2f(src[HD] - m_use);
         l += src[HD + 1] * f;
@@ -387,7 +418,7 @@ HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q
                                         const int* seg_rows, const int* seg_positions, const int* seg_tables,
                                         int num_segments, const int* block_tables, int bt_stride,
                                         int num_heads, int kv_heads, int page_size, float scale, int window,
-                                        float* partial, int64_t partial_floats, int num_splits,
+                                        float* partial, int64_t partial_floats, int num_splits, int waves,
                                         hipStream_t stream) {
   HFEE_REQUIRE(num_segments >= 0, "attention_bf16_decode: bad segment count");
   if (num_segments == 0) return 0;
@@ -404,15 +435,20 @@ HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q
   }
   dim3 grid(num_segments, kv_heads, num_splits);
   const int group = num_heads / kv_heads;
-  const size_t lds = (size_t)DECODE_WAVES * (group < 32 ? group : 32) * (HD + 2) * sizeof(float);
+  const size_t per_wave = (size_t)(group < 32 ? group : 32) * (HD + 2) * sizeof(float);
+  HFEE_REQUIRE(waves >= 1 && waves <= DECODE_MAX_WAVES, "attention_bf16_decode: 1..%d waves, got %d",
+               DECODE_MAX_WAVES, waves);
+  while (waves > 1 && waves * per_wave > 60 * 1024) waves /= 2;     // the waves' states must fit in LDS
+  const size_t lds = waves * per_wave;
   static bool raised = false;
   if (lds > 48 * 1024 && !raised) {
     hipError_t e = hipFuncSetAttribute((const void*)decode_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)(DECODE_WAVES * 32 * (HD + 2) * sizeof(float)));
+                                       (int)(DECODE_MAX_WAVES * 32 * (HD + 2) * sizeof(float) < 160 * 1024
+                                                 ? DECODE_MAX_WAVES * 32 * (HD + 2) * sizeof(float) : 160 * 1024));
     HFEE_REQUIRE(e == hipSuccess, "attention_bf16_decode: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
-  decode_kernel<<<grid, DECODE_WAVES * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
+  decode_kernel<<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
                                          seg_rows, seg_positions, seg_tables, block_tables, bt_stride, num_heads,
                                          scale * LOG2E, window, partial, num_splits);
   HFEE_CHECK_LAUNCH("attention_bf16_decode");

@@ -107,8 +107,11 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 
 // ---- the paged cache's layout -------------------------------------------------
 // One cache layer is [num_pages][2][kv_heads][page_size * head_dim] elements:
-// keys of a (page, head) as [slot][head_dim], values transposed as [head_dim][slot],
-// so that eight consecutive keys of one value column are 16 contiguous bytes in bf16.
+// keys of a (page, head) as [slot][head_dim], values transposed as [head_dim][slot'],
+// where slot' is the slot with bits 2 and 3 exchanged: within every 16 slots the order
+// is 0-3, 8-11, 4-7, 12-15.  The matrix-core attention holds, per lane, the keys
+// 4G..4G+3 and 8+4G..8+4G+3 of a 16-key step; stored this way they are 16 contiguous
+// bytes of one value column in bfloat16.
 struct CacheLayout {
   int64_t page_stride;   // elements between pages: 2 * kv_heads * page_size * head_dim
   int kv_heads;
@@ -119,9 +122,15 @@ struct CacheLayout {
   __host__ __device__ __forceinline__ int64_t key_offset(int page, int kvh, int slot, int d) const {
     return (int64_t)page * page_stride + (int64_t)kvh * page_size * head_dim + (int64_t)slot * head_dim + d;
   }
+  __host__ __device__ static __forceinline__ int value_slot(int slot) {
+    return (slot & ~12) | ((slot & 4) << 1) | ((slot & 8) >> 1);
+  }
+  // first element of value column d of a (page, head): page_size slots follow
+  __host__ __device__ __forceinline__ int64_t value_column(int page, int kvh, int d) const {
+    return (int64_t)page * page_stride + (int64_t)(kv_heads + kvh) * page_size * head_dim + (int64_t)d * page_size;
+  }
   __host__ __device__ __forceinline__ int64_t value_offset(int page, int kvh, int slot, int d) const {
-    return (int64_t)page * page_stride + (int64_t)(kv_heads + kvh) * page_size * head_dim +
-           (int64_t)d * page_size + slot;
+    return value_column(page, kvh, d) + value_slot(slot);
   }
 };
 

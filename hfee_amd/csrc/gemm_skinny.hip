@@ -151,6 +151,68 @@ __device__ __forceinline__ void compute_block(f32x4* acc, float* ss, const Block
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
 
+// What happens to four finished sums: weight rows n .. n+3 of batch row m.
+template <int EPI>
+__device__ __forceinline__ void epilogue(const Args& a, int m, int n, float* v) {
+  if constexpr (EPI == EPI_BF16) {
+    bf16_t* c = (bf16_t*)a.C + (int64_t)m * a.ldc + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < a.N) c[i] = float_to_bf16(v[i]);
+  } else if constexpr (EPI == EPI_F32) {
+    float* c = (float*)a.C + (int64_t)m * a.ldc + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < a.N) c[i] = v[i];
+  } else if constexpr (EPI == EPI_ADD) {
+    float* c = (float*)a.C + (int64_t)m * a.ldc + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < a.N) c[i] += v[i];
+  } else if constexpr (EPI == EPI_SWIGLU) {
+    // rows n, n+1 = gate, up of column n/2; rows n+2, n+3 of column n/2 + 1 (N is even)
+    bf16_t* c = (bf16_t*)a.C + (int64_t)m * a.ldc + (n >> 1);
+    c[0] = float_to_bf16(silu(v[0]) * v[1]);
+    if (n + 2 < a.N) c[1] = float_to_bf16(silu(v[2]) * v[3]);
+  } else {   // EPI_QKV: head sizes are multiples of 4, so the four rows lie in one head
+    const QkvArgs& q = a.qkv;
+    const int hd = q.lay.head_dim;
+    const int head = n / hd, d = n - head * hd;
+    const int pos = q.positions[m];
+    const bool is_v = head >= q.num_heads + q.lay.kv_heads;
+    if (!is_v && q.cos_table != nullptr && d < 2 * q.half) {
+      const float* cs = q.cos_table + (int64_t)pos * q.half + (d >> 1);
+      const float* sn = q.sin_table + (int64_t)pos * q.half + (d >> 1);
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        if (d + 2 * p < 2 * q.half) {
+          const float x0 = v[2 * p], x1 = v[2 * p + 1], c = cs[p], s = sn[p];
+          v[2 * p] = x0 * c - x1 * s;
+          v[2 * p + 1] = x0 * s + x1 * c;
+        }
+      }
+    }
+    bf16_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = float_to_bf16(v[i]);
+    if (head < q.num_heads) {
+      *reinterpret_cast<u32x2*>((bf16_t*)a.C + (int64_t)m * a.ldc + n) = *reinterpret_cast<const u32x2*>(o);
+    } else if (q.cache != nullptr) {
+      const int page = q.block_tables[(int64_t)q.token_segment[m] * q.bt_stride + (pos >> q.lay.page_shift)];
+      const int slot = pos & (q.lay.page_size - 1);
+      bf16_t* cache = (bf16_t*)q.cache;
+      if (!is_v) {
+        *reinterpret_cast<u32x2*>(cache + q.lay.key_offset(page, head - q.num_heads, slot, d)) =
+            *reinterpret_cast<const u32x2*>(o);
+      } else {
+        const int kvh = head - q.num_heads - q.lay.kv_heads;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) cache[q.lay.value_offset(page, kvh, slot, d + i)] = o[i];
+      }
+    }
+  }
+}
+
 template <int MT, bool NORM, int EPI>
 __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   __shared__ float partial[WAVES][MT][64][4];
@@ -263,63 +325,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
       for (int i = 0; i < 4; ++i) v[i] *= scale;
     }
 
-    if constexpr (EPI == EPI_BF16) {
-      bf16_t* c = (bf16_t*)a.C + (int64_t)m * a.ldc + n;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (n + i < a.N) c[i] = float_to_bf16(v[i]);
-    } else if constexpr (EPI == EPI_F32) {
-      float* c = (float*)a.C + (int64_t)m * a.ldc + n;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (n + i < a.N) c[i] = v[i];
-    } else if constexpr (EPI == EPI_ADD) {
-      float* c = (float*)a.C + (int64_t)m * a.ldc + n;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (n + i < a.N) c[i] += v[i];
-    } else if constexpr (EPI == EPI_SWIGLU) {
-      // rows n, n+1 = gate, up of column n/2; rows n+2, n+3 of column n/2 + 1 (N is even)
-      bf16_t* c = (bf16_t*)a.C + (int64_t)m * a.ldc + (n >> 1);
-      c[0] = float_to_bf16(silu(v[0]) * v[1]);
-      if (n + 2 < a.N) c[1] = float_to_bf16(silu(v[2]) * v[3]);
-    } else {   // EPI_QKV: head sizes are multiples of 4, so the four rows lie in one head
-      const QkvArgs& q = a.qkv;
-      const int hd = q.lay.head_dim;
-      const int head = n / hd, d = n - head * hd;
-      const int pos = q.positions[m];
-      const bool is_v = head >= q.num_heads + q.lay.kv_heads;
-      if (!is_v && q.cos_table != nullptr && d < 2 * q.half) {
-        const float* cs = q.cos_table + (int64_t)pos * q.half + (d >> 1);
-        const float* sn = q.sin_table + (int64_t)pos * q.half + (d >> 1);
-#pragma unroll
-        for (int p = 0; p < 2; ++p) {
-          if (d + 2 * p < 2 * q.half) {
-            const float x0 = v[2 * p], x1 = v[2 * p + 1], c = cs[p], s = sn[p];
-            v[2 * p] = x0 * c - x1 * s;
-            v[2 * p + 1] = x0 * s + x1 * c;
-          }
-        }
-      }
-      bf16_t o[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = float_to_bf16(v[i]);
-      if (head < q.num_heads) {
-        *reinterpret_cast<u32x2*>((bf16_t*)a.C + (int64_t)m * a.ldc + n) = *reinterpret_cast<const u32x2*>(o);
-      } else if (q.cache != nullptr) {
-        const int page = q.block_tables[(int64_t)q.token_segment[m] * q.bt_stride + (pos >> q.lay.page_shift)];
-        const int slot = pos & (q.lay.page_size - 1);
-        bf16_t* cache = (bf16_t*)q.cache;
-        if (!is_v) {
-          *reinterpret_cast<u32x2*>(cache + q.lay.key_offset(page, head - q.num_heads, slot, d)) =
-              *reinterpret_cast<const u32x2*>(o);
-        } else {
-          const int kvh = head - q.num_heads - q.lay.kv_heads;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) cache[q.lay.value_offset(page, kvh, slot, d + i)] = o[i];
-        }
-      }
-    }
+    epilogue<EPI>(a, m, n, v);
   }
 }
 
@@ -333,6 +339,165 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
     case EPI_ADD: GO(EPI_ADD); break;
     case EPI_SWIGLU: GO(EPI_SWIGLU); break;
     default: GO(EPI_QKV); break;
+  }
+#undef GO
+}
+
+
+// ------------------------------------------------------------ wide products ---
+// For products with many weight rows (gate/up, the vocabulary head) and at most 16
+// batch rows.  Workgroups are persistent: each walks several groups of 16 weight
+// rows.  The batch rows are turned into matrix operands once per workgroup and stay
+// in registers (with the norm folded in if asked: this makes the fusion free), so
+// the loop streams W only; loads run a fixed number of steps ahead, across the
+// boundary between row groups.  K must be exactly STEPS * 32 * WAVES, so that the
+// loop has no condition in it.
+template <int STEPS, bool NORM, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups) {
+  constexpr int RING = STEPS < 16 ? STEPS : 16;
+  __shared__ float partial[WAVES][64][4];
+  __shared__ float ss_part[WAVES][16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, g = lane >> 4;
+  // local step s of this wave covers columns koff(s) .. koff(s)+31: blocks of four
+  // steps are dealt to the waves in turn
+  auto koff = [&](int s) { return ((((s >> 2) * WAVES + wave) << 2) + (s & 3)) * 32; };
+
+  // ---- the batch rows as operands, once -------------------------------------------
+  Chunk b[STEPS];
+  float ss = 0.f;
+  {
+    int m = min(r16, a.M - 1);
+    if (NORM && a.rows) m = a.rows[m];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int k = koff(s) + g * 8;
+      if constexpr (!NORM) {
+        b[s].u = *reinterpret_cast<const u32x4*>((const bf16_t*)a.A + (int64_t)m * a.lda + k);
+      } else {
+        const float* xr = (const float*)a.A + (int64_t)m * a.lda + k;
+        const f32x4 x0 = load_f4(xr), x1 = load_f4(xr + 4);
+        float nw[8];
+        if (a.norm_weight_is_f32) {
+          const f32x4 n0 = load_f4((const float*)a.norm_weight + k), n1 = load_f4((const float*)a.norm_weight + k + 4);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) { nw[i] = n0[i]; nw[4 + i] = n1[i]; }
+        } else {
+          Chunk c;
+          c.u = *reinterpret_cast<const u32x4*>((const bf16_t*)a.norm_weight + k);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) nw[i] = bf16_to_float(c.e[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          ss = fmaf(x0[i], x0[i], ss);
+          ss = fmaf(x1[i], x1[i], ss);
+          b[s].e[i] = float_to_bf16(x0[i] * nw[i]);
+          b[s].e[4 + i] = float_to_bf16(x1[i] * nw[4 + i]);
+        }
+      }
+    }
+  }
+  float scale = 1.f;
+  if (NORM) {
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if (g == 0) ss_part[wave][r16] = ss;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) t += ss_part[w][r16];
+    scale = 1.0f / sqrtf(t / (float)a.K + a.eps);     // for this lane's batch row (lane % 16)
+  }
+
+  // ---- stream W ---------------------------------------------------------------------
+  auto row_ptr = [&](int rg) { return a.W + (int64_t)min(rg * ROWS + r16, a.N - 1) * a.ldw + g * 8; };
+  int rg = blockIdx.x;                       // the host launches at most row_groups workgroups
+  const bf16_t* w_cur = row_ptr(rg);
+  Chunk ring[RING];
+#pragma unroll
+  for (int s = 0; s < RING; ++s) ring[s].u = *reinterpret_cast<const u32x4*>(w_cur + koff(s));
+
+  while (rg < row_groups) {
+    const int rg_next = rg + gridDim.x;
+    // after the last group the loads ahead re-read it: harmless, and the loop stays free of conditions
+    const bf16_t* w_next = row_ptr(rg_next < row_groups ? rg_next : rg);
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % RING].v, b[s].v, acc, 0, 0, 0);
+      const int ahead = s + RING;          // refill the slot RING steps ahead
+      ring[s % RING].u = ahead < STEPS ? *reinterpret_cast<const u32x4*>(w_cur + koff(ahead))
+                                       : *reinterpret_cast<const u32x4*>(w_next + koff(ahead - STEPS));
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) partial[wave][lane][i] = acc[i];
+    __syncthreads();
+    if (wave == 0) {
+      // register i of lane l: weight row 4*(l/16) + i, batch row l%16
+      const int m = r16, n = rg * ROWS + 4 * g;
+      if (m < a.M && n < a.N) {
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float t = 0.f;
+#pragma unroll
+          for (int w = 0; w < WAVES; ++w) t += partial[w][lane][i];
+          v[i] = t * scale;
+        }
+        epilogue<EPI>(a, m, n, v);
+      }
+    }
+    __syncthreads();
+    rg = rg_next;
+    w_cur = w_next;
+  }
+}
+
+template <bool NORM, int EPI>
+bool launch_wide_steps(const Args& a, int row_groups, int grid, hipStream_t stream) {
+  const int steps = a.K / (32 * WAVES);      // local steps per wave; K == steps * 32 * WAVES was checked
+  if (steps == 4) wide_kernel<4, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
+  else if (steps == 8) wide_kernel<8, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
+  else if (steps == 12) wide_kernel<12, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
+  else if (steps == 16) wide_kernel<16, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
+  else return false;      // other widths: the streaming kernel takes them
+  return true;
+}
+
+// Returns true if the wide kernel took the product.
+bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return false;
+    num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  const int row_groups = (a.N + ROWS - 1) / ROWS;
+  if (a.M > 16 || a.K % (128 * WAVES) != 0 || a.K > 16 * 32 * WAVES) return false;
+  // converting the batch rows once per workgroup pays when a workgroup walks several
+  // row groups; with the norm folded in it pays from two on
+  const int per = (row_groups + num_cus - 1) / num_cus;       // row groups per workgroup, all but equal
+  if (per < (norm ? 2 : 4)) return false;
+  const int grid = (row_groups + per - 1) / per;
+#define GO(NORM_, E) return launch_wide_steps<NORM_, E>(a, row_groups, grid, stream)
+  if (norm) {
+    switch (epi) {
+      case EPI_BF16: GO(true, EPI_BF16);
+      case EPI_F32: GO(true, EPI_F32);
+      case EPI_ADD: GO(true, EPI_ADD);
+      case EPI_SWIGLU: GO(true, EPI_SWIGLU);
+      default: GO(true, EPI_QKV);
+    }
+  }
+  switch (epi) {
+    case EPI_BF16: GO(false, EPI_BF16);
+    case EPI_F32: GO(false, EPI_F32);
+    case EPI_ADD: GO(false, EPI_ADD);
+    case EPI_SWIGLU: GO(false, EPI_SWIGLU);
+    default: GO(false, EPI_QKV);
   }
 #undef GO
 }
@@ -387,6 +552,10 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
     HFEE_REQUIRE(ldc >= N, "gemm_skinny: ldc is shorter than a row");
   }
   const int mt = (M + 15) / 16;
+  if (launch_wide(a, norm, epi, stream)) {
+    HFEE_CHECK_LAUNCH("gemm_skinny(wide)");
+    return 0;
+  }
   if (norm) launch_epi<1, true>(a, epi, stream);
   else if (mt == 1) launch_epi<1, false>(a, epi, stream);
   else if (mt == 2) launch_epi<2, false>(a, epi, stream);

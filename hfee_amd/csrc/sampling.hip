@@ -86,7 +86,17 @@ __device__ __forceinline__ MaxIdx better(MaxIdx a, MaxIdx b) {   // greater valu
 
 __device__ MaxIdx block_argmax(const float* __restrict__ lg, int V, MaxIdx* scratch) {
   MaxIdx best{-INFINITY, 0x7fffffff};
-  for (int j = threadIdx.x; j < V; j += blockDim.x) {
+  const int stride = blockDim.x;
+  int j = threadIdx.x;
+  for (; j + 7 * stride < V; j += 8 * stride) {      // eight loads in flight, compared in ascending j
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = lg[j + u * stride];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (v[u] > best.v) best = MaxIdx{v[u], j + u * stride};
+  }
+  for (; j < V; j += stride) {
     const float v = lg[j];
     if (v > best.v) best = MaxIdx{v, j};   // ascending j per thread: strict '>' keeps the first
   }

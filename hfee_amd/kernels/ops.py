@@ -254,8 +254,10 @@ def attention_bf16_prefill(out, q, cache_layer, tiles, block_tables, num_heads: 
 
 def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tables, block_tables,
                           num_heads: int, kv_heads: int, head_dim: int, page_size: int, scale: float,
-                          window: int, partial, num_splits: int):
-    """One query token per listed segment; keys split over num_splits waves."""
+                          window: int, partial, num_splits: int, waves: int = 4):
+    """One query token per listed segment.  A workgroup of `waves` waves (at most 4)
+    shares the keys of one (segment, KV head, split) and joins them in LDS; with
+    num_splits > 1 a second kernel joins the splits."""
     n, ldq, ldo = _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size)
     count = seg_rows.numel()
     _i32(seg_rows, "attention seg_rows")
@@ -268,7 +270,7 @@ def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tabl
         "hfee_attention_bf16_decode", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(seg_rows),
         _ptr(seg_positions), _ptr(seg_tables), count, _ptr(block_tables), block_tables.stride(0),
         num_heads, kv_heads, page_size, float(scale), int(window), _ptr(partial),
-        0 if partial is None else partial.numel(), int(num_splits), _stream())
+        0 if partial is None else partial.numel(), int(num_splits), int(waves), _stream())
 
 
 # ------------------------------------------------------- fused decode products (M <= 64)
@@ -278,6 +280,18 @@ FUSED_NORM_MAX_ROWS = 16
 # folding the norm into the product makes every workgroup convert the activations
 # itself; beyond this many weight rows a separate norm kernel is cheaper
 FUSED_NORM_MAX_N = 8192
+_cus = None
+
+
+def norm_fusion_pays(n_rows: int, k: int) -> bool:
+    """Whether folding the norm into a product with n_rows weight rows is cheaper than
+    a norm kernel of its own: narrow products, and the wide ones that the persistent
+    kernel takes (there the activations are converted once per workgroup)."""
+    global _cus
+    if _cus is None:
+        _cus = torch.cuda.get_device_properties(0).multi_processor_count
+    wide = n_rows > 16 * _cus and k % 1024 == 0 and k <= 4096
+    return wide or n_rows <= FUSED_NORM_MAX_N
 _EPI = {"bf16": 0, "f32": 1, "add": 2, "swiglu": 3, "qkv": 4}
 
 

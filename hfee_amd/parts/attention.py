@@ -28,8 +28,9 @@ from ..kernels import ops
 from ..weights.spec import TensorSpec
 from .base import LazyNorm, Mixer, lookup, register_mixer
 
-_TILE = 32            # query rows per workgroup of the prefill kernel
-_DECODE_WAVES = 1024  # waves the decode kernel aims for when it splits the keys
+_TILE = 32            # query rows per workgroup of the prefill kernel, keys per tile
+_DECODE_WAVES = 4     # waves of a decode workgroup; each takes every 4th key tile
+_TILES_PER_WAVE = 16  # beyond this many tiles per wave the keys are split over workgroups
 
 
 @register_mixer("attention")
@@ -131,7 +132,7 @@ class Attention(Mixer):
         if fused:
             # norm, projections, rotation and the cache write in one launch
             norm = h.fusable() if (isinstance(h, LazyNorm) and n <= ops.FUSED_NORM_MAX_ROWS
-                                   and self.w_qkv.shape[0] <= ops.FUSED_NORM_MAX_N) else None
+                                   and ops.norm_fusion_pays(*self.w_qkv.shape)) else None
             a = h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
             ops.linear_fused(q, a, self.w_qkv, "qkv", norm_weight=norm[0] if norm else None,
                              eps=norm[1] if norm else 0.0,
@@ -166,11 +167,11 @@ class Attention(Mixer):
                 if self.window > 0:
                     span = min(span, self.window + _TILE)
                 key_tiles = (span + _TILE - 1) // _TILE
-                splits = max(1, min(key_tiles, _DECODE_WAVES // max(1, nseg * K)))
+                splits = max(1, -(-key_tiles // (_DECODE_WAVES * _TILES_PER_WAVE)))
                 partial = None
                 if splits > 1:
                     partial = ctx.workspace.flat("attention.partial", nseg * H * splits * (hd + 2), torch.float32)
                 ops.attention_bf16_decode(att, q, cache, rows, ctx.extra["attention.decode_positions"],
                                           ctx.extra["attention.decode_tables"], tables, H, K, hd,
-                                          ctx.page_size, self.scale, self.window, partial, splits)
+                                          ctx.page_size, self.scale, self.window, partial, splits, _DECODE_WAVES)
         ops.linear(x, att, self.w_o, accumulate=True)

@@ -51,7 +51,7 @@ class Head(Part):
         w = logits.shape[0]
         fused = getattr(self.norm, "fused_form", lambda: None)()
         if (fused and self.dtype == torch.bfloat16 and w <= ops.FUSED_NORM_MAX_ROWS and self.hidden % 8 == 0
-                and self.weight.dtype == torch.bfloat16 and self.vocab <= ops.FUSED_NORM_MAX_N):
+                and self.weight.dtype == torch.bfloat16 and ops.norm_fusion_pays(self.vocab, self.hidden)):
             ops.linear_fused(logits, x, self.weight, "f32", norm_weight=fused[0], eps=fused[1], rows=rows, m=w)
             return
         normed = ctx.rows("head.normed", self.hidden, n=w)

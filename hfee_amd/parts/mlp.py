@@ -44,7 +44,7 @@ class GatedMLP(FeedForward):
         act = ctx.rows("mlp.act", F)
         if self.dtype == torch.bfloat16 and ctx.n <= ops.SKINNY_MAX_ROWS and self.hidden % 8 == 0:
             norm = h.fusable() if (isinstance(h, LazyNorm) and ctx.n <= ops.FUSED_NORM_MAX_ROWS
-                                   and self.w_gate_up.shape[0] <= ops.FUSED_NORM_MAX_N) else None
+                                   and ops.norm_fusion_pays(*self.w_gate_up.shape)) else None
             a = h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
             ops.linear_fused(act, a, self.w_gate_up, "swiglu", norm_weight=norm[0] if norm else None,
                              eps=norm[1] if norm else 0.0)

@@ -10,6 +10,11 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+def vslot(s):
+    """Where the cache keeps slot s of a value column: bits 2 and 3 exchanged."""
+    return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1)
+
+
 def close(a, b, tol):
     """|a - b| <= tol * (1 + |b|), the reference's form (/root/reference/internal/ggml/q8_test.go:24-26)."""
     a, b = a.double().cpu(), b.double().cpu()
@@ -109,6 +114,97 @@ def test_gemm_bf16_tiled_large(M, N, K):
     assert (err <= 1e-5 * (1 + mag)).all(), float((err / (1 + mag)).max())
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 48, 64), (8, 344, 96), (16, 100, 256), (3, 16400, 1024), (16, 16500, 2048),
+                                   (5, 17000, 4096), (2, 16390, 3072), (33, 200, 128), (64, 52, 1024)])
+@pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu"])
+@pytest.mark.parametrize("norm", [False, True])
+def test_fused_decode_products(M, N, K, epilogue, norm):
+    """The streaming and the persistent kernel with every epilogue, with and without
+    the norm in front, against the unfused formulas."""
+    from hfee_amd.kernels import ops
+    if norm and M > 16:
+        pytest.skip("the fused norm takes at most 16 rows")
+    if epilogue == "swiglu" and N % 2:
+        N += 1
+    g = torch.Generator().manual_seed(M + 3 * N + 7 * K)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    if norm:
+        xs = torch.randn(M + 3, K, generator=g) * 2
+        nw = (1 + 0.1 * torch.randn(K, generator=g)).to(torch.bfloat16 if K % 64 else torch.float32)
+        rows = torch.randperm(M + 3, generator=g)[:M].to(torch.int32)
+        x = xs[rows.long()]
+        h = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-5) * nw.double()
+    else:
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        h = x.double()
+    ref = h @ w.double().t()
+    mag = h.abs() @ w.double().abs().t()
+    c0 = torch.randn(M, N, generator=g)
+    if epilogue == "swiglu":
+        ref = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
+        mag = (mag[:, 0::2] + 1) * (mag[:, 1::2] + 1)
+        out = torch.zeros(M, N // 2, dtype=torch.bfloat16, device=DEV)
+    elif epilogue == "add":
+        ref = ref + c0.double()
+        out = c0.clone().to(DEV)
+    else:
+        out = torch.zeros(M, N, dtype=torch.bfloat16 if epilogue == "bf16" else torch.float32, device=DEV)
+    if norm:
+        ops.linear_fused(out, xs.to(DEV), w.to(DEV), epilogue, norm_weight=nw.to(DEV), eps=1e-5, rows=rows.to(DEV), m=M)
+    else:
+        ops.linear_fused(out, x.to(DEV), w.to(DEV), epilogue)
+    tol = 2e-2 if epilogue in ("bf16", "swiglu") or norm else 1e-5
+    err = (out.double().cpu() - ref).abs()
+    assert (err <= tol * (1 + mag)).all(), float((err / (1 + mag)).max())
+
+
+@pytest.mark.parametrize("H,K,hd,half,M", [(4, 2, 16, 8, 5), (3, 1, 32, 16, 16), (6, 3, 48, 8, 1), (2, 2, 128, 64, 9)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_fused_qkv_rotation_and_cache_write(H, K, hd, half, M, norm):
+    """Projection + rotation (pairs 2i, 2i+1) + cache write in one launch against the
+    separate steps."""
+    from plain_llama import plain_rope
+    from hfee_amd.kernels import ops
+    d, ps = 96, 16
+    g = torch.Generator().manual_seed(H + hd + M)
+    N = (H + 2 * K) * hd
+    w = (torch.randn(N, d, generator=g) / math.sqrt(d)).to(torch.bfloat16)
+    pos = torch.randint(0, 60, (M,), generator=g).to(torch.int32)
+    seg = torch.arange(M, dtype=torch.int32)
+    tables = torch.stack([torch.randperm(M * 4, generator=g)[:4] for _ in range(M)]).to(torch.int32)   # each row its own pages
+    tables = (tables // 4 * 0 + torch.arange(M * 4).reshape(M, 4)[:, torch.randperm(4, generator=g)]).to(torch.int32)
+    inv = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float64) * 2 / (2 * half)))
+    ang = torch.arange(64, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    if norm:
+        x = torch.randn(M, d, generator=g) * 2
+        nw = 1 + 0.1 * torch.randn(d, generator=g)
+        h = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-6) * nw.double()
+    else:
+        x = torch.randn(M, d, generator=g).to(torch.bfloat16)
+        h = x.double()
+    y = h @ w.double().t()
+    q_ref = y[:, :H * hd].reshape(M, H, hd).clone()
+    k_ref = y[:, H * hd:(H + K) * hd].reshape(M, K, hd).clone()
+    v_ref = y[:, (H + K) * hd:].reshape(M, K, hd)
+    q_ref[..., :2 * half] = plain_rope(q_ref[..., :2 * half], pos.tolist(), inv, "interleaved")
+    k_ref[..., :2 * half] = plain_rope(k_ref[..., :2 * half], pos.tolist(), inv, "interleaved")
+    layer = torch.zeros(M * 4, 2, K, ps * hd, dtype=torch.bfloat16, device=DEV)
+    q_out = torch.zeros(M, H * hd, dtype=torch.bfloat16, device=DEV)
+    ops.linear_fused(q_out, x.to(DEV), w.to(DEV), "qkv", norm_weight=nw.to(DEV) if norm else None, eps=1e-6,
+                     qkv=dict(positions=pos.to(DEV), token_segment=seg.to(DEV), block_tables=tables.to(DEV), cos=cos, sin=sin,
+                              cache_layer=layer, num_heads=H, kv_heads=K, head_dim=hd, page_size=ps))
+    close(q_out, q_ref.reshape(M, H * hd), 2e-2)
+    lay = layer.cpu()
+    for m in range(M):
+        p = int(pos[m])
+        page, slot = int(tables[m, p // ps]), p % ps
+        for kh in range(K):
+            close(lay[page, 0, kh].view(ps, hd)[slot], k_ref[m, kh], 2e-2)
+            close(lay[page, 1, kh].view(hd, ps)[:, vslot(slot)], v_ref[m, kh], 2e-2)
+    assert int((lay != 0).sum()) <= M * 2 * K * hd, "nothing but the tokens' own slots is written"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_and_add(dtype):
     from hfee_amd.kernels import ops
@@ -119,6 +215,9 @@ def test_swiglu_and_add(dtype):
     ops.swiglu(out, gud[:, :173], gud[:, 173:])
     ref = torch.nn.functional.silu(gu[:, :173].double()) * gu[:, 173:].double()
     close(out, ref, 1e-6 if dtype == torch.float32 else 1e-2)
+    out2 = torch.empty(9, 173, dtype=dtype, device=DEV)          # gate and up in alternating columns
+    ops.swiglu(out2, gud[:, 0::2], gud[:, 1::2])
+    close(out2, torch.nn.functional.silu(gu[:, 0::2].double()) * gu[:, 1::2].double(), 1e-6 if dtype == torch.float32 else 1e-2)
     x = torch.randn(9, 173, generator=g)
     xd = x.clone().to(DEV)
     ops.residual_add(xd, out)
@@ -149,7 +248,7 @@ def _paged(kv, page_size, pages_order):
             t = b * page_size + s
             for h in range(K):
                 layer[p, 0, h].view(page_size, hd)[s] = kv[0][t, h]
-                layer[p, 1, h].view(hd, page_size)[:, s] = kv[1][t, h]
+                layer[p, 1, h].view(hd, page_size)[:, vslot(s)] = kv[1][t, h]
     return layer, torch.tensor([pages_order[:nblocks]], dtype=torch.int32)
 
 
@@ -226,7 +325,7 @@ def test_rope_cache_write(pairing, dtype):
         page, slot = [2, 0, 3, 1][p // ps], p % ps
         for h in range(K):
             close(lay[page, 0, h].view(ps, hd)[slot], k_ref[t, h], tol)
-            assert torch.equal(lay[page, 1, h].view(hd, ps)[:, slot], v[t].view(K, hd)[h])
+            assert torch.equal(lay[page, 1, h].view(hd, ps)[:, vslot(slot)], v[t].view(K, hd)[h])
 
 
 def test_argmax_first_maximum_wins():

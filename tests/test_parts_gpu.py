@@ -17,6 +17,11 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+def vslot(s):
+    """Where the cache keeps slot s of a value column: bits 2 and 3 exchanged."""
+    return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1)
+
+
 def rel(a, b):
     a = a.double().cpu() if isinstance(a, torch.Tensor) else torch.as_tensor(np.asarray(a)).double()
     b = b.double().cpu() if isinstance(b, torch.Tensor) else torch.as_tensor(np.asarray(b)).double()
@@ -373,7 +378,7 @@ def test_attention_finds_a_far_key_among_hundreds():
             for t in range(T):
                 p, s = order[t // ps], t % ps
                 layer[p, 0].view(K, ps, hd)[:, s] = k[t]
-                layer[p, 1].view(K, hd, ps)[:, :, s] = v[t]
+                layer[p, 1].view(K, hd, ps)[:, :, vslot(s)] = v[t]
             layer = layer.to(dtype).to(DEV)
             table = torch.tensor([order], dtype=torch.int32, device=DEV)
             qd = q.reshape(T, H * hd).to(dtype).to(DEV)
