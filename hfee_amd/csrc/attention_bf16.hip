@@ -66,17 +66,39 @@ struct TileOps {
   Op v[2][NDT];
 };
 
+// 64 consecutive entries of a sequence's block table, one per lane, so that a tile's
+// page numbers come from a register shuffle instead of a load that the tile's own loads
+// would have to wait for.
+struct PageWindow {
+  int base;      // first block held; -1: nothing yet
+  int page;      // this lane's entry: block base + lane
+
+  __device__ __forceinline__ void fill(const int* __restrict__ bt, int bt_stride, int block) {
+    base = block;
+    const int mine = block + (int)(threadIdx.x & 63);
+    page = mine < bt_stride ? bt[mine] : 0;
+  }
+  // the page of `block`, which must lie in base .. base + 63
+  __device__ __forceinline__ int of(int block) const { return __shfl(page, block - base, 64); }
+};
+
 // Issues every load of the tile k0 .. k0+31.  kv_first..kv_last: the keys whose pages
 // may be touched at all (a window group has given back the pages before kv_first;
 // nothing exists after kv_last); the rest reads as zeros.
 __device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict__ cache, const CacheLayout& lay,
-                                          const int* __restrict__ bt, int kvh, int k0, int kv_first, int kv_last) {
+                                          const int* __restrict__ bt, int bt_stride, PageWindow& pages, int kvh,
+                                          int k0, int kv_first, int kv_last) {
   const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+  {
+    // the tile's blocks (uniform over the wave): refill the window when the tile leaves it
+    const int b0 = k0 >> lay.page_shift, b1 = (k0 + 31) >> lay.page_shift;
+    if (pages.base < 0 || b0 < pages.base || b1 >= pages.base + 64) pages.fill(bt, bt_stride, b0);
+  }
   {
     const int key = k0 + r32;
     const bool ok = key <= kv_last && key >= kv_first;
-    const bf16_t* krow = ok ? cache + lay.key_offset(bt[key >> lay.page_shift], kvh, key & (lay.page_size - 1), 0)
-                            : cache;
+    const int page = pages.of(key >> lay.page_shift);
+    const bf16_t* krow = ok ? cache + lay.key_offset(page, kvh, key & (lay.page_size - 1), 0) : cache;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       ops.k[c].u = u32x4{0u, 0u, 0u, 0u};
@@ -87,7 +109,7 @@ __device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict
   for (int u = 0; u < 2; ++u) {
     const int kb = k0 + 16 * u;
     const bool ok = kb <= kv_last && kb + 15 >= kv_first;
-    const int page = ok ? bt[kb >> lay.page_shift] : 0;
+    const int page = pages.of(kb >> lay.page_shift);
     const int first = (kb & (lay.page_size - 1)) + 8 * G;      // stored order: 4G.., 8+4G.. are adjacent
 #pragma unroll
     for (int t = 0; t < NDT; ++t) {
@@ -155,23 +177,25 @@ __device__ __forceinline__ void compute_tile(Tile& st, const Op* q_op, const Til
 // for kernels that run one wave per SIMD anyway); otherwise tile by tile.
 template <bool AHEAD>
 __device__ __forceinline__ void attend_tiles(Tile& st, const Op* q_op, const bf16_t* __restrict__ cache,
-                                             const CacheLayout& lay, const int* __restrict__ bt, int kvh,
-                                             int first, int end, int step, int kv_first, int kv_last, int pos,
-                                             int lo, float scale_log2) {
+                                             const CacheLayout& lay, const int* __restrict__ bt, int bt_stride,
+                                             int kvh, int first, int end, int step, int kv_first, int kv_last,
+                                             int pos, int lo, float scale_log2) {
   if (first >= end) return;
+  PageWindow pages;
+  pages.base = -1;
   if constexpr (AHEAD) {
     TileOps cur, nxt;
-    load_tile(cur, cache, lay, bt, kvh, first * 32, kv_first, kv_last);
+    load_tile(cur, cache, lay, bt, bt_stride, pages, kvh, first * 32, kv_first, kv_last);
     for (int t = first; t < end; t += step) {
       const int tn = t + step;
-      if (tn < end) load_tile(nxt, cache, lay, bt, kvh, tn * 32, kv_first, kv_last);
+      if (tn < end) load_tile(nxt, cache, lay, bt, bt_stride, pages, kvh, tn * 32, kv_first, kv_last);
       compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2);
       cur = nxt;
     }
   } else {
     for (int t = first; t < end; t += step) {
       TileOps cur;
-      load_tile(cur, cache, lay, bt, kvh, t * 32, kv_first, kv_last);
+      load_tile(cur, cache, lay, bt, bt_stride, pages, kvh, t * 32, kv_first, kv_last);
       compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2);
     }
   }
@@ -221,7 +245,7 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
   init_tile(st);
   const int kv_last = pos0 + rows - 1;
   const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
-  attend_tiles<false>(st, q_op, cache, lay, bt, kvh, kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
+  attend_tiles<false>(st, q_op, cache, lay, bt, bt_stride, kvh, kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
                scale_log2);
 
   if (slot_ok) {
@@ -279,7 +303,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
     load_query(q_op, q + (int64_t)row * ldq + h * HD, slot_ok);
     Tile st;
     init_tile(st);
-    attend_tiles<true>(st, q_op, cache, lay, bt, kvh, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
+    attend_tiles<true>(st, q_op, cache, lay, bt, bt_stride, kvh, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
                  scale_log2);
 
     // this wave's state into LDS
