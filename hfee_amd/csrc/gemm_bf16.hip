@@ -15,6 +15,8 @@
 // add of /root/reference/internal/llm/forward.go:106-107 fused into the epilogue).
 #include "common.h"
 
+#include <type_traits>
+
 using namespace hfee;
 
 namespace {
@@ -158,6 +160,169 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(void* __restrict__
     }
 }
 
+
+// ---------------------------------------------------------- tiled, pipelined ---
+// The prefill product for aligned operands.  Four waves in a 2x2 grid, each with
+// TM x TN tiles of 32x32 (a workgroup tile of 64 TM x 64 TN), K in steps of 64.
+// Global loads run STAGES K steps ahead of the matrix instructions (a ring of
+// register stages), the LDS holds two steps.  Epilogues: bfloat16 store, float32
+// store, float32 accumulate, and the SiLU gate for weights whose rows alternate
+// gate/up (C[m, j] = silu(row 2j) * row 2j+1).
+constexpr int PBK = 64, PPITCH = 72;   // pitch 144 bytes: no bank conflicts
+constexpr int XCDS = 8;                // accelerator dies of an MI355X
+enum { OUT_SWIGLU = 3 };
+
+template <int TM, int TN>
+struct PStage {
+  u32x4 a[2 * TM], w[2 * TN];      // this thread's 16-byte chunks of the A tile and of the W tile
+};
+
+template <int MODE, int TM, int TN, int STAGES>
+__global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restrict__ C, int64_t ldc,
+                                                                  const bf16_t* __restrict__ A, int64_t lda,
+                                                                  const bf16_t* __restrict__ W, int64_t ldw,
+                                                                  int M, int N, int K) {
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  extern __shared__ __attribute__((aligned(16))) bf16_t lds_tiles[];
+  auto a_tile = [&](int buf) { return lds_tiles + buf * (BM * PPITCH); };
+  auto w_tile = [&](int buf) { return lds_tiles + 2 * BM * PPITCH + buf * (BN * PPITCH); };
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // Workgroups go to the eight XCDs in turn, and each XCD has an L2 of its own.  Give
+  // every XCD a contiguous run of tiles, rows of the batch varying fastest: the
+  // workgroups that run together on an XCD then share a few W tiles, and W comes from
+  // HBM once.
+  int m0, n0;
+  {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const int total = tiles_m * tiles_n, per_xcd = (total + XCDS - 1) / XCDS;
+    const int t = (int)(blockIdx.x % XCDS) * per_xcd + (int)(blockIdx.x / XCDS);
+    if (t >= total) return;
+    m0 = (t % tiles_m) * BM;
+    n0 = (t / tiles_m) * BN;
+  }
+
+  // staging: a tile row is 8 chunks; thread -> row tid/8 + 32p, chunk tid%8
+  const int srow = tid >> 3, schunk = (tid & 7) * 8;
+  const bf16_t* a_ptr[2 * TM];
+  const bf16_t* w_ptr[2 * TN];
+#pragma unroll
+  for (int p = 0; p < 2 * TM; ++p)   // rows beyond M or N read the last valid row; their results are not stored
+    a_ptr[p] = A + (int64_t)min(m0 + srow + 32 * p, M - 1) * lda + schunk;
+#pragma unroll
+  for (int p = 0; p < 2 * TN; ++p)
+    w_ptr[p] = W + (int64_t)min(n0 + srow + 32 * p, N - 1) * ldw + schunk;
+  const int ktiles = (K + PBK - 1) / PBK;
+  auto load_stage = [&](PStage<TM, TN>& st, int kt) {
+    const int k = kt * PBK;
+    const bool in = k + schunk < K;        // K is a multiple of 8: a chunk is inside or outside
+#pragma unroll
+    for (int p = 0; p < 2 * TM; ++p) {
+      st.a[p] = u32x4{0u, 0u, 0u, 0u};
+      if (in) st.a[p] = *reinterpret_cast<const u32x4*>(a_ptr[p] + k);
+    }
+#pragma unroll
+    for (int p = 0; p < 2 * TN; ++p) {
+      st.w[p] = u32x4{0u, 0u, 0u, 0u};
+      if (in) st.w[p] = *reinterpret_cast<const u32x4*>(w_ptr[p] + k);
+    }
+  };
+  auto store_stage = [&](const PStage<TM, TN>& st, int buf) {
+#pragma unroll
+    for (int p = 0; p < 2 * TM; ++p)
+      *reinterpret_cast<u32x4*>(a_tile(buf) + (srow + 32 * p) * PPITCH + schunk) = st.a[p];
+#pragma unroll
+    for (int p = 0; p < 2 * TN; ++p)
+      *reinterpret_cast<u32x4*>(w_tile(buf) + (srow + 32 * p) * PPITCH + schunk) = st.w[p];
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  PStage<TM, TN> ring[STAGES];
+#pragma unroll
+  for (int s = 0; s < STAGES; ++s)
+    if (s < ktiles) load_stage(ring[s], s);
+  store_stage(ring[0], 0);
+  __syncthreads();
+
+  const int lrow = lane & 31, lk = (lane >> 5) * 8;
+  auto step = [&](auto slot_c, int kt) {
+    constexpr int SLOT = decltype(slot_c)::value;
+    const int buf = kt & 1;
+    if (kt + STAGES < ktiles) load_stage(ring[SLOT], kt + STAGES);     // ring[SLOT] went to LDS one step ago
+#pragma unroll
+    for (int ks = 0; ks < PBK / 16; ++ks) {
+      bf16x8 a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        a[i] = *reinterpret_cast<const bf16x8*>(a_tile(buf) + (wm * 32 * TM + i * 32 + lrow) * PPITCH + ks * 16 + lk);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[j] = *reinterpret_cast<const bf16x8*>(w_tile(buf) + (wn * 32 * TN + j * 32 + lrow) * PPITCH + ks * 16 + lk);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < ktiles) store_stage(ring[(SLOT + 1) % STAGES], buf ^ 1);
+    __syncthreads();
+  };
+  for (int kt = 0; kt < ktiles; kt += STAGES) {
+    step(std::integral_constant<int, 0>{}, kt);
+    if (STAGES > 1 && kt + 1 < ktiles) step(std::integral_constant<int, 1 % STAGES>{}, kt + 1);
+    if (STAGES > 2 && kt + 2 < ktiles) step(std::integral_constant<int, 2 % STAGES>{}, kt + 2);
+  }
+
+  // D layout of the 32x32 tile: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn * 32 * TN + j * 32 + lrow;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 32 * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        float v = acc[i][j][r];
+        if (MODE == OUT_SWIGLU) {
+          // the odd neighbour holds the up row: swap inside lane pairs (DPP quad_perm 1,0,3,2)
+          const float up = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+          if ((lane & 1) == 0 && m < M && n < N)
+            ((bf16_t*)C)[(int64_t)m * ldc + (n >> 1)] = float_to_bf16(v * __frcp_rn(1.0f + __expf(-v)) * up);
+        } else if (m < M && n < N) {
+          store_out<MODE>(C, ldc, m, n, v);
+        }
+      }
+    }
+}
+
+template <int MODE>
+int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
+                     int M, int N, int K, hipStream_t stream) {
+  // 128 x 128 tiles, two workgroups per CU.  (128 x 256 tiles halve the LDS reads per
+  // matrix instruction but leave one wave per SIMD, and measured 20 % slower.)
+  constexpr int TM = 2, TN = 2, STAGES = 3;
+  const size_t lds = (size_t)2 * (64 * TM + 64 * TN) * PPITCH * sizeof(bf16_t);
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail("gemm_bf16: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
+  if (tiles > (1 << 30)) return fail("gemm_bf16: too many tiles");
+  dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
+  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
+  return 0;
+}
+
 // ------------------------------------------------------------------ skinny ---
 constexpr int SK_WAVES = 8, SK_ROWS = 16, SK_UNROLL = 4;
 
@@ -222,10 +387,15 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(
   }
 }
 
+// Up to 16 rows the streaming kernel always wins.  From 17 to 64 rows it re-reads the
+// batch for every 16 weight rows, and the tiled kernel (which wastes matrix
+// instructions but not bandwidth) wins once there are enough tiles to fill the chip.
+inline bool skinny_pays(int M, int N) { return M <= 16 || (M <= 64 && N < 16384); }
+
 template <int MODE, bool VEC>
 int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
            int M, int N, int K, int force_kernel, hipStream_t stream) {
-  const bool skinny = force_kernel == 1 || (force_kernel == 0 && M <= 64);
+  const bool skinny = force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N));
   if (skinny) {
     const int mt = (M + 15) / 16;
     dim3 grid((N + SK_ROWS - 1) / SK_ROWS);
@@ -243,6 +413,8 @@ int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, 
   } else {
     dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM);
     if (grid.y > 65535) return fail("gemm_bf16: too many rows (%d)", M);
+    if (VEC && force_kernel != 3)
+      return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, stream);
     gemm_bf16_tiled_kernel<MODE, VEC><<<grid, 256, 0, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
   }
   return 0;
@@ -258,18 +430,30 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                               int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
                               int page_size, hipStream_t stream);
 
-// out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate.
-// force_kernel: 0 choose by M, 1 skinny, 2 tiled (for tests of each kernel alone).
+// out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate (the
+// rows of W alternate gate/up; C is [M, N/2] bfloat16; aligned operands and M > 64 only).
+// force_kernel: 0 choose by M, 1 skinny, 2 tiled, 3 the simple tiled kernel (for tests
+// of each kernel alone).
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
                             int64_t ldw, int M, int N, int K, int force_kernel, hipStream_t stream) {
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
-  HFEE_REQUIRE(ldc >= N && lda >= K && ldw >= K, "gemm_bf16: a leading dimension is shorter than its row");
-  HFEE_REQUIRE(out_mode >= 0 && out_mode <= 2, "gemm_bf16: unknown output mode %d", out_mode);
-  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 2, "gemm_bf16: unknown kernel choice %d", force_kernel);
+  HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16: a leading dimension is shorter than its row");
+  HFEE_REQUIRE(out_mode >= 0 && out_mode <= 3, "gemm_bf16: unknown output mode %d", out_mode);
+  HFEE_REQUIRE(ldc >= (out_mode == 3 ? N / 2 : N), "gemm_bf16: ldc is shorter than a row of the result");
+  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 3, "gemm_bf16: unknown kernel choice %d", force_kernel);
   if (M == 0) return 0;
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) &&
                    ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
-  if (vec && M <= 64 && force_kernel != 2)      // the streaming kernel with prefetch (gemm_skinny.hip)
+  if (out_mode == 3) {
+    HFEE_REQUIRE(N % 2 == 0 && vec, "gemm_bf16: the SiLU gate needs an even N and aligned operands");
+    if (skinny_pays(M, N))
+      return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, 3, nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr,
+                              0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, stream);
+    if (launch_pipelined<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, stream)) return 1;
+    HFEE_CHECK_LAUNCH("gemm_bf16");
+    return 0;
+  }
+  if (vec && M <= 64 && (force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N))))   // gemm_skinny.hip
     return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, out_mode, nullptr, 0, 0.f, nullptr, nullptr, nullptr,
                             nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, stream);
   const bf16_t* a = (const bf16_t*)A;

@@ -102,18 +102,27 @@ def residual_add(x: torch.Tensor, y: torch.Tensor):
 
 # ---------------------------------------------------------------- matrix product
 
-def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate: bool = False, kernel: int = 0):
+def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate: bool = False, kernel: int = 0,
+           gate: bool = False):
     """out (+)= x @ weight.T, weight stored [out_features, in_features].
 
     float32 x and weight: the true 32-bit product, out float32.
     bfloat16 x and weight: matrix cores with float32 accumulation; out bfloat16, or
     float32 (required when accumulating: the residual stream).
-    kernel: 0 automatic, 1 skinny, 2 tiled (bfloat16 only)."""
+    gate (bfloat16, aligned shapes): the rows of weight alternate gate/up and
+    out[m, j] = silu(row 2j) * row 2j+1, out [M, N/2].
+    kernel: 0 automatic, 1 skinny, 2 tiled, 3 the simple tiled kernel (bfloat16 only)."""
     _gpu(out, x, weight)
     M, K, lda = _rows2d(x, "linear x")
     N, Kw, ldw = _rows2d(weight, "linear weight")
     Mo, No, ldc = _rows2d(out, "linear out")
-    _check(Kw == K and Mo == M and No == N, f"linear: shapes x{list(x.shape)} w{list(weight.shape)} out{list(out.shape)}")
+    _check(Kw == K and Mo == M and No == (N // 2 if gate else N),
+           f"linear: shapes x{list(x.shape)} w{list(weight.shape)} out{list(out.shape)}")
+    if gate:
+        _check(x.dtype == weight.dtype == out.dtype == torch.bfloat16 and not accumulate and N % 2 == 0,
+               "linear: the gate epilogue takes bfloat16 operands and an even number of weight rows")
+        lib.core().call("hfee_gemm_bf16", _ptr(out), 3, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K, 0, _stream())
+        return
     _check(x.dtype == weight.dtype, "linear: x and weight dtypes differ")
     if x.dtype == torch.float32:
         _check(out.dtype == torch.float32, "linear: float32 product needs a float32 out")

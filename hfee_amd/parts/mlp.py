@@ -42,15 +42,19 @@ class GatedMLP(FeedForward):
     def forward_add(self, ctx, x, h):
         F = self.intermediate
         act = ctx.rows("mlp.act", F)
-        if self.dtype == torch.bfloat16 and ctx.n <= ops.SKINNY_MAX_ROWS and self.hidden % 8 == 0:
-            norm = h.fusable() if (isinstance(h, LazyNorm) and ctx.n <= ops.FUSED_NORM_MAX_ROWS
-                                   and ops.norm_fusion_pays(*self.w_gate_up.shape)) else None
-            a = h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
-            ops.linear_fused(act, a, self.w_gate_up, "swiglu", norm_weight=norm[0] if norm else None,
-                             eps=norm[1] if norm else 0.0)
+        aligned = self.dtype == torch.bfloat16 and self.hidden % 8 == 0
+        norm = None
+        if aligned and isinstance(h, LazyNorm) and ctx.n <= ops.FUSED_NORM_MAX_ROWS \
+                and ops.norm_fusion_pays(*self.w_gate_up.shape):
+            norm = h.fusable()
+        if norm:          # norm, both projections and the gate in one launch
+            ops.linear_fused(act, h.x, self.w_gate_up, "swiglu", norm_weight=norm[0], eps=norm[1])
         else:
             hn = h.tensor() if isinstance(h, LazyNorm) else h
-            gate_up = ctx.rows("mlp.gate_up", 2 * F)
-            ops.linear(gate_up, hn, self.w_gate_up)
-            ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
+            if aligned:   # the gate in the product's epilogue
+                ops.linear(act, hn, self.w_gate_up, gate=True)
+            else:
+                gate_up = ctx.rows("mlp.gate_up", 2 * F)
+                ops.linear(gate_up, hn, self.w_gate_up)
+                ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
         ops.linear(x, act, self.w_down, accumulate=True)

@@ -100,18 +100,32 @@ def test_gemm_bf16(M, N, K, kernel, mode):
     assert (err <= tol * (1 + mag)).all(), float((err / (1 + mag)).max())
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 128, 32), (300, 200, 520), (2048, 512, 1024), (129, 257, 72)])
-def test_gemm_bf16_tiled_large(M, N, K):
+@pytest.mark.parametrize("M,N,K", [(128, 128, 32), (300, 200, 520), (2048, 512, 1024), (129, 258, 72), (65, 130, 200),
+                                   (257, 384, 64), (1000, 96, 4096)])
+@pytest.mark.parametrize("kernel", [0, 3])
+def test_gemm_bf16_tiled_large(M, N, K, kernel):
+    """The pipelined kernel (0) and the simple tiled one (3), with every epilogue."""
     from hfee_amd.kernels import ops
     g = torch.Generator().manual_seed(M + N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
-    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
     ref = x.double() @ w.double().t()
-    out = torch.zeros(M, N, dtype=torch.float32, device=DEV)
-    ops.linear(out, x.to(DEV), w.to(DEV))
     mag = x.abs().double() @ w.abs().double().t()
+    out = torch.zeros(M, N, dtype=torch.float32, device=DEV)
+    ops.linear(out, x.to(DEV), w.to(DEV), kernel=kernel)
     err = (out.double().cpu() - ref).abs()
     assert (err <= 1e-5 * (1 + mag)).all(), float((err / (1 + mag)).max())
+    c0 = torch.randn(M, N, generator=g)
+    acc = c0.clone().to(DEV)
+    ops.linear(acc, x.to(DEV), w.to(DEV), accumulate=True, kernel=kernel)
+    err = (acc.double().cpu() - ref - c0.double()).abs()
+    assert (err <= 1e-5 * (1 + mag)).all()
+    if kernel == 0:
+        gated = torch.zeros(M, N // 2, dtype=torch.bfloat16, device=DEV)
+        ops.linear(gated, x.to(DEV), w.to(DEV), gate=True)
+        want = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
+        err = (gated.double().cpu() - want).abs()
+        assert (err <= 2e-2 * (1 + mag[:, 0::2]) * (1 + mag[:, 1::2])).all()
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (8, 344, 96), (16, 100, 256), (3, 16400, 1024), (16, 16500, 2048),
