@@ -403,3 +403,58 @@ def test_attention_finds_a_far_key_among_hundreds():
                     outs[f"decode{splits}"] = out[T - 1]
             for name, o in outs.items():
                 assert torch.allclose(o.float().cpu(), want, atol=2e-2), (dtype, far, name)
+
+
+def test_attention_window_edge():
+    """A window of W keys: the key at distance W-1 is the last one seen, the key at
+    distance W is not.  Both are made to stand out in turn; the result must be that
+    key's value in the first case and must not feel it in the second (all kernels,
+    window edges inside a page, on a page's edge and across a 32-key tile)."""
+    from plain_llama import plain_attention
+    from hfee_amd.kernels import ops
+    H, K, hd, ps = 2, 1, 32, 16
+    for dtype in (torch.float32, torch.bfloat16):
+        for T, W in ((100, 20), (97, 33), (130, 64), (64, 16), (50, 49)):
+            for inside in (True, False):
+                g = torch.Generator().manual_seed(T + W)
+                q = torch.randn(T, H, hd, generator=g) * 0.1
+                k = torch.randn(T, K, hd, generator=g) * 0.1
+                v = torch.randn(T, K, hd, generator=g)
+                direction = torch.randn(hd, generator=g)
+                direction /= direction.norm()
+                edge = T - W if inside else T - W - 1
+                k[edge] = 40 * direction
+                q[T - 1] = 40 * direction
+                want = plain_attention(q.to(dtype), k.to(dtype), v.to(dtype), 1.0, window=W)[T - 1].reshape(-1).float()
+                if inside:
+                    assert torch.allclose(want, v[edge].to(dtype).float().repeat(H, 1).reshape(-1), atol=2e-2)
+                nblocks = (T + ps - 1) // ps
+                order = torch.randperm(nblocks + 2, generator=g)[:nblocks].tolist()
+                layer = torch.full((nblocks + 2, 2, K, ps * hd), 9.0)
+                for t in range(T):
+                    p, sl = order[t // ps], t % ps
+                    layer[p, 0].view(K, ps, hd)[:, sl] = k[t]
+                    layer[p, 1].view(K, hd, ps)[:, :, vslot(sl)] = v[t]
+                layer = layer.to(dtype).to(DEV)
+                table = torch.tensor([order], dtype=torch.int32, device=DEV)
+                qd = q.reshape(T, H * hd).to(dtype).to(DEV)
+                positions = torch.arange(T, dtype=torch.int32, device=DEV)
+                seg = torch.zeros(T, dtype=torch.int32, device=DEV)
+                outs = {}
+                out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+                ops.attention_plain(out, qd, layer, positions, seg, table, H, K, hd, ps, 1.0, W)
+                outs["plain"] = out[T - 1]
+                if dtype == torch.bfloat16:
+                    tiles = torch.tensor([(o, min(32, T - o), o, 0) for o in range(0, T, 32)], dtype=torch.int32, device=DEV)
+                    out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+                    ops.attention_bf16_prefill(out, qd, layer, tiles, table, H, K, hd, ps, 1.0, W)
+                    outs["prefill"] = out[T - 1]
+                    rows = torch.tensor([T - 1], dtype=torch.int32, device=DEV)
+                    for splits in (1, 2):
+                        out = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+                        partial = torch.zeros(H * splits * (hd + 2), dtype=torch.float32, device=DEV)
+                        ops.attention_bf16_decode(out, qd, layer, rows, rows.clone(), torch.zeros(1, dtype=torch.int32, device=DEV),
+                                                  table, H, K, hd, ps, 1.0, W, partial, splits)
+                        outs[f"decode{splits}"] = out[T - 1]
+                for name, o in outs.items():
+                    assert torch.allclose(o.float().cpu(), want, atol=3e-2), (dtype, T, W, inside, name)
