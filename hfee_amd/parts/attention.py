@@ -30,7 +30,8 @@ from .base import LazyNorm, Mixer, lookup, register_mixer
 
 _TILE = 32            # query rows per workgroup of the prefill kernel, keys per tile
 _DECODE_WAVES = 4     # waves of a decode workgroup; each takes every 4th key tile
-_TILES_PER_WAVE = 16  # beyond this many tiles per wave the keys are split over workgroups
+_TILES_PER_WAVE = 16  # beyond this many tiles per wave the keys are always split over workgroups
+_DECODE_WORKGROUPS = 256   # with fewer (segment, KV head) pairs than this the keys are split to fill the chip
 
 
 @register_mixer("attention")
@@ -167,7 +168,8 @@ class Attention(Mixer):
                 if self.window > 0:
                     span = min(span, self.window + _TILE)
                 key_tiles = (span + _TILE - 1) // _TILE
-                splits = max(1, -(-key_tiles // (_DECODE_WAVES * _TILES_PER_WAVE)))
+                splits = max(-(-key_tiles // (_DECODE_WAVES * _TILES_PER_WAVE)),
+                             min(_DECODE_WORKGROUPS // max(1, nseg * K), -(-key_tiles // _DECODE_WAVES)), 1)
                 partial = None
                 if splits > 1:
                     partial = ctx.workspace.flat("attention.partial", nseg * H * splits * (hd + 2), torch.float32)
