@@ -18,6 +18,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import numpy as np
+
 
 class OutOfPages(RuntimeError):
     """A reservation needs more pages than the pool has free."""
@@ -86,6 +88,20 @@ class RequestCache:
     length: int = 0                                   # committed tokens
     tables: list = field(default_factory=list)        # per group: page id per block, -1 once released
     first_live_block: list = field(default_factory=list)   # per group
+    arrays: list = field(default_factory=list)        # per group: the table as int32 (released blocks read 0),
+                                                      # kept in step with `tables` for the step's upload
+
+    def table_array(self, group: int) -> np.ndarray:
+        return self.arrays[group][:len(self.tables[group])]
+
+    def _append(self, group: int, page: int) -> None:
+        arr, n = self.arrays[group], len(self.tables[group])
+        if n >= arr.shape[0]:
+            grown = np.zeros(max(16, 2 * arr.shape[0]), dtype=np.int32)
+            grown[:n] = arr[:n]
+            self.arrays[group] = arr = grown
+        arr[n] = page
+        self.tables[group].append(page)
 
 
 class CacheManager:
@@ -110,7 +126,8 @@ class CacheManager:
         if not self._free_slots:
             raise CacheError(f"all {self.max_requests} state slots are in use")
         rc = RequestCache(request_id, self._free_slots.pop(),
-                          tables=[[] for _ in self.groups], first_live_block=[0] * len(self.groups))
+                          tables=[[] for _ in self.groups], first_live_block=[0] * len(self.groups),
+                          arrays=[np.zeros(16, dtype=np.int32) for _ in self.groups])
         self.requests[request_id] = rc
         return rc
 
@@ -168,7 +185,7 @@ class CacheManager:
                                  f"{pool.num_free} are free")
         for g, n in enumerate(need):
             for _ in range(n):
-                rc.tables[g].append(self.pools[g].take(request_id))
+                rc._append(g, self.pools[g].take(request_id))
 
     def commit(self, request_id, n_new: int) -> None:
         """The step has written n_new tokens: advance the length and return the
@@ -188,6 +205,7 @@ class CacheManager:
                 if table[b] >= 0:
                     self.pools[g].give_back(table[b], request_id)
                     table[b] = -1
+                    rc.arrays[g][b] = 0
             rc.first_live_block[g] = max(rc.first_live_block[g], min(dead_until, len(table)))
 
     def truncate(self, request_id, length: int) -> None:

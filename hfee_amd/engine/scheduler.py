@@ -50,7 +50,7 @@ class Stats:
     preemptions: int = 0
 
 
-@dataclass
+@dataclass(eq=False)      # a request is itself, not its contents: membership tests must not compare prompts
 class Request:
     request_id: object
     prompt: list
@@ -165,24 +165,27 @@ class Scheduler:
         batch: list = []     # (request, tokens, wants_logits)
 
         # decoding requests first, oldest first; preempt from the young end if pages run out
+        ps = self.cache.page_size
         for r in [x for x in self.running if x.decoding]:
             if r not in self.running:
                 continue          # preempted while an older request was served
             if budget == 0:
                 break
-            while self._room(r) < 1:
-                victim = self.running[-1]
-                if victim is r:
-                    others = [x for x in self.running if x is not r]
-                    if not others:
-                        break
-                    victim = others[-1]
-                batch = [b for b in batch if b[0] is not victim]
-                self._preempt(victim)
-            if self._room(r) < 1:
-                self._finish(r, "length", finished, "the cache cannot hold this request even alone")
-                continue
-            self.cache.reserve(r.request_id, 1)
+            rc = self.cache.requests[r.request_id]
+            if any(len(t) * ps <= rc.length for t in rc.tables):      # its next token starts a new page
+                while self._room(r) < 1:
+                    victim = self.running[-1]
+                    if victim is r:
+                        others = [x for x in self.running if x is not r]
+                        if not others:
+                            break
+                        victim = others[-1]
+                    batch = [b for b in batch if b[0] is not victim]
+                    self._preempt(victim)
+                if self._room(r) < 1:
+                    self._finish(r, "length", finished, "the cache cannot hold this request even alone")
+                    continue
+                self.cache.reserve(r.request_id, 1)
             batch.append((r, r.feed[:1], True))
             budget -= 1
         budget = self.max_batch_tokens - sum(len(t) for _, t, _ in batch)

@@ -117,17 +117,19 @@ class Engine:
             if rc.length + len(e.tokens) > self.num_positions:
                 raise StepError(f"request {e.request_id!r} would reach position "
                                 f"{rc.length + len(e.tokens) - 1}, the context holds {self.num_positions}")
-            for t in e.tokens:
-                if not 0 <= t < self.vocab:
-                    raise StepError(f"token id {t} is outside the vocabulary of {self.vocab}")
-            for w in e.want:
-                if not 0 <= w < len(e.tokens):
-                    raise StepError(f"request {e.request_id!r} wants logits at {w} of {len(e.tokens)} tokens")
+            if min(e.tokens) < 0 or max(e.tokens) >= self.vocab:
+                raise StepError(f"a token id of request {e.request_id!r} is outside the vocabulary of {self.vocab}")
+            if e.want and (min(e.want) < 0 or max(e.want) >= len(e.tokens)):
+                raise StepError(f"request {e.request_id!r} wants logits outside its {len(e.tokens)} tokens")
             total += len(e.tokens)
         if total > self.max_batch_tokens:
             raise StepError(f"{total} tokens in one step, the engine was made for {self.max_batch_tokens}")
 
     def _reserve(self, entries):
+        ps = self.page_size
+        if all(len(t) * ps >= rc.length + len(e.tokens)
+               for e in entries for rc in (self.cache.requests[e.request_id],) for t in rc.tables):
+            return                      # every token already has a place (the scheduler reserved it)
         need = [0] * len(self.groups)
         for e in entries:
             for g, k in enumerate(self.cache.pages_needed(e.request_id, len(e.tokens))):
@@ -176,38 +178,41 @@ class Engine:
         self._check(entries)
         self._reserve(entries)
 
-        segments, tokens, positions, token_segment, logit_rows = [], [], [], [], []
+        segments, tokens, logit_rows = [], [], []
         row = 0
-        for s, e in enumerate(entries):
+        for e in entries:
             rc = self.cache.get(e.request_id)
             segments.append(Segment(e.request_id, rc.slot, rc.length, len(e.tokens), row))
-            tokens += list(e.tokens)
-            positions += range(rc.length, rc.length + len(e.tokens))
-            token_segment += [s] * len(e.tokens)
+            tokens += e.tokens
             logit_rows += [row + w for w in e.want]
             row += len(e.tokens)
         n = row
+        starts = np.fromiter((s.start for s in segments), dtype=np.int32, count=len(segments))
+        lengths = np.fromiter((s.length for s in segments), dtype=np.int32, count=len(segments))
+        rows0 = np.fromiter((s.row0 for s in segments), dtype=np.int32, count=len(segments))
+        token_segment = np.repeat(np.arange(len(segments), dtype=np.int32), lengths)
+        positions = np.arange(n, dtype=np.int32) - np.repeat(rows0 - starts, lengths)
 
         plan = StepPlan(segments)
         plan.add("token_ids", np.asarray(tokens))
-        plan.add("positions", np.asarray(positions))
-        plan.add("token_segment", np.asarray(token_segment))
-        plan.add("segment_slots", np.asarray([s.slot for s in segments]))
-        plan.add("segment_starts", np.asarray([s.start for s in segments]))
-        plan.add("segment_lengths", np.asarray([s.length for s in segments]))
-        plan.add("segment_rows", np.asarray([s.row0 for s in segments]))
+        plan.add("positions", positions)
+        plan.add("token_segment", token_segment)
+        plan.add("segment_slots", np.fromiter((s.slot for s in segments), dtype=np.int32, count=len(segments)))
+        plan.add("segment_starts", starts)
+        plan.add("segment_lengths", lengths)
+        plan.add("segment_rows", rows0)
         plan.add("logit_rows", np.asarray(logit_rows))
         decode_only = self.use_graphs and all(s.length == 1 for s in segments)
         widths = []
         for g in range(len(self.groups)):
-            tables = [self.cache.block_table(s.request_id, g) for s in segments]
+            tables = [self.cache.get(s.request_id).table_array(g) for s in segments]
             width = max(1, max(len(t) for t in tables))
             if decode_only:      # few distinct widths, so that few graphs are captured
                 width = min(max(8, 1 << (width - 1).bit_length()), max(width, self._max_blocks()))
             widths.append(width)
             bt = np.zeros((len(segments), width), dtype=np.int32)
             for i, t in enumerate(tables):
-                bt[i, :len(t)] = [max(p, 0) for p in t]   # pages a window has given back are never read
+                bt[i, :len(t)] = t          # blocks that a window has given back hold 0 and are never read
             plan.add(f"block_tables.{g}", bt)
         if decode_only:
             plan.host["graph.max_context"] = max(widths) * self.page_size
@@ -225,7 +230,7 @@ class Engine:
             segment_slots=dev["segment_slots"], segment_starts=dev["segment_starts"],
             segment_lengths=dev["segment_lengths"], segment_rows=dev["segment_rows"],
             block_tables=[dev[f"block_tables.{g}"] for g in range(len(self.groups))],
-            max_position=max(positions), storage=self.storage, workspace=self.workspace,
+            max_position=int(positions.max()), storage=self.storage, workspace=self.workspace,
             page_size=self.page_size, extra=dev, host=plan.host)
 
         w = len(logit_rows)
