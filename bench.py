@@ -38,6 +38,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=BASE_8B["num_hidden_layers"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the 2,048-token prefill (for profiling); prints its own short line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -114,6 +116,11 @@ def main() -> int:
             engine.release(rid)
             best = dt if best is None else min(best, dt)
         return best
+
+    if args.prefill_only:
+        pt = prefill_run()
+        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": PREFILL, "layers": L}), flush=True)
+        return 0
 
     dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3

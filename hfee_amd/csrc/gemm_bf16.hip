@@ -213,27 +213,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
   for (int p = 0; p < 2 * TN; ++p)
     w_ptr[p] = W + (int64_t)min(n0 + srow + 32 * p, N - 1) * ldw + schunk;
   const int ktiles = (K + PBK - 1) / PBK;
+  // The main loop has no branch around its loads and nothing that reads a loaded value
+  // before it goes to the LDS: the compiler can then count the loads and wait only for
+  // the stage it needs.  A chunk beyond K (K is a multiple of 8: it is inside or outside
+  // as a whole) is read from the row's last chunk; only the last steps, which run after
+  // the main loop, can hold such a chunk, and they replace it by zeros on its way to the LDS.
+  auto inside = [&](int kt) { return kt * PBK + schunk < K; };
   auto load_stage = [&](PStage<TM, TN>& st, int kt) {
-    const int k = kt * PBK;
-    const bool in = k + schunk < K;        // K is a multiple of 8: a chunk is inside or outside
+    const int ks = inside(kt) ? kt * PBK : K - 8 - schunk;
 #pragma unroll
-    for (int p = 0; p < 2 * TM; ++p) {
-      st.a[p] = u32x4{0u, 0u, 0u, 0u};
-      if (in) st.a[p] = *reinterpret_cast<const u32x4*>(a_ptr[p] + k);
-    }
+    for (int p = 0; p < 2 * TM; ++p) st.a[p] = *reinterpret_cast<const u32x4*>(a_ptr[p] + ks);
 #pragma unroll
-    for (int p = 0; p < 2 * TN; ++p) {
-      st.w[p] = u32x4{0u, 0u, 0u, 0u};
-      if (in) st.w[p] = *reinterpret_cast<const u32x4*>(w_ptr[p] + k);
-    }
+    for (int p = 0; p < 2 * TN; ++p) st.w[p] = *reinterpret_cast<const u32x4*>(w_ptr[p] + ks);
   };
-  auto store_stage = [&](const PStage<TM, TN>& st, int buf) {
+  auto store_stage = [&](const PStage<TM, TN>& st, int buf, bool in) {
+    const u32x4 zero{0u, 0u, 0u, 0u};
 #pragma unroll
     for (int p = 0; p < 2 * TM; ++p)
-      *reinterpret_cast<u32x4*>(a_tile(buf) + (srow + 32 * p) * PPITCH + schunk) = st.a[p];
+      *reinterpret_cast<u32x4*>(a_tile(buf) + (srow + 32 * p) * PPITCH + schunk) = in ? st.a[p] : zero;
 #pragma unroll
     for (int p = 0; p < 2 * TN; ++p)
-      *reinterpret_cast<u32x4*>(w_tile(buf) + (srow + 32 * p) * PPITCH + schunk) = st.w[p];
+      *reinterpret_cast<u32x4*>(w_tile(buf) + (srow + 32 * p) * PPITCH + schunk) = in ? st.w[p] : zero;
   };
 
   f32x16 acc[TM][TN];
@@ -246,16 +246,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
 
   PStage<TM, TN> ring[STAGES];
 #pragma unroll
-  for (int s = 0; s < STAGES; ++s)
-    if (s < ktiles) load_stage(ring[s], s);
-  store_stage(ring[0], 0);
+  for (int s = 0; s < STAGES; ++s) load_stage(ring[s], s);
+  store_stage(ring[0], 0, inside(0));
   __syncthreads();
 
   const int lrow = lane & 31, lk = (lane >> 5) * 8;
-  auto step = [&](auto slot_c, int kt) {
+  auto step = [&](auto slot_c, auto last_c, int kt) {
     constexpr int SLOT = decltype(slot_c)::value;
+    constexpr bool LAST = decltype(last_c)::value;
     const int buf = kt & 1;
-    if (kt + STAGES < ktiles) load_stage(ring[SLOT], kt + STAGES);     // ring[SLOT] went to LDS one step ago
+    load_stage(ring[SLOT], kt + STAGES);     // ring[SLOT] went to LDS one step ago
 #pragma unroll
     for (int ks = 0; ks < PBK / 16; ++ks) {
       bf16x8 a[TM], b[TN];
@@ -271,14 +271,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
-    if (kt + 1 < ktiles) store_stage(ring[(SLOT + 1) % STAGES], buf ^ 1);
+    store_stage(ring[(SLOT + 1) % STAGES], buf ^ 1, LAST ? inside(kt + 1) : true);
     __syncthreads();
   };
-  for (int kt = 0; kt < ktiles; kt += STAGES) {
-    step(std::integral_constant<int, 0>{}, kt);
-    if (STAGES > 1 && kt + 1 < ktiles) step(std::integral_constant<int, 1 % STAGES>{}, kt + 1);
-    if (STAGES > 2 && kt + 2 < ktiles) step(std::integral_constant<int, 2 % STAGES>{}, kt + 2);
+  static_assert(STAGES == 3, "the loop is written out for three stages");
+  using std::integral_constant;
+  int kt = 0;
+  for (; kt + 4 < ktiles; kt += STAGES) {      // these steps store K steps before the last one: whole chunks only
+    step(integral_constant<int, 0>{}, std::false_type{}, kt);
+    step(integral_constant<int, 1>{}, std::false_type{}, kt + 1);
+    step(integral_constant<int, 2>{}, std::false_type{}, kt + 2);
   }
+  if (kt < ktiles) step(integral_constant<int, 0>{}, std::true_type{}, kt);        // one to four steps are left
+  if (kt + 1 < ktiles) step(integral_constant<int, 1>{}, std::true_type{}, kt + 1);
+  if (kt + 2 < ktiles) step(integral_constant<int, 2>{}, std::true_type{}, kt + 2);
+  if (kt + 3 < ktiles) step(integral_constant<int, 0>{}, std::true_type{}, kt + 3);
 
   // D layout of the 32x32 tile: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
 #pragma unroll
