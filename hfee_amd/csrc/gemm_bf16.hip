@@ -256,20 +256,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
     constexpr bool LAST = decltype(last_c)::value;
     const int buf = kt & 1;
     load_stage(ring[SLOT], kt + STAGES);     // ring[SLOT] went to LDS one step ago
-#pragma unroll
-    for (int ks = 0; ks < PBK / 16; ++ks) {
-      bf16x8 a[TM], b[TN];
+    // operands of the next 16 columns are read from the LDS while this 16's products run
+    bf16x8 a[2][TM], b[2][TN];
+    auto read_operands = [&](int ks, bf16x8* af, bf16x8* bf) {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        a[i] = *reinterpret_cast<const bf16x8*>(a_tile(buf) + (wm * 32 * TM + i * 32 + lrow) * PPITCH + ks * 16 + lk);
+        af[i] = *reinterpret_cast<const bf16x8*>(a_tile(buf) + (wm * 32 * TM + i * 32 + lrow) * PPITCH + ks * 16 + lk);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        b[j] = *reinterpret_cast<const bf16x8*>(w_tile(buf) + (wn * 32 * TN + j * 32 + lrow) * PPITCH + ks * 16 + lk);
+        bf[j] = *reinterpret_cast<const bf16x8*>(w_tile(buf) + (wn * 32 * TN + j * 32 + lrow) * PPITCH + ks * 16 + lk);
+    };
+    read_operands(0, a[0], b[0]);
+#pragma unroll
+    for (int ks = 0; ks < PBK / 16; ++ks) {
+      if (ks + 1 < PBK / 16) read_operands(ks + 1, a[(ks + 1) & 1], b[(ks + 1) & 1]);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
     }
     store_stage(ring[(SLOT + 1) % STAGES], buf ^ 1, LAST ? inside(kt + 1) : true);
     __syncthreads();
