@@ -25,6 +25,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 enum { OUT_BF16 = 0, OUT_F32 = 1, OUT_ADD_F32 = 2 };
 
@@ -335,6 +336,251 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
   return 0;
 }
 
+// Tells the scheduler to issue N matrix instructions with R instructions of another
+// group (0x100 LDS read, 0x200 LDS write, 0x020 global load) spread evenly between them.
+template <int OTHER, int N, int R, int G = 0>
+struct Interleave {
+  static __device__ __forceinline__ void emit() {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    constexpr int c = (R * (G + 1)) / N - (R * G) / N;
+    if constexpr (c > 0) __builtin_amdgcn_sched_group_barrier(OTHER, c, 0);
+    Interleave<OTHER, N, R, G + 1>::emit();
+  }
+};
+template <int OTHER, int N, int R>
+struct Interleave<OTHER, N, R, N> {
+  static __device__ __forceinline__ void emit() {}
+};
+
+// Stores a 32 x 32 tile that was formed transposed: register r of lane l holds
+// C[m_base + l % 32][n_base + 8 (r / 4) + 4 (l / 32) + r % 4], so four registers are
+// four consecutive columns.  `vec`: rows of C start 16-byte aligned (8 for bfloat16).
+template <int MODE>
+__device__ __forceinline__ void store_tile_t(void* C, int64_t ldc, int M, int N, int m, int n_base, int lane,
+                                             const f32x16& t, bool vec) {
+  if (m >= M) return;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int n = n_base + 8 * q + 4 * (lane >> 5);
+    if (n >= N) continue;
+    float v[4] = {t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+    if (MODE == OUT_SWIGLU) {          // columns n, n+1 are gate, up of output column n / 2
+      bf16_t* c = (bf16_t*)C + (int64_t)m * ldc + (n >> 1);
+      const bf16_t o0 = float_to_bf16(v[0] * __frcp_rn(1.0f + __expf(-v[0])) * v[1]);
+      const bf16_t o1 = float_to_bf16(v[2] * __frcp_rn(1.0f + __expf(-v[2])) * v[3]);
+      if (vec && n + 3 < N) {
+        *reinterpret_cast<uint32_t*>(c) = (uint32_t)o0 | ((uint32_t)o1 << 16);
+      } else {
+        c[0] = o0;
+        if (n + 3 < N) c[1] = o1;
+      }
+    } else if (MODE == OUT_BF16) {
+      bf16_t* c = (bf16_t*)C + (int64_t)m * ldc + n;
+      if (vec && n + 3 < N) {
+        u32x2 o;
+        o[0] = (uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16);
+        o[1] = (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16);
+        *reinterpret_cast<u32x2*>(c) = o;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) c[i] = float_to_bf16(v[i]);
+      }
+    } else {
+      float* c = (float*)C + (int64_t)m * ldc + n;
+      if (vec && n + 3 < N) {
+        f32x4 o = {v[0], v[1], v[2], v[3]};
+        if (MODE == OUT_ADD_F32) o += *reinterpret_cast<const f32x4*>(c);
+        *reinterpret_cast<f32x4*>(c) = o;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) c[i] = MODE == OUT_ADD_F32 ? c[i] + v[i] : v[i];
+      }
+    }
+  }
+}
+
+// ------------------------------------ tiled, one wave a SIMD, loads into the LDS ---
+// Products with enough tiles of 256 rows to fill the chip.  A 128 x 128 tile at the
+// full matrix rate asks the L1 for 64 bytes a clock, which is all a CU has, and the LDS
+// for one 16-byte read per lane and matrix instruction; a wave tile of 128 x 128
+// (TM = TN = 4: 256 accumulator registers, so one wave a SIMD) halves both.
+//
+// With one wave a SIMD nothing hides latency but distance and the order of issue:
+//  * A K step (32 columns) goes from global memory straight into the LDS
+//    (buffer_load_dwordx4 ... lds: lane l of a wave writes bytes 16 l .. 16 l + 15 of a
+//    1 KB block), so no register stage and no LDS write instruction stands between the
+//    matrix instructions.  Four LDS buffers of one K step each: a step is asked from
+//    memory three steps before it is multiplied.
+//  * A 1 KB block is 16 tile rows of 64 bytes, unpadded; the four 16-byte chunks of row
+//    r are stored in the order c ^ f(r), f(r) = ((r >> 1) ^ (r >> 3)) & 3, which keeps
+//    the 16-byte operand reads of 8 or 16 consecutive rows on distinct banks.
+//  * The one barrier of a step stands where the wave has nothing outstanding in the LDS,
+//    and carries no fence (a fence would wait for every load in flight); what must have
+//    landed is waited for by count.
+//  * The order of issue is spelled out with scheduling groups: what does not stand
+//    between two matrix instructions is not overlapped with them.
+//  * The products are formed transposed (weights as the row operand): a lane then holds
+//    four consecutive columns of one row of C and stores them with one instruction.
+// K must be a multiple of 32 and every row's byte offset must fit 31 bits.
+constexpr int DBK = 32, DROW = DBK * 2;      // bytes of a tile row in a buffer
+
+__device__ __forceinline__ uint32_t swizzle(uint32_t row) { return ((row >> 1) ^ (row >> 3)) & 3u; }
+
+template <int MODE, int TM, int TN>
+__global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict__ C, int64_t ldc,
+                                                               const bf16_t* __restrict__ A, int64_t lda,
+                                                               const bf16_t* __restrict__ W, int64_t ldw,
+                                                               int M, int N, int K) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass has no buffer resources; it only needs the stub
+  constexpr int BM = 64 * TM, BN = 64 * TN, CA = BM / 64, CW = BN / 64;
+  constexpr int BUF = (BM + BN) * DROW;            // bytes of one LDS buffer (A tile, then W tile)
+  extern __shared__ __attribute__((aligned(1024))) char lds_bytes[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  int m0, n0;
+  {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const int total = tiles_m * tiles_n, per_xcd = (total + XCDS - 1) / XCDS;
+    const int t = (int)(blockIdx.x % XCDS) * per_xcd + (int)(blockIdx.x / XCDS);
+    if (t >= total) return;
+    m0 = (t % tiles_m) * BM;
+    n0 = (t / tiles_m) * BN;
+  }
+  // A wave's load p fills tile rows 64 p + 16 wave .. + 15: lane -> row lane / 4, LDS chunk lane % 4,
+  // which holds the row's chunk (lane % 4) ^ f(row).  Rows beyond the edge read the last row.
+  const int lr = 64 * 0 + 16 * wave + (lane >> 2);             // row within the first 64 rows
+  uint32_t a_off[CA], w_off[CW];
+#pragma unroll
+  for (int p = 0; p < CA; ++p) {
+    const uint32_t row = (uint32_t)(lr + 64 * p), chunk = (uint32_t)(lane & 3) ^ swizzle(row);
+    a_off[p] = (uint32_t)(((int64_t)min(m0 + (int)row, M - 1) * lda + chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int p = 0; p < CW; ++p) {
+    const uint32_t row = (uint32_t)(lr + 64 * p), chunk = (uint32_t)(lane & 3) ^ swizzle(row);
+    w_off[p] = (uint32_t)(((int64_t)min(n0 + (int)row, N - 1) * ldw + chunk * 8) * 2);
+  }
+  const int ktiles = K / DBK;
+  // Buffer loads: the row offset is a 32-bit register that never changes, the K step a
+  // scalar; nothing is computed per load.  (0x00020000: a raw buffer of 32-bit data.)
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  const __amdgpu_buffer_rsrc_t a_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)(((int64_t)(M - 1) * lda + K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)(((int64_t)(N - 1) * ldw + K) * 2), 0x00020000);
+  auto load_step = [&](int kt) {
+    const int buf = kt & 3;
+    const int koff = min(kt, ktiles - 1) * DROW;          // past the end: a repeat that nobody uses
+    char* dst = lds_bytes + buf * BUF + wave * 1024;
+#pragma unroll
+    for (int p = 0; p < CA; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(dst + p * 4096), 16, a_off[p], koff, 0, 0);
+#pragma unroll
+    for (int p = 0; p < CW; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)(dst + BM * DROW + p * 4096), 16, w_off[p], koff, 0, 0);
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int lrow = lane & 31, h = lane >> 5;
+  // byte offsets of this lane's operand chunk for columns 0..15 and 16..31 of a step
+  uint32_t rd[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) rd[ks] = (uint32_t)(lrow * DROW) + (((uint32_t)(ks * 2 + h) ^ swizzle((uint32_t)lrow)) << 4);
+  const uint32_t a_rd = (uint32_t)(wm * 32 * TM * DROW), w_rd = (uint32_t)(BM * DROW + wn * 32 * TN * DROW);
+  bf16x8 a[2][TM], b[2][TN];
+  auto read_operands = [&](int buf, int ks, bf16x8* af, bf16x8* bf) {
+    const char* tile = lds_bytes + buf * BUF + rd[ks];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 32 * DROW);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * DROW);
+  };
+  auto multiply = [&](const bf16x8* af, const bf16x8* bf, int from, int to) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        if (i * TN + j >= from && i * TN + j < to)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);   // transposed
+  };
+
+  constexpr int RD = TM + TN, MF = TM * TN, LD = CA + CW, HALF = MF / 2;
+  load_step(0);
+  load_step(1);
+  load_step(2);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LD) : "memory");     // K step 0 has landed
+  __builtin_amdgcn_s_barrier();
+  read_operands(0, 0, a[0], b[0]);
+
+  // One step: columns 0..15 with the reads of columns 16..31 under them; the first half
+  // of columns 16..31 with the requests for K step kt + 3 (its buffer was last read in
+  // step kt - 1, before that step's barrier); then the barrier, and the second half with
+  // the first reads of the next step.  At the barrier this wave's part of K step kt + 1
+  // (asked for two steps ago) has landed: at most the loads of two steps are outstanding.
+  // After the barrier everybody's has, and nobody reads this step's buffer any more.
+  // No fence: it would wait for every load in flight.
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int buf = kt & 3;
+    read_operands(buf, 1, a[1], b[1]);
+    multiply(a[0], b[0], 0, MF);
+    Interleave<0x100, MF, RD>::emit();
+    multiply(a[1], b[1], 0, HALF);
+    load_step(kt + 3);
+    Interleave<0x020, HALF, LD>::emit();
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * LD) : "memory");
+    __builtin_amdgcn_s_barrier();
+    read_operands((kt + 1) & 3, 0, a[0], b[0]);
+    multiply(a[1], b[1], HALF, MF);
+    Interleave<0x100, MF - HALF, RD>::emit();
+  }
+  // the repeats asked for past the end still write into this workgroup's LDS: let them
+  // land before the wave can end and the LDS go to another workgroup
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  const bool vec = MODE == OUT_SWIGLU ? (ldc % 2 == 0 && (uintptr_t)C % 4 == 0)
+                 : MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0)
+                                    : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+#endif
+}
+
+template <int MODE, int TM, int TN>
+int launch_direct(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
+                  int M, int N, int K, hipStream_t stream) {
+  const size_t lds = (size_t)4 * (64 * TM + 64 * TN) * DROW;
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_direct_kernel<MODE, TM, TN>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail("gemm_bf16: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
+  dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
+  gemm_bf16_direct_kernel<MODE, TM, TN><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
+  return 0;
+}
+
+// The large tiles take a product whose K is a multiple of 32, whose byte offsets fit 32
+// bits, and which has enough of them.
+inline bool large_fits(int64_t lda, int64_t ldw, int M, int N, int K) {
+  return K % DBK == 0 && (int64_t)M * lda < (1ll << 30) && (int64_t)N * ldw < (1ll << 30);
+}
+
 // ------------------------------------------------------------------ skinny ---
 constexpr int SK_WAVES = 8, SK_ROWS = 16, SK_UNROLL = 4;
 
@@ -399,6 +645,44 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(
   }
 }
 
+// Which tiled kernel takes an aligned product: force_kernel 2 the 128 x 128 tiles, 4 the
+// 256 x 256 tiles, 5 the 256 x 128 tiles, anything else the one expected to be fastest:
+// rounds of tiles over the chip times the time of a tile, with the share of the matrix
+// peak that each kernel was measured to reach on a busy CU (128 x 128: two workgroups a
+// CU; the large tiles reach more the longer K is, and a tile of empty rows costs as
+// much as a full one).
+inline int fastest_tiled(int M, int N, int K, bool large_ok) {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+           prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+  }
+  if (!large_ok) return 2;
+  auto tiles = [&](int bm, int bn) { return (double)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  auto rounds = [&](double t, int slots) { return (double)(int64_t)((t + slots - 1) / slots); };
+  const double t2 = tiles(128, 128), t4 = tiles(256, 256), t5 = tiles(256, 128);
+  const double c2 = t2 <= cus ? 128.0 * 128 / 0.22 : rounds(t2, 2 * cus) * 2 * 128 * 128 / 0.31;
+  const double fill = K >= 512 ? 1.0 : 0.6;            // the four-buffer pipeline needs a few steps to pay
+  const double c4 = rounds(t4, cus) * 256 * 256 / (0.50 * fill);
+  const double c5 = rounds(t5, cus) * 256 * 128 / (0.37 * fill);
+  if (c4 <= c5 && c4 <= c2) return 4;
+  return c5 <= c2 ? 5 : 2;
+}
+
+template <int MODE>
+int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
+                   int M, int N, int K, int force_kernel, hipStream_t stream) {
+  int choice = force_kernel;
+  const bool large_ok = large_fits(lda, ldw, M, N, K);
+  if (choice != 2 && choice != 4 && choice != 5) choice = fastest_tiled(M, N, K, large_ok);
+  if (choice >= 4 && !large_ok) choice = 2;
+  if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, stream);
+  if (choice == 5) return launch_direct<MODE, 4, 2>(C, ldc, A, lda, W, ldw, M, N, K, stream);
+  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, stream);
+}
+
 // Up to 16 rows the streaming kernel always wins.  From 17 to 64 rows it re-reads the
 // batch for every 16 weight rows, and the tiled kernel (which wastes matrix
 // instructions but not bandwidth) wins once there are enough tiles to fill the chip.
@@ -426,7 +710,7 @@ int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, 
     dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM);
     if (grid.y > 65535) return fail("gemm_bf16: too many rows (%d)", M);
     if (VEC && force_kernel != 3)
-      return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, stream);
+      return launch_aligned<MODE>(C, ldc, A, lda, W, ldw, M, N, K, force_kernel, stream);
     gemm_bf16_tiled_kernel<MODE, VEC><<<grid, 256, 0, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
   }
   return 0;
@@ -444,15 +728,16 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
 
 // out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate (the
 // rows of W alternate gate/up; C is [M, N/2] bfloat16; aligned operands and M > 64 only).
-// force_kernel: 0 choose by M, 1 skinny, 2 tiled, 3 the simple tiled kernel (for tests
-// of each kernel alone).
+// force_kernel: 0 choose by the sizes, 1 skinny, 2 tiled 128 x 128, 3 the simple tiled
+// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128 (for tests of each kernel alone; 4 and 5
+// fall back to 2 where they do not apply).
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
                             int64_t ldw, int M, int N, int K, int force_kernel, hipStream_t stream) {
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16: a leading dimension is shorter than its row");
   HFEE_REQUIRE(out_mode >= 0 && out_mode <= 3, "gemm_bf16: unknown output mode %d", out_mode);
   HFEE_REQUIRE(ldc >= (out_mode == 3 ? N / 2 : N), "gemm_bf16: ldc is shorter than a row of the result");
-  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 3, "gemm_bf16: unknown kernel choice %d", force_kernel);
+  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 5, "gemm_bf16: unknown kernel choice %d", force_kernel);
   if (M == 0) return 0;
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) &&
                    ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
@@ -461,7 +746,7 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
     if (skinny_pays(M, N))
       return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, 3, nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr,
                               0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, stream);
-    if (launch_pipelined<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, stream)) return 1;
+    if (launch_aligned<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, force_kernel, stream)) return 1;
     HFEE_CHECK_LAUNCH("gemm_bf16");
     return 0;
   }

@@ -111,7 +111,8 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
     float32 (required when accumulating: the residual stream).
     gate (bfloat16, aligned shapes): the rows of weight alternate gate/up and
     out[m, j] = silu(row 2j) * row 2j+1, out [M, N/2].
-    kernel: 0 automatic, 1 skinny, 2 tiled, 3 the simple tiled kernel (bfloat16 only)."""
+    kernel (bfloat16 only): 0 automatic, 1 skinny, 2 tiled 128x128, 3 the simple tiled
+    kernel, 4 tiled 256x256, 5 tiled 256x128."""
     _gpu(out, x, weight)
     M, K, lda = _rows2d(x, "linear x")
     N, Kw, ldw = _rows2d(weight, "linear weight")
@@ -121,7 +122,7 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
     if gate:
         _check(x.dtype == weight.dtype == out.dtype == torch.bfloat16 and not accumulate and N % 2 == 0,
                "linear: the gate epilogue takes bfloat16 operands and an even number of weight rows")
-        lib.core().call("hfee_gemm_bf16", _ptr(out), 3, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K, 0, _stream())
+        lib.core().call("hfee_gemm_bf16", _ptr(out), 3, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K, kernel, _stream())
         return
     _check(x.dtype == weight.dtype, "linear: x and weight dtypes differ")
     if x.dtype == torch.float32:

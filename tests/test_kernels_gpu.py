@@ -101,10 +101,13 @@ def test_gemm_bf16(M, N, K, kernel, mode):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 32), (300, 200, 520), (2048, 512, 1024), (129, 258, 72), (65, 130, 200),
-                                   (257, 384, 64), (1000, 96, 4096)])
-@pytest.mark.parametrize("kernel", [0, 3])
+                                   (257, 384, 64), (1000, 96, 4096), (600, 520, 192), (256, 512, 64),
+                                   (513, 258, 320)])
+@pytest.mark.parametrize("kernel", [0, 2, 3, 4, 5])
 def test_gemm_bf16_tiled_large(M, N, K, kernel):
-    """The pipelined kernel (0) and the simple tiled one (3), with every epilogue."""
+    """The tiled kernels each alone (2: 128x128 tiles, 3: the simple one, 4: 256x256, 5:
+    256x128; 4 and 5 hand a K that is no multiple of 64 to 2) and the automatic choice,
+    with every epilogue."""
     from hfee_amd.kernels import ops
     g = torch.Generator().manual_seed(M + N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -120,9 +123,9 @@ def test_gemm_bf16_tiled_large(M, N, K, kernel):
     ops.linear(acc, x.to(DEV), w.to(DEV), accumulate=True, kernel=kernel)
     err = (acc.double().cpu() - ref - c0.double()).abs()
     assert (err <= 1e-5 * (1 + mag)).all()
-    if kernel == 0:
+    if kernel != 3:
         gated = torch.zeros(M, N // 2, dtype=torch.bfloat16, device=DEV)
-        ops.linear(gated, x.to(DEV), w.to(DEV), gate=True)
+        ops.linear(gated, x.to(DEV), w.to(DEV), gate=True, kernel=kernel)
         want = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
         err = (gated.double().cpu() - want).abs()
         assert (err <= 2e-2 * (1 + mag[:, 0::2]) * (1 + mag[:, 1::2])).all()
