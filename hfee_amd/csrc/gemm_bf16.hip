@@ -575,10 +575,168 @@ int launch_direct(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16
   return 0;
 }
 
-// The large tiles take a product whose K is a multiple of 32, whose byte offsets fit 32
+// The same, with K steps of 64 columns: a tile row is a whole 128-byte line, so the L2
+// sees half as many requests, and there is one barrier per 64 columns.  It pays with
+// three buffers, which the LDS holds for 256 x 128 tiles (with the two that fit for
+// 256 x 256 tiles it measured slower than four buffers of 32 columns).
+constexpr int EROW = 128;                    // bytes of a tile row in a buffer
+// depends on the low five bits of the row only: a lane's operand rows are 32 apart
+__device__ __forceinline__ uint32_t swizzle8(uint32_t row) { return (row ^ ((row >> 3) & 3u)) & 7u; }
+
+template <int MODE, int TM, int TN, int NBUF>
+__global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restrict__ C, int64_t ldc,
+                                                                 const bf16_t* __restrict__ A, int64_t lda,
+                                                                 const bf16_t* __restrict__ W, int64_t ldw,
+                                                                 int M, int N, int K) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int BM = 64 * TM, BN = 64 * TN, CA = BM / 32, CW = BN / 32;
+  constexpr int BUF = (BM + BN) * EROW;
+  extern __shared__ __attribute__((aligned(1024))) char lds_bytes[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  int m0, n0;
+  {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const int total = tiles_m * tiles_n, per_xcd = (total + XCDS - 1) / XCDS;
+    const int t = (int)(blockIdx.x % XCDS) * per_xcd + (int)(blockIdx.x / XCDS);
+    if (t >= total) return;
+    m0 = (t % tiles_m) * BM;
+    n0 = (t / tiles_m) * BN;
+  }
+  // A wave's load p fills tile rows 32 p + 8 wave .. + 7: lane -> row lane / 8, LDS chunk lane % 8,
+  // which holds the row's chunk (lane % 8) ^ f(row).
+  const int lr = 8 * wave + (lane >> 3);
+  uint32_t a_off[CA], w_off[CW];
+#pragma unroll
+  for (int p = 0; p < CA; ++p) {
+    const uint32_t row = (uint32_t)(lr + 32 * p), chunk = (uint32_t)(lane & 7) ^ swizzle8(row);
+    a_off[p] = (uint32_t)(((int64_t)min(m0 + (int)row, M - 1) * lda + chunk * 8) * 2);
+  }
+#pragma unroll
+  for (int p = 0; p < CW; ++p) {
+    const uint32_t row = (uint32_t)(lr + 32 * p), chunk = (uint32_t)(lane & 7) ^ swizzle8(row);
+    w_off[p] = (uint32_t)(((int64_t)min(n0 + (int)row, N - 1) * ldw + chunk * 8) * 2);
+  }
+  const int ktiles = K / 64;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  const __amdgpu_buffer_rsrc_t a_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)(((int64_t)(M - 1) * lda + K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t w_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)(((int64_t)(N - 1) * ldw + K) * 2), 0x00020000);
+  auto load_step = [&](int kt, int buf) {
+    const int koff = min(kt, ktiles - 1) * EROW;
+    char* dst = lds_bytes + buf * BUF + wave * 1024;
+#pragma unroll
+    for (int p = 0; p < CA; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(dst + p * 4096), 16, a_off[p], koff, 0, 0);
+#pragma unroll
+    for (int p = 0; p < CW; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)(dst + BM * EROW + p * 4096), 16, w_off[p], koff, 0, 0);
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int lrow = lane & 31, h = lane >> 5;
+  uint32_t rd[4];       // byte offsets of this lane's operand chunk for each 16 columns of a step
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) rd[ks] = (uint32_t)(lrow * EROW) + (((uint32_t)(ks * 2 + h) ^ swizzle8((uint32_t)lrow)) << 4);
+  const uint32_t a_rd = (uint32_t)(wm * 32 * TM * EROW), w_rd = (uint32_t)(BM * EROW + wn * 32 * TN * EROW);
+  bf16x8 a[2][TM], b[2][TN];
+  auto read_operands = [&](int buf, int ks, bf16x8* af, bf16x8* bf) {
+    const char* tile = lds_bytes + buf * BUF + rd[ks];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 32 * EROW);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * EROW);
+  };
+  auto multiply = [&](const bf16x8* af, const bf16x8* bf, int from, int to) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        if (i * TN + j >= from && i * TN + j < to)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);   // transposed
+  };
+
+  constexpr int RD = TM + TN, MF = TM * TN, LD = CA + CW, HALF = MF / 2;
+#pragma unroll
+  for (int s = 0; s < NBUF - 1; ++s) load_step(s, s);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 2) * LD) : "memory");     // K step 0 has landed
+  __builtin_amdgcn_s_barrier();
+  read_operands(0, 0, a[0], b[0]);
+
+  // One step of 64 columns in four quarters.  The requests for K step kt + NBUF - 1 go out
+  // under the first quarter (its buffer was last read in step kt - 1, before that step's
+  // barrier).  The barrier stands in the middle of the last quarter: this wave's part of
+  // K step kt + 1 has landed when at most the loads of NBUF - 2 steps are outstanding;
+  // after it everybody's has, and nobody reads this step's buffer any more.
+  int rb = 0;                                   // kt % NBUF
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int lb = rb == 0 ? NBUF - 1 : rb - 1, nb = rb == NBUF - 1 ? 0 : rb + 1;
+    read_operands(rb, 1, a[1], b[1]);
+    multiply(a[0], b[0], 0, MF);
+    load_step(kt + NBUF - 1, lb);
+    Interleave<0x100, HALF, RD>::emit();
+    __builtin_amdgcn_sched_group_barrier(0x008, MF - HALF, 0);
+    // (the loads follow the reads in program order; the scheduler places them between the
+    // products of the next quarter)
+    read_operands(rb, 2, a[0], b[0]);
+    multiply(a[1], b[1], 0, MF);
+    Interleave<0x020, MF, LD>::emit();
+    __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);
+    read_operands(rb, 3, a[1], b[1]);
+    multiply(a[0], b[0], 0, MF);
+    Interleave<0x100, MF, RD>::emit();
+    multiply(a[1], b[1], 0, HALF);
+    __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NBUF - 2) * LD) : "memory");
+    __builtin_amdgcn_s_barrier();
+    read_operands(nb, 0, a[0], b[0]);
+    multiply(a[1], b[1], HALF, MF);
+    Interleave<0x100, MF - HALF, RD>::emit();
+    rb = nb;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  const bool vec = MODE == OUT_SWIGLU ? (ldc % 2 == 0 && (uintptr_t)C % 4 == 0)
+                 : MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0)
+                                    : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+#endif
+}
+
+template <int MODE, int TM, int TN, int NBUF>
+int launch_direct64(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
+                    int M, int N, int K, hipStream_t stream) {
+  const size_t lds = (size_t)NBUF * (64 * TM + 64 * TN) * EROW;
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail("gemm_bf16: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
+  dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
+  gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
+  return 0;
+}
+
+// The large tiles take a product whose K is a multiple of 64, whose byte offsets fit 32
 // bits, and which has enough of them.
 inline bool large_fits(int64_t lda, int64_t ldw, int M, int N, int K) {
-  return K % DBK == 0 && (int64_t)M * lda < (1ll << 30) && (int64_t)N * ldw < (1ll << 30);
+  return K % 64 == 0 && (int64_t)M * lda < (1ll << 30) && (int64_t)N * ldw < (1ll << 30);
 }
 
 // ------------------------------------------------------------------ skinny ---
@@ -665,8 +823,8 @@ inline int fastest_tiled(int M, int N, int K, bool large_ok) {
   const double t2 = tiles(128, 128), t4 = tiles(256, 256), t5 = tiles(256, 128);
   const double c2 = t2 <= cus ? 128.0 * 128 / 0.22 : rounds(t2, 2 * cus) * 2 * 128 * 128 / 0.31;
   const double fill = K >= 512 ? 1.0 : 0.6;            // the four-buffer pipeline needs a few steps to pay
-  const double c4 = rounds(t4, cus) * 256 * 256 / (0.50 * fill);
-  const double c5 = rounds(t5, cus) * 256 * 128 / (0.37 * fill);
+  const double c4 = rounds(t4, cus) * 256 * 256 / (0.46 * fill);
+  const double c5 = rounds(t5, cus) * 256 * 128 / (0.42 * fill);
   if (c4 <= c5 && c4 <= c2) return 4;
   return c5 <= c2 ? 5 : 2;
 }
@@ -679,7 +837,7 @@ int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf1
   if (choice != 2 && choice != 4 && choice != 5) choice = fastest_tiled(M, N, K, large_ok);
   if (choice >= 4 && !large_ok) choice = 2;
   if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, stream);
-  if (choice == 5) return launch_direct<MODE, 4, 2>(C, ldc, A, lda, W, ldw, M, N, K, stream);
+  if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, stream);
   return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, stream);
 }
 
