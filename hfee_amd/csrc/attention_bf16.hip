@@ -266,6 +266,53 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
   }
 }
 
+// Joins the splits of one (segment, head) in ascending split order: lane s holds the
+// weight of split s, every lane then walks the splits for its own dims.  One wave.
+// COHERENT: the partial results were written by other workgroups of this launch, so
+// they are read at device scope.
+template <bool COHERENT>
+__device__ __forceinline__ float read_partial(const float* p) {
+  if constexpr (COHERENT) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else return *p;
+}
+
+template <bool COHERENT>
+__device__ __forceinline__ void combine_head(bf16_t* __restrict__ orow, const float* __restrict__ pr, int num_splits) {
+  const int lane = threadIdx.x & 63;
+  float m = -INFINITY, l = 0.f;
+  float o[(HD + 63) / 64];
+#pragma unroll
+  for (int j = 0; j < (HD + 63) / 64; ++j) o[j] = 0.f;
+  for (int s0 = 0; s0 < num_splits; s0 += 64) {          // 64 splits at a time
+    const int mine = s0 + lane;
+    const float ms = mine < num_splits ? read_partial<COHERENT>(pr + (int64_t)mine * (HD + 2) + HD) : -INFINITY;
+    const float ls = mine < num_splits ? read_partial<COHERENT>(pr + (int64_t)mine * (HD + 2) + HD + 1) : 0.f;
+    const float m_new = fmaxf(m, wave_max(ms));
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float rescale = exp2f(m - m_use);
+    const float f = exp2f(ms - m_use);                    // this lane's split weight
+    l = l * rescale + wave_sum(ls * f);
+#pragma unroll
+    for (int j = 0; j < (HD + 63) / 64; ++j) o[j] *= rescale;
+    const int count = min(64, num_splits - s0);
+    for (int s = 0; s < count; ++s) {
+      const float fs = __shfl(f, s, 64);
+#pragma unroll
+      for (int j = 0; j < (HD + 63) / 64; ++j) {
+        const int d = lane + 64 * j;
+        if (d < HD) o[j] += read_partial<COHERENT>(pr + (int64_t)(s0 + s) * (HD + 2) + d) * fs;
+      }
+    }
+    m = m_new;
+  }
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int j = 0; j < (HD + 63) / 64; ++j) {
+    const int d = lane + 64 * j;
+    if (d < HD) orow[d] = float_to_bf16(o[j] * inv);
+  }
+}
+
 // -------------------------------------------------------------------- decode ---
 // One workgroup of up to four waves per (decode segment, KV head, split).  The slots
 // are the heads of the group, 32 at a time.  The workgroup's key tiles are dealt to its
@@ -279,7 +326,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
     const bf16_t* __restrict__ cache, CacheLayout lay, const int* __restrict__ seg_rows,
     const int* __restrict__ seg_positions, const int* __restrict__ seg_tables,
     const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2, int window,
-    float* __restrict__ partial, int num_splits) {
+    float* __restrict__ partial, int num_splits, int* __restrict__ counters) {
   extern __shared__ float lds[];   // [waves][slots][HD + 2]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r32 = lane & 31, G = lane >> 5;
   const int waves = blockDim.x >> 6;
@@ -347,59 +394,50 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
         for (int i = 0; i < 4; ++i) v4[i] = float_to_bf16(o[i] * inv);
         *reinterpret_cast<u32x2*>(out + (int64_t)row * ld_out + head * HD + d) = *reinterpret_cast<const u32x2*>(v4);
       } else {
+        // stores of device scope: they go through to memory, where the workgroup that
+        // joins the splits (on any XCD) reads them
         float* pr = partial + ((int64_t)(sidx * num_heads + head) * num_splits + split) * (HD + 2);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) pr[d + i] = o[i];
+        for (int i = 0; i < 4; ++i) __hip_atomic_store(pr + d + i, o[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (d == 0) {
-          pr[HD] = m;
-          pr[HD + 1] = l;
+          __hip_atomic_store(pr + HD, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(pr + HD + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
     }
   }
+
+  // The split that finishes last joins the splits of its (segment, KV head), so that no
+  // second launch is needed: every workgroup publishes its partial results and counts
+  // itself; nobody waits for anybody.  The counter is back at zero afterwards.
+  if (num_splits > 1 && counters != nullptr) {
+    __shared__ int is_last;
+    // The partial results were stored at device scope and are complete when the store
+    // counter is zero; the joining workgroup reads them with loads of device scope.  No
+    // fence: a release would write the whole L2 back and an acquire would empty it, under
+    // the workgroups that still stream keys.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int* counter = counters + sidx * lay.kv_heads + kvh;
+    if (threadIdx.x == 0) is_last = atomicAdd(counter, 1) == num_splits - 1;
+    __syncthreads();
+    if (is_last) {
+      for (int hh = wave; hh < group; hh += waves)
+        combine_head<true>(out + (int64_t)row * ld_out + (kvh * group + hh) * HD,
+                           partial + (int64_t)(sidx * num_heads + kvh * group + hh) * num_splits * (HD + 2), num_splits);
+      if (threadIdx.x == 0) atomicExch(counter, 0);
+    }
+  }
 }
 
-// Joins the splits of one (segment, head) in ascending split order: lane s holds the
-// weight of split s, every lane then walks the splits for its own dims.
+// The same join as a launch of its own (for callers that bring no counters).
 __global__ __launch_bounds__(64) void combine_kernel(bf16_t* __restrict__ out, int64_t ld_out,
                                                      const int* __restrict__ seg_rows,
                                                      const float* __restrict__ partial, int num_heads,
                                                      int num_splits) {
-  const int sidx = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const float* pr = partial + (int64_t)(sidx * num_heads + h) * num_splits * (HD + 2);
-  float m = -INFINITY, l = 0.f;
-  float o[(HD + 63) / 64];
-#pragma unroll
-  for (int j = 0; j < (HD + 63) / 64; ++j) o[j] = 0.f;
-  for (int s0 = 0; s0 < num_splits; s0 += 64) {          // 64 splits at a time
-    const int mine = s0 + lane;
-    const float ms = mine < num_splits ? pr[(int64_t)mine * (HD + 2) + HD] : -INFINITY;
-    const float ls = mine < num_splits ? pr[(int64_t)mine * (HD + 2) + HD + 1] : 0.f;
-    const float m_new = fmaxf(m, wave_max(ms));
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float rescale = exp2f(m - m_use);
-    const float f = exp2f(ms - m_use);                    // this lane's split weight
-    l = l * rescale + wave_sum(ls * f);
-#pragma unroll
-    for (int j = 0; j < (HD + 63) / 64; ++j) o[j] *= rescale;
-    const int count = min(64, num_splits - s0);
-    for (int s = 0; s < count; ++s) {
-      const float fs = __shfl(f, s, 64);
-#pragma unroll
-      for (int j = 0; j < (HD + 63) / 64; ++j) {
-        const int d = lane + 64 * j;
-        if (d < HD) o[j] += pr[(int64_t)(s0 + s) * (HD + 2) + d] * fs;
-      }
-    }
-    m = m_new;
-  }
-  const float inv = 1.0f / l;
-  bf16_t* orow = out + (int64_t)seg_rows[sidx] * ld_out + h * HD;
-#pragma unroll
-  for (int j = 0; j < (HD + 63) / 64; ++j) {
-    const int d = lane + 64 * j;
-    if (d < HD) orow[d] = float_to_bf16(o[j] * inv);
-  }
+  const int sidx = blockIdx.x, h = blockIdx.y;
+  combine_head<false>(out + (int64_t)seg_rows[sidx] * ld_out + h * HD,
+                      partial + (int64_t)(sidx * num_heads + h) * num_splits * (HD + 2), num_splits);
 }
 
 }  // namespace
@@ -438,12 +476,15 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
 // seg_rows / seg_positions / seg_tables: per decode segment its row in the batch,
 // its position and its block-table row.  partial: at least
 // num_segments * num_heads * num_splits * (head_dim + 2) floats when num_splits > 1.
+// counters: null, or at least num_segments * kv_heads int32 that are zero (and are zero
+// again when the kernel has run): the splits are then joined by the workgroup that
+// finishes last instead of by a second launch.
 HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
                                         const int* seg_rows, const int* seg_positions, const int* seg_tables,
                                         int num_segments, const int* block_tables, int bt_stride,
                                         int num_heads, int kv_heads, int page_size, float scale, int window,
                                         float* partial, int64_t partial_floats, int num_splits, int waves,
-                                        hipStream_t stream) {
+                                        int* counters, int num_counters, hipStream_t stream) {
   HFEE_REQUIRE(num_segments >= 0, "attention_bf16_decode: bad segment count");
   if (num_segments == 0) return 0;
   CacheLayout lay;
@@ -458,6 +499,7 @@ HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q
                  (long long)partial_floats, (long long)need);
   }
   dim3 grid(num_segments, kv_heads, num_splits);
+  const bool in_kernel_join = counters != nullptr && num_counters >= num_segments * kv_heads;
   const int group = num_heads / kv_heads;
   const size_t per_wave = (size_t)(group < 32 ? group : 32) * (HD + 2) * sizeof(float);
   HFEE_REQUIRE(waves >= 1 && waves <= DECODE_MAX_WAVES, "attention_bf16_decode: 1..%d waves, got %d",
@@ -474,9 +516,9 @@ HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q
   }
   decode_kernel<<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
                                          seg_rows, seg_positions, seg_tables, block_tables, bt_stride, num_heads,
-                                         scale * LOG2E, window, partial, num_splits);
+                                         scale * LOG2E, window, partial, num_splits, in_kernel_join ? counters : nullptr);
   HFEE_CHECK_LAUNCH("attention_bf16_decode");
-  if (num_splits > 1) {
+  if (num_splits > 1 && !in_kernel_join) {
     dim3 cgrid(num_segments, num_heads);
     combine_kernel<<<cgrid, 64, 0, stream>>>((bf16_t*)out, ld_out, seg_rows, partial, num_heads, num_splits);
     HFEE_CHECK_LAUNCH("attention_bf16_decode(combine)");

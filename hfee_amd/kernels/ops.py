@@ -264,10 +264,12 @@ def attention_bf16_prefill(out, q, cache_layer, tiles, block_tables, num_heads: 
 
 def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tables, block_tables,
                           num_heads: int, kv_heads: int, head_dim: int, page_size: int, scale: float,
-                          window: int, partial, num_splits: int, waves: int = 4):
+                          window: int, partial, num_splits: int, waves: int = 4, counters=None):
     """One query token per listed segment.  A workgroup of `waves` waves (at most 4)
     shares the keys of one (segment, KV head, split) and joins them in LDS; with
-    num_splits > 1 a second kernel joins the splits."""
+    num_splits > 1 the splits are joined by a second kernel, or, given `counters` (at
+    least segments x kv_heads int32 that are zero, and are zero again afterwards), by
+    the workgroup of each (segment, KV head) that finishes last."""
     n, ldq, ldo = _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size)
     count = seg_rows.numel()
     _i32(seg_rows, "attention seg_rows")
@@ -276,11 +278,15 @@ def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tabl
     if num_splits > 1:
         _check(partial is not None and partial.dtype == torch.float32 and partial.is_contiguous(),
                "attention: float32 partial buffer expected")
+    if counters is not None:
+        _check(counters.dtype == torch.int32 and counters.is_contiguous() and counters.is_cuda,
+               "attention: int32 counters expected")
     lib.attention_bf16(head_dim).call(
         "hfee_attention_bf16_decode", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(seg_rows),
         _ptr(seg_positions), _ptr(seg_tables), count, _ptr(block_tables), block_tables.stride(0),
         num_heads, kv_heads, page_size, float(scale), int(window), _ptr(partial),
-        0 if partial is None else partial.numel(), int(num_splits), int(waves), _stream())
+        0 if partial is None else partial.numel(), int(num_splits), int(waves),
+        _ptr(counters), 0 if counters is None else counters.numel(), _stream())
 
 
 # ------------------------------------------------------- fused decode products (M <= 64)

@@ -170,10 +170,12 @@ class Attention(Mixer):
                 key_tiles = (span + _TILE - 1) // _TILE
                 splits = max(-(-key_tiles // (_DECODE_WAVES * _TILES_PER_WAVE)),
                              min(_DECODE_WORKGROUPS // max(1, nseg * K), -(-key_tiles // _DECODE_WAVES)), 1)
-                partial = None
+                partial = counters = None
                 if splits > 1:
                     partial = ctx.workspace.flat("attention.partial", nseg * H * splits * (hd + 2), torch.float32)
+                    counters = ctx.workspace.counters("attention.splits", nseg * K)
                 ops.attention_bf16_decode(att, q, cache, rows, ctx.extra["attention.decode_positions"],
                                           ctx.extra["attention.decode_tables"], tables, H, K, hd,
-                                          ctx.page_size, self.scale, self.window, partial, splits, _DECODE_WAVES)
+                                          ctx.page_size, self.scale, self.window, partial, splits, _DECODE_WAVES,
+                                          counters)
         ops.linear(x, att, self.w_o, accumulate=True)

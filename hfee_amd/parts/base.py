@@ -171,6 +171,18 @@ class Workspace:
             buf = self._buffers[key] = torch.empty((count,), dtype=dtype, device=self.device)
         return buf[:count]
 
+    def counters(self, name: str, count: int) -> torch.Tensor:
+        """`count` int32 that are zero, for kernels whose workgroups count themselves
+        (the one that finishes last does a final piece of work and sets the counter
+        back to zero, so the buffer is zero again whenever a kernel has run)."""
+        key = (name, "counters", torch.int32)
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < count:
+            if buf is not None:
+                self._retired.append(buf)
+            buf = self._buffers[key] = torch.zeros((max(count, 256),), dtype=torch.int32, device=self.device)
+        return buf[:count]
+
 
 @dataclass
 class StepContext:

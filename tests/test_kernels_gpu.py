@@ -302,13 +302,17 @@ def test_attention_kernels(H, K, hd, T, window, dtype):
         ops.attention_bf16_prefill(out2, qd, layer, tiles, table, H, K, hd, ps, scale, window)
         close(out2, ref, tol)
         # decode kernel: the last rows as single queries, with and without split keys
-        for splits in (1, 3):
+        # (joined by a second launch, and by the workgroup that finishes last: twice, the
+        # second time on the counters that the first call left)
+        counters = torch.zeros(3 * K, dtype=torch.int32, device=DEV)
+        for splits, cnt in ((1, None), (3, None), (3, counters), (4, counters)):
             rows = torch.tensor([T - 1, T // 2, 0], dtype=torch.int32, device=DEV)
             out3 = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
             partial = torch.zeros(3 * H * splits * (hd + 2), dtype=torch.float32, device=DEV)
             ops.attention_bf16_decode(out3, qd, layer, rows, rows.clone(), torch.zeros(3, dtype=torch.int32, device=DEV),
-                                      table, H, K, hd, ps, scale, window, partial, splits)
+                                      table, H, K, hd, ps, scale, window, partial, splits, counters=cnt)
             close(out3[[T - 1, T // 2, 0]], ref[[T - 1, T // 2, 0]], tol)
+            assert int(counters.abs().sum()) == 0
 
 
 @pytest.mark.parametrize("pairing", ["half", "interleaved"])
