@@ -51,7 +51,7 @@ union Op {          // one matrix-instruction operand: eight bfloat16
 
 struct Tile {
   // running state of 32 query slots; this lane's slot is lane % 32
-  float m;              // running maximum of the scaled scores (log2 domain)
+  float m;              // reference of the exponentials: at most SLACK below the running maximum (log2 domain)
   float l;              // running sum
   f32x16 o[NDT];        // O^T: register r of tile t is dim 32t + 8*(r/4) + 4*(lane/32) + r%4
 };
@@ -121,11 +121,13 @@ __device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict
   }
 }
 
-// Adds the keys k0 .. k0+31 (already loaded) to the running state.  q_op: this slot's
-// query, pre-loaded as NC operands.  pos: this slot's position (keys lo..pos are
-// visible; -1 for an unused slot).
-__device__ __forceinline__ void compute_tile(Tile& st, const Op* q_op, const TileOps& ops, int k0, int pos, int lo,
-                                             float scale_log2) {
+// Adds the keys k0 .. k0+31 to the running state.  q_op: this slot's query, pre-loaded
+// as NC operands.  pos: this slot's position (keys lo..pos are visible; -1 for an unused
+// slot).  key_op(c) and value_op(u, t) hand over the tile's operands: from registers, or
+// from a tile in LDS that several waves share.
+template <class KeyOp, class ValueOp>
+__device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyOp key_op, ValueOp value_op, int k0,
+                                                  int pos, int lo, float scale_log2, bool all_visible) {
   const int lane = threadIdx.x & 63, G = lane >> 5;
 
   // ---- S^T = K Q^T ------------------------------------------------------------
@@ -133,53 +135,84 @@ __device__ __forceinline__ void compute_tile(Tile& st, const Op* q_op, const Til
 #pragma unroll
   for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
-  for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops.k[c].v, q_op[c].v, s, 0, 0, 0);
+  for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(key_op(c), q_op[c].v, s, 0, 0, 0);
 
   // ---- mask, running maximum and sum ------------------------------------------
+  // all_visible (the same for the whole wave): every key of the tile is visible to every
+  // slot in use, so the comparisons are left out.  (A slot that is not in use then holds
+  // numbers without meaning; they stay in its own lanes and are never stored.)
   float tile_max = -INFINITY;
+  if (all_visible) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int key = k0 + 8 * (r >> 2) + 4 * G + (r & 3);
-    const bool visible = key <= pos && key >= lo;
-    s[r] = visible ? s[r] * scale_log2 : -INFINITY;
-    tile_max = fmaxf(tile_max, s[r]);
+    for (int r = 0; r < 16; ++r) {
+      s[r] *= scale_log2;
+      tile_max = fmaxf(tile_max, s[r]);
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = k0 + 8 * (r >> 2) + 4 * G + (r & 3);
+      const bool visible = key <= pos && key >= lo;
+      s[r] = visible ? s[r] * scale_log2 : -INFINITY;
+      tile_max = fmaxf(tile_max, s[r]);
+    }
   }
   tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-  const float m_new = fmaxf(st.m, tile_max);
-  const float m_use = m_new == -INFINITY ? 0.f : m_new;
-  const float alpha = exp2f(st.m - m_use);          // st.m == -inf gives 0
+  // st.m is the reference that the exponentials are taken against, not always the exact
+  // maximum: it moves (and the sums are rescaled) only when some slot's scores rise more
+  // than SLACK above it, for every slot of the wave at once.  Below that the terms are at
+  // most 2^SLACK, which float32 sums and bfloat16 factors hold as well as terms below 1;
+  // the quotient o / l does not depend on the reference.  After the first tiles a
+  // maximum seldom moves that far, so the rescaling of O is rare.
+  constexpr float SLACK = 8.0f;
+  if (__builtin_amdgcn_ballot_w64(tile_max > st.m + SLACK) != 0) {
+    const float m_new = fmaxf(st.m, tile_max);
+    // 2^x by the hardware instruction alone: its arguments here are <= 0, and a result
+    // too small for a normal number may become zero
+    const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(st.m - m_new);   // st.m == -inf gives 0
+    st.l *= alpha;
+    st.m = m_new;
+#pragma unroll
+    for (int t = 0; t < NDT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
+  }
+  const float m_use = st.m == -INFINITY ? 0.f : st.m;
   float psum = 0.f;
   Op p[2];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const float e = exp2f(s[r] - m_use);
+    const float e = __builtin_amdgcn_exp2f(s[r] - m_use);
     psum += e;
     p[r >> 3].e[r & 7] = float_to_bf16(e);
   }
   psum += __shfl_xor(psum, 32, 64);
-  st.l = st.l * alpha + psum;
-  st.m = m_new;
-#pragma unroll
-  for (int t = 0; t < NDT; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) st.o[t][r] *= alpha;
+  st.l += psum;
 
   // ---- O^T += V^T P^T ----------------------------------------------------------
 #pragma unroll
   for (int u = 0; u < 2; ++u)
 #pragma unroll
     for (int t = 0; t < NDT; ++t)
-      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops.v[u][t].v, p[u].v, st.o[t], 0, 0, 0);
+      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(value_op(u, t), p[u].v, st.o[t], 0, 0, 0);
+}
+
+__device__ __forceinline__ void compute_tile(Tile& st, const Op* q_op, const TileOps& ops, int k0, int pos, int lo,
+                                             float scale_log2, bool all_visible) {
+  compute_tile_with(st, q_op, [&](int c) { return ops.k[c].v; }, [&](int u, int t) { return ops.v[u][t].v; }, k0, pos, lo,
+                    scale_log2, all_visible);
 }
 
 // The tiles first, first + step, ... < end of one sequence.  AHEAD: each tile's loads
 // are issued while the tile before it is computed (two tiles' operands in registers:
 // for kernels that run one wave per SIMD anyway); otherwise tile by tile.
+// all_first..all_last: the keys that every slot in use sees (a tile inside this range
+// needs no mask).
 template <bool AHEAD>
 __device__ __forceinline__ void attend_tiles(Tile& st, const Op* q_op, const bf16_t* __restrict__ cache,
                                              const CacheLayout& lay, const int* __restrict__ bt, int bt_stride,
                                              int kvh, int first, int end, int step, int kv_first, int kv_last,
-                                             int pos, int lo, float scale_log2) {
+                                             int pos, int lo, float scale_log2, int all_first, int all_last) {
   if (first >= end) return;
   PageWindow pages;
   pages.base = -1;
@@ -189,14 +222,14 @@ __device__ __forceinline__ void attend_tiles(Tile& st, const Op* q_op, const bf1
     for (int t = first; t < end; t += step) {
       const int tn = t + step;
       if (tn < end) load_tile(nxt, cache, lay, bt, bt_stride, pages, kvh, tn * 32, kv_first, kv_last);
-      compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2);
+      compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2, t * 32 >= all_first && t * 32 + 31 <= all_last);
       cur = nxt;
     }
   } else {
     for (int t = first; t < end; t += step) {
       TileOps cur;
       load_tile(cur, cache, lay, bt, bt_stride, pages, kvh, t * 32, kv_first, kv_last);
-      compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2);
+      compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2, t * 32 >= all_first && t * 32 + 31 <= all_last);
     }
   }
 }
@@ -225,13 +258,26 @@ __device__ __forceinline__ void init_tile(Tile& st) {
 __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, int64_t ld_out,
                                                      const bf16_t* __restrict__ q, int64_t ldq,
                                                      const bf16_t* __restrict__ cache, CacheLayout lay,
-                                                     const int* __restrict__ work,
+                                                     const int* __restrict__ work, int num_tiles,
                                                      const int* __restrict__ block_tables, int bt_stride,
                                                      int num_heads, float scale_log2, int window) {
   const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
-  const int* wk = work + 4 * blockIdx.x;
+  // Workgroups go to the eight XCDs in turn, and each XCD has an L2 of its own.  Every
+  // XCD gets a contiguous run of the work, ordered by KV head first: the keys and values
+  // of a head are then read through one L2 (with eight KV heads, one head per XCD).
+  // Within a head the later row tiles, which see more keys, come first.
+  int tile, h;
+  {
+    const int total = num_tiles * num_heads, per_xcd = (total + 7) / 8;
+    const int u = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (u >= total) return;
+    const int group = num_heads / lay.kv_heads, per_kv = num_tiles * group;
+    const int kv = u / per_kv, rest = u - kv * per_kv;
+    tile = num_tiles - 1 - rest / group;
+    h = kv * group + rest % group;
+  }
+  const int* wk = work + 4 * tile;
   const int row0 = wk[0], rows = wk[1], pos0 = wk[2], seg = wk[3];
-  const int h = blockIdx.y;
   const int kvh = h / (num_heads / lay.kv_heads);
   const int* bt = block_tables + (int64_t)seg * bt_stride;
 
@@ -245,8 +291,152 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
   init_tile(st);
   const int kv_last = pos0 + rows - 1;
   const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
+  // every row in use sees the keys from the last row's window start to the first row's position
   attend_tiles<false>(st, q_op, cache, lay, bt, bt_stride, kvh, kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
-               scale_log2);
+               scale_log2, window > 0 ? max(0, kv_last - window + 1) : 0, pos0);
+
+  if (slot_ok) {
+    const float inv = 1.0f / st.l;
+    bf16_t* orow = out + (int64_t)(row0 + r32) * ld_out + h * HD;
+#pragma unroll
+    for (int t = 0; t < NDT; ++t)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int d = 32 * t + 8 * b + 4 * G;
+        if (d < HD) {
+          bf16_t v4[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v4[i] = float_to_bf16(st.o[t][4 * b + i] * inv);
+          *reinterpret_cast<u32x2*>(orow + d) = *reinterpret_cast<const u32x2*>(v4);
+        }
+      }
+  }
+}
+
+// --------------------------------------------- prefill, key tiles shared in LDS ---
+// The heads that share a KV head read the same keys and values.  A workgroup takes a
+// tile of 32 rows for up to four such heads, one wave a head, and brings every key
+// tile into LDS once: each lane asks for exactly the 16 bytes that it would have loaded
+// as its own operand, but straight into LDS (lane l of a 1 KB block), and every wave
+// then reads its operands from there, a block being one operand of the whole wave,
+// contiguous.  Two tiles of LDS: the next tile's loads are in flight while this one is
+// multiplied, without a register for them.  Lanes whose key or value does not exist
+// read a place that does (masked keys count for nothing; the cache never holds anything
+// but finite numbers, so a masked value times zero is zero).
+constexpr int KV_BLOCKS = NC + 2 * NDT;           // 1 KB blocks of one key tile: keys, then values
+constexpr int SHARED_WAVES = 4;
+
+// What of a lane's addresses does not change from tile to tile (in elements from the
+// start of a page): the tile adds the page and a uniform slot offset.
+struct LaneOffsets {
+  int64_t key;              // this lane's key row within a page (k0 % page_size == 0), its half of a chunk
+  int64_t value[NDT];       // this lane's value column of each 32-wide part of the head, its half of the slots
+};
+
+__device__ __forceinline__ LaneOffsets lane_offsets(const CacheLayout& lay, int kvh) {
+  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+  LaneOffsets o;
+  o.key = lay.key_offset(0, kvh, r32 & (lay.page_size - 1), 0) + G * 8;
+#pragma unroll
+  for (int t = 0; t < NDT; ++t)
+    o.value[t] = lay.value_column(0, kvh, min(32 * t + r32, HD - 1)) + 8 * G;   // rows beyond the head repeat its last one
+  return o;
+}
+
+__device__ __forceinline__ void request_tile(char* __restrict__ tile_lds, const bf16_t* __restrict__ cache,
+                                             const CacheLayout& lay, const LaneOffsets& off,
+                                             const int* __restrict__ bt, int bt_stride, PageWindow& pages, int k0,
+                                             int kv_first, int kv_last, int wave, int waves) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef const __attribute__((address_space(1))) void* global_ptr;
+  const int r32 = threadIdx.x & 31;
+  {
+    const int b0 = k0 >> lay.page_shift, b1 = (k0 + 31) >> lay.page_shift;
+    if (pages.base < 0 || b0 < pages.base || b1 >= pages.base + 64) pages.fill(bt, bt_stride, b0);
+  }
+  // Keys outside kv_first..kv_last read page 0.  A key's slot in its page is
+  // (k0 + r32) % page_size = k0 % page_size + r32 % page_size: k0 is a multiple of 32.
+  const int key = k0 + r32;
+  const bool key_ok = key <= kv_last && key >= kv_first;
+  const int key_page = pages.of(key >> lay.page_shift);
+  const bf16_t* krow = cache + (key_ok ? key_page * lay.page_stride : 0) + off.key +
+                       (int64_t)(k0 & (lay.page_size - 1)) * lay.head_dim;
+  const bf16_t* vbase[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int kb = k0 + 16 * u;
+    const bool ok = kb <= kv_last && kb + 15 >= kv_first;
+    const int page = pages.of(kb >> lay.page_shift);
+    vbase[u] = cache + (ok ? page * lay.page_stride + (kb & (lay.page_size - 1)) : 0);
+  }
+  // the blocks are dealt to the waves in turn (the test is uniform over a wave)
+  int turn = 0;
+#pragma unroll
+  for (int b = 0; b < KV_BLOCKS; ++b) {
+    if (turn == wave) {
+      const bf16_t* src = b < NC ? krow + b * 16 : vbase[(b - NC) / NDT] + off.value[(b - NC) % NDT];
+      __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)(tile_lds + b * 1024), 16, 0, 0);
+    }
+    turn = turn + 1 == waves ? 0 : turn + 1;
+  }
+}
+
+// work: per row tile 4 ints (first row, rows <= 32, first position, block-table row).
+__global__ __launch_bounds__(SHARED_WAVES * 64) void prefill_shared_kernel(
+    bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
+    const bf16_t* __restrict__ cache, CacheLayout lay, const int* __restrict__ work, int num_tiles,
+    const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2, int window) {
+  extern __shared__ __attribute__((aligned(1024))) char kv_lds[];     // two tiles of KV_BLOCKS KB
+  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), waves = blockDim.x >> 6;
+  const int group = num_heads / lay.kv_heads, chunks = (group + waves - 1) / waves;
+  // Workgroups go to the eight XCDs in turn; every XCD gets a contiguous run of the work,
+  // ordered by KV head first (its keys then live in one L2), later row tiles first.
+  int tile, kvh, chunk;
+  {
+    const int per_kv = num_tiles * chunks, total = per_kv * lay.kv_heads, per_xcd = (total + 7) / 8;
+    const int u = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (u >= total) return;
+    kvh = u / per_kv;
+    const int rest = u - kvh * per_kv;
+    tile = num_tiles - 1 - rest / chunks;
+    chunk = rest % chunks;
+  }
+  const int* wk = work + 4 * tile;
+  const int row0 = wk[0], rows = wk[1], pos0 = wk[2], seg = wk[3];
+  const int* bt = block_tables + (int64_t)seg * bt_stride;
+  const bool head_ok = chunk * waves + wave < group;      // a wave without a head still loads its share
+  const int h = kvh * group + (head_ok ? chunk * waves + wave : 0);
+
+  const bool slot_ok = r32 < rows && head_ok;
+  const int pos = slot_ok ? pos0 + r32 : -1;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  Op q_op[NC];
+  load_query(q_op, q + (int64_t)(row0 + (slot_ok ? r32 : 0)) * ldq + h * HD, slot_ok);
+
+  Tile st;
+  init_tile(st);
+  const int kv_last = pos0 + rows - 1;
+  const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int t_first = kv_first >> 5, t_end = (kv_last >> 5) + 1;
+  const int all_first = window > 0 ? max(0, kv_last - window + 1) : 0;   // every row in use sees all_first .. pos0
+  PageWindow pages;
+  pages.base = -1;
+  constexpr int TILE_BYTES = KV_BLOCKS * 1024;
+  const LaneOffsets off = lane_offsets(lay, kvh);
+  request_tile(kv_lds, cache, lay, off, bt, bt_stride, pages, t_first * 32, kv_first, kv_last, wave, waves);
+  __syncthreads();               // waits for the loads too
+  for (int t = t_first; t < t_end; ++t) {
+    const char* cur = kv_lds + ((t - t_first) & 1) * TILE_BYTES + lane * 16;
+    if (t + 1 < t_end)
+      request_tile(kv_lds + ((t + 1 - t_first) & 1) * TILE_BYTES, cache, lay, off, bt, bt_stride, pages, (t + 1) * 32,
+                   kv_first, kv_last, wave, waves);
+    compute_tile_with(
+        st, q_op, [&](int c) { return *reinterpret_cast<const bf16x8*>(cur + c * 1024); },
+        [&](int u, int tt) { return *reinterpret_cast<const bf16x8*>(cur + (NC + u * NDT + tt) * 1024); }, t * 32, pos, lo,
+        scale_log2, t * 32 >= all_first && t * 32 + 31 <= pos0);
+    __syncthreads();             // the next tile has landed; nobody reads this one any more
+  }
 
   if (slot_ok) {
     const float inv = 1.0f / st.l;
@@ -351,7 +541,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
     Tile st;
     init_tile(st);
     attend_tiles<true>(st, q_op, cache, lay, bt, bt_stride, kvh, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
-                 scale_log2);
+                 scale_log2, lo, pos);
 
     // this wave's state into LDS
     if (g0 > 0) __syncthreads();
@@ -457,18 +647,39 @@ static int check_common(const char* name, int64_t ld_out, int64_t ldq, int num_h
 }
 
 // work: num_tiles x 4 int32 (first row, rows <= 32, first position, block-table row).
+// variant: 0 choose, 1 one wave per (tile, head), 2 key tiles shared in LDS by the heads
+// of a KV head (for tests of each kernel alone).
 HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* q, int64_t ldq,
                                          const void* cache, const int* work, int num_tiles,
                                          const int* block_tables, int bt_stride, int num_heads, int kv_heads,
-                                         int page_size, float scale, int window, hipStream_t stream) {
+                                         int page_size, float scale, int window, int variant, hipStream_t stream) {
   HFEE_REQUIRE(num_tiles >= 0, "attention_bf16_prefill: bad tile count");
+  HFEE_REQUIRE(variant >= 0 && variant <= 2, "attention_bf16_prefill: unknown kernel choice %d", variant);
   if (num_tiles == 0) return 0;
   CacheLayout lay;
   if (check_common("attention_bf16_prefill", ld_out, ldq, num_heads, kv_heads, page_size, window, out, q, &lay))
     return 1;
-  dim3 grid(num_tiles, num_heads);
-  prefill_kernel<<<grid, 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
-                                          work, block_tables, bt_stride, num_heads, scale * LOG2E, window);
+  HFEE_REQUIRE((int64_t)num_tiles * num_heads < (1ll << 30), "attention_bf16_prefill: too much work for one launch");
+  const int group = num_heads / kv_heads;
+  if (variant == 1 || (variant == 0 && group == 1)) {      // nothing to share: one wave per (tile, head)
+    dim3 grid((unsigned)(((int64_t)num_tiles * num_heads + 7) / 8 * 8));
+    prefill_kernel<<<grid, 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
+                                            work, num_tiles, block_tables, bt_stride, num_heads, scale * LOG2E, window);
+  } else {
+    const int waves = group < SHARED_WAVES ? group : SHARED_WAVES, chunks = (group + waves - 1) / waves;
+    const size_t lds = (size_t)2 * KV_BLOCKS * 1024;
+    static bool raised = false;
+    if (lds > 48 * 1024 && !raised) {
+      hipError_t e = hipFuncSetAttribute((const void*)prefill_shared_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds);
+      HFEE_REQUIRE(e == hipSuccess, "attention_bf16_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
+      raised = true;
+    }
+    dim3 grid((unsigned)(((int64_t)num_tiles * kv_heads * chunks + 7) / 8 * 8));
+    prefill_shared_kernel<<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
+                                                             (const bf16_t*)cache, lay, work, num_tiles, block_tables,
+                                                             bt_stride, num_heads, scale * LOG2E, window);
+  }
   HFEE_CHECK_LAUNCH("attention_bf16_prefill");
   return 0;
 }

@@ -251,15 +251,17 @@ def _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, he
 
 
 def attention_bf16_prefill(out, q, cache_layer, tiles, block_tables, num_heads: int, kv_heads: int,
-                           head_dim: int, page_size: int, scale: float, window: int = 0):
-    """tiles: [num_tiles, 4] int32 (first row, rows <= 32, first position, block-table row)."""
+                           head_dim: int, page_size: int, scale: float, window: int = 0, kernel: int = 0):
+    """tiles: [num_tiles, 4] int32 (first row, rows <= 32, first position, block-table row).
+    kernel: 0 automatic, 1 one wave per (tile, head), 2 the heads of a KV head share its
+    key tiles through LDS."""
     n, ldq, ldo = _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size)
     _check(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
            "attention: tiles must be [num_tiles, 4] int32")
     lib.attention_bf16(head_dim).call(
         "hfee_attention_bf16_prefill", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(tiles),
         tiles.shape[0], _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, page_size,
-        float(scale), int(window), _stream())
+        float(scale), int(window), int(kernel), _stream())
 
 
 def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tables, block_tables,

@@ -271,7 +271,8 @@ def _paged(kv, page_size, pages_order):
 
 @pytest.mark.parametrize("H,K,hd,T,window", [(4, 2, 16, 37, 0), (3, 1, 32, 100, 0), (6, 3, 48, 70, 0),
                                              (2, 2, 64, 33, 0), (4, 1, 128, 130, 0), (4, 2, 16, 90, 20),
-                                             (5, 5, 80, 40, 0), (1, 1, 256, 35, 0)])
+                                             (5, 5, 80, 40, 0), (1, 1, 256, 35, 0), (12, 2, 64, 200, 0),
+                                             (8, 1, 256, 70, 33)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_kernels(H, K, hd, T, window, dtype):
     """Plain kernel (both dtypes) and the matrix-core kernels (bfloat16) against
@@ -298,9 +299,10 @@ def test_attention_kernels(H, K, hd, T, window, dtype):
     close(out, ref, tol)
     if dtype == torch.bfloat16:
         tiles = torch.tensor([(o, min(32, T - o), o, 0) for o in range(0, T, 32)], dtype=torch.int32, device=DEV)
-        out2 = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
-        ops.attention_bf16_prefill(out2, qd, layer, tiles, table, H, K, hd, ps, scale, window)
-        close(out2, ref, tol)
+        for kernel in (0, 1, 2):       # the automatic choice, one wave per (tile, head), tiles shared in LDS
+            out2 = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
+            ops.attention_bf16_prefill(out2, qd, layer, tiles, table, H, K, hd, ps, scale, window, kernel=kernel)
+            close(out2, ref, tol)
         # decode kernel: the last rows as single queries, with and without split keys
         # (joined by a second launch, and by the workgroup that finishes last: twice, the
         # second time on the counters that the first call left)
