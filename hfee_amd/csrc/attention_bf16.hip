@@ -141,23 +141,22 @@ __device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyO
   // all_visible (the same for the whole wave): every key of the tile is visible to every
   // slot in use, so the comparisons are left out.  (A slot that is not in use then holds
   // numbers without meaning; they stay in its own lanes and are never stored.)
+  // (the scale, which is positive, is applied to the maximum here and to each score
+  // inside its exponential below: one multiplication fewer per score)
   float tile_max = -INFINITY;
   if (all_visible) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      s[r] *= scale_log2;
-      tile_max = fmaxf(tile_max, s[r]);
-    }
+    for (int r = 0; r < 16; ++r) tile_max = fmaxf(tile_max, s[r]);
   } else {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int key = k0 + 8 * (r >> 2) + 4 * G + (r & 3);
       const bool visible = key <= pos && key >= lo;
-      s[r] = visible ? s[r] * scale_log2 : -INFINITY;
+      s[r] = visible ? s[r] : -INFINITY;
       tile_max = fmaxf(tile_max, s[r]);
     }
   }
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64)) * scale_log2;
   // st.m is the reference that the exponentials are taken against, not always the exact
   // maximum: it moves (and the sums are rescaled) only when some slot's scores rise more
   // than SLACK above it, for every slot of the wave at once.  Below that the terms are at
@@ -182,7 +181,7 @@ __device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyO
   Op p[2];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const float e = __builtin_amdgcn_exp2f(s[r] - m_use);
+    const float e = __builtin_amdgcn_exp2f(fmaf(s[r], scale_log2, -m_use));
     psum += e;
     p[r >> 3].e[r & 7] = float_to_bf16(e);
   }
@@ -635,7 +634,8 @@ __global__ __launch_bounds__(64) void combine_kernel(bf16_t* __restrict__ out, i
 HFEE_API int hfee_attention_bf16_head_dim() { return HD; }
 
 static int check_common(const char* name, int64_t ld_out, int64_t ldq, int num_heads, int kv_heads,
-                        int page_size, int window, const void* out, const void* q, CacheLayout* lay) {
+                        int page_size, int window, float scale, const void* out, const void* q, CacheLayout* lay) {
+  HFEE_REQUIRE(scale > 0.f && scale < INFINITY, "%s: the score scale must be positive, got %g", name, (double)scale);
   HFEE_REQUIRE(num_heads > 0 && kv_heads > 0 && num_heads % kv_heads == 0,
                "%s: %d heads are not a multiple of %d kv heads", name, num_heads, kv_heads);
   HFEE_REQUIRE(num_heads <= 65535, "%s: too many heads", name);
@@ -657,7 +657,7 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
   HFEE_REQUIRE(variant >= 0 && variant <= 2, "attention_bf16_prefill: unknown kernel choice %d", variant);
   if (num_tiles == 0) return 0;
   CacheLayout lay;
-  if (check_common("attention_bf16_prefill", ld_out, ldq, num_heads, kv_heads, page_size, window, out, q, &lay))
+  if (check_common("attention_bf16_prefill", ld_out, ldq, num_heads, kv_heads, page_size, window, scale, out, q, &lay))
     return 1;
   HFEE_REQUIRE((int64_t)num_tiles * num_heads < (1ll << 30), "attention_bf16_prefill: too much work for one launch");
   const int group = num_heads / kv_heads;
@@ -699,7 +699,7 @@ HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q
   HFEE_REQUIRE(num_segments >= 0, "attention_bf16_decode: bad segment count");
   if (num_segments == 0) return 0;
   CacheLayout lay;
-  if (check_common("attention_bf16_decode", ld_out, ldq, num_heads, kv_heads, page_size, window, out, q, &lay))
+  if (check_common("attention_bf16_decode", ld_out, ldq, num_heads, kv_heads, page_size, window, scale, out, q, &lay))
     return 1;
   HFEE_REQUIRE(num_splits >= 1 && num_splits <= 65535, "attention_bf16_decode: bad split count %d", num_splits);
   HFEE_REQUIRE(kv_heads <= 65535, "attention_bf16_decode: too many kv heads");
