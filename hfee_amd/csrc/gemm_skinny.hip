@@ -16,6 +16,12 @@
 //   EPI_ADD      C (float32) += result        (/root/reference/internal/llm/forward.go:106-107)
 //   EPI_SWIGLU   rows of W alternate gate/up: C[m, j] = silu(gate_j) * up_j
 //                                             (/root/reference/internal/ggml/ops.go:159-165)
+//   EMIT   (with EPI_ADD) a norm that follows the residual add, in two halves so that
+//          nobody waits for a whole row: the product that adds into the stream also
+//          writes bfloat16(x_new * w_next) and, per workgroup, its columns' share of every
+//          row's sum of squares.  The product that consumes the row (ROW SCALE) adds the
+//          shares up, in a fixed order, and scales its finished sums by
+//          1/sqrt(mean + eps): the same numbers as NORM gives, with no norm of its own.
 //   EPI_QKV      rows of W are q, k, v heads with rotation pairs adjacent (2i, 2i+1):
 //                rotate q and k at the token's position, write q to C, k and v into the
 //                token's slot of the paged cache
@@ -67,7 +73,19 @@ struct Args {
   float eps;
   const int* rows;            // NORM: row m of the product is row rows[m] of A (null: m)
   QkvArgs qkv;
+  // EMIT (EPI_ADD only; emit_out null: nothing is emitted)
+  const void* emit_weight;    // [N] weight of the norm that follows
+  int emit_weight_is_f32;
+  bf16_t* emit_out;           // [M, N] bfloat16(x_new * weight)
+  int64_t ld_emit;
+  float* emit_ss;             // [workgroups][SS_STRIDE] this workgroup's columns' sum of squares per row
+  // ROW SCALE (scale_ss null: none)
+  const float* scale_ss;      // [scale_blocks][SS_STRIDE] shares of the rows' sums of squares
+  int scale_blocks;
+  float scale_eps;
 };
+
+constexpr int SS_STRIDE = 64;   // rows of a product of this file
 
 struct Block {                // one wave's operands for one K block
   Chunk w[UNROLL];
@@ -150,6 +168,20 @@ __device__ __forceinline__ void compute_block(f32x4* acc, float* ss, const Block
 }
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
+
+// ROW SCALE: 1/sqrt(mean of squares + eps) of every batch row from the shares that the
+// product before this one left, into `out` (LDS, SS_STRIDE floats).  Wave w takes rows
+// w, w + WAVES, ...; lane l adds shares l, l + 64, ... and the lanes meet in a fixed tree,
+// so the sum does not depend on anything but the shares.  The caller synchronises.
+__device__ __forceinline__ void row_scales(const Args& a, float* out) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int m = wave; m < a.M; m += WAVES) {
+    float t = 0.f;
+    for (int b = lane; b < a.scale_blocks; b += 64) t += a.scale_ss[(int64_t)b * SS_STRIDE + m];
+    t = wave_sum(t);
+    if (lane == 0) out[m] = 1.0f / sqrtf(t / (float)a.K + a.scale_eps);
+  }
+}
 
 // What happens to four finished sums: weight rows n .. n+3 of batch row m.
 template <int EPI>
@@ -289,6 +321,8 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   }
 
   // ---- partial sums meet in LDS ---------------------------------------------------
+  __shared__ float row_scale[SS_STRIDE];
+  if (!NORM && a.scale_ss != nullptr) row_scales(a, row_scale);
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
 #pragma unroll
@@ -303,11 +337,12 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   __syncthreads();
 
   // D layout of the 16x16 tile: register i of lane l is weight row 4*(l/16) + i, batch row l%16
+  // (MT * 64 is a multiple of the wave size: whole waves walk the loop, as the shuffles of EMIT need)
   for (int idx = threadIdx.x; idx < MT * 64; idx += WAVES * 64) {
     const int t = idx >> 6, l = idx & 63;
     const int m = t * 16 + (l & 15);
     const int n = n0 + 4 * (l >> 4);
-    if (m >= a.M || n >= a.N) continue;
+    const bool live = m < a.M && n < a.N;
     float v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -323,9 +358,36 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
       const float scale = 1.0f / sqrtf(s / (float)a.K + a.eps);
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= scale;
+    } else if (a.scale_ss != nullptr) {
+      const float scale = row_scale[min(m, SS_STRIDE - 1)];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= scale;
     }
 
-    epilogue<EPI>(a, m, n, v);
+    if (EPI == EPI_ADD && a.emit_out != nullptr) {
+      // the residual add, and the first half of the norm that follows it
+      float ss = 0.f;
+      if (live) {
+        float* c = (float*)a.C + (int64_t)m * a.ldc + n;
+        bf16_t* e = a.emit_out + (int64_t)m * a.ld_emit + n;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (n + i < a.N) {
+            const float x = c[i] + v[i];
+            c[i] = x;
+            ss = fmaf(x, x, ss);
+            const float w = a.emit_weight_is_f32 ? ((const float*)a.emit_weight)[n + i]
+                                                 : bf16_to_float(((const bf16_t*)a.emit_weight)[n + i]);
+            e[i] = float_to_bf16(x * w);
+          }
+        }
+      }
+      ss += __shfl_xor(ss, 16, 64);          // the four column groups of this row
+      ss += __shfl_xor(ss, 32, 64);
+      if ((l >> 4) == 0 && m < a.M) a.emit_ss[(int64_t)blockIdx.x * SS_STRIDE + m] = ss;
+    } else if (live) {
+      epilogue<EPI>(a, m, n, v);
+    }
   }
 }
 
@@ -409,6 +471,11 @@ __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) t += ss_part[w][r16];
     scale = 1.0f / sqrtf(t / (float)a.K + a.eps);     // for this lane's batch row (lane % 16)
+  } else if (a.scale_ss != nullptr) {
+    __shared__ float row_scale[SS_STRIDE];
+    row_scales(a, row_scale);
+    __syncthreads();
+    scale = row_scale[min(r16, a.M - 1)];
   }
 
   // ---- stream W ---------------------------------------------------------------------
@@ -506,13 +573,19 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 
 // One entry point for every variant.  a_is_f32 != 0 selects the fused RMSNorm (M <= 16).
 // epi: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate, 4 q/k/v.
+// emit_out (with epi 2): also write bfloat16(C_new * emit_weight) to emit_out [M, N] and this
+// product's shares of the rows' sums of squares to emit_ss (ceil(N / 16) x 64 floats).
+// scale_ss: shares left by such a product (scale_blocks x 64 floats) over rows of width K:
+// the finished sums are scaled by 1 / sqrt(sum / K + scale_eps).
 HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
                               int64_t ldw, int M, int N, int K, int epi,
                               const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
                               const int* positions, const int* token_segment, const int* block_tables,
                               int bt_stride, const float* cos_table, const float* sin_table, int half,
                               int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
-                              int page_size, hipStream_t stream) {
+                              int page_size, const void* emit_weight, int emit_weight_is_f32, void* emit_out,
+                              int64_t ld_emit, float* emit_ss, const float* scale_ss, int scale_blocks,
+                              float scale_eps, hipStream_t stream) {
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
   if (M == 0) return 0;
   HFEE_REQUIRE(M <= 64, "gemm_skinny: at most 64 rows, got %d", M);
@@ -551,8 +624,18 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
   } else {
     HFEE_REQUIRE(ldc >= N, "gemm_skinny: ldc is shorter than a row");
   }
+  if (emit_out != nullptr) {
+    HFEE_REQUIRE(epi == EPI_ADD && !norm, "gemm_skinny: a following norm is emitted by the accumulating product only");
+    HFEE_REQUIRE(emit_weight != nullptr && emit_ss != nullptr && ld_emit >= N, "gemm_skinny: incomplete arguments for the emitted norm");
+    a.emit_weight = emit_weight; a.emit_weight_is_f32 = emit_weight_is_f32; a.emit_out = (bf16_t*)emit_out;
+    a.ld_emit = ld_emit; a.emit_ss = emit_ss;
+  }
+  if (scale_ss != nullptr) {
+    HFEE_REQUIRE(!norm && scale_blocks > 0 && scale_eps >= 0.f, "gemm_skinny: a row scale needs its shares and no norm of its own");
+    a.scale_ss = scale_ss; a.scale_blocks = scale_blocks; a.scale_eps = scale_eps;
+  }
   const int mt = (M + 15) / 16;
-  if (launch_wide(a, norm, epi, stream)) {
+  if (emit_out == nullptr && launch_wide(a, norm, epi, stream)) {
     HFEE_CHECK_LAUNCH("gemm_skinny(wide)");
     return 0;
   }

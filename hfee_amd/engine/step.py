@@ -272,8 +272,17 @@ class Engine:
     def _forward(self, ctx, n: int, w: int, dev: dict):
         x = self.workspace.rows("residual", n, self.model.spec.hidden, torch.float32)
         self.model.embedding.forward(ctx, x)
-        for entry in self.model.schedule:
-            self.model.blocks[entry.layer].forward(ctx, x, entry)
+        schedule, blocks = self.model.schedule, self.model.blocks
+        carried = None          # the next block's normed input, if the block before has begun it
+        for i, entry in enumerate(schedule):
+            block = blocks[entry.layer]
+            if getattr(block, "chains_norms", False):
+                after = blocks[schedule[i + 1].layer] if i + 1 < len(schedule) else None
+                next_norm = after.first_norm() if getattr(after, "chains_norms", False) else None
+                carried = block.forward(ctx, x, entry, carried, next_norm)
+            else:
+                block.forward(ctx, x, entry)
+                carried = None
         if not w:
             return None
         logits = self.workspace.rows("logits", w, self.vocab, torch.float32)

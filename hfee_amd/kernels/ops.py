@@ -321,8 +321,18 @@ def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0.0, rows=None, m=None, qkv=None):
+SS_STRIDE = 64     # rows of a table of sum-of-squares shares (one row of the table per 16 weight rows)
+
+
+def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0.0, rows=None, m=None, qkv=None,
+                 emit=None, row_scale=None):
     """out = epilogue(norm(x) @ weight.T) in one launch, for at most 64 rows.
+
+    emit (with "add"): dict(weight, out, shares): the norm that follows the residual add, in
+    two halves: this product also writes bfloat16(out_new * weight) to emit["out"] [M, N] and
+    its shares of the rows' sums of squares to emit["shares"] (float32, at least
+    ceil(N / 16) * 64).  row_scale: dict(shares, blocks, eps): the other half: x is such an
+    emitted tensor, and the finished sums are scaled by 1 / sqrt(sum of shares / K + eps).
 
     x: bfloat16 [M, K]; or, with norm_weight, the float32 residual stream (at most 16
     rows; `rows` optionally gathers them, then `m` is their number).
@@ -350,6 +360,26 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
     want = {"bf16": torch.bfloat16, "f32": torch.float32, "add": torch.float32, "swiglu": torch.bfloat16,
             "qkv": torch.bfloat16}[epilogue]
     _check(out.dtype == want, f"linear_fused: out must be {want} for {epilogue!r}")
+    e_args = [None, 0, None, 0, None]
+    if emit is not None:
+        _gpu(emit["weight"], emit["out"], emit["shares"])
+        _check(epilogue == "add" and not fused_norm, "linear_fused: only the accumulating product emits a norm")
+        eo, es, ew = emit["out"], emit["shares"], emit["weight"]
+        Me, Ne, lde = _rows2d(eo, "linear_fused emit out")
+        _check(eo.dtype == torch.bfloat16 and Me >= M and Ne == N, "linear_fused: emit out must be bfloat16 [M, N]")
+        _check(ew.numel() == N and ew.is_contiguous() and ew.dtype in (torch.float32, torch.bfloat16),
+               "linear_fused: emit weight")
+        _check(es.dtype == torch.float32 and es.is_contiguous() and es.numel() >= ((N + 15) // 16) * SS_STRIDE,
+               "linear_fused: the shares need ceil(N / 16) * 64 float32")
+        e_args = [_ptr(ew), int(ew.dtype == torch.float32), _ptr(eo), lde, _ptr(es)]
+    s_args = [None, 0, 0.0]
+    if row_scale is not None:
+        _gpu(row_scale["shares"])
+        _check(not fused_norm, "linear_fused: a row scale and a fused norm exclude each other")
+        ss, blocks = row_scale["shares"], int(row_scale["blocks"])
+        _check(ss.dtype == torch.float32 and ss.is_contiguous() and blocks > 0 and ss.numel() >= blocks * SS_STRIDE,
+               "linear_fused: row scale shares")
+        s_args = [_ptr(ss), blocks, float(row_scale["eps"])]
     q = qkv or {}
     if epilogue == "qkv":
         H, KV, hd, ps = q["num_heads"], q["kv_heads"], q["head_dim"], q["page_size"]
@@ -369,9 +399,9 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
                         epi, _ptr(norm_weight), int(fused_norm and norm_weight.dtype == torch.float32), float(eps),
                         _ptr(rows), _ptr(q["positions"]), _ptr(q.get("token_segment")), _ptr(bt),
                         0 if bt is None else bt.stride(0), _ptr(cos), _ptr(sin), half, table_positions,
-                        _ptr(cache), H, KV, hd, ps, _stream())
+                        _ptr(cache), H, KV, hd, ps, *e_args, *s_args, _stream())
         return
     _check(No == (N // 2 if epilogue == "swiglu" else N), "linear_fused: out width")
     lib.core().call("hfee_gemm_skinny", _ptr(out), ldc, _ptr(x), int(fused_norm), lda, _ptr(weight), ldw, M, N, K, epi,
                     _ptr(norm_weight), int(fused_norm and norm_weight.dtype == torch.float32), float(eps), _ptr(rows),
-                    None, None, None, 0, None, None, 0, 0, None, 0, 0, 0, 0, _stream())
+                    None, None, None, 0, None, None, 0, 0, None, 0, 0, 0, 0, *e_args, *s_args, _stream())

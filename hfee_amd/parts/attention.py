@@ -38,6 +38,7 @@ _DECODE_WORKGROUPS = 256   # with fewer (segment, KV head) pairs than this the k
 class Attention(Mixer):
     graph_safe = True
     takes_lazy_norm = True
+    emits_norm = True
 
     def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
@@ -119,7 +120,7 @@ class Attention(Mixer):
         plan.host["attention.decode_max_position"] = max(d_pos) if d_pos else 0
 
     # ---- the layer
-    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool, then=None):
         H, K, hd = self.num_heads, self.kv_heads, self.head_dim
         n = ctx.n
         group = ctx.storage.group_of(cache_layer)
@@ -132,11 +133,13 @@ class Attention(Mixer):
         q = qkv[:, :self.q_width]
         if fused:
             # norm, projections, rotation and the cache write in one launch
-            norm = h.fusable() if (isinstance(h, LazyNorm) and n <= ops.FUSED_NORM_MAX_ROWS
+            few = n <= ops.FUSED_NORM_MAX_ROWS
+            halves = h.row_scale() if (few and isinstance(h, LazyNorm)) else None     # first half done before
+            norm = h.fusable() if (halves is None and few and isinstance(h, LazyNorm)
                                    and ops.norm_fusion_pays(*self.w_qkv.shape)) else None
-            a = h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
+            a = halves[0] if halves else h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
             ops.linear_fused(q, a, self.w_qkv, "qkv", norm_weight=norm[0] if norm else None,
-                             eps=norm[1] if norm else 0.0,
+                             eps=norm[1] if norm else 0.0, row_scale=halves[1] if halves else None,
                              qkv=dict(positions=ctx.positions, token_segment=ctx.token_segment, block_tables=tables,
                                       cos=cos, sin=sin, cache_layer=cache if writes_cache else None,
                                       num_heads=H, kv_heads=K, head_dim=hd, page_size=ctx.page_size))
@@ -178,4 +181,11 @@ class Attention(Mixer):
                                           ctx.extra["attention.decode_tables"], tables, H, K, hd,
                                           ctx.page_size, self.scale, self.window, partial, splits, _DECODE_WAVES,
                                           counters)
-        ops.linear(x, att, self.w_o, accumulate=True)
+        emit = None
+        if then is not None and self.dtype == torch.bfloat16 and n <= ops.FUSED_NORM_MAX_ROWS \
+                and self.hidden % 8 == 0 and self.q_width % 8 == 0:
+            emit = then.offer()
+        if emit:       # the output projection adds into x and begins the norm that follows
+            ops.linear_fused(x, att, self.w_o, "add", emit=emit)
+        else:
+            ops.linear(x, att, self.w_o, accumulate=True)

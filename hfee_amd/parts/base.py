@@ -69,6 +69,9 @@ class Part:
     graph_safe = False
     # True if forward_add accepts a LazyNorm in place of the normed tensor.
     takes_lazy_norm = False
+    # True if forward_add accepts `then=` (the LazyNorm of the norm that follows this
+    # part) and may do that norm's first half in its last product.
+    emits_norm = False
 
     def tensor_specs(self) -> list:
         return []
@@ -114,18 +117,48 @@ class LazyNorm:
     """A normed copy of the residual stream that is made only when someone asks for
     it.  A part that sets `takes_lazy_norm = True` gets one of these instead of a
     tensor and may fold the norm into its first product (`fusable()`), or call
-    `tensor()` for the materialised rows."""
+    `tensor()` for the materialised rows.
+
+    The norm may also be done in two halves around it, without a launch of its own: a
+    part whose last step adds into the residual stream (`emits_norm = True`) is handed
+    the LazyNorm of what follows it as `then`; if `then.offer()` returns arguments, its
+    adding product also writes bfloat16(x_new * weight) and the rows' sums of squares
+    (`ops.linear_fused(..., emit=...)`).  The part that consumes the norm then finds
+    `pending` set and gives it to its first product as `row_scale`."""
 
     def __init__(self, ctx, norm, x):
         self.ctx, self.norm, self.x = ctx, norm, x
         self._tensor = None
+        self.pending = None      # dict(out, shares, blocks, eps) once a producer has done the first half
 
     def fusable(self):
         """(weight, eps) if the norm is y = x / sqrt(mean(x^2) + eps) * weight, else None."""
         return getattr(self.norm, "fused_form", lambda: None)()
 
+    def offer(self):
+        """For the part that adds into x last: the `emit` arguments of its adding product,
+        or None if this norm cannot be split (then nothing changes for anybody)."""
+        form = self.fusable()
+        if form is None or self.x.dtype != torch.float32:
+            return None
+        weight, eps = form
+        width = self.x.shape[1]
+        blocks = (width + 15) // 16
+        out = self.ctx.rows("block.emitted", width, torch.bfloat16)
+        shares = self.ctx.workspace.flat("block.emitted_shares", blocks * 64, torch.float32)
+        self.pending = dict(out=out, shares=shares, blocks=blocks, eps=eps)
+        return dict(weight=weight, out=out, shares=shares)
+
+    def row_scale(self):
+        """For the consuming part: (emitted tensor, `row_scale` arguments) if a producer has
+        done the first half, else None."""
+        if self.pending is None:
+            return None
+        p = self.pending
+        return p["out"], dict(shares=p["shares"], blocks=p["blocks"], eps=p["eps"])
+
     def tensor(self):
-        if self._tensor is None:
+        if self._tensor is None:       # (also after an offer: x is complete, the whole norm is always right)
             self._tensor = self.ctx.rows("block.normed", self.x.shape[1])
             self.norm.forward(self.ctx, self._tensor, self.x)
         return self._tensor

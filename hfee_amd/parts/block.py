@@ -34,9 +34,25 @@ class PreNormBlock(Part):
         for p in self.parts():
             p.bind(tensors)
 
-    def forward(self, ctx, x, entry):
-        h = LazyNorm(ctx, self.mixer_norm, x)
-        self.mixer.forward_add(ctx, x, h if self.mixer.takes_lazy_norm else h.tensor(), entry.cache,
-                               entry.writes_cache)
-        h = LazyNorm(ctx, self.feed_forward_norm, x)
-        self.feed_forward.forward_add(ctx, x, h if self.feed_forward.takes_lazy_norm else h.tensor())
+    # forward takes the normed input that the block before may have prepared, and the
+    # first norm of the block after (the engine passes both to blocks that say so)
+    chains_norms = True
+
+    def first_norm(self):
+        return self.mixer_norm
+
+    def forward(self, ctx, x, entry, h_in=None, next_norm=None):
+        h = h_in if h_in is not None else LazyNorm(ctx, self.mixer_norm, x)
+        h2 = LazyNorm(ctx, self.feed_forward_norm, x)
+        self._run(self.mixer, ctx, x, h, h2, entry.cache, entry.writes_cache)
+        h3 = LazyNorm(ctx, next_norm, x) if next_norm is not None else None
+        self._run(self.feed_forward, ctx, x, h2, h3)
+        return h3
+
+    @staticmethod
+    def _run(part, ctx, x, h, then, *args):
+        h = h if part.takes_lazy_norm else h.tensor()
+        if then is not None and part.emits_norm:
+            part.forward_add(ctx, x, h, *args, then=then)
+        else:
+            part.forward_add(ctx, x, h, *args)

@@ -17,6 +17,7 @@ from .base import FeedForward, LazyNorm, register_feed_forward
 class GatedMLP(FeedForward):
     graph_safe = True
     takes_lazy_norm = True
+    emits_norm = True
 
     def __init__(self, spec: FeedForwardSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
@@ -39,15 +40,18 @@ class GatedMLP(FeedForward):
                                      dim=1).reshape(2 * self.intermediate, self.hidden).contiguous()
         self.w_down = tensors.pop(p + "down_proj.weight").contiguous()
 
-    def forward_add(self, ctx, x, h):
+    def forward_add(self, ctx, x, h, then=None):
         F = self.intermediate
         act = ctx.rows("mlp.act", F)
-        aligned = self.dtype == torch.bfloat16 and self.hidden % 8 == 0
+        aligned = self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and F % 8 == 0
+        few = ctx.n <= ops.FUSED_NORM_MAX_ROWS
+        halves = h.row_scale() if (aligned and few and isinstance(h, LazyNorm)) else None
         norm = None
-        if aligned and isinstance(h, LazyNorm) and ctx.n <= ops.FUSED_NORM_MAX_ROWS \
-                and ops.norm_fusion_pays(*self.w_gate_up.shape):
+        if halves is None and aligned and few and isinstance(h, LazyNorm) and ops.norm_fusion_pays(*self.w_gate_up.shape):
             norm = h.fusable()
-        if norm:          # norm, both projections and the gate in one launch
+        if halves:        # the norm's first half came with the product before; both projections and the gate
+            ops.linear_fused(act, halves[0], self.w_gate_up, "swiglu", row_scale=halves[1])
+        elif norm:        # norm, both projections and the gate in one launch
             ops.linear_fused(act, h.x, self.w_gate_up, "swiglu", norm_weight=norm[0], eps=norm[1])
         else:
             hn = h.tensor() if isinstance(h, LazyNorm) else h
@@ -57,4 +61,8 @@ class GatedMLP(FeedForward):
                 gate_up = ctx.rows("mlp.gate_up", 2 * F)
                 ops.linear(gate_up, hn, self.w_gate_up)
                 ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
-        ops.linear(x, act, self.w_down, accumulate=True)
+        emit = then.offer() if (then is not None and aligned and few) else None
+        if emit:          # the down projection adds into x and begins the norm that follows
+            ops.linear_fused(x, act, self.w_down, "add", emit=emit)
+        else:
+            ops.linear(x, act, self.w_down, accumulate=True)

@@ -175,6 +175,54 @@ def test_fused_decode_products(M, N, K, epilogue, norm):
     assert (err <= tol * (1 + mag)).all(), float((err / (1 + mag)).max())
 
 
+@pytest.mark.parametrize("M,N,K,N2", [(1, 64, 96, 48), (8, 200, 256, 344), (16, 4096, 1024, 16400), (33, 104, 64, 72),
+                                       (64, 520, 128, 100)])
+@pytest.mark.parametrize("epilogue2", ["bf16", "swiglu", "add"])
+def test_norm_in_two_halves(M, N, K, N2, epilogue2):
+    """A norm between two products, without a launch of its own: the product that adds
+    into the residual stream also writes bfloat16(x_new * w_norm) and its shares of the
+    rows' sums of squares; the next product reads that and scales its finished sums.
+    Against residual add, RMSNorm and product done apart."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(M + 3 * N + 7 * K + N2)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    x0 = torch.randn(M, N, generator=g) * 2
+    nw = (1 + 0.1 * torch.randn(N, generator=g)).to(torch.float32 if N % 64 else torch.bfloat16)
+    w2 = (torch.randn(N2, N, generator=g) / math.sqrt(N)).to(torch.bfloat16)
+    eps = 1e-5
+    x1 = x0.double() + a.double() @ w1.double().t()
+    h = x1 / torch.sqrt((x1 ** 2).mean(-1, keepdim=True) + eps) * nw.double()
+    ref = h @ w2.double().t()
+    mag = h.abs() @ w2.double().abs().t()
+    # first product
+    x = x0.clone().to(DEV)
+    emitted = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    blocks = (N + 15) // 16
+    shares = torch.full((blocks * 64,), float("nan"), dtype=torch.float32, device=DEV)
+    ops.linear_fused(x, a.to(DEV), w1.to(DEV), "add", emit=dict(weight=nw.to(DEV), out=emitted, shares=shares))
+    err = (x.double().cpu() - x1).abs()
+    assert (err <= 1e-5 * (1 + x0.abs().double() + a.abs().double() @ w1.abs().double().t())).all()
+    got_ss = shares.view(blocks, 64)[:, :M].double().sum(0).cpu()
+    assert torch.allclose(got_ss, (x1 ** 2).sum(-1), rtol=1e-5)
+    close(emitted, x1 * nw.double(), 1e-2)
+    # second product
+    scale = dict(shares=shares, blocks=blocks, eps=eps)
+    if epilogue2 == "swiglu":
+        out = torch.zeros(M, N2 // 2, dtype=torch.bfloat16, device=DEV)
+        ref = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
+        mag = (mag[:, 0::2] + 1) * (mag[:, 1::2] + 1)
+    elif epilogue2 == "add":
+        c0 = torch.randn(M, N2, generator=g)
+        out = c0.clone().to(DEV)
+        ref = ref + c0.double()
+    else:
+        out = torch.zeros(M, N2, dtype=torch.bfloat16, device=DEV)
+    ops.linear_fused(out, emitted, w2.to(DEV), epilogue2, row_scale=scale)
+    err = (out.double().cpu() - ref).abs()
+    assert (err <= 2e-2 * (1 + mag)).all(), float((err / (1 + mag)).max())
+
+
 @pytest.mark.parametrize("H,K,hd,half,M", [(4, 2, 16, 8, 5), (3, 1, 32, 16, 16), (6, 3, 48, 8, 1), (2, 2, 128, 64, 9)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rotation_and_cache_write(H, K, hd, half, M, norm):
