@@ -91,7 +91,7 @@ class Attention(Mixer):
     def key_layout(self):
         """What two layers must share to read one cache layer."""
         pos = self.position
-        return (self.kv_heads, self.head_dim, None if pos is None else (pos.rotary_dim, pos.theta, pos.scaling))
+        return (self.kv_heads, self.head_dim, None if pos is None else pos.signature())
 
     # ---- cache
     def cache_spec(self):

@@ -62,6 +62,10 @@ class Rotary(Part):
         self.inv_freq = rope_frequencies(self.rotary_dim, self.theta, self.scaling)
         self.cos = self.sin = None
 
+    def signature(self):
+        """What two mixers must share to read one another's rotated keys."""
+        return ("rope", self.rotary_dim, self.theta, self.scaling)
+
     def prepare(self, num_positions: int, device) -> None:
         if self.cos is not None and self.cos.shape[0] >= num_positions and self.cos.device == torch.device(device):
             return

@@ -290,6 +290,130 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         ToyConfig.from_dict({"architectures": ["ToyForCausalLM"]})
 
 
+def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path):
+    """A feed-forward that routes every token to one of three experts, and a position
+    encoding that is not the architecture's (rotation by sqrt(position) * frequency), in
+    a toy architecture; both registered here, built by the registries, stepped in
+    portions and compared with a plain computation.  Nothing of the framework changes."""
+    import numpy as np
+    import hfee_amd  # noqa: F401
+    from hfee_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
+                                 ScheduleEntry, params, register_architecture)
+    from hfee_amd.config.base import KeyReader
+    from hfee_amd.engine import Engine, StepEntry, load_model
+    from hfee_amd.parts import FeedForward, Part, register_feed_forward, register_position
+    from hfee_amd.weights import TensorSpec, write_model_folder
+    from plain_llama import plain_attention, plain_rmsnorm, plain_rope
+
+    @register_position("toy_sqrt_rope")
+    class SqrtRope(Part):
+        def __init__(self, spec):
+            self.head_dim = self.rotary_dim = spec.get("head_dim")
+            self.base = float(spec.get("base"))
+            self.pairing = 0               # pairs (i, i + head_dim / 2)
+            self.cos = self.sin = None
+
+        def signature(self):
+            return ("toy_sqrt_rope", self.head_dim, self.base)
+
+        def frequencies(self):
+            return np.array([self.base ** (-2 * i / self.head_dim) for i in range(self.head_dim // 2)])
+
+        def prepare(self, num_positions, device):
+            angles = np.sqrt(np.arange(num_positions, dtype=np.float64))[:, None] * self.frequencies()[None, :]
+            self.cos = torch.from_numpy(np.cos(angles).astype(np.float32)).to(device)
+            self.sin = torch.from_numpy(np.sin(angles).astype(np.float32)).to(device)
+
+    @register_feed_forward("toy_top1_experts")
+    class Top1Experts(FeedForward):
+        def __init__(self, spec, prefix, dtype):
+            self.hidden, self.experts, self.prefix = spec.get("hidden"), spec.get("experts"), prefix
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + "router.weight", (self.experts, self.hidden)),
+                    TensorSpec(self.prefix + "experts.weight", (self.experts * self.hidden, self.hidden))]
+
+        def bind(self, tensors):
+            self.router = tensors.pop(self.prefix + "router.weight")
+            self.w = tensors.pop(self.prefix + "experts.weight").view(self.experts, self.hidden, self.hidden)
+
+        def forward_add(self, ctx, x, h):
+            choice = (h.float() @ self.router.float().t()).argmax(-1)          # router logits in 32-bit
+            for e in range(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    x[rows] += h[rows].float() @ self.w[e].float().t()
+
+    @dataclass(frozen=True)
+    class RoutedConfig:
+        architecture: str
+        hidden: int
+        layers: int
+        vocab: int
+        experts: int
+
+        @staticmethod
+        def from_dict(d, where="config.json"):
+            r = KeyReader(d, where)
+            c = RoutedConfig("ToyRoutedForCausalLM", r.int("r_hidden"), r.int("r_layers"), r.int("r_vocab"), r.int("r_experts"))
+            r.finish()
+            return c
+
+        def to_dict(self):
+            return {"architectures": ["ToyRoutedForCausalLM"], "r_hidden": self.hidden, "r_layers": self.layers,
+                    "r_vocab": self.vocab, "r_experts": self.experts}
+
+    H, KV, HD = 3, 1, 16
+
+    def routed_spec(c):
+        norm = NormSpec("rmsnorm", c.hidden, 1e-6)
+        ffn = FeedForwardSpec("toy_top1_experts", params(hidden=c.hidden, experts=c.experts))
+        att = MixerSpec("attention", params(hidden=c.hidden, num_heads=H, num_kv_heads=KV, head_dim=HD, scale=0.2, window=0),
+                        position=PositionSpec("toy_sqrt_rope", params(head_dim=HD, base=50.0)))
+        layers = tuple(LayerSpec("prenorm", c.hidden, att, ffn, norm, norm, f"r.{i}.") for i in range(c.layers))
+        return ModelSpec("ToyRoutedForCausalLM", c.hidden, c.vocab, layers, tuple(ScheduleEntry(i, i) for i in range(c.layers)),
+                         norm, "r.embed.weight", "r.norm.weight", None, max_positions=256)
+
+    register_architecture("ToyRoutedForCausalLM", RoutedConfig, routed_spec)
+    cfg = RoutedConfig("ToyRoutedForCausalLM", 40, 2, 70, 3)
+    folder = write_model_folder(str(tmp_path / "routed"), cfg, seed=5, std=0.2)
+    model, _ = load_model(folder, "float32")
+    eng = Engine(model, num_pages=8, page_size=16, max_requests=2, max_batch_tokens=64)
+    toks = tu.make_requests(70, [45], seed=8)["r0"]
+    eng.admit("a")
+    got, i = [], 0
+    for n in [7, 1, 20, 2, 15]:
+        got.append(eng.step([StepEntry("a", toks[i:i + n], list(range(n)))]).double().cpu())
+        i += n
+    got = torch.cat(got)
+
+    # the plain computation, whole sequence, float64
+    from hfee_amd.weights import Checkpoint
+    ck = Checkpoint(folder)
+    t = {n: ck.tensor(n).double() for n in ck.names()}
+    x = t["r.embed.weight"][toks]
+    pos = list(range(len(toks)))
+    inv_freq = torch.tensor([50.0 ** (-2 * j / HD) for j in range(HD // 2)], dtype=torch.float64)
+    used = set()
+    for l in range(cfg.layers):
+        p = f"r.{l}."
+        h = plain_rmsnorm(x, t[p + "mixer_norm.weight"], 1e-6)
+        q = (h @ t[p + "mixer.q_proj.weight"].t()).view(-1, H, HD)
+        k = (h @ t[p + "mixer.k_proj.weight"].t()).view(-1, KV, HD)
+        v = (h @ t[p + "mixer.v_proj.weight"].t()).view(-1, KV, HD)
+        sqrt_pos = [math.sqrt(i) for i in pos]
+        q, k = plain_rope(q, sqrt_pos, inv_freq, "half"), plain_rope(k, sqrt_pos, inv_freq, "half")
+        x = x + plain_attention(q, k, v, 0.2).reshape(len(toks), H * HD) @ t[p + "mixer.o_proj.weight"].t()
+        h = plain_rmsnorm(x, t[p + "feed_forward_norm.weight"], 1e-6)
+        choice = (h @ t[p + "feed_forward.router.weight"].t()).argmax(-1)
+        used |= set(choice.tolist())
+        w = t[p + "feed_forward.experts.weight"].view(cfg.experts, cfg.hidden, cfg.hidden)
+        x = x + torch.stack([h[r] @ w[int(choice[r])].t() for r in range(len(toks))])
+    want = plain_rmsnorm(x, t["r.norm.weight"], 1e-6) @ t["r.embed.weight"].t()
+    assert len(used) > 1, "the test is meant to route to more than one expert"
+    assert torch.allclose(got, want, atol=2e-4, rtol=2e-4), float((got - want).abs().max())
+
+
 # -------------------------------------------------------------- the sampler ---
 
 def test_sampler_kernel_follows_the_plain_rules():
