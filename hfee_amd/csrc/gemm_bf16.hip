@@ -14,6 +14,7 @@
 // Output modes: bfloat16 store, float32 store, float32 accumulate (the residual
 // add of /root/reference/internal/llm/forward.go:106-107 fused into the epilogue).
 #include "common.h"
+#include "qkv_epilogue.h"
 
 #include <type_traits>
 
@@ -27,7 +28,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-enum { OUT_BF16 = 0, OUT_F32 = 1, OUT_ADD_F32 = 2 };
+enum { OUT_BF16 = 0, OUT_F32 = 1, OUT_ADD_F32 = 2, OUT_SWIGLU = 3, OUT_QKV = 4 };
 
 union Chunk {           // eight bfloat16 values = 16 bytes
   u32x4 u;
@@ -162,6 +163,125 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(void* __restrict__
 }
 
 
+// Stores a 32 x 32 tile that was formed transposed: register r of lane l holds
+// C[m_base + l % 32][n_base + 8 (r / 4) + 4 (l / 32) + r % 4], so four registers are
+// four consecutive columns.  `vec`: rows of C start 16-byte aligned (8 for bfloat16).
+template <int MODE>
+__device__ __forceinline__ void store_tile_t(void* C, int64_t ldc, int M, int N, int m, int n_base, int lane,
+                                             const f32x16& t, bool vec) {
+  if (m >= M) return;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int n = n_base + 8 * q + 4 * (lane >> 5);
+    if (n >= N) continue;
+    float v[4] = {t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+    if (MODE == OUT_SWIGLU) {          // columns n, n+1 are gate, up of output column n / 2
+      bf16_t* c = (bf16_t*)C + (int64_t)m * ldc + (n >> 1);
+      const bf16_t o0 = float_to_bf16(v[0] * __frcp_rn(1.0f + __expf(-v[0])) * v[1]);
+      const bf16_t o1 = float_to_bf16(v[2] * __frcp_rn(1.0f + __expf(-v[2])) * v[3]);
+      if (vec && n + 3 < N) {
+        *reinterpret_cast<uint32_t*>(c) = (uint32_t)o0 | ((uint32_t)o1 << 16);
+      } else {
+        c[0] = o0;
+        if (n + 3 < N) c[1] = o1;
+      }
+    } else if (MODE == OUT_BF16) {
+      bf16_t* c = (bf16_t*)C + (int64_t)m * ldc + n;
+      if (vec && n + 3 < N) {
+        u32x2 o;
+        o[0] = (uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16);
+        o[1] = (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16);
+        *reinterpret_cast<u32x2*>(c) = o;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) c[i] = float_to_bf16(v[i]);
+      }
+    } else {
+      float* c = (float*)C + (int64_t)m * ldc + n;
+      if (vec && n + 3 < N) {
+        f32x4 o = {v[0], v[1], v[2], v[3]};
+        if (MODE == OUT_ADD_F32) o += *reinterpret_cast<const f32x4*>(c);
+        *reinterpret_cast<f32x4*>(c) = o;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) c[i] = MODE == OUT_ADD_F32 ? c[i] + v[i] : v[i];
+      }
+    }
+  }
+}
+
+// The q/k/v epilogue for a wave's TM x TN tiles of transposed 32 x 32 products: what
+// belongs to a row (position, page, slot) is fetched once per row, what belongs to four
+// columns (head, place in the head, q or k or v) once per four columns.
+template <int TM, int TN>
+__device__ __forceinline__ void store_wave_qkv(void* C, int64_t ldc, int M, int N, int m_first, int n_first, int lane,
+                                               const f32x16 (&acc)[TM][TN], const QkvArgs& qkv) {
+  const int lrow = lane & 31, hd = qkv.lay.head_dim;
+  int pos[TM], slot[TM];
+  int64_t page_base[TM];
+  bool row_ok[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m_first + i * 32 + lrow;
+    row_ok[i] = m < M;
+    const int mm = row_ok[i] ? m : M - 1;
+    pos[i] = qkv.positions[mm];
+    slot[i] = pos[i] & (qkv.lay.page_size - 1);
+    page_base[i] = 0;
+    if (qkv.cache != nullptr)
+      page_base[i] = (int64_t)qkv.block_tables[(int64_t)qkv.token_segment[mm] * qkv.bt_stride + (pos[i] >> qkv.lay.page_shift)] *
+                     qkv.lay.page_stride;
+  }
+  bf16_t* cache = (bf16_t*)qkv.cache;
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n_first + j * 32 + 8 * q + 4 * (lane >> 5);
+      if (n >= N) continue;
+      const int head = n / hd, d = n - head * hd;
+      const bool is_q = head < qkv.num_heads, is_v = head >= qkv.num_heads + qkv.lay.kv_heads;
+      const bool rotate = !is_v && qkv.cos_table != nullptr && d < 2 * qkv.half;
+      const bool second = d + 2 < 2 * qkv.half;              // the second pair is inside the rotated part too
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        if (!row_ok[i]) continue;
+        float v[4] = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+        if (rotate) {
+          const float* cs = qkv.cos_table + (int64_t)pos[i] * qkv.half + (d >> 1);
+          const float* sn = qkv.sin_table + (int64_t)pos[i] * qkv.half + (d >> 1);
+          const float x0 = v[0], x1 = v[1], c0 = cs[0], s0 = sn[0];
+          v[0] = x0 * c0 - x1 * s0;
+          v[1] = x0 * s0 + x1 * c0;
+          if (second) {
+            const float x2 = v[2], x3 = v[3], c1 = cs[1], s1 = sn[1];
+            v[2] = x2 * c1 - x3 * s1;
+            v[3] = x2 * s1 + x3 * c1;
+          }
+        }
+        u32x2 o;
+        o[0] = (uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16);
+        o[1] = (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16);
+        const int m = m_first + i * 32 + lrow;
+        if (is_q) {
+          *reinterpret_cast<u32x2*>((bf16_t*)C + (int64_t)m * ldc + n) = o;
+        } else if (cache != nullptr) {
+          if (!is_v) {
+            *reinterpret_cast<u32x2*>(cache + page_base[i] + qkv.lay.key_offset(0, head - qkv.num_heads, slot[i], d)) = o;
+          } else {
+            bf16_t* col = cache + page_base[i] + qkv.lay.value_offset(0, head - qkv.num_heads - qkv.lay.kv_heads, slot[i], d);
+            col[0] = (bf16_t)(o[0] & 0xffff);
+            col[qkv.lay.page_size] = (bf16_t)(o[0] >> 16);
+            col[2 * qkv.lay.page_size] = (bf16_t)(o[1] & 0xffff);
+            col[3 * qkv.lay.page_size] = (bf16_t)(o[1] >> 16);
+          }
+        }
+      }
+    }
+}
+
 // ---------------------------------------------------------- tiled, pipelined ---
 // The prefill product for aligned operands.  Four waves in a 2x2 grid, each with
 // TM x TN tiles of 32x32 (a workgroup tile of 64 TM x 64 TN), K in steps of 64.
@@ -171,7 +291,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(void* __restrict__
 // gate/up (C[m, j] = silu(row 2j) * row 2j+1).
 constexpr int PBK = 64, PPITCH = 72;   // pitch 144 bytes: no bank conflicts
 constexpr int XCDS = 8;                // accelerator dies of an MI355X
-enum { OUT_SWIGLU = 3 };
 
 template <int TM, int TN>
 struct PStage {
@@ -182,7 +301,7 @@ template <int MODE, int TM, int TN, int STAGES>
 __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restrict__ C, int64_t ldc,
                                                                   const bf16_t* __restrict__ A, int64_t lda,
                                                                   const bf16_t* __restrict__ W, int64_t ldw,
-                                                                  int M, int N, int K) {
+                                                                  int M, int N, int K, QkvArgs qkv) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
   extern __shared__ __attribute__((aligned(16))) bf16_t lds_tiles[];
   auto a_tile = [&](int buf) { return lds_tiles + buf * (BM * PPITCH); };
@@ -275,7 +394,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[ks & 1][j], a[ks & 1][i], acc[i][j], 0, 0, 0);   // transposed
     }
     store_stage(ring[(SLOT + 1) % STAGES], buf ^ 1, LAST ? inside(kt + 1) : true);
     __syncthreads();
@@ -293,31 +412,24 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
   if (kt + 2 < ktiles) step(integral_constant<int, 2>{}, std::true_type{}, kt + 2);
   if (kt + 3 < ktiles) step(integral_constant<int, 0>{}, std::true_type{}, kt + 3);
 
-  // D layout of the 32x32 tile: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
+  // the products were formed transposed: a lane holds four consecutive columns of a row
+  const bool vec = MODE == OUT_SWIGLU ? (ldc % 2 == 0 && (uintptr_t)C % 4 == 0)
+                 : MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0)
+                                    : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
+  if constexpr (MODE == OUT_QKV) {
+    store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
+  } else {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wn * 32 * TN + j * 32 + lrow;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 32 * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        float v = acc[i][j][r];
-        if (MODE == OUT_SWIGLU) {
-          // the odd neighbour holds the up row: swap inside lane pairs (DPP quad_perm 1,0,3,2)
-          const float up = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-          if ((lane & 1) == 0 && m < M && n < N)
-            ((bf16_t*)C)[(int64_t)m * ldc + (n >> 1)] = float_to_bf16(v * __frcp_rn(1.0f + __expf(-v)) * up);
-        } else if (m < M && n < N) {
-          store_out<MODE>(C, ldc, m, n, v);
-        }
-      }
-    }
+      for (int j = 0; j < TN; ++j)
+        store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+  }
 }
 
 template <int MODE>
 int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                     int M, int N, int K, hipStream_t stream) {
+                     int M, int N, int K, const QkvArgs& qkv, hipStream_t stream) {
   // 128 x 128 tiles, two workgroups per CU.  (128 x 256 tiles halve the LDS reads per
   // matrix instruction but leave one wave per SIMD, and measured 20 % slower.)
   constexpr int TM = 2, TN = 2, STAGES = 3;
@@ -332,7 +444,7 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
   const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
   if (tiles > (1 << 30)) return fail("gemm_bf16: too many tiles");
   dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
-  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
+  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv);
   return 0;
 }
 
@@ -351,55 +463,6 @@ template <int OTHER, int N, int R>
 struct Interleave<OTHER, N, R, N> {
   static __device__ __forceinline__ void emit() {}
 };
-
-// Stores a 32 x 32 tile that was formed transposed: register r of lane l holds
-// C[m_base + l % 32][n_base + 8 (r / 4) + 4 (l / 32) + r % 4], so four registers are
-// four consecutive columns.  `vec`: rows of C start 16-byte aligned (8 for bfloat16).
-template <int MODE>
-__device__ __forceinline__ void store_tile_t(void* C, int64_t ldc, int M, int N, int m, int n_base, int lane,
-                                             const f32x16& t, bool vec) {
-  if (m >= M) return;
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int n = n_base + 8 * q + 4 * (lane >> 5);
-    if (n >= N) continue;
-    float v[4] = {t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
-    if (MODE == OUT_SWIGLU) {          // columns n, n+1 are gate, up of output column n / 2
-      bf16_t* c = (bf16_t*)C + (int64_t)m * ldc + (n >> 1);
-      const bf16_t o0 = float_to_bf16(v[0] * __frcp_rn(1.0f + __expf(-v[0])) * v[1]);
-      const bf16_t o1 = float_to_bf16(v[2] * __frcp_rn(1.0f + __expf(-v[2])) * v[3]);
-      if (vec && n + 3 < N) {
-        *reinterpret_cast<uint32_t*>(c) = (uint32_t)o0 | ((uint32_t)o1 << 16);
-      } else {
-        c[0] = o0;
-        if (n + 3 < N) c[1] = o1;
-      }
-    } else if (MODE == OUT_BF16) {
-      bf16_t* c = (bf16_t*)C + (int64_t)m * ldc + n;
-      if (vec && n + 3 < N) {
-        u32x2 o;
-        o[0] = (uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16);
-        o[1] = (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16);
-        *reinterpret_cast<u32x2*>(c) = o;
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (n + i < N) c[i] = float_to_bf16(v[i]);
-      }
-    } else {
-      float* c = (float*)C + (int64_t)m * ldc + n;
-      if (vec && n + 3 < N) {
-        f32x4 o = {v[0], v[1], v[2], v[3]};
-        if (MODE == OUT_ADD_F32) o += *reinterpret_cast<const f32x4*>(c);
-        *reinterpret_cast<f32x4*>(c) = o;
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (n + i < N) c[i] = MODE == OUT_ADD_F32 ? c[i] + v[i] : v[i];
-      }
-    }
-  }
-}
 
 // ------------------------------------ tiled, one wave a SIMD, loads into the LDS ---
 // Products with enough tiles of 256 rows to fill the chip.  A 128 x 128 tile at the
@@ -432,7 +495,7 @@ template <int MODE, int TM, int TN>
 __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict__ C, int64_t ldc,
                                                                const bf16_t* __restrict__ A, int64_t lda,
                                                                const bf16_t* __restrict__ W, int64_t ldw,
-                                                               int M, int N, int K) {
+                                                               int M, int N, int K, QkvArgs qkv) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass has no buffer resources; it only needs the stub
   constexpr int BM = 64 * TM, BN = 64 * TN, CA = BM / 64, CW = BN / 64;
   constexpr int BUF = (BM + BN) * DROW;            // bytes of one LDS buffer (A tile, then W tile)
@@ -550,17 +613,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
   const bool vec = MODE == OUT_SWIGLU ? (ldc % 2 == 0 && (uintptr_t)C % 4 == 0)
                  : MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0)
                                     : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
+  if constexpr (MODE == OUT_QKV) {
+    store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
+  } else {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-      store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+      for (int j = 0; j < TN; ++j)
+        store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+  }
 #endif
 }
 
 template <int MODE, int TM, int TN>
 int launch_direct(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                  int M, int N, int K, hipStream_t stream) {
+                  int M, int N, int K, const QkvArgs& qkv, hipStream_t stream) {
   const size_t lds = (size_t)4 * (64 * TM + 64 * TN) * DROW;
   static bool raised = false;
   if (!raised) {
@@ -571,7 +638,7 @@ int launch_direct(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16
   }
   const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
   dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
-  gemm_bf16_direct_kernel<MODE, TM, TN><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
+  gemm_bf16_direct_kernel<MODE, TM, TN><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv);
   return 0;
 }
 
@@ -587,7 +654,7 @@ template <int MODE, int TM, int TN, int NBUF>
 __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restrict__ C, int64_t ldc,
                                                                  const bf16_t* __restrict__ A, int64_t lda,
                                                                  const bf16_t* __restrict__ W, int64_t ldw,
-                                                                 int M, int N, int K) {
+                                                                 int M, int N, int K, QkvArgs qkv) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int BM = 64 * TM, BN = 64 * TN, CA = BM / 32, CW = BN / 32;
   constexpr int BUF = (BM + BN) * EROW;
@@ -708,17 +775,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
   const bool vec = MODE == OUT_SWIGLU ? (ldc % 2 == 0 && (uintptr_t)C % 4 == 0)
                  : MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0)
                                     : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
+  if constexpr (MODE == OUT_QKV) {
+    store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
+  } else {
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-      store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+      for (int j = 0; j < TN; ++j)
+        store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+  }
 #endif
 }
 
 template <int MODE, int TM, int TN, int NBUF>
 int launch_direct64(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                    int M, int N, int K, hipStream_t stream) {
+                    int M, int N, int K, const QkvArgs& qkv, hipStream_t stream) {
   const size_t lds = (size_t)NBUF * (64 * TM + 64 * TN) * EROW;
   static bool raised = false;
   if (!raised) {
@@ -729,7 +800,7 @@ int launch_direct64(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf
   }
   const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
   dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
-  gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
+  gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv);
   return 0;
 }
 
@@ -831,14 +902,14 @@ inline int fastest_tiled(int M, int N, int K, bool large_ok) {
 
 template <int MODE>
 int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                   int M, int N, int K, int force_kernel, hipStream_t stream) {
+                   int M, int N, int K, int force_kernel, hipStream_t stream, const QkvArgs& qkv = QkvArgs{}) {
   int choice = force_kernel;
   const bool large_ok = large_fits(lda, ldw, M, N, K);
   if (choice != 2 && choice != 4 && choice != 5) choice = fastest_tiled(M, N, K, large_ok);
   if (choice >= 4 && !large_ok) choice = 2;
-  if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, stream);
-  if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, stream);
-  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, stream);
+  if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
 }
 
 // Up to 16 rows the streaming kernel always wins.  From 17 to 64 rows it re-reads the
@@ -925,5 +996,20 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
 #undef GO
   if (rc) return rc;
   HFEE_CHECK_LAUNCH("gemm_bf16");
+  return 0;
+}
+
+// The q/k/v product of more than 64 rows: C = q part of A W^T rotated, k and v rotated
+// and written into the paged cache by the product's epilogue (see qkv_epilogue.h).
+// Operands must be aligned as the tiled kernels need them.  For the callers of
+// hfee_gemm_skinny, which hands such products here.
+HFEE_API int hfee_gemm_bf16_qkv(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int64_t ldw, int M,
+                                int N, int K, const QkvArgs* qkv, int force_kernel, hipStream_t stream) {
+  HFEE_REQUIRE(M > 0 && N > 0 && K > 0 && qkv != nullptr, "gemm_bf16_qkv: bad arguments");
+  HFEE_REQUIRE((K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0),
+               "gemm_bf16_qkv: K and the leading dimensions must be multiples of 8 and the operands 16-byte aligned");
+  if (launch_aligned<OUT_QKV>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, force_kernel, stream, *qkv))
+    return 1;
+  HFEE_CHECK_LAUNCH("gemm_bf16_qkv");
   return 0;
 }

@@ -27,6 +27,7 @@
 //                token's slot of the paged cache
 //                                             (/root/reference/internal/llm/forward.go:96-101)
 #include "common.h"
+#include "qkv_epilogue.h"
 
 using namespace hfee;
 
@@ -45,19 +46,6 @@ union Chunk {
   u32x4 u;
   bf16x8 v;
   bf16_t e[8];
-};
-
-struct QkvArgs {
-  const int* positions;       // [M]
-  const int* token_segment;   // [M]
-  const int* block_tables;
-  int bt_stride;
-  const float* cos_table;     // [positions][half] or null
-  const float* sin_table;
-  int half;                   // rotated pairs per head
-  void* cache;                // one cache layer, or null (keys and values are not written)
-  CacheLayout lay;
-  int num_heads;
 };
 
 struct Args {
@@ -206,42 +194,8 @@ __device__ __forceinline__ void epilogue(const Args& a, int m, int n, float* v) 
     bf16_t* c = (bf16_t*)a.C + (int64_t)m * a.ldc + (n >> 1);
     c[0] = float_to_bf16(silu(v[0]) * v[1]);
     if (n + 2 < a.N) c[1] = float_to_bf16(silu(v[2]) * v[3]);
-  } else {   // EPI_QKV: head sizes are multiples of 4, so the four rows lie in one head
-    const QkvArgs& q = a.qkv;
-    const int hd = q.lay.head_dim;
-    const int head = n / hd, d = n - head * hd;
-    const int pos = q.positions[m];
-    const bool is_v = head >= q.num_heads + q.lay.kv_heads;
-    if (!is_v && q.cos_table != nullptr && d < 2 * q.half) {
-      const float* cs = q.cos_table + (int64_t)pos * q.half + (d >> 1);
-      const float* sn = q.sin_table + (int64_t)pos * q.half + (d >> 1);
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        if (d + 2 * p < 2 * q.half) {
-          const float x0 = v[2 * p], x1 = v[2 * p + 1], c = cs[p], s = sn[p];
-          v[2 * p] = x0 * c - x1 * s;
-          v[2 * p + 1] = x0 * s + x1 * c;
-        }
-      }
-    }
-    bf16_t o[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = float_to_bf16(v[i]);
-    if (head < q.num_heads) {
-      *reinterpret_cast<u32x2*>((bf16_t*)a.C + (int64_t)m * a.ldc + n) = *reinterpret_cast<const u32x2*>(o);
-    } else if (q.cache != nullptr) {
-      const int page = q.block_tables[(int64_t)q.token_segment[m] * q.bt_stride + (pos >> q.lay.page_shift)];
-      const int slot = pos & (q.lay.page_size - 1);
-      bf16_t* cache = (bf16_t*)q.cache;
-      if (!is_v) {
-        *reinterpret_cast<u32x2*>(cache + q.lay.key_offset(page, head - q.num_heads, slot, d)) =
-            *reinterpret_cast<const u32x2*>(o);
-      } else {
-        const int kvh = head - q.num_heads - q.lay.kv_heads;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) cache[q.lay.value_offset(page, kvh, slot, d + i)] = o[i];
-      }
-    }
+  } else {   // EPI_QKV
+    qkv_store(a.qkv, a.C, a.ldc, m, n, v);
   }
 }
 
@@ -571,6 +525,9 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 
 }  // namespace
 
+HFEE_API int hfee_gemm_bf16_qkv(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int64_t ldw, int M,
+                                int N, int K, const QkvArgs* qkv, int force_kernel, hipStream_t stream);   // gemm_bf16.hip
+
 // One entry point for every variant.  a_is_f32 != 0 selects the fused RMSNorm (M <= 16).
 // epi: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate, 4 q/k/v.
 // emit_out (with epi 2): also write bfloat16(C_new * emit_weight) to emit_out [M, N] and this
@@ -588,8 +545,8 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                               float scale_eps, hipStream_t stream) {
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
   if (M == 0) return 0;
-  HFEE_REQUIRE(M <= 64, "gemm_skinny: at most 64 rows, got %d", M);
   HFEE_REQUIRE(epi >= 0 && epi <= 4, "gemm_skinny: unknown epilogue %d", epi);
+  HFEE_REQUIRE(M <= 64 || epi == EPI_QKV, "gemm_skinny: at most 64 rows (more for q/k/v only), got %d", M);
   HFEE_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0,
                "gemm_skinny: K and the leading dimensions must be multiples of 8 and the operands 16-byte aligned");
   HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_skinny: a leading dimension is shorter than its row");
@@ -621,6 +578,11 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
     a.qkv.positions = positions; a.qkv.token_segment = token_segment; a.qkv.block_tables = block_tables;
     a.qkv.bt_stride = bt_stride; a.qkv.cos_table = cos_table; a.qkv.sin_table = sin_table; a.qkv.half = half;
     a.qkv.cache = cache; a.qkv.num_heads = num_heads;
+    if (M > 64) {       // a prefill portion: the tiled kernels, with the same epilogue
+      HFEE_REQUIRE(!norm && emit_out == nullptr && scale_ss == nullptr,
+                   "gemm_skinny: more than 64 rows take neither a fused norm nor a row scale");
+      return hfee_gemm_bf16_qkv(C, ldc, A, lda, W, ldw, M, N, K, &a.qkv, 0, stream);
+    }
   } else {
     HFEE_REQUIRE(ldc >= N, "gemm_skinny: ldc is shorter than a row");
   }

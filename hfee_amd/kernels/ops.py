@@ -326,7 +326,8 @@ SS_STRIDE = 64     # rows of a table of sum-of-squares shares (one row of the ta
 
 def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0.0, rows=None, m=None, qkv=None,
                  emit=None, row_scale=None):
-    """out = epilogue(norm(x) @ weight.T) in one launch, for at most 64 rows.
+    """out = epilogue(norm(x) @ weight.T) in one launch, for at most 64 rows ("qkv": any
+    number of rows; more than 64 take the tiled kernels with the same epilogue).
 
     emit (with "add"): dict(weight, out, shares): the norm that follows the residual add, in
     two halves: this product also writes bfloat16(out_new * weight) to emit["out"] [M, N] and

@@ -223,13 +223,16 @@ def test_norm_in_two_halves(M, N, K, N2, epilogue2):
     assert (err <= 2e-2 * (1 + mag)).all(), float((err / (1 + mag)).max())
 
 
-@pytest.mark.parametrize("H,K,hd,half,M", [(4, 2, 16, 8, 5), (3, 1, 32, 16, 16), (6, 3, 48, 8, 1), (2, 2, 128, 64, 9)])
+@pytest.mark.parametrize("H,K,hd,half,M", [(4, 2, 16, 8, 5), (3, 1, 32, 16, 16), (6, 3, 48, 8, 1), (2, 2, 128, 64, 9),
+                                           (4, 2, 16, 8, 100), (6, 3, 48, 8, 130), (2, 2, 128, 64, 300), (5, 1, 64, 32, 65)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rotation_and_cache_write(H, K, hd, half, M, norm):
     """Projection + rotation (pairs 2i, 2i+1) + cache write in one launch against the
-    separate steps."""
+    separate steps: the streaming kernels (up to 64 rows) and the tiled ones."""
     from plain_llama import plain_rope
     from hfee_amd.kernels import ops
+    if norm and M > 16:
+        pytest.skip("the fused norm takes at most 16 rows")
     d, ps = 96, 16
     g = torch.Generator().manual_seed(H + hd + M)
     N = (H + 2 * K) * hd
