@@ -875,7 +875,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(
 }
 
 // Which tiled kernel takes an aligned product: force_kernel 2 the 128 x 128 tiles, 4 the
-// 256 x 256 tiles, 5 the 256 x 128 tiles, anything else the one expected to be fastest:
+// 256 x 256 tiles, 5 the 256 x 128 tiles, 6 the 256 x 192 tiles, anything else the one
+// expected to be fastest:
 // rounds of tiles over the chip times the time of a tile, with the share of the matrix
 // peak that each kernel was measured to reach on a busy CU (128 x 128: two workgroups a
 // CU; the large tiles reach more the longer K is, and a tile of empty rows costs as
@@ -891,13 +892,18 @@ inline int fastest_tiled(int M, int N, int K, bool large_ok) {
   if (!large_ok) return 2;
   auto tiles = [&](int bm, int bn) { return (double)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   auto rounds = [&](double t, int slots) { return (double)(int64_t)((t + slots - 1) / slots); };
-  const double t2 = tiles(128, 128), t4 = tiles(256, 256), t5 = tiles(256, 128);
+  const double t2 = tiles(128, 128), t4 = tiles(256, 256), t5 = tiles(256, 128), t6 = tiles(256, 192);
   const double c2 = t2 <= cus ? 128.0 * 128 / 0.22 : rounds(t2, 2 * cus) * 2 * 128 * 128 / 0.31;
   const double fill = K >= 512 ? 1.0 : 0.6;            // the four-buffer pipeline needs a few steps to pay
   const double c4 = rounds(t4, cus) * 256 * 256 / (0.46 * fill);
   const double c5 = rounds(t5, cus) * 256 * 128 / (0.42 * fill);
-  if (c4 <= c5 && c4 <= c2) return 4;
-  return c5 <= c2 ? 5 : 2;
+  const double c6 = rounds(t6, cus) * 256 * 192 / (0.44 * fill);
+  int best = 2;
+  double cost = c2;
+  if (c5 < cost) { best = 5; cost = c5; }
+  if (c6 < cost) { best = 6; cost = c6; }
+  if (c4 <= cost) best = 4;
+  return best;
 }
 
 template <int MODE>
@@ -905,8 +911,9 @@ int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf1
                    int M, int N, int K, int force_kernel, hipStream_t stream, const QkvArgs& qkv = QkvArgs{}) {
   int choice = force_kernel;
   const bool large_ok = large_fits(lda, ldw, M, N, K);
-  if (choice != 2 && choice != 4 && choice != 5) choice = fastest_tiled(M, N, K, large_ok);
+  if (choice != 2 && (choice < 4 || choice > 6)) choice = fastest_tiled(M, N, K, large_ok);
   if (choice >= 4 && !large_ok) choice = 2;
+  if (choice == 6) return launch_direct<MODE, 4, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
@@ -960,15 +967,15 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
 // out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate (the
 // rows of W alternate gate/up; C is [M, N/2] bfloat16; aligned operands and M > 64 only).
 // force_kernel: 0 choose by the sizes, 1 skinny, 2 tiled 128 x 128, 3 the simple tiled
-// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128 (for tests of each kernel alone; 4 and 5
-// fall back to 2 where they do not apply).
+// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192 (for tests of each
+// kernel alone; 4 to 6 fall back to 2 where they do not apply).
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
                             int64_t ldw, int M, int N, int K, int force_kernel, hipStream_t stream) {
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16: a leading dimension is shorter than its row");
   HFEE_REQUIRE(out_mode >= 0 && out_mode <= 3, "gemm_bf16: unknown output mode %d", out_mode);
   HFEE_REQUIRE(ldc >= (out_mode == 3 ? N / 2 : N), "gemm_bf16: ldc is shorter than a row of the result");
-  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 5, "gemm_bf16: unknown kernel choice %d", force_kernel);
+  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 6, "gemm_bf16: unknown kernel choice %d", force_kernel);
   if (M == 0) return 0;
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) &&
                    ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
