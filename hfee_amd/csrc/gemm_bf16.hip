@@ -489,6 +489,15 @@ struct Interleave<OTHER, N, R, N> {
 // K must be a multiple of 32 and every row's byte offset must fit 31 bits.
 constexpr int DBK = 32, DROW = DBK * 2;      // bytes of a tile row in a buffer
 
+// A workgroup barrier without a fence.  The barrier instruction does not count as a
+// memory access for the compiler, so the empty statements on both sides keep the LDS
+// reads and the loads into the LDS where they were written, relative to it.
+__device__ __forceinline__ void barrier_no_fence() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 __device__ __forceinline__ uint32_t swizzle(uint32_t row) { return ((row >> 1) ^ (row >> 3)) & 3u; }
 
 template <int MODE, int TM, int TN>
@@ -582,7 +591,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
   load_step(1);
   load_step(2);
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LD) : "memory");     // K step 0 has landed
-  __builtin_amdgcn_s_barrier();
+  barrier_no_fence();
   read_operands(0, 0, a[0], b[0]);
 
   // One step: columns 0..15 with the reads of columns 16..31 under them; the first half
@@ -601,7 +610,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
     load_step(kt + 3);
     Interleave<0x020, HALF, LD>::emit();
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * LD) : "memory");
-    __builtin_amdgcn_s_barrier();
+    barrier_no_fence();
     read_operands((kt + 1) & 3, 0, a[0], b[0]);
     multiply(a[1], b[1], HALF, MF);
     Interleave<0x100, MF - HALF, RD>::emit();
@@ -736,7 +745,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
 #pragma unroll
   for (int s = 0; s < NBUF - 1; ++s) load_step(s, s);
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 2) * LD) : "memory");     // K step 0 has landed
-  __builtin_amdgcn_s_barrier();
+  barrier_no_fence();
   read_operands(0, 0, a[0], b[0]);
 
   // One step of 64 columns in four quarters.  The requests for K step kt + NBUF - 1 go out
@@ -764,7 +773,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
     multiply(a[1], b[1], 0, HALF);
     __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NBUF - 2) * LD) : "memory");
-    __builtin_amdgcn_s_barrier();
+    barrier_no_fence();
     read_operands(nb, 0, a[0], b[0]);
     multiply(a[1], b[1], HALF, MF);
     Interleave<0x100, MF - HALF, RD>::emit();
