@@ -971,7 +971,8 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                               int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
                               int page_size, const void* emit_weight, int emit_weight_is_f32, void* emit_out,
                               int64_t ld_emit, float* emit_ss, const float* scale_ss, int scale_blocks,
-                              float scale_eps, hipStream_t stream);
+                              float scale_eps, float* scratch, int64_t scratch_floats, int* counters,
+                              int num_counters, hipStream_t stream);
 
 // out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate (the
 // rows of W alternate gate/up; C is [M, N/2] bfloat16; aligned operands and M > 64 only).
@@ -992,14 +993,14 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
     HFEE_REQUIRE(N % 2 == 0 && vec, "gemm_bf16: the SiLU gate needs an even N and aligned operands");
     if (skinny_pays(M, N))
       return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, 3, nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr,
-                              0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, stream);
+                              0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, nullptr, 0, nullptr, 0, stream);
     if (launch_aligned<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, force_kernel, stream)) return 1;
     HFEE_CHECK_LAUNCH("gemm_bf16");
     return 0;
   }
   if (vec && M <= 64 && (force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N))))   // gemm_skinny.hip
     return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, out_mode, nullptr, 0, 0.f, nullptr, nullptr, nullptr,
-                            nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, stream);
+                            nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, nullptr, 0, nullptr, 0, stream);
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   int rc;

@@ -199,6 +199,38 @@ __device__ __forceinline__ void epilogue(const Args& a, int m, int n, float* v) 
   }
 }
 
+// What every kernel of this file does with four finished sums of a whole wave's lanes
+// (lane l: batch row m, weight rows n .. n+3, `live` if they exist): the residual add
+// with the first half of the norm that follows it (EMIT), or the plain epilogue.
+// `block`: this group of 16 weight rows (the row of the shares table).  All lanes of the
+// wave come here together: the shares are summed by shuffles.
+template <int EPI>
+__device__ __forceinline__ void finish_rows(const Args& a, int m, int n, bool live, float* v, int block, int l) {
+  if (EPI == EPI_ADD && a.emit_out != nullptr) {
+    float ss = 0.f;
+    if (live) {
+      float* c = (float*)a.C + (int64_t)m * a.ldc + n;
+      bf16_t* e = a.emit_out + (int64_t)m * a.ld_emit + n;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (n + i < a.N) {
+          const float x = c[i] + v[i];
+          c[i] = x;
+          ss = fmaf(x, x, ss);
+          const float w = a.emit_weight_is_f32 ? ((const float*)a.emit_weight)[n + i]
+                                               : bf16_to_float(((const bf16_t*)a.emit_weight)[n + i]);
+          e[i] = float_to_bf16(x * w);
+        }
+      }
+    }
+    ss += __shfl_xor(ss, 16, 64);          // the four column groups of this row
+    ss += __shfl_xor(ss, 32, 64);
+    if ((l >> 4) == 0 && m < a.M) a.emit_ss[(int64_t)block * SS_STRIDE + m] = ss;
+  } else if (live) {
+    epilogue<EPI>(a, m, n, v);
+  }
+}
+
 template <int MT, bool NORM, int EPI>
 __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   __shared__ float partial[WAVES][MT][64][4];
@@ -318,30 +350,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
       for (int i = 0; i < 4; ++i) v[i] *= scale;
     }
 
-    if (EPI == EPI_ADD && a.emit_out != nullptr) {
-      // the residual add, and the first half of the norm that follows it
-      float ss = 0.f;
-      if (live) {
-        float* c = (float*)a.C + (int64_t)m * a.ldc + n;
-        bf16_t* e = a.emit_out + (int64_t)m * a.ld_emit + n;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (n + i < a.N) {
-            const float x = c[i] + v[i];
-            c[i] = x;
-            ss = fmaf(x, x, ss);
-            const float w = a.emit_weight_is_f32 ? ((const float*)a.emit_weight)[n + i]
-                                                 : bf16_to_float(((const bf16_t*)a.emit_weight)[n + i]);
-            e[i] = float_to_bf16(x * w);
-          }
-        }
-      }
-      ss += __shfl_xor(ss, 16, 64);          // the four column groups of this row
-      ss += __shfl_xor(ss, 32, 64);
-      if ((l >> 4) == 0 && m < a.M) a.emit_ss[(int64_t)blockIdx.x * SS_STRIDE + m] = ss;
-    } else if (live) {
-      epilogue<EPI>(a, m, n, v);
-    }
+    finish_rows<EPI>(a, m, n, live, v, blockIdx.x, l);
   }
 }
 
@@ -359,6 +368,166 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 #undef GO
 }
 
+
+// ------------------------------------------------------------ 17 to 64 rows ---
+// With more than 16 batch rows the streaming kernel reads the batch again for every 16
+// weight rows, and that traffic (from L2) outgrows the weights.  Here K is cut into
+// slices of 1,024 columns, each with workgroups of its own.  A workgroup keeps its slice
+// of the batch, all rows, in LDS; each of its waves walks over groups of 16 weight rows
+// on its own: the weights come straight from global memory through a ring of 16 loads
+// that runs across group boundaries, the batch operands from LDS; no barrier stands in
+// the loop.  The slices' partial sums of a row group meet in a scratch buffer: every
+// wave stores its share at device scope and counts itself, and the wave that finishes a
+// row group last adds the shares in the order of the slices and runs the epilogue.
+// Nobody waits for anybody; the counters are back at zero afterwards.
+constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32, MID_RING = 16;
+constexpr int MID_PITCH = MID_KS + 8;        // LDS row pitch of the batch slice in elements: rows 16 bytes askew
+
+constexpr size_t mid_lds_bytes(int mt) { return (size_t)mt * 16 * MID_PITCH * sizeof(bf16_t); }
+
+template <int MT, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups, int slices, float* __restrict__ scratch,
+                                                         int* __restrict__ counters) {
+  extern __shared__ __attribute__((aligned(16))) char mid_lds[];
+  bf16_t* xs = (bf16_t*)mid_lds;                                                    // [MT * 16][MID_PITCH]
+  __shared__ float row_scale[SS_STRIDE];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, g = lane >> 4;
+  const int slice = blockIdx.x % slices;                     // the host launches a multiple of `slices`
+  const int stride = (gridDim.x / slices) * WAVES;           // waves of this slice
+  const int k0 = slice * MID_KS;
+
+  // ---- the first weights go out before anything else ---------------------------------
+  auto row_ptr = [&](int rg) {       // rows beyond N read the last row; what they produce is never stored
+    return a.W + (int64_t)min(rg * ROWS + r16, a.N - 1) * a.ldw + k0 + g * 8;
+  };
+  int rg = (blockIdx.x / slices) * WAVES + wave;
+  const bf16_t* w_cur = row_ptr(min(rg, row_groups - 1));
+  Chunk ring[MID_RING];
+#pragma unroll
+  for (int st = 0; st < MID_RING; ++st) ring[st].u = *reinterpret_cast<const u32x4*>(w_cur + st * 32);
+
+  // ---- the batch slice into LDS (rows beyond M as zeros) -------------------------------
+  for (int idx = threadIdx.x; idx < MT * 16 * (MID_KS / 8); idx += WAVES * 64) {
+    const int row = idx / (MID_KS / 8), c = idx - row * (MID_KS / 8);
+    u32x4 v = u32x4{0u, 0u, 0u, 0u};
+    if (row < a.M) v = *reinterpret_cast<const u32x4*>((const bf16_t*)a.A + (int64_t)row * a.lda + k0 + c * 8);
+    *reinterpret_cast<u32x4*>(xs + row * MID_PITCH + c * 8) = v;
+  }
+  if (a.scale_ss != nullptr) row_scales(a, row_scale);
+  __syncthreads();
+
+  const bf16_t* x_lane = xs + r16 * MID_PITCH + g * 8;
+  while (rg < row_groups) {
+    const int rg_next = rg + stride;
+    const bf16_t* w_next = row_ptr(rg_next < row_groups ? rg_next : rg);    // past the end: a repeat that nobody uses
+    f32x4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < MID_STEPS; ++st) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const bf16x8 b = *reinterpret_cast<const bf16x8*>(x_lane + t * 16 * MID_PITCH + st * 32);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st % MID_RING].v, b, acc[t], 0, 0, 0);
+      }
+      const int ahead = st + MID_RING;
+      ring[st % MID_RING].u = ahead < MID_STEPS ? *reinterpret_cast<const u32x4*>(w_cur + ahead * 32)
+                                                : *reinterpret_cast<const u32x4*>(w_next + (ahead - MID_STEPS) * 32);
+    }
+    // The order of issue, spelled out (groups: 0x008 matrix, 0x100 LDS read, 0x020 global
+    // load): the batch operands of a step are read under the products of the step before,
+    // and a ring slot is refilled as soon as its step has been multiplied.
+    __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+#pragma unroll
+    for (int st = 0; st < MID_STEPS; ++st) {
+      if (st + 1 < MID_STEPS) __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+
+    bool finish = true;
+    if (slices > 1) {
+      // this slice's share, at device scope; then count; the last one adds all shares in order
+      // (a wave's store of one register is 256 contiguous bytes: whole lines go through to memory)
+      float* mine = scratch + ((int64_t)(rg * slices + slice) * MT) * 256 + lane;
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          __hip_atomic_store(mine + (t * 4 + i) * 64, acc[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // (the stores are complete when every load issued before them is too: the ring refills after this)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      int arrived = 0;
+      if (lane == 0) arrived = atomicAdd(counters + rg, 1);
+      finish = __builtin_amdgcn_readfirstlane(arrived) == slices - 1;
+      if (finish) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int sl = 0; sl < slices; ++sl) {
+          const float* theirs = scratch + ((int64_t)(rg * slices + sl) * MT) * 256 + lane;
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              acc[t][i] += __hip_atomic_load(theirs + (t * 4 + i) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane == 0) atomicExch(counters + rg, 0);
+      }
+    }
+    if (finish) {
+      // register i of lane l: weight row 4*(l/16) + i, batch row l%16
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + r16, n = rg * ROWS + 4 * g;
+        float v[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        if (a.scale_ss != nullptr) {
+          const float scale = row_scale[m];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] *= scale;
+        }
+        finish_rows<EPI>(a, m, n, m < a.M && n < a.N, v, rg, lane);
+      }
+    }
+    rg = rg_next;
+    w_cur = w_next;
+  }
+}
+
+// Returns true if the kernel for 17 to 64 rows took the product.
+template <int MT>
+bool launch_mid_rows(const Args& a, int epi, float* scratch, int64_t scratch_floats, int* counters, int num_counters,
+                     int num_cus, hipStream_t stream) {
+  const int row_groups = (a.N + ROWS - 1) / ROWS, slices = a.K / MID_KS;
+  if (slices > 1 && (scratch == nullptr || counters == nullptr || num_counters < row_groups ||
+                     scratch_floats < (int64_t)row_groups * slices * MT * 256))
+    return false;
+  int per_slice = num_cus / slices;                         // workgroups per slice: eight row groups at a time each
+  if (per_slice < 1) per_slice = 1;
+  if (per_slice > (row_groups + WAVES - 1) / WAVES) per_slice = (row_groups + WAVES - 1) / WAVES;
+  const size_t lds = mid_lds_bytes(MT);
+#define GO(E)                                                                                                  \
+  do {                                                                                                         \
+    static bool raised = false;                                                                                \
+    if (!raised) {                                                                                             \
+      if (hipFuncSetAttribute((const void*)mid_kernel<MT, E>, hipFuncAttributeMaxDynamicSharedMemorySize,      \
+                              (int)lds) != hipSuccess)                                                        \
+        return false;                                                                                          \
+      raised = true;                                                                                           \
+    }                                                                                                          \
+    mid_kernel<MT, E><<<per_slice * slices, WAVES * 64, lds, stream>>>(a, row_groups, slices, scratch, counters); \
+  } while (0)
+  switch (epi) {
+    case EPI_BF16: GO(EPI_BF16); break;
+    case EPI_F32: GO(EPI_F32); break;
+    case EPI_ADD: GO(EPI_ADD); break;
+    case EPI_SWIGLU: GO(EPI_SWIGLU); break;
+    default: GO(EPI_QKV); break;
+  }
+#undef GO
+  return true;
+}
 
 // ------------------------------------------------------------ wide products ---
 // For products with many weight rows (gate/up, the vocabulary head) and at most 16
@@ -534,6 +703,11 @@ HFEE_API int hfee_gemm_bf16_qkv(void* C, int64_t ldc, const void* A, int64_t lda
 // product's shares of the rows' sums of squares to emit_ss (ceil(N / 16) x 64 floats).
 // scale_ss: shares left by such a product (scale_blocks x 64 floats) over rows of width K:
 // the finished sums are scaled by 1 / sqrt(sum / K + scale_eps).
+// scratch, counters: for 17 to 64 rows and K a multiple of 1,024, a faster kernel that
+// needs ceil(N / 16) * (K / 1024) * ceil(M / 16) * 256 floats of scratch and ceil(N / 16)
+// int32 counters that are zero (and are zero again afterwards); without them, or for
+// other sizes, or where it would not pay, the streaming kernel takes the product (a
+// negative num_counters takes the faster kernel wherever it applies: for tests).
 HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
                               int64_t ldw, int M, int N, int K, int epi,
                               const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
@@ -542,8 +716,11 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                               int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
                               int page_size, const void* emit_weight, int emit_weight_is_f32, void* emit_out,
                               int64_t ld_emit, float* emit_ss, const float* scale_ss, int scale_blocks,
-                              float scale_eps, hipStream_t stream) {
+                              float scale_eps, float* scratch, int64_t scratch_floats, int* counters,
+                              int num_counters, hipStream_t stream) {
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
+  const bool force_mid = num_counters < 0;          // (for tests of that kernel alone)
+  if (force_mid) num_counters = -num_counters;
   if (M == 0) return 0;
   HFEE_REQUIRE(epi >= 0 && epi <= 4, "gemm_skinny: unknown epilogue %d", epi);
   HFEE_REQUIRE(M <= 64 || epi == EPI_QKV, "gemm_skinny: at most 64 rows (more for q/k/v only), got %d", M);
@@ -597,6 +774,26 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
     a.scale_ss = scale_ss; a.scale_blocks = scale_blocks; a.scale_eps = scale_eps;
   }
   const int mt = (M + 15) / 16;
+  // Where the kernel with the batch in LDS was measured to win: products that are large
+  // enough to pay for its set-up (q/k/v and down of an 8B model, not the output product),
+  // and not so wide that the tiled kernel fills the chip (gate/up).
+  const bool mid_pays = (int64_t)N * K >= (int64_t)24 << 20 && N < 16384;
+  if (!norm && mt > 1 && K % MID_KS == 0 && (mid_pays || force_mid)) {
+    static int num_cus = 0;
+    if (num_cus == 0) {
+      int dev = 0;
+      hipDeviceProp_t prop;
+      num_cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+                 prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    }
+    const bool took = mt == 2 ? launch_mid_rows<2>(a, epi, scratch, scratch_floats, counters, num_counters, num_cus, stream)
+                    : mt == 3 ? launch_mid_rows<3>(a, epi, scratch, scratch_floats, counters, num_counters, num_cus, stream)
+                              : launch_mid_rows<4>(a, epi, scratch, scratch_floats, counters, num_counters, num_cus, stream);
+    if (took) {
+      HFEE_CHECK_LAUNCH("gemm_skinny(17 to 64 rows)");
+      return 0;
+    }
+  }
   if (emit_out == nullptr && launch_wide(a, norm, epi, stream)) {
     HFEE_CHECK_LAUNCH("gemm_skinny(wide)");
     return 0;

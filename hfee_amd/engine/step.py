@@ -278,8 +278,9 @@ class Engine:
             block = blocks[entry.layer]
             if getattr(block, "chains_norms", False):
                 after = blocks[schedule[i + 1].layer] if i + 1 < len(schedule) else None
-                next_norm = after.first_norm() if getattr(after, "chains_norms", False) else None
-                carried = block.forward(ctx, x, entry, carried, next_norm)
+                following = after.begin(ctx, x) if getattr(after, "chains_norms", False) else None
+                block.forward(ctx, x, entry, carried, following)
+                carried = following
             else:
                 block.forward(ctx, x, entry)
                 carried = None

@@ -324,8 +324,16 @@ def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
 SS_STRIDE = 64     # rows of a table of sum-of-squares shares (one row of the table per 16 weight rows)
 
 
+def mid_rows_scratch(n_rows: int, n_weight_rows: int, k: int) -> int:
+    """float32 words of scratch that a product of 17 to 64 rows wants for its faster kernel
+    (0: it has no use for scratch)."""
+    if n_rows <= 16 or n_rows > SKINNY_MAX_ROWS or k % 1024 or k == 1024:
+        return 0
+    return ((n_weight_rows + 15) // 16) * (k // 1024) * ((n_rows + 15) // 16) * 256
+
+
 def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0.0, rows=None, m=None, qkv=None,
-                 emit=None, row_scale=None):
+                 emit=None, row_scale=None, scratch=None, counters=None, force_mid_rows=False):
     """out = epilogue(norm(x) @ weight.T) in one launch, for at most 64 rows ("qkv": any
     number of rows; more than 64 take the tiled kernels with the same epilogue).
 
@@ -334,6 +342,10 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
     its shares of the rows' sums of squares to emit["shares"] (float32, at least
     ceil(N / 16) * 64).  row_scale: dict(shares, blocks, eps): the other half: x is such an
     emitted tensor, and the finished sums are scaled by 1 / sqrt(sum of shares / K + eps).
+    scratch (float32, `mid_rows_scratch` words) and counters (int32 zeros, ceil(N / 16); zero
+    again afterwards): let products of 17 to 64 rows over K % 1024 == 0 take a kernel that
+    keeps the batch in LDS and cuts K over workgroups, where that pays (force_mid_rows:
+    wherever it applies, for tests).
 
     x: bfloat16 [M, K]; or, with norm_weight, the float32 residual stream (at most 16
     rows; `rows` optionally gathers them, then `m` is their number).
@@ -381,6 +393,12 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
         _check(ss.dtype == torch.float32 and ss.is_contiguous() and blocks > 0 and ss.numel() >= blocks * SS_STRIDE,
                "linear_fused: row scale shares")
         s_args = [_ptr(ss), blocks, float(row_scale["eps"])]
+    w_args = [None, 0, None, 0]
+    if scratch is not None and counters is not None:
+        _gpu(scratch, counters)
+        _check(scratch.dtype == torch.float32 and scratch.is_contiguous() and counters.dtype == torch.int32
+               and counters.is_contiguous(), "linear_fused: float32 scratch and int32 counters expected")
+        w_args = [_ptr(scratch), scratch.numel(), _ptr(counters), -counters.numel() if force_mid_rows else counters.numel()]
     q = qkv or {}
     if epilogue == "qkv":
         H, KV, hd, ps = q["num_heads"], q["kv_heads"], q["head_dim"], q["page_size"]
@@ -400,9 +418,9 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
                         epi, _ptr(norm_weight), int(fused_norm and norm_weight.dtype == torch.float32), float(eps),
                         _ptr(rows), _ptr(q["positions"]), _ptr(q.get("token_segment")), _ptr(bt),
                         0 if bt is None else bt.stride(0), _ptr(cos), _ptr(sin), half, table_positions,
-                        _ptr(cache), H, KV, hd, ps, *e_args, *s_args, _stream())
+                        _ptr(cache), H, KV, hd, ps, *e_args, *s_args, *w_args, _stream())
         return
     _check(No == (N // 2 if epilogue == "swiglu" else N), "linear_fused: out width")
     lib.core().call("hfee_gemm_skinny", _ptr(out), ldc, _ptr(x), int(fused_norm), lda, _ptr(weight), ldw, M, N, K, epi,
                     _ptr(norm_weight), int(fused_norm and norm_weight.dtype == torch.float32), float(eps), _ptr(rows),
-                    None, None, None, 0, None, None, 0, 0, None, 0, 0, 0, 0, *e_args, *s_args, _stream())
+                    None, None, None, 0, None, None, 0, 0, None, 0, 0, 0, 0, *e_args, *s_args, *w_args, _stream())

@@ -39,6 +39,7 @@ class Attention(Mixer):
     graph_safe = True
     takes_lazy_norm = True
     emits_norm = True
+    second_half_rows = ops.SKINNY_MAX_ROWS
 
     def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
@@ -138,7 +139,7 @@ class Attention(Mixer):
         if fused:
             # norm, projections, rotation and the cache write in one launch
             few = n <= ops.FUSED_NORM_MAX_ROWS
-            halves = h.row_scale() if (few and isinstance(h, LazyNorm)) else None     # first half done before
+            halves = h.row_scale() if isinstance(h, LazyNorm) else None     # first half done before
             norm = h.fusable() if (halves is None and few and isinstance(h, LazyNorm)
                                    and ops.norm_fusion_pays(*self.w_qkv.shape)) else None
             a = halves[0] if halves else h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
@@ -146,7 +147,8 @@ class Attention(Mixer):
                              eps=norm[1] if norm else 0.0, row_scale=halves[1] if halves else None,
                              qkv=dict(positions=ctx.positions, token_segment=ctx.token_segment, block_tables=tables,
                                       cos=cos, sin=sin, cache_layer=cache if writes_cache else None,
-                                      num_heads=H, kv_heads=K, head_dim=hd, page_size=ctx.page_size))
+                                      num_heads=H, kv_heads=K, head_dim=hd, page_size=ctx.page_size),
+                             **ctx.workspace.product_scratch(n, self.w_qkv))
         else:
             hn = h.tensor() if isinstance(h, LazyNorm) else h
             if writes_cache:
@@ -186,10 +188,10 @@ class Attention(Mixer):
                                           ctx.page_size, self.scale, self.window, partial, splits, _DECODE_WAVES,
                                           counters)
         emit = None
-        if then is not None and self.dtype == torch.bfloat16 and n <= ops.FUSED_NORM_MAX_ROWS \
+        if then is not None and self.dtype == torch.bfloat16 and n <= ops.SKINNY_MAX_ROWS \
                 and self.hidden % 8 == 0 and self.q_width % 8 == 0:
             emit = then.offer()
         if emit:       # the output projection adds into x and begins the norm that follows
-            ops.linear_fused(x, att, self.w_o, "add", emit=emit)
+            ops.linear_fused(x, att, self.w_o, "add", emit=emit, **ctx.workspace.product_scratch(n, self.w_o))
         else:
             ops.linear(x, att, self.w_o, accumulate=True)

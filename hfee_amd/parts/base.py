@@ -72,6 +72,9 @@ class Part:
     # True if forward_add accepts `then=` (the LazyNorm of the norm that follows this
     # part) and may do that norm's first half in its last product.
     emits_norm = False
+    # Up to how many rows in a step forward_add finishes a norm whose first half a part
+    # before it has done (LazyNorm.row_scale); 0: never.
+    second_half_rows = 0
 
     def tensor_specs(self) -> list:
         return []
@@ -126,8 +129,9 @@ class LazyNorm:
     (`ops.linear_fused(..., emit=...)`).  The part that consumes the norm then finds
     `pending` set and gives it to its first product as `row_scale`."""
 
-    def __init__(self, ctx, norm, x):
+    def __init__(self, ctx, norm, x, second_half_rows: int = 0):
         self.ctx, self.norm, self.x = ctx, norm, x
+        self.second_half_rows = second_half_rows      # of the part that will consume this norm
         self._tensor = None
         self.pending = None      # dict(out, shares, blocks, eps) once a producer has done the first half
 
@@ -139,7 +143,7 @@ class LazyNorm:
         """For the part that adds into x last: the `emit` arguments of its adding product,
         or None if this norm cannot be split (then nothing changes for anybody)."""
         form = self.fusable()
-        if form is None or self.x.dtype != torch.float32:
+        if form is None or self.x.dtype != torch.float32 or self.ctx.n > self.second_half_rows:
             return None
         weight, eps = form
         width = self.x.shape[1]
@@ -203,6 +207,16 @@ class Workspace:
                 self._retired.append(buf)
             buf = self._buffers[key] = torch.empty((count,), dtype=dtype, device=self.device)
         return buf[:count]
+
+    def product_scratch(self, n_rows: int, weight: torch.Tensor) -> dict:
+        """The `scratch` and `counters` arguments of `ops.linear_fused` for a product of
+        n_rows rows with this weight (empty where it has no use for them)."""
+        from ..kernels import ops
+        words = ops.mid_rows_scratch(n_rows, weight.shape[0], weight.shape[1])
+        if not words:
+            return {}
+        return dict(scratch=self.flat("product.partial", words, torch.float32),
+                    counters=self.counters("product.slices", (weight.shape[0] + 15) // 16))
 
     def counters(self, name: str, count: int) -> torch.Tensor:
         """`count` int32 that are zero, for kernels whose workgroups count themselves

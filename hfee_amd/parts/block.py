@@ -34,20 +34,20 @@ class PreNormBlock(Part):
         for p in self.parts():
             p.bind(tensors)
 
-    # forward takes the normed input that the block before may have prepared, and the
-    # first norm of the block after (the engine passes both to blocks that say so)
+    # forward takes the normed input that the block before may have begun, and that of
+    # the block after, which this block's last part may begin (the engine makes both with
+    # `begin` for blocks that say so)
     chains_norms = True
 
-    def first_norm(self):
-        return self.mixer_norm
+    def begin(self, ctx, x):
+        """The block's normed input, not yet computed."""
+        return LazyNorm(ctx, self.mixer_norm, x, self.mixer.second_half_rows)
 
-    def forward(self, ctx, x, entry, h_in=None, next_norm=None):
-        h = h_in if h_in is not None else LazyNorm(ctx, self.mixer_norm, x)
-        h2 = LazyNorm(ctx, self.feed_forward_norm, x)
+    def forward(self, ctx, x, entry, h_in=None, h_next=None):
+        h = h_in if h_in is not None else self.begin(ctx, x)
+        h2 = LazyNorm(ctx, self.feed_forward_norm, x, self.feed_forward.second_half_rows)
         self._run(self.mixer, ctx, x, h, h2, entry.cache, entry.writes_cache)
-        h3 = LazyNorm(ctx, next_norm, x) if next_norm is not None else None
-        self._run(self.feed_forward, ctx, x, h2, h3)
-        return h3
+        self._run(self.feed_forward, ctx, x, h2, h_next)
 
     @staticmethod
     def _run(part, ctx, x, h, then, *args):

@@ -18,6 +18,7 @@ class GatedMLP(FeedForward):
     graph_safe = True
     takes_lazy_norm = True
     emits_norm = True
+    second_half_rows = ops.FUSED_NORM_MAX_ROWS
 
     def __init__(self, spec: FeedForwardSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
@@ -61,8 +62,11 @@ class GatedMLP(FeedForward):
                 gate_up = ctx.rows("mlp.gate_up", 2 * F)
                 ops.linear(gate_up, hn, self.w_gate_up)
                 ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
-        emit = then.offer() if (then is not None and aligned and few) else None
+        n = ctx.n
+        emit = then.offer() if (then is not None and aligned and n <= ops.SKINNY_MAX_ROWS) else None
         if emit:          # the down projection adds into x and begins the norm that follows
-            ops.linear_fused(x, act, self.w_down, "add", emit=emit)
+            ops.linear_fused(x, act, self.w_down, "add", emit=emit, **ctx.workspace.product_scratch(n, self.w_down))
+        elif aligned and ops.FUSED_NORM_MAX_ROWS < n <= ops.SKINNY_MAX_ROWS:
+            ops.linear_fused(x, act, self.w_down, "add", **ctx.workspace.product_scratch(n, self.w_down))
         else:
             ops.linear(x, act, self.w_down, accumulate=True)

@@ -175,6 +175,64 @@ def test_fused_decode_products(M, N, K, epilogue, norm):
     assert (err <= tol * (1 + mag)).all(), float((err / (1 + mag)).max())
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 48, 1024), (33, 200, 2048), (64, 344, 3072), (40, 6150, 4096), (64, 100, 1024),
+                                   (48, 30, 2048)])
+@pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu", "emit", "scaled"])
+def test_products_of_17_to_64_rows(M, N, K, epilogue):
+    """The kernel that keeps the batch in LDS and cuts K over workgroups (17 to 64 rows,
+    K a multiple of 1,024), with every epilogue, twice in a row on the same scratch and
+    counters, against the unfused formulas."""
+    from hfee_amd.kernels import ops
+    if epilogue == "swiglu" and N % 2:
+        N += 1
+    g = torch.Generator().manual_seed(M + 3 * N + 7 * K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    ref = x.double() @ w.double().t()
+    mag = x.double().abs() @ w.double().abs().t()
+    words = ops.mid_rows_scratch(M, N, K)
+    assert (words > 0) == (K > 1024)
+    scratch = torch.full((max(words, 1),), float("nan"), dtype=torch.float32, device=DEV)
+    counters = torch.zeros((N + 15) // 16, dtype=torch.int32, device=DEV)
+    kw = dict(scratch=scratch, counters=counters, force_mid_rows=True)
+    c0 = torch.randn(M, N, generator=g)
+    for _ in range(2):
+        if epilogue == "swiglu":
+            want = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
+            bound = 2e-2 * (mag[:, 0::2] + 1) * (mag[:, 1::2] + 1)
+            out = torch.zeros(M, N // 2, dtype=torch.bfloat16, device=DEV)
+            ops.linear_fused(out, x.to(DEV), w.to(DEV), "swiglu", **kw)
+        elif epilogue in ("add", "emit"):
+            want, bound = ref + c0.double(), 1e-5 * (1 + mag + c0.abs().double())
+            out = c0.clone().to(DEV)
+            emit = None
+            if epilogue == "emit":
+                nw = (1 + 0.1 * torch.randn(N, generator=g)).float()
+                emitted = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+                shares = torch.zeros(((N + 15) // 16) * 64, dtype=torch.float32, device=DEV)
+                emit = dict(weight=nw.to(DEV), out=emitted, shares=shares)
+            ops.linear_fused(out, x.to(DEV), w.to(DEV), "add", emit=emit, **kw)
+            if emit:
+                close(emitted, want * nw.double(), 1e-2)
+                got = shares.view(-1, 64)[:, :M].double().sum(0).cpu()
+                assert torch.allclose(got, (want ** 2).sum(-1), rtol=1e-5)
+        elif epilogue == "scaled":
+            # x stands for an emitted tensor; the shares are made up so that every row has its own scale
+            blocks = 5
+            shares = torch.rand(blocks * 64, generator=g) + 0.5
+            scale = 1 / torch.sqrt(shares.view(blocks, 64)[:, :M].double().sum(0) / K + 1e-5)
+            want, bound = ref * scale[:, None], 2e-2 * (1 + mag * scale[:, None])
+            out = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+            ops.linear_fused(out, x.to(DEV), w.to(DEV), "bf16", row_scale=dict(shares=shares.to(DEV), blocks=blocks, eps=1e-5), **kw)
+        else:
+            want, bound = ref, (2e-2 if epilogue == "bf16" else 1e-5) * (1 + mag)
+            out = torch.zeros(M, N, dtype=torch.bfloat16 if epilogue == "bf16" else torch.float32, device=DEV)
+            ops.linear_fused(out, x.to(DEV), w.to(DEV), epilogue, **kw)
+        err = (out.double().cpu() - want).abs()
+        assert (err <= bound).all(), float((err / bound).max())
+        assert int(counters.abs().sum()) == 0
+
+
 @pytest.mark.parametrize("M,N,K,N2", [(1, 64, 96, 48), (8, 200, 256, 344), (16, 4096, 1024, 16400), (33, 104, 64, 72),
                                        (64, 520, 128, 100)])
 @pytest.mark.parametrize("epilogue2", ["bf16", "swiglu", "add"])
@@ -229,11 +287,26 @@ def test_norm_in_two_halves(M, N, K, N2, epilogue2):
 def test_fused_qkv_rotation_and_cache_write(H, K, hd, half, M, norm):
     """Projection + rotation (pairs 2i, 2i+1) + cache write in one launch against the
     separate steps: the streaming kernels (up to 64 rows) and the tiled ones."""
-    from plain_llama import plain_rope
-    from hfee_amd.kernels import ops
     if norm and M > 16:
         pytest.skip("the fused norm takes at most 16 rows")
-    d, ps = 96, 16
+    _check_fused_qkv(H, K, hd, half, M, norm, 96)
+
+
+@pytest.mark.parametrize("H,K,hd,half,M,d", [(4, 2, 16, 8, 17, 2048), (5, 1, 64, 32, 64, 1024), (6, 3, 48, 8, 40, 3072)])
+def test_fused_qkv_with_the_batch_in_lds(H, K, hd, half, M, d):
+    """The same through the kernel for 17 to 64 rows that cuts K over workgroups."""
+    from hfee_amd.kernels import ops
+    N = (H + 2 * K) * hd
+    scratch = torch.full((max(ops.mid_rows_scratch(M, N, d), 1),), float("nan"), dtype=torch.float32, device=DEV)
+    counters = torch.zeros((N + 15) // 16, dtype=torch.int32, device=DEV)
+    _check_fused_qkv(H, K, hd, half, M, False, d, scratch=scratch, counters=counters, force_mid_rows=True)
+    assert int(counters.abs().sum()) == 0
+
+
+def _check_fused_qkv(H, K, hd, half, M, norm, d, **kw):
+    from plain_llama import plain_rope
+    from hfee_amd.kernels import ops
+    ps = 16
     g = torch.Generator().manual_seed(H + hd + M)
     N = (H + 2 * K) * hd
     w = (torch.randn(N, d, generator=g) / math.sqrt(d)).to(torch.bfloat16)
@@ -261,7 +334,7 @@ def test_fused_qkv_rotation_and_cache_write(H, K, hd, half, M, norm):
     q_out = torch.zeros(M, H * hd, dtype=torch.bfloat16, device=DEV)
     ops.linear_fused(q_out, x.to(DEV), w.to(DEV), "qkv", norm_weight=nw.to(DEV) if norm else None, eps=1e-6,
                      qkv=dict(positions=pos.to(DEV), token_segment=seg.to(DEV), block_tables=tables.to(DEV), cos=cos, sin=sin,
-                              cache_layer=layer, num_heads=H, kv_heads=K, head_dim=hd, page_size=ps))
+                              cache_layer=layer, num_heads=H, kv_heads=K, head_dim=hd, page_size=ps), **kw)
     close(q_out, q_ref.reshape(M, H * hd), 2e-2)
     lay = layer.cpu()
     for m in range(M):
