@@ -25,6 +25,17 @@ BASE_8B = dict(num_hidden_layers=32, hidden_size=4096, num_attention_heads=32, n
                rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
                rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                              "high_freq_factor": 4.0, "original_max_position_embeddings": 8192})
+# other shapes of the same architecture, for looking at kernels away from the default sizes
+SHAPES = {
+    "llama-3.1-8b": BASE_8B,
+    "llama-3.2-1b": dict(BASE_8B, num_hidden_layers=16, hidden_size=2048, head_dim=64, intermediate_size=8192,
+                         tie_word_embeddings=True,
+                         rope_scaling=dict(BASE_8B["rope_scaling"], factor=32.0)),
+    "llama-2-13b": dict(BASE_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40,
+                        num_key_value_heads=40, intermediate_size=13824, vocab_size=32000,
+                        max_position_embeddings=4096, rope_theta=10000.0, rope_scaling=None),
+}
+SHAPE_NAMES = {"llama-3.1-8b": "Llama-3.1-8B", "llama-3.2-1b": "Llama-3.2-1B", "llama-2-13b": "Llama-2-13B"}
 CONTEXT = 8192
 PROMPT = 1024
 PREFILL = 2048
@@ -36,8 +47,12 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=BASE_8B["num_hidden_layers"])
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.1-8b")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--serving", type=int, default=0, metavar="R",
+                    help="instead of the default run: R requests at once under continuous batching, prompts of "
+                         "64 to 2,048 tokens, 128 new tokens each, context 4,096; prints its own line")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own short line")
     args = ap.parse_args()
@@ -52,7 +67,9 @@ def main() -> int:
     from hfee_amd.engine import Engine, Request, Scheduler, random_model
     from hfee_amd.sampling import Sampler, SamplingParams
 
-    cj = dict(BASE_8B, architectures=["LlamaForCausalLM"], num_hidden_layers=args.layers)
+    base = SHAPES[args.shape]
+    context = min(CONTEXT, base["max_position_embeddings"])
+    cj = dict(base, architectures=["LlamaForCausalLM"], num_hidden_layers=args.layers or base["num_hidden_layers"])
     cfg = config_from_dict(cj)
     t0 = time.perf_counter()
     model = random_model(cfg, seed=0, dtype="bfloat16", device="cuda:0", std=0.02)
@@ -64,18 +81,21 @@ def main() -> int:
     layer_params = d * (H + 2 * K) * hd + H * hd * d + 3 * d * F
     weight_bytes = 2 * (L * layer_params + V * d)              # every matrix a decode step reads, once
     kv_bytes_per_token = L * 2 * K * hd * 2
-    max_batch = max(64, args.batch)
+    max_batch = max(64, args.batch, args.serving)
     steps_total = args.steps + args.warmup
 
     page_size = 16
     tokens_cached = max_batch * (PROMPT + steps_total + page_size) + PREFILL + page_size
+    if args.serving:
+        context = min(context, 4096)
+        tokens_cached = args.serving * (2048 + 128 + page_size)
     engine = Engine(model, cache_tokens=tokens_cached, page_size=page_size, max_requests=max_batch,
-                    max_batch_tokens=PREFILL, num_positions=CONTEXT)
+                    max_batch_tokens=PREFILL, num_positions=context)
     sampler = Sampler(V, engine.device, max_rows=max_batch)
     gen = torch.Generator().manual_seed(0)
 
     def decode_run(batch: int, steps: int, warmup: int):
-        sched = Scheduler(engine, sampler, max_num_seqs=batch, max_batch_tokens=PREFILL, num_ctx=CONTEXT)
+        sched = Scheduler(engine, sampler, max_num_seqs=batch, max_batch_tokens=PREFILL, num_ctx=context)
         params = SamplingParams.greedy(num_predict=-1, ignore_eos=True)
         for i in range(batch):
             prompt = torch.randint(0, V, (PROMPT,), generator=gen).tolist()
@@ -117,6 +137,37 @@ def main() -> int:
             best = dt if best is None else min(best, dt)
         return best
 
+    def serving_run(count: int):
+        """All requests arrive at once; portions of prompts run beside decoded tokens until
+        the last request has its 128 tokens."""
+        sched = Scheduler(engine, sampler, max_num_seqs=count, max_batch_tokens=PREFILL, num_ctx=context)
+        params = SamplingParams.greedy(num_predict=128, ignore_eos=True)
+        lengths = torch.randint(64, 2049, (count,), generator=gen).tolist()
+        for i, n in enumerate(lengths):
+            sched.add(Request(("serving", i), torch.randint(0, V, (n,), generator=gen).tolist(), params, seed=i))
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        steps = made = 0
+        while sched.has_work():
+            for fin in sched.step():
+                made += len(fin.request.generated)
+            steps += 1
+        torch.cuda.synchronize()
+        return time.perf_counter() - t, sum(lengths), made, steps
+
+    if args.serving:
+        serving_run(min(args.serving, 8))        # (compiles nothing, but captures graphs and sizes buffers)
+        dt, prompt_tokens, made, steps = serving_run(args.serving)
+        print(json.dumps({
+            "metric": "continuous batching, generated tok/s (%s bf16)" % SHAPE_NAMES[args.shape],
+            "value": round(made / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "seconds": round(dt, 3),
+            "all_tokens_per_s": round((prompt_tokens + made) / dt, 1), "dtype": "bf16",
+            "data": "synthetic (seeded uniform random token ids, random N(0,0.02) weights)",
+            "config": {"model": SHAPE_NAMES[args.shape] + "-shaped", "layers": L, "requests": args.serving,
+                       "prompt_tokens_total": prompt_tokens, "generated_total": made, "seq_len": context,
+                       "max_batch_tokens": PREFILL, "page_size": page_size}}), flush=True)
+        return 0
+
     if args.prefill_only:
         pt = prefill_run()
         print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": PREFILL, "layers": L}), flush=True)
@@ -128,13 +179,13 @@ def main() -> int:
     step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
     achieved = step_bytes / (dt / args.steps)
     line = {
-        "metric": "decode tok/s @ batch 1/8/64; prefill tok/s @ 2,048 tokens (Llama-3.1-8B bf16)",
+        "metric": "decode tok/s @ batch 1/8/64; prefill tok/s @ 2,048 tokens (%s bf16)" % SHAPE_NAMES[args.shape],
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (seeded uniform random token ids, random N(0,0.02) weights)",
-        "config": {"model": "Llama-3.1-8B-shaped", "layers": L, "layers_of_config": BASE_8B["num_hidden_layers"],
+        "config": {"model": SHAPE_NAMES[args.shape] + "-shaped", "layers": L, "layers_of_config": base["num_hidden_layers"],
                    "hidden": d, "heads": H, "kv_heads": K, "head_dim": hd, "intermediate": F, "vocab": V,
-                   "global_batch": args.batch, "seq_len": CONTEXT, "prompt_tokens": PROMPT,
+                   "global_batch": args.batch, "seq_len": context, "prompt_tokens": PROMPT,
                    "mean_context_in_timed_steps": round(mean_ctx, 1), "page_size": page_size,
                    "max_batch_tokens": PREFILL, "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",

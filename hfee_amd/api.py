@@ -91,17 +91,28 @@ class LLM:
         outputs: dict = {}
         for req in requests:
             self.scheduler.add(req)
-        while self.scheduler.has_work():
-            for fin in self.scheduler.step():
-                h = helpers[fin.request.request_id]
-                text = None
-                if self.tokenizer is not None:
-                    tail = h["stop"].flush() + h["utf8"].flush()
-                    if tail and fin.reason != "stop-string":
-                        h["text"].append(tail)
-                    text = "".join(h["text"])
-                outputs[fin.request.request_id] = Output(list(fin.request.generated), text, fin.request.stats,
-                                                         fin.reason, fin.error)
+        try:
+            while self.scheduler.has_work():
+                for fin in self.scheduler.step():
+                    h = helpers[fin.request.request_id]
+                    text = None
+                    if self.tokenizer is not None:
+                        tail = h["stop"].flush() + h["utf8"].flush()
+                        if tail and fin.reason != "stop-string":
+                            h["text"].append(tail)
+                        text = "".join(h["text"])
+                    outputs[fin.request.request_id] = Output(list(fin.request.generated), text, fin.request.stats,
+                                                             fin.reason, fin.error)
+        except BaseException:
+            # interrupted (Ctrl-C, an error in on_token): what is unfinished is cancelled, as the
+            # reference ends a request whose caller has gone (/root/reference/internal/llm/runner.go:244-247),
+            # so that its pages are free for the next call
+            for req in requests:
+                if req.request_id not in outputs:
+                    self.scheduler.cancel(req.request_id)
+            while self.scheduler.has_work():
+                self.scheduler.step()
+            raise
         return [outputs[r.request_id] for r in requests]
 
     def _make_emit(self, h, on_token):

@@ -67,7 +67,6 @@ def run(argv) -> int:
     args = ap.parse_args(argv)
 
     from .api import LLM
-    from .sampling import SamplingParams
 
     t0 = time.perf_counter()
     llm = LLM(args.model, random_weights=args.random_weights, seed=args.seed, dtype=args.dtype,
@@ -81,6 +80,8 @@ def run(argv) -> int:
         text = " ".join(args.prompt)
         if not sys.stdin.isatty():
             text = (sys.stdin.read().strip() + "\n\n" + text).strip()      # run.go:46-53
+        if not text and sys.stdin.isatty() and llm.tokenizer is not None:
+            return interactive(llm, make_params(args), args.verbose, load)
         if not text:
             print("usage: hfee run <model> [prompt]   (or --tokens 1,2,3)", file=sys.stderr)
             return 1
@@ -89,11 +90,21 @@ def run(argv) -> int:
             return 1
         prompt = text
 
-    params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
-                            repeat_penalty=args.repeat_penalty, repeat_last_n=args.repeat_last_n,
-                            seed=args.sample_seed, num_predict=args.num_predict, stop=tuple(args.stop),
-                            ignore_eos=args.ignore_eos)
+    answer(llm, prompt, make_params(args), args.verbose, load, t0)
+    return 0
 
+
+def make_params(args):
+    from .sampling import SamplingParams
+    return SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
+                          repeat_penalty=args.repeat_penalty, repeat_last_n=args.repeat_last_n,
+                          seed=args.sample_seed, num_predict=args.num_predict, stop=tuple(args.stop),
+                          ignore_eos=args.ignore_eos)
+
+
+def answer(llm, prompt, params, verbose: bool, load: float, t0: float):
+    """Generates from one prompt, printing the pieces as they come, and with --verbose the
+    counts and rates of /root/reference/cmd/hfee/run.go:210-223."""
     def show(index, token, text):
         if llm.tokenizer is not None:
             if text:
@@ -102,10 +113,8 @@ def run(argv) -> int:
             print(token, end=" ", flush=True)
 
     out = llm.generate([prompt], params, on_token=show)[0]
-    if llm.tokenizer is not None and out.text is not None:
-        pass
     print("\n")
-    if args.verbose:
+    if verbose:
         s = out.stats
         total = time.perf_counter() - t0
 
@@ -118,7 +127,58 @@ def run(argv) -> int:
         print(f"eval count:           {s.eval_tokens} token(s)")
         print(f"eval rate:            {rate(s.eval_tokens, s.eval_duration)}")
         print(f"done reason:          {out.done_reason}\n")
-    return 0
+    return out
+
+
+def read_message(readline, prompt_more=lambda: print("... ", end="", flush=True)):
+    """One line, or several between \"\"\" markers (/root/reference/cmd/hfee/run.go:154-175).
+    None at the end of the input."""
+    line = readline()
+    if not line:
+        return None
+    line = line.strip()
+    if not line.startswith('"""'):
+        return line
+    body = line[3:]
+    while not body.strip().endswith('"""') or not body:
+        prompt_more()
+        more = readline()
+        if not more:
+            return None
+        body += "\n" + more.rstrip("\r\n")
+    return body.strip()[:-3].strip()
+
+
+def interactive(llm, params, verbose: bool, load: float) -> int:
+    """`hfee run <model>` without a prompt on a terminal: messages are read one after the
+    other (/root/reference/cmd/hfee/run.go:69-152).  Every message is a prompt of its
+    own: the reference keeps a conversation through its server's chat template, and the
+    server is no part of this engine, so /clear and /system have nothing to act on."""
+    print('Type a message, or /? for help. Use """ to begin a multi-line message.')
+    while True:
+        print(">>> ", end="", flush=True)
+        try:
+            line = read_message(sys.stdin.readline)
+        except KeyboardInterrupt:
+            print("\nUse Ctrl + d or /bye to exit.")
+            continue
+        if line is None:
+            print()
+            return 0
+        if line == "":
+            continue
+        if line in ("/bye", "/exit"):
+            return 0
+        if line in ("/?", "/help"):
+            print('  /bye            Exit\n  """             Start or end a multi-line message')
+            continue
+        if line.startswith("/"):
+            print(f"Unknown command {line.split()[0]}. Type /? for help.")
+            continue
+        try:
+            answer(llm, line, params, verbose, load, time.perf_counter())
+        except KeyboardInterrupt:
+            print()
 
 
 def main(argv=None) -> int:

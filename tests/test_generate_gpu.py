@@ -84,3 +84,29 @@ def test_stop_on_eos_and_context_limit(model_folders, tmp_path):
     assert o.done_reason == "length" and len(prompt) + len(o.token_ids) == 21
     with pytest.raises(ValueError, match="context window"):
         small.generate([list(range(20))], SamplingParams.greedy())
+
+
+def test_an_interrupted_call_leaves_nothing_behind(model_folders):
+    """An error from the caller's on_token ends the call; its requests are cancelled and
+    their pages freed, and the next call gives the usual tokens."""
+    from hfee_amd import LLM, SamplingParams
+    folder = model_folders[("A", "float32")]
+    prompts = list(tu.make_requests(256, [9, 20], seed=4).values())
+    llm = LLM(folder, dtype="float32", num_ctx=128, num_parallel=2)
+    want = [o.token_ids for o in llm.generate(prompts, SamplingParams.greedy(num_predict=10))]
+
+    class Stop(Exception):
+        pass
+
+    seen = []
+
+    def on_token(index, token, text):
+        seen.append(token)
+        if len(seen) == 5:
+            raise Stop()
+
+    with pytest.raises(Stop):
+        llm.generate(prompts, SamplingParams.greedy(num_predict=10), on_token=on_token)
+    assert not llm.scheduler.has_work() and not llm.engine.cache.requests
+    llm.engine.cache.check()
+    assert [o.token_ids for o in llm.generate(prompts, SamplingParams.greedy(num_predict=10))] == want

@@ -182,3 +182,21 @@ def test_eos_stops_without_keeping_the_token_and_cancel_frees():
     assert done["c"].reason == "cancelled"
     eng.cache.check()
     assert eng.cache.free_pages() == [32] and eng.cache.num_free_slots == 2
+
+
+def test_the_command_line_reads_messages_of_one_or_several_lines():
+    """/root/reference/cmd/hfee/run.go:154-175: a line, or what stands between two markers."""
+    from hfee_amd.cli import read_message
+
+    def reader(text):
+        lines = iter(text.splitlines(keepends=True))
+        return lambda: next(lines, "")
+
+    quiet = lambda: None
+    assert read_message(reader("  hello there \n"), quiet) == "hello there"
+    assert read_message(reader("\n"), quiet) == ""
+    assert read_message(reader(""), quiet) is None
+    assert read_message(reader('"""first\nsecond line\n  third"""\nnext\n'), quiet) == "first\nsecond line\n  third"
+    assert read_message(reader('"""\nalone\n"""\n'), quiet) == "alone"
+    assert read_message(reader('"""one line"""\n'), quiet) == "one line"
+    assert read_message(reader('"""never closed\n'), quiet) is None
