@@ -146,6 +146,26 @@ class Scheduler:
             self.running.remove(request)
         finished.append(Finished(request, reason, error))
 
+    def _plan_ahead(self, batch) -> None:
+        """If the next step can only be "every request of this one decodes one more token"
+        (nobody waits for a place, no prompt is unfinished, nobody reaches its limit of
+        tokens, nobody is at the end of the context), the engine plans that step now, while the
+        GPU is busy with this one.  A guess that fails (an end-of-sequence token, a
+        cancellation) costs nothing but the planning."""
+        if self.waiting or len(batch) != len(self.running):
+            return
+        shape = []
+        for (r, toks, want), q in zip(batch, self.running):
+            if r is not q or not want or len(r.feed) != 0 or r.cancelled:
+                return
+            limit = r.params.num_predict
+            if limit >= 0 and len(r.generated) + 1 >= limit:
+                return
+            if self.cache.get(r.request_id).length + 1 > self.num_ctx:
+                return
+            shape.append((r.request_id, 1, [0]))
+        self.engine.prepare(shape)
+
     # ------------------------------------------------------------------- step
     def step(self) -> list:
         """One pass: admit, batch, run, sample.  Returns the requests that finished."""
@@ -248,7 +268,9 @@ class Scheduler:
             if want:
                 owners.append(r)
                 rows.append(SampleRow(r.params, r.seed, r.draws, r.history, len(rows)))
-        ids = self.sampler.sample(logits, rows) if rows else []
+        pending = self.sampler.launch(logits, rows)
+        self._plan_ahead(batch)          # while the GPU runs this step
+        ids = self.sampler.collect(pending)
         now = self.clock()
         for r, token in zip(owners, ids):
             if not r.decoding:

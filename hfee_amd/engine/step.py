@@ -38,6 +38,7 @@ class StepPlan:
         self.segments = segments
         self.arrays: dict = {}
         self.host: dict = {}
+        self.packed = None        # set by the engine once the arrays lie in a pinned buffer
 
     def add(self, key: str, array: np.ndarray):
         if key in self.arrays:
@@ -76,6 +77,8 @@ class Engine:
                 self.storage.add_state(name, shape, dt)
         model.prepare(info)
         self._meta_capacity = 0
+        self._meta_views: dict = {}        # layout of a step's metadata -> (offsets, views of the device buffer)
+        self._prepared = None              # (signature, plan) of a step planned ahead
         self._meta_ring, self._meta_device = [], None
         self.steps_run = 0
         # decode-only steps are replayed as captured HIP graphs, one per
@@ -90,10 +93,12 @@ class Engine:
     def admit(self, request_id):
         rc = self.cache.admit(request_id)
         self.storage.clear_slot(rc.slot)
+        self._prepared = None
         return rc
 
     def release(self, request_id):
         self.cache.release(request_id)
+        self._prepared = None
 
     def is_live(self, request_id) -> bool:
         return request_id in self.cache.requests
@@ -141,13 +146,10 @@ class Engine:
         for e in entries:
             self.cache.reserve(e.request_id, len(e.tokens))
 
-    def _upload(self, plan: StepPlan) -> dict:
-        """All planned arrays in one pinned buffer, one copy to the device."""
-        offsets, total = {}, 0
-        for key, a in plan.arrays.items():
-            offsets[key] = total
-            total += (a.size + 3) // 4 * 4
-        total = max(total, 4)
+    def _pack(self, plan: StepPlan) -> None:
+        """Lays the planned arrays out in the pinned buffer of the coming step."""
+        layout = tuple((key, a.shape) for key, a in plan.arrays.items())
+        total = max(sum((a.size + 3) // 4 * 4 for a in plan.arrays.values()), 4)
         if total > self._meta_capacity:
             cap = max(total * 2, self._meta_bound())
             # a ring of pinned buffers: the copy of step k may still be in flight
@@ -156,36 +158,47 @@ class Engine:
                                for _ in range(4)]
             self._meta_device = torch.empty(cap, dtype=torch.int32, device=self.device)
             self._meta_capacity = cap
+            self._meta_views.clear()
             self._graphs.clear()      # captured graphs point into the old buffer
+        views = self._meta_views.get(layout)
+        if views is None:             # where each array lies, and its view of the device buffer
+            if len(self._meta_views) > 256:
+                self._meta_views.clear()
+            offsets, dev, at = {}, {}, 0
+            for key, a in plan.arrays.items():
+                offsets[key] = at
+                dev[key] = self._meta_device[at:at + a.size].view(a.shape)
+                at += (a.size + 3) // 4 * 4
+            views = self._meta_views[layout] = (offsets, dev)
+        offsets, dev = views
         pinned, event = self._meta_ring[self.steps_run % len(self._meta_ring)]
         event.synchronize()
         host = pinned.numpy()
         for key, a in plan.arrays.items():
             host[offsets[key]:offsets[key] + a.size] = a.reshape(-1)
+        plan.packed = (self.steps_run, self._meta_device, pinned, event, total, dev, host[offsets["token_ids"]:])
+
+    def _upload(self, plan: StepPlan, tokens) -> dict:
+        """All planned arrays in one pinned buffer, one copy to the device."""
+        if plan.packed is None or plan.packed[0] != self.steps_run or plan.packed[1] is not self._meta_device:
+            self._pack(plan)
+        _, _, pinned, event, total, dev, token_place = plan.packed
+        token_place[:len(tokens)] = tokens
         self._meta_device[:total].copy_(pinned[:total], non_blocking=True)
         event.record()
-        out = {}
-        for key, a in plan.arrays.items():
-            out[key] = self._meta_device[offsets[key]:offsets[key] + a.size].view(a.shape)
-        return out
+        return dev
 
-    def begin(self, entries):
-        """Checks the entries, takes their pages, sends the step's metadata to the
-        device and returns (context, number of wanted rows, key for graph capture or
-        None).  step() is begin + the model + commit; tests of single parts call
-        begin() themselves."""
-        entries = list(entries)
-        self._check(entries)
-        self._reserve(entries)
-
-        segments, tokens, logit_rows = [], [], []
+    def _plan(self, shape) -> StepPlan:
+        """The metadata of a step whose entries are `shape`: (request id, number of tokens,
+        wanted places) each; everything but the token ids themselves.  The requests' pages
+        are reserved already."""
+        segments, logit_rows = [], []
         row = 0
-        for e in entries:
-            rc = self.cache.get(e.request_id)
-            segments.append(Segment(e.request_id, rc.slot, rc.length, len(e.tokens), row))
-            tokens += e.tokens
-            logit_rows += [row + w for w in e.want]
-            row += len(e.tokens)
+        for rid, count, want in shape:
+            rc = self.cache.get(rid)
+            segments.append(Segment(rid, rc.slot, rc.length, count, row))
+            logit_rows += [row + w for w in want]
+            row += count
         n = row
         starts = np.fromiter((s.start for s in segments), dtype=np.int32, count=len(segments))
         lengths = np.fromiter((s.length for s in segments), dtype=np.int32, count=len(segments))
@@ -194,7 +207,7 @@ class Engine:
         positions = np.arange(n, dtype=np.int32) - np.repeat(rows0 - starts, lengths)
 
         plan = StepPlan(segments)
-        plan.add("token_ids", np.asarray(tokens))
+        plan.add("token_ids", np.zeros(n, dtype=np.int32))
         plan.add("positions", positions)
         plan.add("token_segment", token_segment)
         plan.add("segment_slots", np.fromiter((s.slot for s in segments), dtype=np.int32, count=len(segments)))
@@ -222,22 +235,67 @@ class Engine:
             if id(mixer) not in seen:
                 seen.add(id(mixer))
                 mixer.plan(plan)
+        plan.n, plan.wanted, plan.max_position = n, len(logit_rows), int(positions.max())
+        plan.graph_key = None
+        if decode_only:
+            plan.graph_key = (n, tuple(widths), plan.wanted, tuple(sorted((k, a.shape) for k, a in plan.arrays.items())))
+        return plan
 
-        dev = self._upload(plan)
+    def _signature(self, shape) -> tuple:
+        """What a plan depends on beside the pages that its requests hold."""
+        return tuple((rid, self.cache.get(rid).length, count, tuple(want)) for rid, count, want in shape)
+
+    def prepare(self, shape) -> bool:
+        """For a caller that knows the shape of its next step before it knows the tokens
+        (a scheduler, while the GPU still runs the step before): reserves the pages and
+        plans the step now, so that begin() has only the tokens left to fill in.  shape:
+        (request id, number of tokens, wanted places) for each entry.  Nothing is lost if
+        the next step turns out differently: begin() then plans anew (pages that were
+        reserved stay with their requests).  False if the pages do not suffice."""
+        self._prepared = None
+        shape = [(rid, count, list(want)) for rid, count, want in shape]
+        need = [0] * len(self.groups)
+        for rid, count, _ in shape:
+            if rid not in self.cache.requests or self.cache.get(rid).length + count > self.num_positions:
+                return False
+            for g, k in enumerate(self.cache.pages_needed(rid, count)):
+                need[g] += k
+        free = self.cache.free_pages()
+        if any(need[g] > free[g] for g in range(len(self.groups))):
+            return False
+        for rid, count, _ in shape:
+            self.cache.reserve(rid, count)
+        plan = self._plan(shape)
+        self._pack(plan)
+        self._prepared = (self._signature(shape), plan)
+        return True
+
+    def begin(self, entries):
+        """Checks the entries, takes their pages, sends the step's metadata to the
+        device and returns (context, number of wanted rows, key for graph capture or
+        None).  step() is begin + the model + commit; tests of single parts call
+        begin() themselves."""
+        entries = list(entries)
+        self._check(entries)
+        self._reserve(entries)
+
+        shape = [(e.request_id, len(e.tokens), e.want) for e in entries]
+        prepared, self._prepared = self._prepared, None
+        if prepared is not None and prepared[0] == self._signature(shape):
+            plan = prepared[1]
+        else:
+            plan = self._plan(shape)
+        tokens = entries[0].tokens if len(entries) == 1 else [t for e in entries for t in e.tokens]
+        dev = self._upload(plan, tokens)
         ctx = StepContext(
-            n=n, dtype=self.dtype, device=self.device, segments=segments,
+            n=plan.n, dtype=self.dtype, device=self.device, segments=plan.segments,
             token_ids=dev["token_ids"], positions=dev["positions"], token_segment=dev["token_segment"],
             segment_slots=dev["segment_slots"], segment_starts=dev["segment_starts"],
             segment_lengths=dev["segment_lengths"], segment_rows=dev["segment_rows"],
             block_tables=[dev[f"block_tables.{g}"] for g in range(len(self.groups))],
-            max_position=int(positions.max()), storage=self.storage, workspace=self.workspace,
+            max_position=plan.max_position, storage=self.storage, workspace=self.workspace,
             page_size=self.page_size, extra=dev, host=plan.host)
-
-        w = len(logit_rows)
-        key = None
-        if decode_only:
-            key = (n, tuple(widths), w, tuple(sorted((k, a.shape) for k, a in plan.arrays.items())))
-        return ctx, w, key
+        return ctx, plan.wanted, plan.graph_key
 
     def commit(self, entries) -> None:
         for e in entries:

@@ -68,25 +68,41 @@ class Sampler:
     def __init__(self, vocab: int, device, max_rows: int):
         self.vocab, self.device, self.max_rows = vocab, device, max_rows
         self._out = torch.empty(max_rows, dtype=torch.int32, device=device)
+        self._host = torch.empty(max_rows, dtype=torch.int32, pin_memory=True)
+        self._done = torch.cuda.Event()
         self._scratch = None
 
     def sample(self, logits: torch.Tensor, rows) -> list:
         """logits: float32 [*, vocab] on the device (changed in place by the repeat
         penalty, as the reference changes them).  Returns one id per row."""
+        return self.collect(self.launch(logits, rows))
+
+    def launch(self, logits: torch.Tensor, rows):
+        """Starts the sampling of `rows` and returns what collect() takes: the caller may
+        do other work on the host between the two while the GPU runs."""
         n = len(rows)
         if n == 0:
-            return []
+            return 0
         if n > self.max_rows:
             raise ValueError(f"{n} rows to sample, the sampler was made for {self.max_rows}")
         plain_greedy = all(r.params.temperature <= 0 and (r.params.repeat_penalty == 1 or r.params.repeat_last_n == 0)
                            for r in rows)
         if plain_greedy and [r.logits_row for r in rows] == list(range(logits.shape[0])):
             ops.argmax(self._out, logits)
-            return self._out[:n].tolist()
-        params, hist = pack_rows(rows)
-        if self._scratch is None:
-            self._scratch = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
-        dparams = torch.from_numpy(params).to(self.device)
-        dhist = torch.from_numpy(hist).to(self.device)
-        ops.sample(self._out, logits, dparams, dhist, self._scratch)
-        return self._out[:n].tolist()
+        else:
+            params, hist = pack_rows(rows)
+            if self._scratch is None:
+                self._scratch = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
+            dparams = torch.from_numpy(params).to(self.device)
+            dhist = torch.from_numpy(hist).to(self.device)
+            ops.sample(self._out, logits, dparams, dhist, self._scratch)
+        self._host[:n].copy_(self._out[:n], non_blocking=True)
+        self._done.record()
+        return n
+
+    def collect(self, n: int) -> list:
+        """Waits for the ids of the last launch()."""
+        if n == 0:
+            return []
+        self._done.synchronize()
+        return self._host[:n].tolist()

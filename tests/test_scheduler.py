@@ -18,6 +18,8 @@ class FakeEngine:
         self.cache = CacheManager([CacheGroupSpec("full", 1, 16, (0,))], page_size, num_pages, max_requests)
         self.fed = {}          # request -> tokens in its cache
         self.batches = []      # per step: [(request, n tokens, wants logits)]
+        self.prepared = None   # the shape that the scheduler announced for the next step
+        self.guesses = []      # per announced shape: did the next step have it?
 
     def admit(self, rid):
         self.fed[rid] = []
@@ -30,9 +32,24 @@ class FakeEngine:
     def is_live(self, rid):
         return rid in self.cache.requests
 
+    def prepare(self, shape):
+        """As the engine: reserves the pages of the announced step if they are there."""
+        shape = [(rid, n, list(want)) for rid, n, want in shape]
+        assert all(rid in self.cache.requests for rid, _, _ in shape)
+        need = sum(self.cache.pages_needed(rid, n)[0] for rid, n, _ in shape)
+        if need > self.cache.free_pages()[0]:
+            return False
+        for rid, n, _ in shape:
+            self.cache.reserve(rid, n)
+        self.prepared = shape
+        return True
+
     def step(self, entries):
         rows = []
         assert len({e.request_id for e in entries}) == len(entries)
+        if self.prepared is not None:
+            self.guesses.append(self.prepared == [(e.request_id, len(e.tokens), list(e.want)) for e in entries])
+            self.prepared = None
         for e in entries:
             assert len(self.fed[e.request_id]) == self.cache.get(e.request_id).length
             self.cache.reserve(e.request_id, len(e.tokens))
@@ -47,6 +64,12 @@ class FakeEngine:
 
 
 class FakeSampler:
+    def launch(self, logits, rows):
+        return self.sample(logits, rows)
+
+    def collect(self, pending):
+        return pending
+
     def sample(self, logits, rows):
         out = []
         for r in rows:
@@ -200,3 +223,39 @@ def test_the_command_line_reads_messages_of_one_or_several_lines():
     assert read_message(reader('"""\nalone\n"""\n'), quiet) == "alone"
     assert read_message(reader('"""one line"""\n'), quiet) == "one line"
     assert read_message(reader('"""never closed\n'), quiet) is None
+
+
+def test_decode_steps_are_announced_ahead_and_a_wrong_guess_costs_nothing():
+    """While every live request decodes and nobody waits, the scheduler tells the engine
+    the shape of the next step before it knows the tokens; it does not when a request is
+    about to reach its limit, and an end-of-sequence token merely makes a guess wrong."""
+    class EosSampler(FakeSampler):
+        def sample(self, logits, rows):
+            return [EOS if (r.seed == 2 and r.draw == 5) else t for r, t in zip(rows, super().sample(logits, rows))]
+    eng = FakeEngine(32, 3)
+    s = Scheduler(eng, EosSampler(), max_num_seqs=3, max_batch_tokens=64, num_ctx=128, eos_token_ids=(EOS,),
+                  clock=lambda: 0.0)
+    s.add(Request("a", [1, 2, 3], SamplingParams.greedy(num_predict=20), seed=1))
+    s.add(Request("b", list(range(20)), SamplingParams.greedy(num_predict=30), seed=2))
+    s.add(Request("c", [7], SamplingParams.greedy(num_predict=12), seed=3))
+    done = run_all(s)
+    assert [len(done[k].request.generated) for k in "abc"] == [20, 5, 12] and done["b"].reason == "stop"
+    # steps: 1 prompt step, then decode steps until "a" has its 20 tokens
+    assert len(eng.batches) == 20
+    assert eng.guesses.count(False) == 1          # the step after b's end-of-sequence token
+    # a guess after each of the steps 1..19 but step 12, whose token is c's last (a's last is step 20's)
+    assert len(eng.guesses) == 18
+    eng.cache.check()
+    assert eng.cache.free_pages() == [32]
+
+    # the same requests without any announcement give the same tokens
+    eng2 = FakeEngine(32, 3)
+    eng2.prepare = lambda shape: False
+    s2 = Scheduler(eng2, EosSampler(), max_num_seqs=3, max_batch_tokens=64, num_ctx=128, eos_token_ids=(EOS,),
+                   clock=lambda: 0.0)
+    s2.add(Request("a", [1, 2, 3], SamplingParams.greedy(num_predict=20), seed=1))
+    s2.add(Request("b", list(range(20)), SamplingParams.greedy(num_predict=30), seed=2))
+    s2.add(Request("c", [7], SamplingParams.greedy(num_predict=12), seed=3))
+    done2 = run_all(s2)
+    assert all(done2[k].request.generated == done[k].request.generated for k in "abc")
+    assert eng2.batches == eng.batches
