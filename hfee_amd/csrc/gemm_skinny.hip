@@ -158,16 +158,42 @@ __device__ __forceinline__ void compute_block(f32x4* acc, float* ss, const Block
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
 
 // ROW SCALE: 1/sqrt(mean of squares + eps) of every batch row from the shares that the
-// product before this one left, into `out` (LDS, SS_STRIDE floats).  Wave w takes rows
-// w, w + WAVES, ...; lane l adds shares l, l + 64, ... and the lanes meet in a fixed tree,
-// so the sum does not depend on anything but the shares.  The caller synchronises.
+// product before this one left, into `out` (LDS, SS_STRIDE floats).  All threads of the
+// workgroup come here; the caller synchronises before it reads `out`.  Lane l of wave w
+// takes batch rows l % 16 (+16, +32, +48) and the shares 4w + l/16, + 32, ...: every load
+// is on its own (nobody waits for a sum before asking for the next share), a row's four
+// lanes meet by shuffles and the waves in LDS, in an order that depends on nothing but
+// the number of shares.
 __device__ __forceinline__ void row_scales(const Args& a, float* out) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int m = wave; m < a.M; m += WAVES) {
-    float t = 0.f;
-    for (int b = lane; b < a.scale_blocks; b += 64) t += a.scale_ss[(int64_t)b * SS_STRIDE + m];
-    t = wave_sum(t);
-    if (lane == 0) out[m] = 1.0f / sqrtf(t / (float)a.K + a.scale_eps);
+  __shared__ float part[WAVES][SS_STRIDE];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, j = lane >> 4;
+  const int tiles = (a.M + 15) >> 4;
+  float s[SS_STRIDE / 16];
+  const float* p[SS_STRIDE / 16];
+#pragma unroll
+  for (int t = 0; t < SS_STRIDE / 16; ++t) {
+    s[t] = 0.f;
+    p[t] = a.scale_ss + min(t * 16 + m16, a.M - 1);      // rows beyond M repeat the last one; nobody uses them
+  }
+#pragma unroll 4
+  for (int b = wave * 4 + j; b < a.scale_blocks; b += WAVES * 4) {
+#pragma unroll
+    for (int t = 0; t < SS_STRIDE / 16; ++t)
+      if (t < tiles) s[t] += p[t][(int64_t)b * SS_STRIDE];
+  }
+#pragma unroll
+  for (int t = 0; t < SS_STRIDE / 16; ++t) {
+    float v = s[t];
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    if (j == 0) part[wave][t * 16 + m16] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < SS_STRIDE) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) v += part[w][threadIdx.x];
+    out[threadIdx.x] = 1.0f / sqrtf(v / (float)a.K + a.scale_eps);
   }
 }
 
@@ -235,6 +261,7 @@ template <int MT, bool NORM, int EPI>
 __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   __shared__ float partial[WAVES][MT][64][4];
   __shared__ float ss_part[WAVES][MT][16];
+  __shared__ float row_scale[SS_STRIDE];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * ROWS;
@@ -263,6 +290,8 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
     XBlock<MT, NORM> xcur, xnxt;
     int kb = wave;
     if (kb < nfull) load_block<MT, NORM>(cur, xcur, w_row, x_rows, a, kb * KBLOCK);
+    // (behind the first loads of W, so that it costs no latency of its own)
+    if (!NORM && a.scale_ss != nullptr) row_scales(a, row_scale);
     while (kb < nfull) {
       const int kn = kb + WAVES;
       if (kn < nfull) load_block<MT, NORM>(nxt, xnxt, w_row, x_rows, a, kn * KBLOCK);
@@ -307,8 +336,6 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   }
 
   // ---- partial sums meet in LDS ---------------------------------------------------
-  __shared__ float row_scale[SS_STRIDE];
-  if (!NORM && a.scale_ss != nullptr) row_scales(a, row_scale);
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
 #pragma unroll
