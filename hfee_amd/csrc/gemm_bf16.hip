@@ -890,7 +890,13 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(
 // peak that each kernel was measured to reach on a busy CU (128 x 128: two workgroups a
 // CU; the large tiles reach more the longer K is, and a tile of empty rows costs as
 // much as a full one).
-inline int fastest_tiled(int M, int N, int K, bool large_ok) {
+struct TiledPlan {
+  int first;       // kernel of the columns 0 .. n1
+  int n1;
+  int second;      // kernel of the columns n1 .. N (0: there are none)
+};
+
+inline TiledPlan plan_tiled(int M, int N, int K, bool large_ok, bool may_split) {
   static int cus = 0;
   if (cus == 0) {
     int dev = 0;
@@ -898,34 +904,73 @@ inline int fastest_tiled(int M, int N, int K, bool large_ok) {
     cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
            prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
   }
-  if (!large_ok) return 2;
-  auto tiles = [&](int bm, int bn) { return (double)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-  auto rounds = [&](double t, int slots) { return (double)(int64_t)((t + slots - 1) / slots); };
-  const double t2 = tiles(128, 128), t4 = tiles(256, 256), t5 = tiles(256, 128), t6 = tiles(256, 192);
-  const double c2 = t2 <= cus ? 128.0 * 128 / 0.22 : rounds(t2, 2 * cus) * 2 * 128 * 128 / 0.31;
+  if (!large_ok) return TiledPlan{2, N, 0};
   const double fill = K >= 512 ? 1.0 : 0.6;            // the four-buffer pipeline needs a few steps to pay
-  const double c4 = rounds(t4, cus) * 256 * 256 / (0.46 * fill);
-  const double c5 = rounds(t5, cus) * 256 * 128 / (0.42 * fill);
-  const double c6 = rounds(t6, cus) * 256 * 192 / (0.44 * fill);
-  int best = 2;
-  double cost = c2;
-  if (c5 < cost) { best = 5; cost = c5; }
-  if (c6 < cost) { best = 6; cost = c6; }
-  if (c4 <= cost) best = 4;
+  auto rounds = [&](double t, int slots) { return (double)(int64_t)((t + slots - 1) / slots); };
+  // time of kernel k on n columns, in tile elements over the share of the peak
+  auto cost = [&](int k, int n) {
+    const int bm = k == 2 ? 128 : 256, bn = k == 2 ? 128 : k == 4 ? 256 : k == 5 ? 128 : 192;
+    const double t = (double)((M + bm - 1) / bm) * ((n + bn - 1) / bn);
+    if (k == 2) return t <= cus ? 128.0 * 128 / 0.22 : rounds(t, 2 * cus) * 2 * 128 * 128 / 0.31;
+    return rounds(t, cus) * bm * bn / ((k == 4 ? 0.46 : k == 5 ? 0.42 : 0.44) * fill);
+  };
+  TiledPlan best{2, N, 0};
+  double best_cost = cost(2, N);
+  for (int k : {5, 6, 4})
+    if (cost(k, N) < best_cost || (k == 4 && cost(k, N) <= best_cost)) {
+      best = TiledPlan{k, N, 0};
+      best_cost = cost(k, N);
+    }
+  // A last round of large tiles that fills a part of the chip only costs as much as a
+  // full one: the columns of the whole rounds go to the large tiles and the rest to a
+  // second launch with the kernel that suits it (for 2,048 x 28,672: three rounds of
+  // 256 x 256 and one of 256 x 128 in place of seven of 256 x 128).
+  if (may_split) {
+    const double launch = 3e-6 / (K * 2.05e-13);       // a second launch, in the same unit
+    const int tile_rows = (M + 255) / 256;
+    for (int a : {4, 6}) {
+      const int bn = a == 4 ? 256 : 192;
+      const int per_round = cus / tile_rows;           // tile columns that one round takes
+      if (per_round < 1) continue;
+      const int whole = (N / bn) / per_round;
+      const int n1 = whole * per_round * bn;
+      if (whole < 1 || n1 >= N) continue;
+      for (int b : {2, 5, 6, 4}) {
+        const double c = cost(a, n1) + cost(b, N - n1) + launch;
+        if (c < best_cost) {
+          best = TiledPlan{a, n1, b};
+          best_cost = c;
+        }
+      }
+    }
+  }
   return best;
+}
+
+template <int MODE>
+int launch_tiled_kernel(int choice, void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
+                        int M, int N, int K, hipStream_t stream, const QkvArgs& qkv) {
+  if (choice == 6) return launch_direct<MODE, 4, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
 }
 
 template <int MODE>
 int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
                    int M, int N, int K, int force_kernel, hipStream_t stream, const QkvArgs& qkv = QkvArgs{}) {
-  int choice = force_kernel;
   const bool large_ok = large_fits(lda, ldw, M, N, K);
-  if (choice != 2 && (choice < 4 || choice > 6)) choice = fastest_tiled(M, N, K, large_ok);
-  if (choice >= 4 && !large_ok) choice = 2;
-  if (choice == 6) return launch_direct<MODE, 4, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
-  if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
-  if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
-  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  if (force_kernel == 2 || (force_kernel >= 4 && force_kernel <= 6))
+    return launch_tiled_kernel<MODE>(force_kernel >= 4 && !large_ok ? 2 : force_kernel, C, ldc, A, lda, W, ldw, M, N, K,
+                                     stream, qkv);
+  // (the q/k/v epilogue finds a column's head by its number: those products stay whole)
+  const TiledPlan plan = plan_tiled(M, N, K, large_ok, MODE != OUT_QKV);
+  if (int rc = launch_tiled_kernel<MODE>(plan.first, C, ldc, A, lda, W, ldw, M, plan.n1, K, stream, qkv)) return rc;
+  if (plan.second == 0) return 0;
+  const int64_t skip = MODE == OUT_SWIGLU ? plan.n1 / 2 : plan.n1;         // output columns of the first part
+  void* c2 = (MODE == OUT_BF16 || MODE == OUT_SWIGLU) ? (void*)((bf16_t*)C + skip) : (void*)((float*)C + skip);
+  return launch_tiled_kernel<MODE>(plan.second, c2, ldc, A, lda, W + (int64_t)plan.n1 * ldw, ldw, M, N - plan.n1, K,
+                                   stream, qkv);
 }
 
 // Up to 16 rows the streaming kernel always wins.  From 17 to 64 rows it re-reads the
@@ -973,6 +1018,18 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                               int64_t ld_emit, float* emit_ss, const float* scale_ss, int scale_blocks,
                               float scale_eps, float* scratch, int64_t scratch_floats, int* counters,
                               int num_counters, hipStream_t stream);
+
+// How an aligned product of more than 64 rows is laid over the tiled kernels when nothing
+// is forced: kernel of the first n1 columns, n1, kernel of the rest (0: none).  For
+// tests and for reading a profile.
+HFEE_API int hfee_gemm_bf16_plan(int M, int N, int K, int* first, int* n1, int* second) {
+  HFEE_REQUIRE(M > 0 && N > 0 && K > 0 && first && n1 && second, "gemm_bf16_plan: bad arguments");
+  const TiledPlan p = plan_tiled(M, N, K, large_fits(K, K, M, N, K), true);
+  *first = p.first;
+  *n1 = p.n1;
+  *second = p.second;
+  return 0;
+}
 
 // out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate (the
 // rows of W alternate gate/up; C is [M, N/2] bfloat16; aligned operands and M > 64 only).

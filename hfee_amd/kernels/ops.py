@@ -142,6 +142,15 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
         raise KernelError(f"linear: unsupported dtype {x.dtype}")
 
 
+def tiled_plan(m: int, n: int, k: int) -> tuple:
+    """(kernel of the first n1 weight rows, n1, kernel of the rest or 0): how `linear`
+    lays an aligned bfloat16 product of more than 64 rows over the tiled kernels."""
+    import ctypes
+    first, n1, second = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    lib.core().call("hfee_gemm_bf16_plan", m, n, k, ctypes.byref(first), ctypes.byref(n1), ctypes.byref(second))
+    return first.value, n1.value, second.value
+
+
 # --------------------------------------------------------- rotation and the cache
 
 def rope_cache_write(q, k, v, positions, token_segment, block_tables, cos, sin, pairing: int,

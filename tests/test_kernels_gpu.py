@@ -131,6 +131,38 @@ def test_gemm_bf16_tiled_large(M, N, K, kernel):
         assert (err <= 2e-2 * (1 + mag[:, 0::2]) * (1 + mag[:, 1::2])).all()
 
 
+def test_gemm_bf16_over_two_launches():
+    """A product whose last round of large tiles would fill a part of the chip only goes
+    to two kernels, split along the weight rows: every epilogue, the seam included."""
+    from hfee_amd.kernels import ops
+    M, N, K = 1024, 24704, 1024
+    first, n1, second = ops.tiled_plan(M, N, K)
+    assert second != 0 and 0 < n1 < N and n1 % 2 == 0, "this shape is meant to be split"
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    ref = x.float() @ w.float().t()                    # (the operands are exact in float32)
+    mag = x.abs().float() @ w.abs().float().t()
+    xd, wd = x.to(DEV), w.to(DEV)
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    ops.linear(out, xd, wd)
+    assert ((out.cpu() - ref).abs() <= 2e-5 * (1 + mag)).all()
+    half = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear(half, xd, wd)
+    assert ((half.float().cpu() - ref).abs() <= 1e-2 * (1 + mag)).all()
+    c0 = torch.randn(M, N, generator=g)
+    acc = c0.clone().to(DEV)
+    ops.linear(acc, xd, wd, accumulate=True)
+    assert ((acc.cpu() - ref - c0).abs() <= 2e-5 * (1 + mag)).all()
+    gated = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear(gated, xd, wd, gate=True)
+    want = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
+    assert ((gated.float().cpu() - want).abs() <= 2e-2 * (1 + mag[:, 0::2]) * (1 + mag[:, 1::2])).all()
+    # the shapes of the benchmark's model: gate/up is split, the others are not
+    assert ops.tiled_plan(2048, 28672, 4096)[2] != 0
+    assert ops.tiled_plan(2048, 4096, 4096)[2] == 0 and ops.tiled_plan(2048, 4096, 14336)[2] == 0
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (8, 344, 96), (16, 100, 256), (3, 16400, 1024), (16, 16500, 2048),
                                    (5, 17000, 4096), (2, 16390, 3072), (33, 200, 128), (64, 52, 1024)])
 @pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu"])
