@@ -212,6 +212,72 @@ __device__ __forceinline__ void store_tile_t(void* C, int64_t ldc, int M, int N,
   }
 }
 
+// The same for a wave's whole TM x TN tiles, through the LDS: a lane holds four
+// consecutive columns of one row, so a store instruction of the plain way writes 16 or
+// 32 bytes each to 32 different rows of C; here a strip of 32 rows is laid down in the
+// wave's own piece of LDS (rows 16 bytes askew) and read back so that 16 bytes a lane
+// make whole rows of C, 256 bytes and more at a time.  For tiles that lie inside C, with
+// rows of C that start 16-byte aligned; the caller has made sure that nobody reads the
+// LDS any more.  lds: the wave's own STAGE_BYTES.
+template <int MODE, int TN>
+struct Stage {
+  static constexpr int ES = (MODE == OUT_BF16 || MODE == OUT_SWIGLU) ? 2 : 4;     // bytes of an element of C
+  static constexpr int OC = MODE == OUT_SWIGLU ? 16 * TN : 32 * TN;              // columns of C in a strip row
+  static constexpr int PITCH = OC * ES + 16;
+  static constexpr int CHUNKS = OC * ES / 16;
+  static constexpr int BYTES = (32 * PITCH + 1023) / 1024 * 1024;
+};
+
+template <int MODE, int TM, int TN>
+__device__ __forceinline__ void store_wave_staged(char* lds, void* C, int64_t ldc, int M, int m_first, int n_first,
+                                                  int lane, const f32x16 (&acc)[TM][TN]) {
+  using S = Stage<MODE, TN>;
+  const int lrow = lane & 31, h = lane >> 5;
+  char* crow = (char*)C + ((int64_t)m_first * ldc + (MODE == OUT_SWIGLU ? n_first / 2 : n_first)) * S::ES;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    char* mine = lds + lrow * S::PITCH;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x16& t = acc[i][j];
+        const float v[4] = {t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+        if constexpr (MODE == OUT_SWIGLU) {
+          const bf16_t o0 = float_to_bf16(v[0] * __frcp_rn(1.0f + __expf(-v[0])) * v[1]);
+          const bf16_t o1 = float_to_bf16(v[2] * __frcp_rn(1.0f + __expf(-v[2])) * v[3]);
+          *reinterpret_cast<uint32_t*>(mine + (j * 16 + 4 * q + 2 * h) * 2) = (uint32_t)o0 | ((uint32_t)o1 << 16);
+        } else if constexpr (MODE == OUT_BF16) {
+          u32x2 o;
+          o[0] = (uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16);
+          o[1] = (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16);
+          *reinterpret_cast<u32x2*>(mine + (j * 32 + 8 * q + 4 * h) * 2) = o;
+        } else {
+          *reinterpret_cast<f32x4*>(mine + (j * 32 + 8 * q + 4 * h) * 4) = f32x4{v[0], v[1], v[2], v[3]};
+        }
+      }
+    // (the same wave wrote what it reads: its LDS instructions keep their order)
+    constexpr int PIECES = 32 * S::CHUNKS / 64;            // 16-byte pieces of the strip per lane
+    static_assert(32 * S::CHUNKS % 64 == 0, "a strip is a whole number of pieces per lane");
+    f32x4* dst[PIECES];
+    f32x4 old[PIECES];
+#pragma unroll
+    for (int it = 0; it < PIECES; ++it) {
+      const int idx = lane + 64 * it, row = idx / S::CHUNKS, c = idx - row * S::CHUNKS;
+      dst[it] = m_first + i * 32 + row < M
+                    ? reinterpret_cast<f32x4*>(crow + (int64_t)(i * 32 + row) * ldc * S::ES + c * 16) : nullptr;
+      // what is added to: every piece asked for before the first is needed
+      if (MODE == OUT_ADD_F32 && dst[it]) old[it] = *dst[it];
+    }
+#pragma unroll
+    for (int it = 0; it < PIECES; ++it) {
+      const int idx = lane + 64 * it, row = idx / S::CHUNKS, c = idx - row * S::CHUNKS;
+      const f32x4 piece = *reinterpret_cast<const f32x4*>(lds + row * S::PITCH + c * 16);
+      if (dst[it]) *dst[it] = MODE == OUT_ADD_F32 ? old[it] + piece : piece;
+    }
+  }
+}
+
 // The q/k/v epilogue for a wave's TM x TN tiles of transposed 32 x 32 products: what
 // belongs to a row (position, page, slot) is fetched once per row, what belongs to four
 // columns (head, place in the head, q or k or v) once per four columns.
@@ -477,8 +543,10 @@ struct Interleave<OTHER, N, R, N> {
 //    matrix instructions.  Four LDS buffers of one K step each: a step is asked from
 //    memory three steps before it is multiplied.
 //  * A 1 KB block is 16 tile rows of 64 bytes, unpadded; the four 16-byte chunks of row
-//    r are stored in the order c ^ f(r), f(r) = ((r >> 1) ^ (r >> 3)) & 3, which keeps
-//    the 16-byte operand reads of 8 or 16 consecutive rows on distinct banks.
+//    r are stored in the order c ^ f(r), f(r) = bit 3 of r | bit 2 of r << 1: of the
+//    functions whose bits are parities of row bits, the hardware's conflict counter
+//    showed none for this one on a wave's 16-byte operand reads (rows lane % 32, chunks
+//    2 ks + lane / 32), and two-way conflicts for e.g. ((r >> 1) ^ (r >> 3)) & 3.
 //  * The one barrier of a step stands where the wave has nothing outstanding in the LDS,
 //    and carries no fence (a fence would wait for every load in flight); what must have
 //    landed is waited for by count.
@@ -498,7 +566,7 @@ __device__ __forceinline__ void barrier_no_fence() {
   asm volatile("" ::: "memory");
 }
 
-__device__ __forceinline__ uint32_t swizzle(uint32_t row) { return ((row >> 1) ^ (row >> 3)) & 3u; }
+__device__ __forceinline__ uint32_t swizzle(uint32_t row) { return ((row >> 3) & 1u) | ((row >> 1) & 2u); }
 
 template <int MODE, int TM, int TN>
 __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict__ C, int64_t ldc,
@@ -625,11 +693,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
   if constexpr (MODE == OUT_QKV) {
     store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
   } else {
+    using S = Stage<MODE, TN>;
+    static_assert(4 * S::BYTES <= 4 * BUF, "the waves' strips fit in the LDS of the buffers");
+    __syncthreads();      // nobody reads operands from the LDS any more
+    const bool whole_rows = (ldc * S::ES) % 16 == 0 && (uintptr_t)C % 16 == 0 && n0 + wn * 32 * TN + 32 * TN <= N;
+    if (whole_rows) {
+      store_wave_staged<MODE, TM, TN>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
+    } else {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+        for (int j = 0; j < TN; ++j)
+          store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+    }
   }
 #endif
 }
@@ -787,11 +863,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
   if constexpr (MODE == OUT_QKV) {
     store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
   } else {
+    using S = Stage<MODE, TN>;
+    static_assert(4 * S::BYTES <= NBUF * BUF, "the waves' strips fit in the LDS of the buffers");
+    __syncthreads();      // nobody reads operands from the LDS any more
+    const bool whole_rows = (ldc * S::ES) % 16 == 0 && (uintptr_t)C % 16 == 0 && n0 + wn * 32 * TN + 32 * TN <= N;
+    if (whole_rows) {
+      store_wave_staged<MODE, TM, TN>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
+    } else {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+        for (int j = 0; j < TN; ++j)
+          store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+    }
   }
 #endif
 }
