@@ -53,6 +53,9 @@ def main() -> int:
     ap.add_argument("--serving", type=int, default=0, metavar="R",
                     help="instead of the default run: R requests at once under continuous batching, prompts of "
                          "64 to 2,048 tokens, 128 new tokens each, context 4,096; prints its own line")
+    ap.add_argument("--context", type=int, default=0, metavar="T",
+                    help="instead of the default run: a prompt of T tokens in portions of 2,048, then decode "
+                         "steps at that context with --batch requests; prints its own line")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own short line")
     args = ap.parse_args()
@@ -89,6 +92,13 @@ def main() -> int:
     if args.serving:
         context = min(context, 4096)
         tokens_cached = args.serving * (2048 + 128 + page_size)
+    if args.context:
+        # the first requests go on decoding while the later ones run their prompts
+        context = args.context + args.batch * (args.context // PREFILL + 2) + steps_total + page_size
+        if context > base["max_position_embeddings"]:
+            print(f"bench.py: --context {args.context} is beyond what the shape allows")
+            return 2
+        tokens_cached = args.batch * (context + page_size)
     engine = Engine(model, cache_tokens=tokens_cached, page_size=page_size, max_requests=max_batch,
                     max_batch_tokens=PREFILL, num_positions=context)
     sampler = Sampler(V, engine.device, max_rows=max_batch)
@@ -166,6 +176,54 @@ def main() -> int:
             "config": {"model": SHAPE_NAMES[args.shape] + "-shaped", "layers": L, "requests": args.serving,
                        "prompt_tokens_total": prompt_tokens, "generated_total": made, "seq_len": context,
                        "max_batch_tokens": PREFILL, "page_size": page_size}}), flush=True)
+        return 0
+
+    def context_run(batch: int, tokens: int, steps: int, warmup: int):
+        """Prompts of `tokens` tokens, the first one timed alone (portions of 2,048 tokens
+        each attend to all that came before), then decode steps at that context."""
+        sched = Scheduler(engine, sampler, max_num_seqs=batch, max_batch_tokens=PREFILL, num_ctx=context)
+        params = SamplingParams.greedy(num_predict=-1, ignore_eos=True)
+        sched.add(Request(("context", 0), torch.randint(0, V, (tokens,), generator=gen).tolist(), params, seed=0))
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        while not sched.running or not sched.running[0].decoding:
+            sched.step()
+        torch.cuda.synchronize()
+        prefill_s = time.perf_counter() - t
+        for i in range(1, batch):
+            sched.add(Request(("context", i), torch.randint(0, V, (tokens,), generator=gen).tolist(), params, seed=i))
+        while any(not r.decoding for r in list(sched.running) + list(sched.waiting)):
+            sched.step()
+        for _ in range(warmup):
+            sched.step()
+        before = sum(len(r.generated) for r in sched.running)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            sched.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        made = sum(len(r.generated) for r in sched.running) - before
+        lengths = [engine.cached_length(r.request_id) for r in sched.running]
+        assert made == batch * steps and len(lengths) == batch and min(lengths) >= tokens, (made, lengths)
+        for r in list(sched.running):
+            sched.cancel(r.request_id)
+        sched.step()
+        return prefill_s, dt
+
+    if args.context:
+        prefill_s, dt = context_run(args.batch, args.context, args.steps, args.warmup)
+        T = args.context
+        flops = 2.0 * T * (L * layer_params) + 2.0 * V * d + L * 4.0 * hd * H * T * (T + 1) / 2
+        step_bytes = weight_bytes + args.batch * (T + args.warmup + args.steps / 2) * kv_bytes_per_token
+        print(json.dumps({
+            "metric": "prefill and decode at a context of %d tokens (%s bf16)" % (T, SHAPE_NAMES[args.shape]),
+            "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 2),
+                        "frac": round(flops / prefill_s / BF16_PEAK, 4)},
+            "decode": {"value": round(args.batch * args.steps / dt, 1), "batch": args.batch,
+                       "ms_per_step": round(dt / args.steps * 1e3, 3),
+                       "hbm_frac": round(step_bytes / (dt / args.steps) / HBM_PEAK, 4)},
+            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": L}), flush=True)
         return 0
 
     if args.prefill_only:

@@ -156,15 +156,17 @@ __device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyO
       tile_max = fmaxf(tile_max, s[r]);
     }
   }
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64)) * scale_log2;
+  tile_max *= scale_log2;          // (of this lane's half of the slot's keys)
   // st.m is the reference that the exponentials are taken against, not always the exact
   // maximum: it moves (and the sums are rescaled) only when some slot's scores rise more
   // than SLACK above it, for every slot of the wave at once.  Below that the terms are at
   // most 2^SLACK, which float32 sums and bfloat16 factors hold as well as terms below 1;
   // the quotient o / l does not depend on the reference.  After the first tiles a
-  // maximum seldom moves that far, so the rescaling of O is rare.
+  // maximum seldom moves that far, so the rescaling of O is rare, and only then do the
+  // two lanes of a slot have to agree on the maximum.
   constexpr float SLACK = 8.0f;
   if (__builtin_amdgcn_ballot_w64(tile_max > st.m + SLACK) != 0) {
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
     const float m_new = fmaxf(st.m, tile_max);
     // 2^x by the hardware instruction alone: its arguments here are <= 0, and a result
     // too small for a normal number may become zero
@@ -185,8 +187,7 @@ __device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyO
     psum += e;
     p[r >> 3].e[r & 7] = float_to_bf16(e);
   }
-  psum += __shfl_xor(psum, 32, 64);
-  st.l += psum;
+  st.l += psum;          // this lane's half of the slot's keys: the halves meet in finish_sum
 
   // ---- O^T += V^T P^T ----------------------------------------------------------
 #pragma unroll
@@ -242,6 +243,9 @@ __device__ __forceinline__ void load_query(Op* q_op, const bf16_t* __restrict__ 
   }
 }
 
+// The sum of a slot's terms: each of its two lanes has added up its own half of the keys.
+__device__ __forceinline__ float finish_sum(const Tile& st) { return st.l + __shfl_xor(st.l, 32, 64); }
+
 __device__ __forceinline__ void init_tile(Tile& st) {
   st.m = -INFINITY;
   st.l = 0.f;
@@ -294,8 +298,9 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
   attend_tiles<false>(st, q_op, cache, lay, bt, bt_stride, kvh, kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
                scale_log2, window > 0 ? max(0, kv_last - window + 1) : 0, pos0);
 
+  const float l_slot = finish_sum(st);
   if (slot_ok) {
-    const float inv = 1.0f / st.l;
+    const float inv = 1.0f / l_slot;
     bf16_t* orow = out + (int64_t)(row0 + r32) * ld_out + h * HD;
 #pragma unroll
     for (int t = 0; t < NDT; ++t)
@@ -380,7 +385,76 @@ __device__ __forceinline__ void request_tile(char* __restrict__ tile_lds, const 
   }
 }
 
+// The same request when the number of waves is known at compile time: which blocks a
+// wave brings, and from where in a page each of its lanes reads them, never changes, so
+// it is worked out once (WaveBlocks).  A tile of 32 keys lies in at most two pages (of its
+// first and of its last 16 keys); their numbers come out of the page window as scalars,
+// and a request is a choice between two bases, an addition and the load: no branch, no
+// shuffle, no multiplication per lane.
+template <int WAVES>
+struct WaveBlocks {
+  static constexpr int J = (KV_BLOCKS + WAVES - 1) / WAVES;
+  int count;                 // blocks of this wave
+  uint32_t lane_off[J];      // this lane's bytes from the start of a page
+  bool second[J];            // this lane reads the page of the tile's last 16 keys
+  int kind[J];               // 0 keys, 1 values of the first 16 keys, 2 values of the last 16 keys
+};
+
+template <int WAVES>
+__device__ __forceinline__ WaveBlocks<WAVES> wave_blocks(const CacheLayout& lay, int kvh, int wave) {
+  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+  WaveBlocks<WAVES> w;
+  w.count = 0;
+#pragma unroll
+  for (int j = 0; j < WaveBlocks<WAVES>::J; ++j) {
+    const int b = min(wave + WAVES * j, KV_BLOCKS - 1);
+    if (wave + WAVES * j < KV_BLOCKS) w.count = j + 1;
+    if (b < NC) {
+      w.kind[j] = 0;
+      w.second[j] = r32 >= 16;
+      w.lane_off[j] = (uint32_t)((lay.key_offset(0, kvh, r32 & (lay.page_size - 1), 0) + b * 16 + G * 8) * 2);
+    } else {
+      const int u = (b - NC) / NDT, t = (b - NC) % NDT;
+      w.kind[j] = 1 + u;
+      w.second[j] = u != 0;
+      // rows beyond the head repeat its last one
+      w.lane_off[j] = (uint32_t)((lay.value_column(0, kvh, min(32 * t + r32, HD - 1)) + 8 * G) * 2);
+    }
+  }
+  return w;
+}
+
+template <int WAVES>
+__device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds, const bf16_t* __restrict__ cache,
+                                                    const CacheLayout& lay, const WaveBlocks<WAVES>& w,
+                                                    const int* __restrict__ bt, int bt_stride, PageWindow& pages,
+                                                    int k0, int kv_first, int kv_last, int wave) {
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  typedef const __attribute__((address_space(1))) void* global_ptr;
+  const int block_a = k0 >> lay.page_shift, block_b = (k0 + 16) >> lay.page_shift;
+  if (pages.base < 0 || block_a < pages.base || block_b >= pages.base + 64) pages.fill(bt, bt_stride, block_a);
+  // pages outside kv_first..kv_last may have been given back: page 0 is read instead
+  const bool ok_a = k0 <= kv_last && k0 + 15 >= kv_first, ok_b = k0 + 16 <= kv_last && k0 + 31 >= kv_first;
+  const int page_a = ok_a ? __builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_a - pages.base)) : 0;
+  const int page_b = ok_b ? __builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_b - pages.base)) : 0;
+  const char* base_a = (const char*)cache + (int64_t)page_a * lay.page_stride * 2;
+  const char* base_b = (const char*)cache + (int64_t)page_b * lay.page_stride * 2;
+  const int in_page = k0 & (lay.page_size - 1);
+  // what the tile's place in its page adds: rows of keys, slots of values
+  const uint32_t add[3] = {(uint32_t)(in_page * lay.head_dim * 2), (uint32_t)(in_page * 2),
+                           (uint32_t)(((k0 + 16) & (lay.page_size - 1)) * 2)};
+#pragma unroll
+  for (int j = 0; j < WaveBlocks<WAVES>::J; ++j) {
+    if (KV_BLOCKS % WAVES == 0 || j < w.count) {
+      const char* src = (w.second[j] ? base_b : base_a) + (w.lane_off[j] + (w.kind[j] == 0 ? add[0] : w.kind[j] == 1 ? add[1] : add[2]));
+      __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)(tile_lds + (wave + WAVES * j) * 1024), 16, 0, 0);
+    }
+  }
+}
+
 // work: per row tile 4 ints (first row, rows <= 32, first position, block-table row).
+// WAVES: the waves of a workgroup if they are SHARED_WAVES, 0 for any other number.
+template <int WAVES>
 __global__ __launch_bounds__(SHARED_WAVES * 64) void prefill_shared_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, CacheLayout lay, const int* __restrict__ work, int num_tiles,
@@ -423,13 +497,17 @@ __global__ __launch_bounds__(SHARED_WAVES * 64) void prefill_shared_kernel(
   pages.base = -1;
   constexpr int TILE_BYTES = KV_BLOCKS * 1024;
   const LaneOffsets off = lane_offsets(lay, kvh);
-  request_tile(kv_lds, cache, lay, off, bt, bt_stride, pages, t_first * 32, kv_first, kv_last, wave, waves);
+  const WaveBlocks<WAVES == 0 ? 1 : WAVES> mine = wave_blocks<WAVES == 0 ? 1 : WAVES>(lay, kvh, wave);
+  auto request = [&](int t) {
+    char* dst = kv_lds + ((t - t_first) & 1) * TILE_BYTES;
+    if constexpr (WAVES != 0) request_wave_blocks<WAVES>(dst, cache, lay, mine, bt, bt_stride, pages, t * 32, kv_first, kv_last, wave);
+    else request_tile(dst, cache, lay, off, bt, bt_stride, pages, t * 32, kv_first, kv_last, wave, waves);
+  };
+  request(t_first);
   __syncthreads();               // waits for the loads too
   for (int t = t_first; t < t_end; ++t) {
     const char* cur = kv_lds + ((t - t_first) & 1) * TILE_BYTES + lane * 16;
-    if (t + 1 < t_end)
-      request_tile(kv_lds + ((t + 1 - t_first) & 1) * TILE_BYTES, cache, lay, off, bt, bt_stride, pages, (t + 1) * 32,
-                   kv_first, kv_last, wave, waves);
+    if (t + 1 < t_end) request(t + 1);
     compute_tile_with(
         st, q_op, [&](int c) { return *reinterpret_cast<const bf16x8*>(cur + c * 1024); },
         [&](int u, int tt) { return *reinterpret_cast<const bf16x8*>(cur + (NC + u * NDT + tt) * 1024); }, t * 32, pos, lo,
@@ -437,8 +515,9 @@ __global__ __launch_bounds__(SHARED_WAVES * 64) void prefill_shared_kernel(
     __syncthreads();             // the next tile has landed; nobody reads this one any more
   }
 
+  const float l_slot = finish_sum(st);
   if (slot_ok) {
-    const float inv = 1.0f / st.l;
+    const float inv = 1.0f / l_slot;
     bf16_t* orow = out + (int64_t)(row0 + r32) * ld_out + h * HD;
 #pragma unroll
     for (int t = 0; t < NDT; ++t)
@@ -543,6 +622,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
                  scale_log2, lo, pos);
 
     // this wave's state into LDS
+    const float l_slot = finish_sum(st);
     if (g0 > 0) __syncthreads();
     if (slot_ok) {
       float* mine = lds + (int64_t)(wave * slots + r32) * (HD + 2);
@@ -555,7 +635,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
         }
       if (G == 0) {
         mine[HD] = st.m;
-        mine[HD + 1] = st.l;
+        mine[HD + 1] = l_slot;
       }
     }
     __syncthreads();
@@ -670,15 +750,23 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
     const size_t lds = (size_t)2 * KV_BLOCKS * 1024;
     static bool raised = false;
     if (lds > 48 * 1024 && !raised) {
-      hipError_t e = hipFuncSetAttribute((const void*)prefill_shared_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+      hipError_t e = hipFuncSetAttribute((const void*)prefill_shared_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                          (int)lds);
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute((const void*)prefill_shared_kernel<SHARED_WAVES>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       HFEE_REQUIRE(e == hipSuccess, "attention_bf16_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
       raised = true;
     }
     dim3 grid((unsigned)(((int64_t)num_tiles * kv_heads * chunks + 7) / 8 * 8));
-    prefill_shared_kernel<<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
-                                                             (const bf16_t*)cache, lay, work, num_tiles, block_tables,
-                                                             bt_stride, num_heads, scale * LOG2E, window);
+    if (waves == SHARED_WAVES)
+      prefill_shared_kernel<SHARED_WAVES><<<grid, waves * 64, lds, stream>>>(
+          (bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, work, num_tiles, block_tables, bt_stride,
+          num_heads, scale * LOG2E, window);
+    else
+      prefill_shared_kernel<0><<<grid, waves * 64, lds, stream>>>(
+          (bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, work, num_tiles, block_tables, bt_stride,
+          num_heads, scale * LOG2E, window);
   }
   HFEE_CHECK_LAUNCH("attention_bf16_prefill");
   return 0;

@@ -433,6 +433,17 @@ def _paged(kv, page_size, pages_order):
 def test_attention_kernels(H, K, hd, T, window, dtype):
     """Plain kernel (both dtypes) and the matrix-core kernels (bfloat16) against
     the reference formula, on pages in scrambled order."""
+    _check_attention(H, K, hd, T, window, dtype, 16)
+
+
+@pytest.mark.parametrize("H,K,hd,T,window,ps", [(4, 1, 128, 130, 0, 32), (8, 2, 64, 150, 40, 64), (4, 1, 48, 300, 0, 128),
+                                                (16, 2, 32, 97, 50, 32)])
+def test_attention_kernels_with_larger_pages(H, K, hd, T, window, ps):
+    """The same with pages of 32, 64 and 128 slots (a tile of 32 keys then lies in one page)."""
+    _check_attention(H, K, hd, T, window, torch.bfloat16, ps)
+
+
+def _check_attention(H, K, hd, T, window, dtype, ps):
     from plain_llama import plain_attention
     from hfee_amd.kernels import ops
     g = torch.Generator().manual_seed(H * 100 + hd + T)
@@ -441,7 +452,6 @@ def test_attention_kernels(H, K, hd, T, window, dtype):
     v = torch.randn(T, K, hd, generator=g).to(dtype)
     scale = 1 / math.sqrt(hd)
     ref = plain_attention(q, k, v, scale, window=window).reshape(T, H * hd)
-    ps = 16
     nblocks = (T + ps - 1) // ps
     order = torch.randperm(nblocks + 5, generator=g)[:nblocks].tolist()
     layer, table = _paged((k, v), ps, order)
