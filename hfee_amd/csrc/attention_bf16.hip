@@ -82,43 +82,50 @@ struct PageWindow {
   __device__ __forceinline__ int of(int block) const { return __shfl(page, block - base, 64); }
 };
 
-// Issues every load of the tile k0 .. k0+31.  kv_first..kv_last: the keys whose pages
-// may be touched at all (a window group has given back the pages before kv_first;
-// nothing exists after kv_last); the rest reads as zeros.
-__device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict__ cache, const CacheLayout& lay,
-                                          const int* __restrict__ bt, int bt_stride, PageWindow& pages, int kvh,
-                                          int k0, int kv_first, int kv_last) {
+// What of a lane's addresses does not change from tile to tile (in elements from the
+// start of a page): the tile adds the page and a uniform slot offset.
+struct LaneOffsets {
+  int64_t key;              // this lane's key row within a page (k0 % page_size == 0), its half of a chunk
+  int64_t value[NDT];       // this lane's value column of each 32-wide part of the head, its half of the slots
+};
+
+__device__ __forceinline__ LaneOffsets lane_offsets(const CacheLayout& lay, int kvh) {
   const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
-  {
-    // the tile's blocks (uniform over the wave): refill the window when the tile leaves it
-    const int b0 = k0 >> lay.page_shift, b1 = (k0 + 31) >> lay.page_shift;
-    if (pages.base < 0 || b0 < pages.base || b1 >= pages.base + 64) pages.fill(bt, bt_stride, b0);
-  }
-  {
-    const int key = k0 + r32;
-    const bool ok = key <= kv_last && key >= kv_first;
-    const int page = pages.of(key >> lay.page_shift);
-    const bf16_t* krow = ok ? cache + lay.key_offset(page, kvh, key & (lay.page_size - 1), 0) : cache;
+  LaneOffsets o;
+  o.key = lay.key_offset(0, kvh, r32 & (lay.page_size - 1), 0) + G * 8;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      ops.k[c].u = u32x4{0u, 0u, 0u, 0u};
-      if (ok) ops.k[c].u = *reinterpret_cast<const u32x4*>(krow + c * 16 + G * 8);
-    }
-  }
+  for (int t = 0; t < NDT; ++t)
+    o.value[t] = lay.value_column(0, kvh, min(32 * t + r32, HD - 1)) + 8 * G;   // rows beyond the head repeat its last one
+  return o;
+}
+
+// Issues every load of the tile k0 .. k0+31 into registers.  kv_first..kv_last: the keys
+// whose pages may be touched at all (a window group has given back the pages before
+// kv_first; nothing exists after kv_last): a page without such a key is replaced by page
+// 0.  What is read beside the keys that a slot sees is masked or multiplied by zero (the
+// cache never holds anything but finite numbers).  The tile lies in at most two pages;
+// their numbers are scalars out of the page window, and a lane's address is one of two
+// bases plus what lane_offsets worked out once.
+__device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict__ cache, const CacheLayout& lay,
+                                          const LaneOffsets& off, const int* __restrict__ bt, int bt_stride,
+                                          PageWindow& pages, int k0, int kv_first, int kv_last) {
+  const int r32 = threadIdx.x & 31;
+  const int block_a = k0 >> lay.page_shift, block_b = (k0 + 16) >> lay.page_shift;
+  if (pages.base < 0 || block_a < pages.base || block_b >= pages.base + 64) pages.fill(bt, bt_stride, block_a);
+  const bool ok_a = k0 <= kv_last && k0 + 15 >= kv_first, ok_b = k0 + 16 <= kv_last && k0 + 31 >= kv_first;
+  const int page_a = ok_a ? __builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_a - pages.base)) : 0;
+  const int page_b = ok_b ? __builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_b - pages.base)) : 0;
+  const bf16_t* base_a = cache + (int64_t)page_a * lay.page_stride;
+  const bf16_t* base_b = cache + (int64_t)page_b * lay.page_stride;
+  const int in_page = k0 & (lay.page_size - 1);
+  const bf16_t* krow = (r32 < 16 ? base_a : base_b) + off.key + in_page * lay.head_dim;
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int kb = k0 + 16 * u;
-    const bool ok = kb <= kv_last && kb + 15 >= kv_first;
-    const int page = pages.of(kb >> lay.page_shift);
-    const int first = (kb & (lay.page_size - 1)) + 8 * G;      // stored order: 4G.., 8+4G.. are adjacent
+  for (int c = 0; c < NC; ++c) ops.k[c].u = *reinterpret_cast<const u32x4*>(krow + c * 16);
+  const bf16_t* vbase[2] = {base_a + in_page, base_b + ((k0 + 16) & (lay.page_size - 1))};
 #pragma unroll
-    for (int t = 0; t < NDT; ++t) {
-      const int d = 32 * t + r32;
-      ops.v[u][t].u = u32x4{0u, 0u, 0u, 0u};
-      if (ok && d < HD)
-        ops.v[u][t].u = *reinterpret_cast<const u32x4*>(cache + lay.value_column(page, kvh, d) + first);
-    }
-  }
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int t = 0; t < NDT; ++t) ops.v[u][t].u = *reinterpret_cast<const u32x4*>(vbase[u] + off.value[t]);
 }
 
 // Adds the keys k0 .. k0+31 to the running state.  q_op: this slot's query, pre-loaded
@@ -211,24 +218,24 @@ __device__ __forceinline__ void compute_tile(Tile& st, const Op* q_op, const Til
 template <bool AHEAD>
 __device__ __forceinline__ void attend_tiles(Tile& st, const Op* q_op, const bf16_t* __restrict__ cache,
                                              const CacheLayout& lay, const int* __restrict__ bt, int bt_stride,
-                                             int kvh, int first, int end, int step, int kv_first, int kv_last,
+                                             const LaneOffsets& off, int first, int end, int step, int kv_first, int kv_last,
                                              int pos, int lo, float scale_log2, int all_first, int all_last) {
   if (first >= end) return;
   PageWindow pages;
   pages.base = -1;
   if constexpr (AHEAD) {
     TileOps cur, nxt;
-    load_tile(cur, cache, lay, bt, bt_stride, pages, kvh, first * 32, kv_first, kv_last);
+    load_tile(cur, cache, lay, off, bt, bt_stride, pages, first * 32, kv_first, kv_last);
     for (int t = first; t < end; t += step) {
       const int tn = t + step;
-      if (tn < end) load_tile(nxt, cache, lay, bt, bt_stride, pages, kvh, tn * 32, kv_first, kv_last);
+      if (tn < end) load_tile(nxt, cache, lay, off, bt, bt_stride, pages, tn * 32, kv_first, kv_last);
       compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2, t * 32 >= all_first && t * 32 + 31 <= all_last);
       cur = nxt;
     }
   } else {
     for (int t = first; t < end; t += step) {
       TileOps cur;
-      load_tile(cur, cache, lay, bt, bt_stride, pages, kvh, t * 32, kv_first, kv_last);
+      load_tile(cur, cache, lay, off, bt, bt_stride, pages, t * 32, kv_first, kv_last);
       compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2, t * 32 >= all_first && t * 32 + 31 <= all_last);
     }
   }
@@ -295,7 +302,7 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
   const int kv_last = pos0 + rows - 1;
   const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
   // every row in use sees the keys from the last row's window start to the first row's position
-  attend_tiles<false>(st, q_op, cache, lay, bt, bt_stride, kvh, kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
+  attend_tiles<false>(st, q_op, cache, lay, bt, bt_stride, lane_offsets(lay, kvh), kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
                scale_log2, window > 0 ? max(0, kv_last - window + 1) : 0, pos0);
 
   const float l_slot = finish_sum(st);
@@ -329,23 +336,6 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
 // but finite numbers, so a masked value times zero is zero).
 constexpr int KV_BLOCKS = NC + 2 * NDT;           // 1 KB blocks of one key tile: keys, then values
 constexpr int SHARED_WAVES = 4;
-
-// What of a lane's addresses does not change from tile to tile (in elements from the
-// start of a page): the tile adds the page and a uniform slot offset.
-struct LaneOffsets {
-  int64_t key;              // this lane's key row within a page (k0 % page_size == 0), its half of a chunk
-  int64_t value[NDT];       // this lane's value column of each 32-wide part of the head, its half of the slots
-};
-
-__device__ __forceinline__ LaneOffsets lane_offsets(const CacheLayout& lay, int kvh) {
-  const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
-  LaneOffsets o;
-  o.key = lay.key_offset(0, kvh, r32 & (lay.page_size - 1), 0) + G * 8;
-#pragma unroll
-  for (int t = 0; t < NDT; ++t)
-    o.value[t] = lay.value_column(0, kvh, min(32 * t + r32, HD - 1)) + 8 * G;   // rows beyond the head repeat its last one
-  return o;
-}
 
 __device__ __forceinline__ void request_tile(char* __restrict__ tile_lds, const bf16_t* __restrict__ cache,
                                              const CacheLayout& lay, const LaneOffsets& off,
@@ -611,6 +601,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
   const int t_begin = tile_first + split * per;
   const int t_end = min(tile_first + tile_count, t_begin + per);
 
+  const LaneOffsets off = lane_offsets(lay, kvh);
   for (int g0 = 0; g0 < group; g0 += 32) {
     const bool slot_ok = g0 + r32 < group;
     const int h = kvh * group + g0 + (slot_ok ? r32 : 0);
@@ -618,7 +609,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
     load_query(q_op, q + (int64_t)row * ldq + h * HD, slot_ok);
     Tile st;
     init_tile(st);
-    attend_tiles<true>(st, q_op, cache, lay, bt, bt_stride, kvh, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
+    attend_tiles<true>(st, q_op, cache, lay, bt, bt_stride, off, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
                  scale_log2, lo, pos);
 
     // this wave's state into LDS
