@@ -427,8 +427,11 @@ __device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds,
   const bool ok_a = k0 <= kv_last && k0 + 15 >= kv_first, ok_b = k0 + 16 <= kv_last && k0 + 31 >= kv_first;
   const int page_a = ok_a ? __builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_a - pages.base)) : 0;
   const int page_b = ok_b ? __builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_b - pages.base)) : 0;
-  const char* base_a = (const char*)cache + (int64_t)page_a * lay.page_stride * 2;
-  const char* base_b = (const char*)cache + (int64_t)page_b * lay.page_stride * 2;
+  // (the two pages' byte offsets as scalars that the compiler takes as given: it would
+  // otherwise choose between the page numbers per lane and multiply in every lane)
+  const uint64_t bytes_a = (uint64_t)page_a * (uint64_t)lay.page_stride * 2, bytes_b = (uint64_t)page_b * (uint64_t)lay.page_stride * 2;
+  const uint32_t a_lo = __builtin_amdgcn_readfirstlane((uint32_t)bytes_a), a_hi = __builtin_amdgcn_readfirstlane((uint32_t)(bytes_a >> 32));
+  const uint32_t b_lo = __builtin_amdgcn_readfirstlane((uint32_t)bytes_b), b_hi = __builtin_amdgcn_readfirstlane((uint32_t)(bytes_b >> 32));
   const int in_page = k0 & (lay.page_size - 1);
   // what the tile's place in its page adds: rows of keys, slots of values
   const uint32_t add[3] = {(uint32_t)(in_page * lay.head_dim * 2), (uint32_t)(in_page * 2),
@@ -436,7 +439,8 @@ __device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds,
 #pragma unroll
   for (int j = 0; j < WaveBlocks<WAVES>::J; ++j) {
     if (KV_BLOCKS % WAVES == 0 || j < w.count) {
-      const char* src = (w.second[j] ? base_b : base_a) + (w.lane_off[j] + (w.kind[j] == 0 ? add[0] : w.kind[j] == 1 ? add[1] : add[2]));
+      const uint64_t page_bytes = ((uint64_t)(w.second[j] ? b_hi : a_hi) << 32) | (w.second[j] ? b_lo : a_lo);
+      const char* src = (const char*)cache + page_bytes + (w.lane_off[j] + (w.kind[j] == 0 ? add[0] : w.kind[j] == 1 ? add[1] : add[2]));
       __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)(tile_lds + (wave + WAVES * j) * 1024), 16, 0, 0);
     }
   }
