@@ -363,11 +363,20 @@ struct PStage {
   u32x4 a[2 * TM], w[2 * TN];      // this thread's 16-byte chunks of the A tile and of the W tile
 };
 
+// The second half of a norm whose first half the product before has done (gemm_skinny.hip,
+// ROW SCALE), for products of at most 64 rows: every row of the result is scaled by
+// 1/sqrt(sum of the row's shares / K + eps).  shares null: no scaling.
+struct RowScale {
+  const float* shares;      // [blocks][64]
+  int blocks;
+  float eps;
+};
+
 template <int MODE, int TM, int TN, int STAGES>
 __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restrict__ C, int64_t ldc,
                                                                   const bf16_t* __restrict__ A, int64_t lda,
                                                                   const bf16_t* __restrict__ W, int64_t ldw,
-                                                                  int M, int N, int K, QkvArgs qkv) {
+                                                                  int M, int N, int K, QkvArgs qkv, RowScale rs) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
   extern __shared__ __attribute__((aligned(16))) bf16_t lds_tiles[];
   auto a_tile = [&](int buf) { return lds_tiles + buf * (BM * PPITCH); };
@@ -433,8 +442,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
   PStage<TM, TN> ring[STAGES];
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) load_stage(ring[s], s);
+  // the rows' scales (at most 64 rows, so m0 == 0), behind the first loads of the tiles:
+  // thread -> row tid % 64, every fourth share
+  __shared__ float row_scale[64];
+  __shared__ float row_scale_part[4][64];
+  if (rs.shares != nullptr) {
+    const int row = min(tid & 63, M - 1), q4 = tid >> 6;
+    float t = 0.f;
+#pragma unroll 8
+    for (int b = q4; b < rs.blocks; b += 4) t += rs.shares[(int64_t)b * 64 + row];
+    row_scale_part[q4][tid & 63] = t;
+  }
   store_stage(ring[0], 0, inside(0));
   __syncthreads();
+  if (rs.shares != nullptr && tid < 64)      // (read after the barriers of the loop below, or the one before the stores)
+    row_scale[tid] = 1.0f / sqrtf((((row_scale_part[0][tid] + row_scale_part[1][tid]) + row_scale_part[2][tid]) +
+                                   row_scale_part[3][tid]) / (float)K + rs.eps);
 
   const int lrow = lane & 31, lk = (lane >> 5) * 8;
   auto step = [&](auto slot_c, auto last_c, int kt) {
@@ -485,6 +508,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
   if constexpr (MODE == OUT_QKV) {
     store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
   } else {
+    if (rs.shares != nullptr) {
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const float scale = row_scale[min(wm * 32 * TM + i * 32 + lrow, 63)];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] *= scale;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -495,7 +529,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
 
 template <int MODE>
 int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                     int M, int N, int K, const QkvArgs& qkv, hipStream_t stream) {
+                     int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, const RowScale& rs = RowScale{}) {
   // 128 x 128 tiles, two workgroups per CU.  (128 x 256 tiles halve the LDS reads per
   // matrix instruction but leave one wave per SIMD, and measured 20 % slower.)
   constexpr int TM = 2, TN = 2, STAGES = 3;
@@ -510,7 +544,7 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
   const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
   if (tiles > (1 << 30)) return fail("gemm_bf16: too many tiles");
   dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
-  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv);
+  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv, rs);
   return 0;
 }
 
@@ -1102,6 +1136,33 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                               int64_t ld_emit, float* emit_ss, const float* scale_ss, int scale_blocks,
                               float scale_eps, float* scratch, int64_t scratch_floats, int* counters,
                               int num_counters, hipStream_t stream);
+
+// The tiled product of at most 64 rows whose result rows are scaled by the second half of
+// a norm (see RowScale): for shapes that are too wide for the streaming kernels.
+// out_mode as hfee_gemm_bf16; operands aligned as for the tiled kernels.
+HFEE_API int hfee_gemm_bf16_scaled(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
+                                   int64_t ldw, int M, int N, int K, const float* shares, int blocks, float eps,
+                                   hipStream_t stream) {
+  HFEE_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_bf16_scaled: 1 to 64 rows, got M=%d N=%d K=%d", M, N, K);
+  HFEE_REQUIRE(out_mode >= 0 && out_mode <= 3, "gemm_bf16_scaled: unknown output mode %d", out_mode);
+  HFEE_REQUIRE(shares != nullptr && blocks > 0 && eps >= 0.f, "gemm_bf16_scaled: no shares");
+  HFEE_REQUIRE((K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) &&
+                   lda >= K && ldw >= K,
+               "gemm_bf16_scaled: K and the leading dimensions must be multiples of 8 and the operands 16-byte aligned");
+  HFEE_REQUIRE(out_mode != 3 || N % 2 == 0, "gemm_bf16_scaled: the SiLU gate needs an even N");
+  HFEE_REQUIRE(ldc >= (out_mode == 3 ? N / 2 : N), "gemm_bf16_scaled: ldc is shorter than a row of the result");
+  const RowScale rs{shares, blocks, eps};
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  int rc;
+  if (out_mode == OUT_BF16) rc = launch_pipelined<OUT_BF16>(C, ldc, a, lda, w, ldw, M, N, K, QkvArgs{}, stream, rs);
+  else if (out_mode == OUT_F32) rc = launch_pipelined<OUT_F32>(C, ldc, a, lda, w, ldw, M, N, K, QkvArgs{}, stream, rs);
+  else if (out_mode == OUT_ADD_F32) rc = launch_pipelined<OUT_ADD_F32>(C, ldc, a, lda, w, ldw, M, N, K, QkvArgs{}, stream, rs);
+  else rc = launch_pipelined<OUT_SWIGLU>(C, ldc, a, lda, w, ldw, M, N, K, QkvArgs{}, stream, rs);
+  if (rc) return rc;
+  HFEE_CHECK_LAUNCH("gemm_bf16_scaled");
+  return 0;
+}
 
 // How an aligned product of more than 64 rows is laid over the tiled kernels when nothing
 // is forced: kernel of the first n1 columns, n1, kernel of the rest (0: none).  For

@@ -723,6 +723,9 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 
 HFEE_API int hfee_gemm_bf16_qkv(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int64_t ldw, int M,
                                 int N, int K, const QkvArgs* qkv, int force_kernel, hipStream_t stream);   // gemm_bf16.hip
+HFEE_API int hfee_gemm_bf16_scaled(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
+                                   int64_t ldw, int M, int N, int K, const float* shares, int blocks, float eps,
+                                   hipStream_t stream);                                                    // gemm_bf16.hip
 
 // One entry point for every variant.  a_is_f32 != 0 selects the fused RMSNorm (M <= 16).
 // epi: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate, 4 q/k/v.
@@ -800,6 +803,10 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
     HFEE_REQUIRE(!norm && scale_blocks > 0 && scale_eps >= 0.f, "gemm_skinny: a row scale needs its shares and no norm of its own");
     a.scale_ss = scale_ss; a.scale_blocks = scale_blocks; a.scale_eps = scale_eps;
   }
+  // More than 16 rows and very many weight rows (gate/up): the streaming kernel would
+  // read the batch again for every 16 of them; the tiled kernel takes the row scale too.
+  if (scale_ss != nullptr && M > 16 && N >= 16384 && emit_out == nullptr && epi != EPI_QKV)
+    return hfee_gemm_bf16_scaled(C, epi, ldc, A, lda, W, ldw, M, N, K, scale_ss, scale_blocks, scale_eps, stream);
   const int mt = (M + 15) / 16;
   // Where the kernel with the batch in LDS was measured to win: products that are large
   // enough to pay for its set-up (q/k/v and down of an 8B model, not the output product),

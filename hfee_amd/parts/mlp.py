@@ -18,7 +18,7 @@ class GatedMLP(FeedForward):
     graph_safe = True
     takes_lazy_norm = True
     emits_norm = True
-    second_half_rows = ops.FUSED_NORM_MAX_ROWS
+    second_half_rows = ops.SKINNY_MAX_ROWS
 
     def __init__(self, spec: FeedForwardSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
@@ -46,7 +46,7 @@ class GatedMLP(FeedForward):
         act = ctx.rows("mlp.act", F)
         aligned = self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and F % 8 == 0
         few = ctx.n <= ops.FUSED_NORM_MAX_ROWS
-        halves = h.row_scale() if (aligned and few and isinstance(h, LazyNorm)) else None
+        halves = h.row_scale() if (aligned and isinstance(h, LazyNorm)) else None      # (offered for few rows only)
         norm = None
         if halves is None and aligned and few and isinstance(h, LazyNorm) and ops.norm_fusion_pays(*self.w_gate_up.shape):
             norm = h.fusable()

@@ -266,7 +266,7 @@ def test_products_of_17_to_64_rows(M, N, K, epilogue):
 
 
 @pytest.mark.parametrize("M,N,K,N2", [(1, 64, 96, 48), (8, 200, 256, 344), (16, 4096, 1024, 16400), (33, 104, 64, 72),
-                                       (64, 520, 128, 100)])
+                                       (64, 520, 128, 100), (40, 200, 64, 16400), (64, 2048, 128, 17000), (17, 96, 64, 16384)])
 @pytest.mark.parametrize("epilogue2", ["bf16", "swiglu", "add"])
 def test_norm_in_two_halves(M, N, K, N2, epilogue2):
     """A norm between two products, without a launch of its own: the product that adds
