@@ -60,13 +60,59 @@ __global__ void rmsnorm_kernel(TOut* __restrict__ out, const float* __restrict__
     o[j] = from_float<TOut>(xr[j] * scale * to_float<TW>(w[j]));
 }
 
+// The same with 16-byte loads and the row kept in registers between the sum and the
+// scaling (d <= 4 * NV * blockDim.x, a multiple of 4; rows 16-byte aligned).
+template <typename TOut, typename TW, int NV>
+__global__ void rmsnorm_rows_kernel(TOut* __restrict__ out, const float* __restrict__ x,
+                                    const TW* __restrict__ w, const int* __restrict__ rows,
+                                    float eps, int d) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const float* xr = x + (int64_t)(rows ? rows[r] : r) * d;
+  f32x4 v[NV];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int j = 4 * (threadIdx.x + i * blockDim.x);
+    v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (j < d) v[i] = *reinterpret_cast<const f32x4*>(xr + j);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) ss = fmaf(v[i][c], v[i][c], ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+  TOut* o = out + (int64_t)r * d;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int j = 4 * (threadIdx.x + i * blockDim.x);
+    if (j < d) {
+      TOut y[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) y[c] = from_float<TOut>(v[i][c] * scale * to_float<TW>(w[j + c]));
+      if constexpr (sizeof(TOut) == 2) *reinterpret_cast<uint2*>(o + j) = *reinterpret_cast<const uint2*>(y);
+      else *reinterpret_cast<f32x4*>(o + j) = *reinterpret_cast<const f32x4*>(y);
+    }
+  }
+}
+
 HFEE_API int hfee_rmsnorm(void* out, int out_dtype, const float* x, const void* w, int w_dtype,
                           const int* rows, float eps, int n, int d, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && d > 0, "rmsnorm: bad sizes n=%d d=%d", n, d);
   HFEE_REQUIRE(eps >= 0.f, "rmsnorm: eps must not be negative");
   if (n == 0) return 0;
   const int threads = d >= 2048 ? 512 : 256;
-#define LAUNCH(TO, TW) rmsnorm_kernel<TO, TW><<<n, threads, 0, stream>>>((TO*)out, x, (const TW*)w, rows, eps, d)
+  // rows that start 16-byte aligned (8 for a bfloat16 result) and fit in registers
+  const bool rows_fit = d % 4 == 0 && d <= 16 * threads && (uintptr_t)x % 16 == 0 &&
+                        (uintptr_t)out % (out_dtype == DT_F32 ? 16 : 8) == 0;
+  const int nv = (d + 4 * threads - 1) / (4 * threads);          // 1 .. 4
+#define LAUNCH(TO, TW)                                                                                              \
+  do {                                                                                                              \
+    if (rows_fit && nv <= 1) rmsnorm_rows_kernel<TO, TW, 1><<<n, threads, 0, stream>>>((TO*)out, x, (const TW*)w, rows, eps, d);      \
+    else if (rows_fit && nv == 2) rmsnorm_rows_kernel<TO, TW, 2><<<n, threads, 0, stream>>>((TO*)out, x, (const TW*)w, rows, eps, d); \
+    else if (rows_fit) rmsnorm_rows_kernel<TO, TW, 4><<<n, threads, 0, stream>>>((TO*)out, x, (const TW*)w, rows, eps, d);            \
+    else rmsnorm_kernel<TO, TW><<<n, threads, 0, stream>>>((TO*)out, x, (const TW*)w, rows, eps, d);                \
+  } while (0)
   if (out_dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
   else if (out_dtype == DT_F32 && w_dtype == DT_BF16) LAUNCH(float, bf16_t);
   else if (out_dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16_t, float);
@@ -193,6 +239,65 @@ __global__ void rope_cache_kernel(T* __restrict__ q, int64_t ldq, const T* __res
   }
 }
 
+// The same for bfloat16 with adjacent pairs (2i, 2i + 1), eight elements (16 bytes, four
+// pairs) per thread and step: head_dim and 2 * half multiples of 8, rows 16-byte aligned.
+__global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, const bf16_t* __restrict__ k, int64_t ldk,
+                                        const bf16_t* __restrict__ v, int64_t ldv,
+                                        const int* __restrict__ positions, const int* __restrict__ token_segment,
+                                        const int* __restrict__ block_tables, int bt_stride,
+                                        const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                                        int half, bf16_t* __restrict__ cache, CacheLayout lay, int num_heads) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  union Eight {
+    u32x4 u;
+    bf16_t e[8];
+  };
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int hd = lay.head_dim, per_head = hd / 8;
+  const float* cs = cos_table ? cos_table + (int64_t)pos * half : nullptr;
+  const float* sn = sin_table ? sin_table + (int64_t)pos * half : nullptr;
+  const int rot = cs != nullptr ? 2 * half : 0;
+  // elements d .. d + 7 of a head: pairs d/2 .. d/2 + 3 (rot is a multiple of 8: all or none are rotated)
+  auto rotate = [&](Eight& x, int d) {
+    if (d >= rot) return;
+    const f32x4 c = *reinterpret_cast<const f32x4*>(cs + (d >> 1)), s = *reinterpret_cast<const f32x4*>(sn + (d >> 1));
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const float x0 = bf16_to_float(x.e[2 * p]), x1 = bf16_to_float(x.e[2 * p + 1]);
+      x.e[2 * p] = float_to_bf16(x0 * c[p] - x1 * s[p]);
+      x.e[2 * p + 1] = float_to_bf16(x0 * s[p] + x1 * c[p]);
+    }
+  };
+  if (q != nullptr && cs != nullptr) {
+    bf16_t* qt = q + (int64_t)t * ldq;
+    for (int w = threadIdx.x; w < num_heads * per_head; w += blockDim.x) {
+      const int d = (w % per_head) * 8;
+      Eight x;
+      x.u = *reinterpret_cast<const u32x4*>(qt + w * 8);
+      rotate(x, d);
+      *reinterpret_cast<u32x4*>(qt + w * 8) = x.u;
+    }
+  }
+  if (k == nullptr || cache == nullptr) return;
+  const int page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
+  const int slot = pos & (lay.page_size - 1);
+  const bf16_t* kt = k + (int64_t)t * ldk;
+  const bf16_t* vt = v + (int64_t)t * ldv;
+  for (int w = threadIdx.x; w < lay.kv_heads * per_head; w += blockDim.x) {
+    const int h = w / per_head, d = (w - h * per_head) * 8;
+    Eight x, y;
+    x.u = *reinterpret_cast<const u32x4*>(kt + w * 8);
+    y.u = *reinterpret_cast<const u32x4*>(vt + w * 8);
+    rotate(x, d);
+    *reinterpret_cast<u32x4*>(cache + lay.key_offset(page, h, slot, d)) = x.u;
+    bf16_t* vc = cache + lay.value_offset(page, h, slot, d);          // column d of the head; the next is page_size on
+#pragma unroll
+    for (int c = 0; c < 8; ++c) vc[(int64_t)c * lay.page_size] = y.e[c];
+  }
+}
+
 HFEE_API int hfee_rope_cache_write(void* q, int64_t ldq, const void* k, int64_t ldk, const void* v, int64_t ldv,
                                    int dtype, const int* positions, const int* token_segment,
                                    const int* block_tables, int bt_stride,
@@ -218,6 +323,12 @@ HFEE_API int hfee_rope_cache_write(void* q, int64_t ldq, const void* k, int64_t 
     rope_cache_kernel<float><<<n, 256, 0, stream>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
         positions, token_segment, block_tables, bt_stride, cos_table, sin_table, half, pairing,
         (float*)cache, lay, num_heads);
+  else if (dtype == DT_BF16 && pairing == 1 && head_dim % 8 == 0 && half % 4 == 0 &&
+           (q == nullptr || (ldq % 8 == 0 && (uintptr_t)q % 16 == 0)) &&
+           (k == nullptr || (ldk % 8 == 0 && ldv % 8 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0)) &&
+           (uintptr_t)cos_table % 16 == 0 && (uintptr_t)sin_table % 16 == 0 && (uintptr_t)cache % 16 == 0)
+    rope_cache_pairs_kernel<<<n, 256, 0, stream>>>((bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv,
+        positions, token_segment, block_tables, bt_stride, cos_table, sin_table, half, (bf16_t*)cache, lay, num_heads);
   else if (dtype == DT_BF16)
     rope_cache_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv,
         positions, token_segment, block_tables, bt_stride, cos_table, sin_table, half, pairing,
