@@ -528,3 +528,50 @@ def test_argmax_first_maximum_wins():
     out = torch.zeros(3, dtype=torch.int32, device=DEV)
     ops.argmax(out, logits.to(DEV))
     assert out.tolist() == [17, 4999, 0]
+
+
+@pytest.mark.parametrize("H,K,hd,ps,ctx", [(8, 2, 128, 16, 9000), (4, 1, 64, 16, 5000), (8, 2, 128, 32, 6000)])
+def test_attention_over_long_contexts(H, K, hd, ps, ctx):
+    """Thousands of keys: the block table no longer fits the 64 entries that a wave holds at
+    a time, so the window moves several times per request.  One key far back is made to
+    stand out for every query, so that a region that is skipped or read twice shows.  The
+    matrix-core kernels (decode with several splits, prefill for the last rows) against the
+    plain kernel, which is itself checked against the formula at small sizes."""
+    from hfee_amd.kernels import ops
+    B = 2
+    g = torch.Generator(device=DEV).manual_seed(ctx + hd)
+    blocks = (ctx + ps - 1) // ps
+    cache = (torch.randn(B * blocks, 2, K, ps * hd, generator=g, device=DEV) * 0.5).to(torch.bfloat16)
+    table = torch.randperm(B * blocks, generator=g, device=DEV).to(torch.int32).reshape(B, blocks)
+    scale = 1 / math.sqrt(hd)
+    # queries: the last 40 rows of request 0 (a prefill portion deep in the context) and one decode row of each request
+    T = 40
+    q = torch.randn(T + B, H * hd, generator=g, device=DEV).to(torch.bfloat16)
+    far = [ctx // 3 + 5, ctx // 2 + 11]
+    for b in range(B):      # key `far[b]` of every kv head points along the queries' mean direction, scaled up
+        page, slot = int(table[b, far[b] // ps]), far[b] % ps
+        for kh in range(K):
+            rows = q[:T] if b == 0 else q[T + b:T + b + 1]
+            mean = rows.float().view(-1, H, hd)[:, kh * (H // K)].mean(0)
+            cache[page, 0, kh].view(ps, hd)[slot] = (mean / mean.norm() * 30).to(torch.bfloat16)
+    positions = torch.cat([torch.arange(ctx - T, ctx), torch.tensor([ctx - 1, ctx - 8])]).to(torch.int32).to(DEV)
+    seg = torch.tensor([0] * T + [0, 1], dtype=torch.int32, device=DEV)
+    ref = torch.zeros(T + B, H * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention_plain(ref, q, cache, positions, seg, table, H, K, hd, ps, scale, 0)
+    out = torch.zeros_like(ref)
+    tiles = torch.tensor([(0, 32, ctx - T, 0), (32, T - 32, ctx - T + 32, 0)], dtype=torch.int32, device=DEV)
+    for kernel in (1, 2):
+        out.zero_()
+        ops.attention_bf16_prefill(out, q, cache, tiles, table, H, K, hd, ps, scale, 0, kernel=kernel)
+        assert (out[:T].float() - ref[:T].float()).abs().max() <= 2e-2 * (1 + ref[:T].float().abs().max())
+    rows = torch.tensor([T, T + 1], dtype=torch.int32, device=DEV)
+    for splits in (1, 5, 16):
+        out.zero_()
+        partial = torch.zeros(B * H * splits * (hd + 2), dtype=torch.float32, device=DEV)
+        counters = torch.zeros(B * K, dtype=torch.int32, device=DEV)
+        ops.attention_bf16_decode(out, q, cache, rows, positions[T:].contiguous(), torch.arange(B, dtype=torch.int32, device=DEV),
+                                  table, H, K, hd, ps, scale, 0, partial, splits, counters=counters if splits > 1 else None)
+        assert (out[T:].float() - ref[T:].float()).abs().max() <= 2e-2 * (1 + ref[T:].float().abs().max())
+        assert int(counters.abs().sum()) == 0
+    # the far key carries weight: without it the result would be another
+    assert ref.float().abs().max() > 0.2
