@@ -621,11 +621,6 @@ __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) t += ss_part[w][r16];
     scale = 1.0f / sqrtf(t / (float)a.K + a.eps);     // for this lane's batch row (lane % 16)
-  } else if (a.scale_ss != nullptr) {
-    __shared__ float row_scale[SS_STRIDE];
-    row_scales(a, row_scale);
-    __syncthreads();
-    scale = row_scale[min(r16, a.M - 1)];
   }
 
   // ---- stream W ---------------------------------------------------------------------
@@ -635,6 +630,12 @@ __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups
   Chunk ring[RING];
 #pragma unroll
   for (int s = 0; s < RING; ++s) ring[s].u = *reinterpret_cast<const u32x4*>(w_cur + koff(s));
+  if (!NORM && a.scale_ss != nullptr) {      // (behind the first loads of W: it costs no latency of its own)
+    __shared__ float row_scale[SS_STRIDE];
+    row_scales(a, row_scale);
+    __syncthreads();
+    scale = row_scale[min(r16, a.M - 1)];
+  }
 
   while (rg < row_groups) {
     const int rg_next = rg + gridDim.x;
