@@ -225,6 +225,64 @@ __device__ __forceinline__ void epilogue(const Args& a, int m, int n, float* v) 
   }
 }
 
+// What the thread that finishes four sums (weight rows n .. n+3 of batch row m) has to
+// read for them: asked for at the start of a kernel, it has arrived when the sums have.
+template <int EPI>
+struct Ahead {
+  float old[4];          // EPI_ADD: what is added to
+  float weight[4];       // EPI_ADD with EMIT: the weight of the norm that follows
+  QkvPlace place;        // EPI_QKV
+};
+
+template <int EPI>
+__device__ __forceinline__ Ahead<EPI> look_ahead(const Args& a, int m, int n, bool live) {
+  Ahead<EPI> h;
+  if constexpr (EPI == EPI_ADD) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool in = live && n + i < a.N;
+      h.old[i] = in ? ((const float*)a.C)[(int64_t)m * a.ldc + n + i] : 0.f;
+      h.weight[i] = !(in && a.emit_out != nullptr) ? 0.f
+                    : a.emit_weight_is_f32 ? ((const float*)a.emit_weight)[n + i]
+                                           : bf16_to_float(((const bf16_t*)a.emit_weight)[n + i]);
+    }
+  } else if constexpr (EPI == EPI_QKV) {
+    if (live) h.place = qkv_place(a.qkv, a.C, a.ldc, m, n);
+  }
+  return h;
+}
+
+// finish_rows with what look_ahead has brought
+template <int EPI>
+__device__ __forceinline__ void finish_rows_ahead(const Args& a, const Ahead<EPI>& h, int m, int n, bool live, float* v,
+                                                  int block, int l) {
+  if constexpr (EPI == EPI_ADD) {
+    float ss = 0.f;
+    if (live) {
+      float* c = (float*)a.C + (int64_t)m * a.ldc + n;
+      bf16_t* e = a.emit_out != nullptr ? a.emit_out + (int64_t)m * a.ld_emit + n : nullptr;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (n + i < a.N) {
+          const float x = h.old[i] + v[i];
+          c[i] = x;
+          ss = fmaf(x, x, ss);
+          if (e != nullptr) e[i] = float_to_bf16(x * h.weight[i]);
+        }
+      }
+    }
+    if (a.emit_out != nullptr) {
+      ss += __shfl_xor(ss, 16, 64);          // the four column groups of this row
+      ss += __shfl_xor(ss, 32, 64);
+      if ((l >> 4) == 0 && m < a.M) a.emit_ss[(int64_t)block * SS_STRIDE + m] = ss;
+    }
+  } else if constexpr (EPI == EPI_QKV) {
+    if (live) qkv_put(h.place, v);
+  } else {
+    if (live) epilogue<EPI>(a, m, n, v);
+  }
+}
+
 // What every kernel of this file does with four finished sums of a whole wave's lanes
 // (lane l: batch row m, weight rows n .. n+3, `live` if they exist): the residual add
 // with the first half of the norm that follows it (EMIT), or the plain epilogue.
@@ -283,6 +341,11 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
     acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     ss[t] = 0.f;
   }
+  // the threads that will finish the sums (the first MT waves, four sums each) ask now for
+  // what they will need then
+  const int f_t = threadIdx.x >> 6, f_m = f_t * 16 + (lane & 15), f_n = n0 + 4 * (lane >> 4);
+  const bool f_live = f_t < MT && f_m < a.M && f_n < a.N;
+  const Ahead<EPI> ahead = look_ahead<EPI>(a, f_m, f_n, f_live);
 
   const int nfull = a.K / KBLOCK;
   {
@@ -377,7 +440,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
       for (int i = 0; i < 4; ++i) v[i] *= scale;
     }
 
-    finish_rows<EPI>(a, m, n, live, v, blockIdx.x, l);
+    finish_rows_ahead<EPI>(a, ahead, m, n, live, v, blockIdx.x, l);      // (idx == threadIdx.x: MT <= WAVES)
   }
 }
 

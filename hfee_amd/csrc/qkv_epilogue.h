@@ -25,41 +25,69 @@ struct QkvArgs {
 };
 
 
-__device__ __forceinline__ void qkv_store(const QkvArgs& q, void* C, int64_t ldc, int m, int n, float* v) {
+// Where four finished sums go and what they are rotated by: everything that has to be
+// read for them, so that a kernel can ask for it before its sums are ready.
+struct QkvPlace {
+  float c[2], s[2];      // cosine and sine of the two pairs (rotate[p] says whether pair p is rotated)
+  bool rotate[2];
+  bf16_t* dst;           // null: nothing to store
+  int step;              // elements between the four values at dst (1: one 8-byte store)
+};
+
+__device__ __forceinline__ QkvPlace qkv_place(const QkvArgs& q, void* C, int64_t ldc, int m, int n) {
+  QkvPlace w;
   const int hd = q.lay.head_dim;
   const int head = n / hd, d = n - head * hd;
   const int pos = q.positions[m];
   const bool is_v = head >= q.num_heads + q.lay.kv_heads;
-  if (!is_v && q.cos_table != nullptr && d < 2 * q.half) {
-    const float* cs = q.cos_table + (int64_t)pos * q.half + (d >> 1);
-    const float* sn = q.sin_table + (int64_t)pos * q.half + (d >> 1);
+  const bool rotated = !is_v && q.cos_table != nullptr && d < 2 * q.half;
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-      if (d + 2 * p < 2 * q.half) {
-        const float x0 = v[2 * p], x1 = v[2 * p + 1], c = cs[p], s = sn[p];
-        v[2 * p] = x0 * c - x1 * s;
-        v[2 * p + 1] = x0 * s + x1 * c;
-      }
-    }
+  for (int p = 0; p < 2; ++p) {
+    w.rotate[p] = rotated && d + 2 * p < 2 * q.half;
+    w.c[p] = w.rotate[p] ? q.cos_table[(int64_t)pos * q.half + (d >> 1) + p] : 1.f;
+    w.s[p] = w.rotate[p] ? q.sin_table[(int64_t)pos * q.half + (d >> 1) + p] : 0.f;
   }
-  bf16_t o[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) o[i] = float_to_bf16(v[i]);
+  w.dst = nullptr;
+  w.step = 1;
   if (head < q.num_heads) {
-    *reinterpret_cast<qkv_u32x2*>((bf16_t*)C + (int64_t)m * ldc + n) = *reinterpret_cast<const qkv_u32x2*>(o);
+    w.dst = (bf16_t*)C + (int64_t)m * ldc + n;
   } else if (q.cache != nullptr) {
     const int page = q.block_tables[(int64_t)q.token_segment[m] * q.bt_stride + (pos >> q.lay.page_shift)];
     const int slot = pos & (q.lay.page_size - 1);
     bf16_t* cache = (bf16_t*)q.cache;
     if (!is_v) {
-      *reinterpret_cast<qkv_u32x2*>(cache + q.lay.key_offset(page, head - q.num_heads, slot, d)) =
-          *reinterpret_cast<const qkv_u32x2*>(o);
+      w.dst = cache + q.lay.key_offset(page, head - q.num_heads, slot, d);
     } else {
-      const int kvh = head - q.num_heads - q.lay.kv_heads;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) cache[q.lay.value_offset(page, kvh, slot, d + i)] = o[i];
+      w.dst = cache + q.lay.value_offset(page, head - q.num_heads - q.lay.kv_heads, slot, d);
+      w.step = q.lay.page_size;          // a head's value columns lie page_size apart
     }
   }
+  return w;
+}
+
+__device__ __forceinline__ void qkv_put(const QkvPlace& w, float* v) {
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    if (w.rotate[p]) {
+      const float x0 = v[2 * p], x1 = v[2 * p + 1];
+      v[2 * p] = x0 * w.c[p] - x1 * w.s[p];
+      v[2 * p + 1] = x0 * w.s[p] + x1 * w.c[p];
+    }
+  }
+  bf16_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = float_to_bf16(v[i]);
+  if (w.dst == nullptr) return;
+  if (w.step == 1) {
+    *reinterpret_cast<qkv_u32x2*>(w.dst) = *reinterpret_cast<const qkv_u32x2*>(o);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w.dst[(int64_t)i * w.step] = o[i];
+  }
+}
+
+__device__ __forceinline__ void qkv_store(const QkvArgs& q, void* C, int64_t ldc, int m, int n, float* v) {
+  qkv_put(qkv_place(q, C, ldc, m, n), v);
 }
 
 }  // namespace hfee
