@@ -316,15 +316,17 @@ __device__ __forceinline__ void finish_rows(const Args& a, int m, int n, bool li
 }
 
 template <int MT, bool NORM, int EPI>
-__global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
+__global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_here) {
   __shared__ float partial[WAVES][MT][64][4];
   __shared__ float ss_part[WAVES][MT][16];
   __shared__ float row_scale[SS_STRIDE];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * ROWS;
+  // rows_here (16, or 12 where that fills the chip more evenly): the weight rows of this
+  // workgroup; with 12, the matrix instruction's last four rows repeat the twelfth and are dropped
+  const int n0 = blockIdx.x * rows_here;
   // rows beyond N or M read a valid row; what they produce is never stored
-  const bf16_t* w_row = a.W + (int64_t)min(n0 + r16, a.N - 1) * a.ldw + g * 8;
+  const bf16_t* w_row = a.W + (int64_t)min(n0 + min(r16, rows_here - 1), a.N - 1) * a.ldw + g * 8;
   const void* x_rows[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -344,7 +346,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   // the threads that will finish the sums (the first MT waves, four sums each) ask now for
   // what they will need then
   const int f_t = threadIdx.x >> 6, f_m = f_t * 16 + (lane & 15), f_n = n0 + 4 * (lane >> 4);
-  const bool f_live = f_t < MT && f_m < a.M && f_n < a.N;
+  const bool f_live = f_t < MT && f_m < a.M && f_n < a.N && 4 * (lane >> 4) < rows_here;
   const Ahead<EPI> ahead = look_ahead<EPI>(a, f_m, f_n, f_live);
 
   const int nfull = a.K / KBLOCK;
@@ -418,7 +420,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
     const int t = idx >> 6, l = idx & 63;
     const int m = t * 16 + (l & 15);
     const int n = n0 + 4 * (l >> 4);
-    const bool live = m < a.M && n < a.N;
+    const bool live = m < a.M && n < a.N && 4 * (l >> 4) < rows_here;
     float v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -446,8 +448,20 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
 
 template <int MT, bool NORM>
 void launch_epi(const Args& a, int epi, hipStream_t stream) {
-  dim3 grid((a.N + ROWS - 1) / ROWS);
-#define GO(E) skinny_kernel<MT, NORM, E><<<grid, WAVES * 64, 0, stream>>>(a)
+  // Twelve rows a workgroup where that takes fewer rounds of rows over the chip than
+  // sixteen (6,144 rows on 256 CUs: two workgroups a CU of 12 rows each instead of one or
+  // two of 16).  Not with EMIT: its shares are counted in groups of 16 rows.
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    num_cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+               prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+  }
+  auto rounds = [&](int rows) { return (((a.N + rows - 1) / rows + num_cus - 1) / num_cus) * rows; };
+  const int rows_here = (a.emit_out == nullptr && rounds(12) < rounds(ROWS)) ? 12 : ROWS;
+  dim3 grid((a.N + rows_here - 1) / rows_here);
+#define GO(E) skinny_kernel<MT, NORM, E><<<grid, WAVES * 64, 0, stream>>>(a, rows_here)
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
