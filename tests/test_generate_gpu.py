@@ -110,3 +110,27 @@ def test_an_interrupted_call_leaves_nothing_behind(model_folders):
     assert not llm.scheduler.has_work() and not llm.engine.cache.requests
     llm.engine.cache.check()
     assert [o.token_ids for o in llm.generate(prompts, SamplingParams.greedy(num_predict=10))] == want
+
+
+def test_the_command_line_generates_from_token_ids(model_folders):
+    """`hfee run <model> --tokens ...` as a user calls it: the ids of the greedy
+    continuation, and with --verbose the counts that the reference prints."""
+    import os, subprocess, sys
+    from plain_llama import PlainLlama
+    folder = model_folders[("A", "float32")]
+    prompt = tu.make_requests(256, [11], seed=8)["r0"]
+    want = PlainLlama(folder).greedy(prompt, 7)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "hfee"), "run", folder, "--tokens",
+                        ",".join(map(str, prompt)), "--dtype", "float32", "--temperature", "0", "--repeat-penalty", "1",
+                        "--num-predict", "7", "--num-ctx", "128", "--verbose"],
+                       capture_output=True, text=True, timeout=300, stdin=subprocess.DEVNULL)
+    assert p.returncode == 0, p.stderr[-2000:]
+    first = p.stdout.strip().splitlines()[0]
+    assert [int(t) for t in first.split()] == want
+    assert "prompt eval count:    11 token(s)" in p.stdout and "eval count:           7 token(s)" in p.stdout
+    assert "done reason:          length" in p.stdout
+    # without a prompt and without a terminal there is nothing to do
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "hfee"), "run", folder, "--dtype", "float32"],
+                       capture_output=True, text=True, timeout=300, stdin=subprocess.DEVNULL)
+    assert p.returncode == 1 and "usage" in p.stderr
