@@ -15,6 +15,7 @@
 // add of /root/reference/internal/llm/forward.go:106-107 fused into the epilogue).
 #include "common.h"
 #include "qkv_epilogue.h"
+#include "gemm_entry.h"
 
 #include <type_traits>
 
@@ -1126,17 +1127,6 @@ int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, 
 
 }  // namespace
 
-HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
-                              int64_t ldw, int M, int N, int K, int epi,
-                              const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
-                              const int* positions, const int* token_segment, const int* block_tables,
-                              int bt_stride, const float* cos_table, const float* sin_table, int half,
-                              int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
-                              int page_size, const void* emit_weight, int emit_weight_is_f32, void* emit_out,
-                              int64_t ld_emit, float* emit_ss, const float* scale_ss, int scale_blocks,
-                              float scale_eps, float* scratch, int64_t scratch_floats, int* counters,
-                              int num_counters, hipStream_t stream);
-
 // The tiled product of at most 64 rows whose result rows are scaled by the second half of
 // a norm (see RowScale): for shapes that are too wide for the streaming kernels.
 // out_mode as hfee_gemm_bf16; operands aligned as for the tiled kernels.
@@ -1195,14 +1185,14 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
     HFEE_REQUIRE(N % 2 == 0 && vec, "gemm_bf16: the SiLU gate needs an even N and aligned operands");
     if (skinny_pays(M, N))
       return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, 3, nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr,
-                              0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, nullptr, 0, nullptr, 0, stream);
+                              0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, nullptr, 0, 0, stream);
     if (launch_aligned<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, force_kernel, stream)) return 1;
     HFEE_CHECK_LAUNCH("gemm_bf16");
     return 0;
   }
   if (vec && M <= 64 && (force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N))))   // gemm_skinny.hip
     return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, out_mode, nullptr, 0, 0.f, nullptr, nullptr, nullptr,
-                            nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, nullptr, 0, nullptr, 0, stream);
+                            nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, nullptr, 0, 0, stream);
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   int rc;

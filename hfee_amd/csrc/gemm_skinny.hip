@@ -28,6 +28,7 @@
 //                                             (/root/reference/internal/llm/forward.go:96-101)
 #include "common.h"
 #include "qkv_epilogue.h"
+#include "gemm_entry.h"
 
 using namespace hfee;
 
@@ -252,7 +253,11 @@ __device__ __forceinline__ Ahead<EPI> look_ahead(const Args& a, int m, int n, bo
   return h;
 }
 
-// finish_rows with what look_ahead has brought
+// What every kernel that looks ahead does with four finished sums of a whole wave's lanes
+// (lane l: batch row m, weight rows n .. n+3, `live` if they exist): the residual add with
+// the first half of the norm that follows it (EMIT), or the plain epilogue, with what
+// look_ahead has brought.  `block`: this group of 16 weight rows (the row of the shares
+// table).  All lanes of the wave come here together: the shares are summed by shuffles.
 template <int EPI>
 __device__ __forceinline__ void finish_rows_ahead(const Args& a, const Ahead<EPI>& h, int m, int n, bool live, float* v,
                                                   int block, int l) {
@@ -280,38 +285,6 @@ __device__ __forceinline__ void finish_rows_ahead(const Args& a, const Ahead<EPI
     if (live) qkv_put(h.place, v);
   } else {
     if (live) epilogue<EPI>(a, m, n, v);
-  }
-}
-
-// What every kernel of this file does with four finished sums of a whole wave's lanes
-// (lane l: batch row m, weight rows n .. n+3, `live` if they exist): the residual add
-// with the first half of the norm that follows it (EMIT), or the plain epilogue.
-// `block`: this group of 16 weight rows (the row of the shares table).  All lanes of the
-// wave come here together: the shares are summed by shuffles.
-template <int EPI>
-__device__ __forceinline__ void finish_rows(const Args& a, int m, int n, bool live, float* v, int block, int l) {
-  if (EPI == EPI_ADD && a.emit_out != nullptr) {
-    float ss = 0.f;
-    if (live) {
-      float* c = (float*)a.C + (int64_t)m * a.ldc + n;
-      bf16_t* e = a.emit_out + (int64_t)m * a.ld_emit + n;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (n + i < a.N) {
-          const float x = c[i] + v[i];
-          c[i] = x;
-          ss = fmaf(x, x, ss);
-          const float w = a.emit_weight_is_f32 ? ((const float*)a.emit_weight)[n + i]
-                                               : bf16_to_float(((const bf16_t*)a.emit_weight)[n + i]);
-          e[i] = float_to_bf16(x * w);
-        }
-      }
-    }
-    ss += __shfl_xor(ss, 16, 64);          // the four column groups of this row
-    ss += __shfl_xor(ss, 32, 64);
-    if ((l >> 4) == 0 && m < a.M) a.emit_ss[(int64_t)block * SS_STRIDE + m] = ss;
-  } else if (live) {
-    epilogue<EPI>(a, m, n, v);
   }
 }
 
@@ -478,20 +451,22 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 // weight rows, and that traffic (from L2) outgrows the weights.  Here K is cut into
 // slices of 1,024 columns, each with workgroups of its own.  A workgroup keeps its slice
 // of the batch, all rows, in LDS; each of its waves walks over groups of 16 weight rows
-// on its own: the weights come straight from global memory through a ring of 16 loads
+// on its own: the weights come straight from global memory through a ring of 8 or 16 loads
 // that runs across group boundaries, the batch operands from LDS; no barrier stands in
-// the loop.  The slices' partial sums of a row group meet in a scratch buffer: every
-// wave stores its share at device scope and counts itself, and the wave that finishes a
-// row group last adds the shares in the order of the slices and runs the epilogue.
-// Nobody waits for anybody; the counters are back at zero afterwards.
-constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32, MID_RING = 16;
+// the loop.  With more than one slice a wave leaves its share of a row group's sums in a
+// scratch buffer and goes on; a second, short kernel (one wave for 16 batch rows of a row
+// group, so that the whole chip takes part) adds the shares in the order of the slices and
+// runs the epilogue.  Nobody waits for anybody, and nothing is counted.
+constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32;
+// loads a wave keeps in flight: with three or four tiles of batch rows a step takes longer,
+// and a shorter ring measured faster (less of the chip's memory queue held by each wave)
+constexpr int mid_ring(int mt) { return mt >= 3 ? 8 : 16; }
 constexpr int MID_PITCH = MID_KS + 8;        // LDS row pitch of the batch slice in elements: rows 16 bytes askew
 
 constexpr size_t mid_lds_bytes(int mt) { return (size_t)mt * 16 * MID_PITCH * sizeof(bf16_t); }
 
 template <int MT, int EPI>
-__global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups, int slices, float* __restrict__ scratch,
-                                                         int* __restrict__ counters) {
+__global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups, int slices, float* __restrict__ scratch) {
   extern __shared__ __attribute__((aligned(16))) char mid_lds[];
   bf16_t* xs = (bf16_t*)mid_lds;                                                    // [MT * 16][MID_PITCH]
   __shared__ float row_scale[SS_STRIDE];
@@ -502,24 +477,43 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   const int stride = (gridDim.x / slices) * WAVES;           // waves of this slice
   const int k0 = slice * MID_KS;
 
-  // ---- the first weights go out before anything else ---------------------------------
+  // ---- the batch slice is asked for first: it comes from L2 and must not wait in line
+  // behind the first weights, which come from memory (a wave's loads return in order).
+  // Every workgroup of a slice wants the same rows: each starts at another one.
+  constexpr int FILL = MT * 16 * (MID_KS / 8) / (WAVES * 64);      // 16-byte chunks a thread brings
+  static_assert(MT * 16 * (MID_KS / 8) % (WAVES * 64) == 0, "the batch slice is whole rounds of the workgroup");
+  constexpr int FILL_ROWS = WAVES * 64 / (MID_KS / 8);             // rows a round of the workgroup covers
+  const int fill_row = threadIdx.x / (MID_KS / 8), fill_c = threadIdx.x % (MID_KS / 8);
+  const int fill_first = (blockIdx.x / slices) % FILL;
+  u32x4 fill[FILL];
+#pragma unroll
+  for (int it = 0; it < FILL; ++it) {
+    const int row = ((it + fill_first) % FILL) * FILL_ROWS + fill_row;
+    fill[it] = u32x4{0u, 0u, 0u, 0u};                             // rows beyond M are zeros
+    if (row < a.M) fill[it] = *reinterpret_cast<const u32x4*>((const bf16_t*)a.A + (int64_t)row * a.lda + k0 + fill_c * 8);
+  }
+
+  // ---- then the first weights: behind every wave's requests for the batch, also in the
+  // queue of loads that the waves of a CU share (the barrier waits for the issue, not the data)
+  __syncthreads();
   auto row_ptr = [&](int rg) {       // rows beyond N read the last row; what they produce is never stored
     return a.W + (int64_t)min(rg * ROWS + r16, a.N - 1) * a.ldw + k0 + g * 8;
   };
-  int rg = (blockIdx.x / slices) * WAVES + wave;
+  // (row groups are dealt out so that every workgroup of a slice gets as many, within one)
+  const int per_slice = gridDim.x / slices;
+  int rg = blockIdx.x / slices + per_slice * wave;
   const bf16_t* w_cur = row_ptr(min(rg, row_groups - 1));
+  constexpr int MID_RING = mid_ring(MT);
   Chunk ring[MID_RING];
 #pragma unroll
   for (int st = 0; st < MID_RING; ++st) ring[st].u = *reinterpret_cast<const u32x4*>(w_cur + st * 32);
 
-  // ---- the batch slice into LDS (rows beyond M as zeros) -------------------------------
-  for (int idx = threadIdx.x; idx < MT * 16 * (MID_KS / 8); idx += WAVES * 64) {
-    const int row = idx / (MID_KS / 8), c = idx - row * (MID_KS / 8);
-    u32x4 v = u32x4{0u, 0u, 0u, 0u};
-    if (row < a.M) v = *reinterpret_cast<const u32x4*>((const bf16_t*)a.A + (int64_t)row * a.lda + k0 + c * 8);
-    *reinterpret_cast<u32x4*>(xs + row * MID_PITCH + c * 8) = v;
+#pragma unroll
+  for (int it = 0; it < FILL; ++it) {
+    const int row = ((it + fill_first) % FILL) * FILL_ROWS + fill_row;
+    *reinterpret_cast<u32x4*>(xs + row * MID_PITCH + fill_c * 8) = fill[it];
   }
-  if (a.scale_ss != nullptr) row_scales(a, row_scale);
+  if (slices == 1 && a.scale_ss != nullptr) row_scales(a, row_scale);
   __syncthreads();
 
   const bf16_t* x_lane = xs + r16 * MID_PITCH + g * 8;
@@ -551,47 +545,25 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
     }
 
-    bool finish = true;
+    const int n = rg * ROWS + 4 * g;
     if (slices > 1) {
-      // this slice's share, at device scope; then count; the last one adds all shares in order
-      // (a wave's store of one register is 256 contiguous bytes: whole lines go through to memory)
-      float* mine = scratch + ((int64_t)(rg * slices + slice) * MT) * 256 + lane;
+      // this slice's share: register i of lane l (weight row 4*(l/16) + i, batch row l%16) of
+      // tile t at [row group][slice][t][l][i], a kilobyte a store
+      float* mine = scratch + ((int64_t)(rg * slices + slice) * MT) * 256 + lane * 4;
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          __hip_atomic_store(mine + (t * 4 + i) * 64, acc[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      // (the stores are complete when every load issued before them is too: the ring refills after this)
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      int arrived = 0;
-      if (lane == 0) arrived = atomicAdd(counters + rg, 1);
-      finish = __builtin_amdgcn_readfirstlane(arrived) == slices - 1;
-      if (finish) {
-#pragma unroll
-        for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int sl = 0; sl < slices; ++sl) {
-          const float* theirs = scratch + ((int64_t)(rg * slices + sl) * MT) * 256 + lane;
-#pragma unroll
-          for (int t = 0; t < MT; ++t)
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              acc[t][i] += __hip_atomic_load(theirs + (t * 4 + i) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        if (lane == 0) atomicExch(counters + rg, 0);
-      }
-    }
-    if (finish) {
-      // register i of lane l: weight row 4*(l/16) + i, batch row l%16
+      for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4*>(mine + t * 256) = acc[t];
+    } else {
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const int m = t * 16 + r16, n = rg * ROWS + 4 * g;
+        const int m = t * 16 + r16;
         float v[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
         if (a.scale_ss != nullptr) {
           const float scale = row_scale[m];
 #pragma unroll
           for (int i = 0; i < 4; ++i) v[i] *= scale;
         }
-        finish_rows<EPI>(a, m, n, m < a.M && n < a.N, v, rg, lane);
+        const bool live = m < a.M && n < a.N;
+        finish_rows_ahead<EPI>(a, look_ahead<EPI>(a, m, n, live), m, n, live, v, rg, lane);
       }
     }
     rg = rg_next;
@@ -599,18 +571,56 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   }
 }
 
-// Returns true if the kernel for 17 to 64 rows took the product.
+// The second kernel of a product cut into slices: wave (row group, t) adds the slices'
+// shares of batch rows 16t .. 16t+15, in the order of the slices, and runs the epilogue.
+// What the epilogue reads and all shares are asked for together.
+template <int MT, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void mid_finish_kernel(Args a, int row_groups, int slices,
+                                                                const float* __restrict__ scratch) {
+  __shared__ float row_scale[SS_STRIDE];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, g = lane >> 4;
+  const int unit = blockIdx.x * WAVES + wave;
+  const int rg = unit / MT, t = unit - rg * MT;
+  const bool here = rg < row_groups;                       // (whole waves; every wave stays for the barrier below)
+  const int m = t * 16 + r16, n = rg * ROWS + 4 * g;
+  const bool live = here && m < a.M && n < a.N;
+  const Ahead<EPI> ahead = look_ahead<EPI>(a, m, n, live);
+  const float* share = scratch + ((int64_t)min(rg, row_groups - 1) * slices * MT + t) * 256 + lane * 4;
+  const int64_t step = (int64_t)MT * 256;
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  constexpr int TOGETHER = 8;
+  for (int s0 = 0; s0 < slices; s0 += TOGETHER) {
+    f32x4 part[TOGETHER];
+#pragma unroll
+    for (int j = 0; j < TOGETHER; ++j)                     // past the end: a repeat that is not added
+      part[j] = *reinterpret_cast<const f32x4*>(share + min(s0 + j, slices - 1) * step);
+#pragma unroll
+    for (int j = 0; j < TOGETHER; ++j)
+      if (s0 + j < slices) acc += part[j];
+  }
+  float v[4] = {acc[0], acc[1], acc[2], acc[3]};
+  if (a.scale_ss != nullptr) {
+    row_scales(a, row_scale);
+    __syncthreads();
+    const float scale = row_scale[m];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] *= scale;
+  }
+  if (here) finish_rows_ahead<EPI>(a, ahead, m, n, live, v, rg, lane);
+}
+
+// Returns true if the kernels for 17 to 64 rows took the product.
 template <int MT>
-bool launch_mid_rows(const Args& a, int epi, float* scratch, int64_t scratch_floats, int* counters, int num_counters,
-                     int num_cus, hipStream_t stream) {
+bool launch_mid_rows(const Args& a, int epi, float* scratch, int64_t scratch_floats, int num_cus, hipStream_t stream) {
   const int row_groups = (a.N + ROWS - 1) / ROWS, slices = a.K / MID_KS;
-  if (slices > 1 && (scratch == nullptr || counters == nullptr || num_counters < row_groups ||
-                     scratch_floats < (int64_t)row_groups * slices * MT * 256))
-    return false;
+  if (slices > 1 && (scratch == nullptr || scratch_floats < (int64_t)row_groups * slices * MT * 256)) return false;
   int per_slice = num_cus / slices;                         // workgroups per slice: eight row groups at a time each
   if (per_slice < 1) per_slice = 1;
   if (per_slice > (row_groups + WAVES - 1) / WAVES) per_slice = (row_groups + WAVES - 1) / WAVES;
   const size_t lds = mid_lds_bytes(MT);
+  const int finish_grid = (row_groups * MT + WAVES - 1) / WAVES;
 #define GO(E)                                                                                                  \
   do {                                                                                                         \
     static bool raised = false;                                                                                \
@@ -620,7 +630,8 @@ bool launch_mid_rows(const Args& a, int epi, float* scratch, int64_t scratch_flo
         return false;                                                                                          \
       raised = true;                                                                                           \
     }                                                                                                          \
-    mid_kernel<MT, E><<<per_slice * slices, WAVES * 64, lds, stream>>>(a, row_groups, slices, scratch, counters); \
+    mid_kernel<MT, E><<<per_slice * slices, WAVES * 64, lds, stream>>>(a, row_groups, slices, scratch);        \
+    if (slices > 1) mid_finish_kernel<MT, E><<<finish_grid, WAVES * 64, 0, stream>>>(a, row_groups, slices, scratch); \
   } while (0)
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
@@ -799,23 +810,16 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 
 }  // namespace
 
-HFEE_API int hfee_gemm_bf16_qkv(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int64_t ldw, int M,
-                                int N, int K, const QkvArgs* qkv, int force_kernel, hipStream_t stream);   // gemm_bf16.hip
-HFEE_API int hfee_gemm_bf16_scaled(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
-                                   int64_t ldw, int M, int N, int K, const float* shares, int blocks, float eps,
-                                   hipStream_t stream);                                                    // gemm_bf16.hip
-
 // One entry point for every variant.  a_is_f32 != 0 selects the fused RMSNorm (M <= 16).
 // epi: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate, 4 q/k/v.
 // emit_out (with epi 2): also write bfloat16(C_new * emit_weight) to emit_out [M, N] and this
 // product's shares of the rows' sums of squares to emit_ss (ceil(N / 16) x 64 floats).
 // scale_ss: shares left by such a product (scale_blocks x 64 floats) over rows of width K:
 // the finished sums are scaled by 1 / sqrt(sum / K + scale_eps).
-// scratch, counters: for 17 to 64 rows and K a multiple of 1,024, a faster kernel that
-// needs ceil(N / 16) * (K / 1024) * ceil(M / 16) * 256 floats of scratch and ceil(N / 16)
-// int32 counters that are zero (and are zero again afterwards); without them, or for
-// other sizes, or where it would not pay, the streaming kernel takes the product (a
-// negative num_counters takes the faster kernel wherever it applies: for tests).
+// scratch: for 17 to 64 rows and K a multiple of 1,024, a faster pair of kernels that needs
+// ceil(N / 16) * (K / 1024) * ceil(M / 16) * 256 floats of scratch (none for K = 1,024);
+// without it, or for other sizes, or where it would not pay, the streaming kernel takes
+// the product (force_mid != 0 takes the faster kernels wherever they apply: for tests).
 HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
                               int64_t ldw, int M, int N, int K, int epi,
                               const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
@@ -824,11 +828,9 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                               int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
                               int page_size, const void* emit_weight, int emit_weight_is_f32, void* emit_out,
                               int64_t ld_emit, float* emit_ss, const float* scale_ss, int scale_blocks,
-                              float scale_eps, float* scratch, int64_t scratch_floats, int* counters,
-                              int num_counters, hipStream_t stream) {
+                              float scale_eps, float* scratch, int64_t scratch_floats, int force_mid,
+                              hipStream_t stream) {
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
-  const bool force_mid = num_counters < 0;          // (for tests of that kernel alone)
-  if (force_mid) num_counters = -num_counters;
   if (M == 0) return 0;
   HFEE_REQUIRE(epi >= 0 && epi <= 4, "gemm_skinny: unknown epilogue %d", epi);
   HFEE_REQUIRE(M <= 64 || epi == EPI_QKV, "gemm_skinny: at most 64 rows (more for q/k/v only), got %d", M);
@@ -886,10 +888,18 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
   if (scale_ss != nullptr && M > 16 && N >= 16384 && emit_out == nullptr && epi != EPI_QKV)
     return hfee_gemm_bf16_scaled(C, epi, ldc, A, lda, W, ldw, M, N, K, scale_ss, scale_blocks, scale_eps, stream);
   const int mt = (M + 15) / 16;
-  // Where the kernel with the batch in LDS was measured to win: products that are large
-  // enough to pay for its set-up (q/k/v and down of an 8B model, not the output product),
-  // and not so wide that the tiled kernel fills the chip (gate/up).
-  const bool mid_pays = (int64_t)N * K >= (int64_t)24 << 20 && N < 16384;
+  // Where the kernels with the batch in LDS win, from fits to measured times in microseconds
+  // (1,024 to 15,360 weight rows, K from 2,048 to 14,336, 17 to 64 batch rows): the streaming
+  // kernel takes the weights' time at 5 TB/s, a launch, and 0.052 a batch row and 1,024
+  // columns for reading the batch again with every 16 weight rows (more where the row
+  // groups outnumber the CUs); the pair of kernels takes 16.5, or the weights' time at
+  // 4.65 TB/s and 4 where that is more, whatever the number of batch rows.  Not for very
+  // many weight rows (gate/up), where the tiled kernel fills the chip.
+  const double weight_mb = 2e-6 * (double)N * (double)K;
+  const double rounds = ((N + ROWS - 1) / ROWS) / 256.0;
+  const double t_streaming = weight_mb / 5.0 + 3.0 + 0.052 * (K / 1024.0) * (rounds > 1.0 ? rounds : 1.0) * M;
+  const double t_pair = weight_mb * 0.215 + 4.0 > 16.5 ? weight_mb * 0.215 + 4.0 : 16.5;
+  const bool mid_pays = t_pair < 0.95 * t_streaming && N < 16384;
   if (!norm && mt > 1 && K % MID_KS == 0 && (mid_pays || force_mid)) {
     static int num_cus = 0;
     if (num_cus == 0) {
@@ -898,9 +908,9 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
       num_cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
                  prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
     }
-    const bool took = mt == 2 ? launch_mid_rows<2>(a, epi, scratch, scratch_floats, counters, num_counters, num_cus, stream)
-                    : mt == 3 ? launch_mid_rows<3>(a, epi, scratch, scratch_floats, counters, num_counters, num_cus, stream)
-                              : launch_mid_rows<4>(a, epi, scratch, scratch_floats, counters, num_counters, num_cus, stream);
+    const bool took = mt == 2 ? launch_mid_rows<2>(a, epi, scratch, scratch_floats, num_cus, stream)
+                    : mt == 3 ? launch_mid_rows<3>(a, epi, scratch, scratch_floats, num_cus, stream)
+                              : launch_mid_rows<4>(a, epi, scratch, scratch_floats, num_cus, stream);
     if (took) {
       HFEE_CHECK_LAUNCH("gemm_skinny(17 to 64 rows)");
       return 0;

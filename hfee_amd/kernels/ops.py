@@ -342,7 +342,7 @@ def mid_rows_scratch(n_rows: int, n_weight_rows: int, k: int) -> int:
 
 
 def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0.0, rows=None, m=None, qkv=None,
-                 emit=None, row_scale=None, scratch=None, counters=None, force_mid_rows=False):
+                 emit=None, row_scale=None, scratch=None, force_mid_rows=False):
     """out = epilogue(norm(x) @ weight.T) in one launch, for at most 64 rows ("qkv": any
     number of rows; more than 64 take the tiled kernels with the same epilogue).
 
@@ -351,10 +351,10 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
     its shares of the rows' sums of squares to emit["shares"] (float32, at least
     ceil(N / 16) * 64).  row_scale: dict(shares, blocks, eps): the other half: x is such an
     emitted tensor, and the finished sums are scaled by 1 / sqrt(sum of shares / K + eps).
-    scratch (float32, `mid_rows_scratch` words) and counters (int32 zeros, ceil(N / 16); zero
-    again afterwards): let products of 17 to 64 rows over K % 1024 == 0 take a kernel that
-    keeps the batch in LDS and cuts K over workgroups, where that pays (force_mid_rows:
-    wherever it applies, for tests).
+    scratch (float32, `mid_rows_scratch` words): lets products of 17 to 64 rows over
+    K % 1024 == 0 take a kernel that keeps the batch in LDS and cuts K over workgroups, and a
+    second one that adds the slices up, where that pays (force_mid_rows: wherever it applies,
+    for tests).
 
     x: bfloat16 [M, K]; or, with norm_weight, the float32 residual stream (at most 16
     rows; `rows` optionally gathers them, then `m` is their number).
@@ -402,12 +402,11 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
         _check(ss.dtype == torch.float32 and ss.is_contiguous() and blocks > 0 and ss.numel() >= blocks * SS_STRIDE,
                "linear_fused: row scale shares")
         s_args = [_ptr(ss), blocks, float(row_scale["eps"])]
-    w_args = [None, 0, None, 0]
-    if scratch is not None and counters is not None:
-        _gpu(scratch, counters)
-        _check(scratch.dtype == torch.float32 and scratch.is_contiguous() and counters.dtype == torch.int32
-               and counters.is_contiguous(), "linear_fused: float32 scratch and int32 counters expected")
-        w_args = [_ptr(scratch), scratch.numel(), _ptr(counters), -counters.numel() if force_mid_rows else counters.numel()]
+    w_args = [None, 0, int(force_mid_rows)]
+    if scratch is not None:
+        _gpu(scratch)
+        _check(scratch.dtype == torch.float32 and scratch.is_contiguous(), "linear_fused: float32 scratch expected")
+        w_args = [_ptr(scratch), scratch.numel(), int(force_mid_rows)]
     q = qkv or {}
     if epilogue == "qkv":
         H, KV, hd, ps = q["num_heads"], q["kv_heads"], q["head_dim"], q["page_size"]

@@ -209,14 +209,13 @@ class Workspace:
         return buf[:count]
 
     def product_scratch(self, n_rows: int, weight: torch.Tensor) -> dict:
-        """The `scratch` and `counters` arguments of `ops.linear_fused` for a product of
-        n_rows rows with this weight (empty where it has no use for them)."""
+        """The `scratch` argument of `ops.linear_fused` for a product of n_rows rows with
+        this weight (empty where it has no use for it)."""
         from ..kernels import ops
         words = ops.mid_rows_scratch(n_rows, weight.shape[0], weight.shape[1])
         if not words:
             return {}
-        return dict(scratch=self.flat("product.partial", words, torch.float32),
-                    counters=self.counters("product.slices", (weight.shape[0] + 15) // 16))
+        return dict(scratch=self.flat("product.partial", words, torch.float32))
 
     def counters(self, name: str, count: int) -> torch.Tensor:
         """`count` int32 that are zero, for kernels whose workgroups count themselves

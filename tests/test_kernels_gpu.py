@@ -212,8 +212,8 @@ def test_fused_decode_products(M, N, K, epilogue, norm):
 @pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu", "emit", "scaled"])
 def test_products_of_17_to_64_rows(M, N, K, epilogue):
     """The kernel that keeps the batch in LDS and cuts K over workgroups (17 to 64 rows,
-    K a multiple of 1,024), with every epilogue, twice in a row on the same scratch and
-    counters, against the unfused formulas."""
+    K a multiple of 1,024) and the kernel that adds its slices up, with every epilogue, twice
+    in a row on the same scratch, against the unfused formulas."""
     from hfee_amd.kernels import ops
     if epilogue == "swiglu" and N % 2:
         N += 1
@@ -225,8 +225,7 @@ def test_products_of_17_to_64_rows(M, N, K, epilogue):
     words = ops.mid_rows_scratch(M, N, K)
     assert (words > 0) == (K > 1024)
     scratch = torch.full((max(words, 1),), float("nan"), dtype=torch.float32, device=DEV)
-    counters = torch.zeros((N + 15) // 16, dtype=torch.int32, device=DEV)
-    kw = dict(scratch=scratch, counters=counters, force_mid_rows=True)
+    kw = dict(scratch=scratch, force_mid_rows=True)
     c0 = torch.randn(M, N, generator=g)
     for _ in range(2):
         if epilogue == "swiglu":
@@ -262,7 +261,6 @@ def test_products_of_17_to_64_rows(M, N, K, epilogue):
             ops.linear_fused(out, x.to(DEV), w.to(DEV), epilogue, **kw)
         err = (out.double().cpu() - want).abs()
         assert (err <= bound).all(), float((err / bound).max())
-        assert int(counters.abs().sum()) == 0
 
 
 @pytest.mark.parametrize("M,N,K,N2", [(1, 64, 96, 48), (8, 200, 256, 344), (16, 4096, 1024, 16400), (33, 104, 64, 72),
@@ -330,9 +328,7 @@ def test_fused_qkv_with_the_batch_in_lds(H, K, hd, half, M, d):
     from hfee_amd.kernels import ops
     N = (H + 2 * K) * hd
     scratch = torch.full((max(ops.mid_rows_scratch(M, N, d), 1),), float("nan"), dtype=torch.float32, device=DEV)
-    counters = torch.zeros((N + 15) // 16, dtype=torch.int32, device=DEV)
-    _check_fused_qkv(H, K, hd, half, M, False, d, scratch=scratch, counters=counters, force_mid_rows=True)
-    assert int(counters.abs().sum()) == 0
+    _check_fused_qkv(H, K, hd, half, M, False, d, scratch=scratch, force_mid_rows=True)
 
 
 def _check_fused_qkv(H, K, hd, half, M, norm, d, **kw):
