@@ -2,7 +2,7 @@
 // reading W once from HBM, with the neighbouring small operations folded in so that a
 // decode step of a layer is five launches instead of ten.
 //
-// A workgroup owns 16 weight rows; its eight waves split K in blocks of 128 and
+// A workgroup owns 16 weight rows; its eight waves split K in blocks of 64 and
 // stream their share of W straight from global memory into the A operand of
 // v_mfma_f32_16x16x32_bf16 (lane l: row l%16, eight consecutive k).  The batch rows are
 // the B operand.  Loads are issued one block ahead of the matrix instructions.
@@ -41,7 +41,9 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_QKV = 4 };
 
-constexpr int WAVES = 8, ROWS = 16, UNROLL = 4, KBLOCK = 32 * UNROLL;
+// (a block of 64 columns: with two blocks of a wave in flight, 256 workgroups hold 8 MB of
+// weights in flight, which measured best; with twice that, long rows (K = 14,336) stream 15% slower)
+constexpr int WAVES = 8, ROWS = 16, UNROLL = 2, KBLOCK = 32 * UNROLL;
 
 union Chunk {
   u32x4 u;
@@ -165,32 +167,41 @@ __device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
 // is on its own (nobody waits for a sum before asking for the next share), a row's four
 // lanes meet by shuffles and the waves in LDS, in an order that depends on nothing but
 // the number of shares.
+template <int TILES>
 __device__ __forceinline__ void row_scales(const Args& a, float* out) {
   __shared__ float part[WAVES][SS_STRIDE];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, j = lane >> 4;
-  const int tiles = (a.M + 15) >> 4;
-  float s[SS_STRIDE / 16];
-  const float* p[SS_STRIDE / 16];
+  float s[TILES];
+  const float* p[TILES];
 #pragma unroll
-  for (int t = 0; t < SS_STRIDE / 16; ++t) {
+  for (int t = 0; t < TILES; ++t) {
     s[t] = 0.f;
     p[t] = a.scale_ss + min(t * 16 + m16, a.M - 1);      // rows beyond M repeat the last one; nobody uses them
   }
-#pragma unroll 4
-  for (int b = wave * 4 + j; b < a.scale_blocks; b += WAVES * 4) {
+  // (no load stands under a condition: the compiler keeps a whole round of them in flight)
+  constexpr int ROUND = 8;
+  for (int b0 = wave * 4 + j; b0 < a.scale_blocks; b0 += ROUND * WAVES * 4) {
+    float v[ROUND][TILES];
 #pragma unroll
-    for (int t = 0; t < SS_STRIDE / 16; ++t)
-      if (t < tiles) s[t] += p[t][(int64_t)b * SS_STRIDE];
+    for (int r = 0; r < ROUND; ++r) {
+      const int b = min(b0 + r * WAVES * 4, a.scale_blocks - 1);       // past the end: a repeat that is not added
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) v[r][t] = p[t][(int64_t)b * SS_STRIDE];
+    }
+#pragma unroll
+    for (int r = 0; r < ROUND; ++r)
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) s[t] += b0 + r * WAVES * 4 < a.scale_blocks ? v[r][t] : 0.f;
   }
 #pragma unroll
-  for (int t = 0; t < SS_STRIDE / 16; ++t) {
+  for (int t = 0; t < TILES; ++t) {
     float v = s[t];
     v += __shfl_xor(v, 16, 64);
     v += __shfl_xor(v, 32, 64);
     if (j == 0) part[wave][t * 16 + m16] = v;
   }
   __syncthreads();
-  if (threadIdx.x < SS_STRIDE) {
+  if (threadIdx.x < TILES * 16) {
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) v += part[w][threadIdx.x];
@@ -293,7 +304,8 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_her
   __shared__ float partial[WAVES][MT][64][4];
   __shared__ float ss_part[WAVES][MT][16];
   __shared__ float row_scale[SS_STRIDE];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
   // rows_here (16, or 12 where that fills the chip more evenly): the weight rows of this
   // workgroup; with 12, the matrix instruction's last four rows repeat the twelfth and are dropped
@@ -324,19 +336,29 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_her
 
   const int nfull = a.K / KBLOCK;
   {
-    Block cur, nxt;
-    XBlock<MT, NORM> xcur, xnxt;
-    int kb = wave;
-    if (kb < nfull) load_block<MT, NORM>(cur, xcur, w_row, x_rows, a, kb * KBLOCK);
+    // Two sets of registers take turns, so that no loaded value is ever copied (a copy
+    // would wait for its load), and no load of the loop stands under a condition (the
+    // wait before a product would then count as if it had not been issued): the
+    // products of a block run while the loads of the next one are in flight.
+    Block b0, b1;
+    XBlock<MT, NORM> x0, x1;
+    const int mine = wave < nfull ? (nfull - 1 - wave) / WAVES + 1 : 0;      // whole blocks of this wave
+    if (mine > 0) load_block<MT, NORM>(b0, x0, w_row, x_rows, a, wave * KBLOCK);
     // (behind the first loads of W, so that it costs no latency of its own)
-    if (!NORM && a.scale_ss != nullptr) row_scales(a, row_scale);
-    while (kb < nfull) {
-      const int kn = kb + WAVES;
-      if (kn < nfull) load_block<MT, NORM>(nxt, xnxt, w_row, x_rows, a, kn * KBLOCK);
-      compute_block<MT, NORM>(acc, ss, cur, xcur);
-      cur = nxt;
-      xcur = xnxt;
-      kb = kn;
+    if (!NORM && a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
+    int i = 0;
+    for (; mine - i >= 3; i += 2) {
+      load_block<MT, NORM>(b1, x1, w_row, x_rows, a, (wave + (i + 1) * WAVES) * KBLOCK);
+      compute_block<MT, NORM>(acc, ss, b0, x0);
+      load_block<MT, NORM>(b0, x0, w_row, x_rows, a, (wave + (i + 2) * WAVES) * KBLOCK);
+      compute_block<MT, NORM>(acc, ss, b1, x1);
+    }
+    if (mine - i == 2) {
+      load_block<MT, NORM>(b1, x1, w_row, x_rows, a, (wave + (i + 1) * WAVES) * KBLOCK);
+      compute_block<MT, NORM>(acc, ss, b0, x0);
+      compute_block<MT, NORM>(acc, ss, b1, x1);
+    } else if (mine - i == 1) {
+      compute_block<MT, NORM>(acc, ss, b0, x0);
     }
   }
   // the last, partial block (K is a multiple of 8: whole chunks are in or out)
@@ -513,7 +535,7 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
     const int row = ((it + fill_first) % FILL) * FILL_ROWS + fill_row;
     *reinterpret_cast<u32x4*>(xs + row * MID_PITCH + fill_c * 8) = fill[it];
   }
-  if (slices == 1 && a.scale_ss != nullptr) row_scales(a, row_scale);
+  if (slices == 1 && a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
   __syncthreads();
 
   const bf16_t* x_lane = xs + r16 * MID_PITCH + g * 8;
@@ -602,7 +624,7 @@ __global__ __launch_bounds__(WAVES * 64) void mid_finish_kernel(Args a, int row_
   }
   float v[4] = {acc[0], acc[1], acc[2], acc[3]};
   if (a.scale_ss != nullptr) {
-    row_scales(a, row_scale);
+    row_scales<MT>(a, row_scale);
     __syncthreads();
     const float scale = row_scale[m];
 #pragma unroll
@@ -720,7 +742,7 @@ __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups
   for (int s = 0; s < RING; ++s) ring[s].u = *reinterpret_cast<const u32x4*>(w_cur + koff(s));
   if (!NORM && a.scale_ss != nullptr) {      // (behind the first loads of W: it costs no latency of its own)
     __shared__ float row_scale[SS_STRIDE];
-    row_scales(a, row_scale);
+    row_scales<1>(a, row_scale);
     __syncthreads();
     scale = row_scale[min(r16, a.M - 1)];
   }
