@@ -907,7 +907,7 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
   }
   // More than 16 rows and very many weight rows (gate/up): the streaming kernel would
   // read the batch again for every 16 of them; the tiled kernel takes the row scale too.
-  if (scale_ss != nullptr && M > 16 && N >= 16384 && emit_out == nullptr && epi != EPI_QKV)
+  if (scale_ss != nullptr && M > 16 && N >= 16384 && emit_out == nullptr && epi != EPI_QKV && !force_mid)
     return hfee_gemm_bf16_scaled(C, epi, ldc, A, lda, W, ldw, M, N, K, scale_ss, scale_blocks, scale_eps, stream);
   const int mt = (M + 15) / 16;
   // Where the kernels with the batch in LDS win, from fits to measured times in microseconds
