@@ -127,7 +127,8 @@ def main() -> int:
         mean_ctx = sum(lengths) / batch + steps / 2
         for r in list(sched.running):
             sched.cancel(r.request_id)
-        sched.step()
+        while sched.has_work():          # (a step launched ahead is read first; the one after frees them)
+            sched.step()
         return dt, mean_ctx
 
     def prefill_run():
@@ -184,12 +185,14 @@ def main() -> int:
         sched = Scheduler(engine, sampler, max_num_seqs=batch, max_batch_tokens=PREFILL, num_ctx=context)
         params = SamplingParams.greedy(num_predict=-1, ignore_eos=True)
         sched.add(Request(("context", 0), torch.randint(0, V, (tokens,), generator=gen).tolist(), params, seed=0))
+        sched.look_ahead = False         # (the prompt's time is not to hold a decode step launched behind it)
         torch.cuda.synchronize()
         t = time.perf_counter()
         while not sched.running or not sched.running[0].decoding:
             sched.step()
         torch.cuda.synchronize()
         prefill_s = time.perf_counter() - t
+        sched.look_ahead = True
         for i in range(1, batch):
             sched.add(Request(("context", i), torch.randint(0, V, (tokens,), generator=gen).tolist(), params, seed=i))
         while any(not r.decoding for r in list(sched.running) + list(sched.waiting)):
@@ -208,7 +211,8 @@ def main() -> int:
         assert made == batch * steps and len(lengths) == batch and min(lengths) >= tokens, (made, lengths)
         for r in list(sched.running):
             sched.cancel(r.request_id)
-        sched.step()
+        while sched.has_work():          # (a step launched ahead is read first; the one after frees them)
+            sched.step()
         return prefill_s, dt
 
     if args.context:

@@ -27,6 +27,18 @@ there.  Here they can, and this is what happens:
      stream goes on where it was, so the tokens it produces are the same);
   4. a request that is alone and still cannot get a page finishes with "length".
 The request admitted first is never preempted, so every step makes progress.
+
+One step ahead.  While every running request only decodes, the next step is known but
+for its tokens, and those lie on the device as soon as the sampler has run.  The
+scheduler then launches step t+1 (its tokens taken from the sampler's output on the
+device) before it reads the tokens of step t: the GPU goes from one step to the next
+without waiting for the host.  If a request turns out to have ended at step t (an
+end-of-sequence token, a stop from its callback), the token that step t+1 made for it
+is dropped; its pages were still its own when that step was queued, and whoever gets
+them next runs after it on the same stream.  Nothing is launched ahead when a request
+waits, a prompt is unfinished, a request is at its limit of tokens or of context, is
+cancelled, samples with a penalty on its own earlier tokens (the host has not seen the
+latest one yet), or when pages are short: then the step is an ordinary one.
 """
 from __future__ import annotations
 
@@ -94,6 +106,9 @@ class Scheduler:
         self.running: list = []          # in admission order
         self._order = 0
         self.last_batch: list = []       # (request_id, tokens in the step) of the latest step, for tests
+        self._ahead = None               # a step that runs already: (owners of its rows, handle of its ids)
+        self.steps_ahead = 0             # how many steps were launched before their tokens were known
+        self.look_ahead = bool(getattr(engine, "takes_device_tokens", False)) and hasattr(sampler, "device_ids")
 
     # ----------------------------------------------------------------- intake
     def add(self, request: Request) -> None:
@@ -109,7 +124,7 @@ class Scheduler:
         self.waiting.append(request)
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.waiting or self.running)       # (a step launched ahead for nobody is just dropped)
 
     def cancel(self, request_id) -> None:
         for r in list(self.waiting) + self.running:
@@ -146,31 +161,63 @@ class Scheduler:
             self.running.remove(request)
         finished.append(Finished(request, reason, error))
 
-    def _plan_ahead(self, batch) -> None:
-        """If the next step can only be "every request of this one decodes one more token"
-        (nobody waits for a place, no prompt is unfinished, nobody reaches its limit of
-        tokens, nobody is at the end of the context), the engine plans that step now, while the
-        GPU is busy with this one.  A guess that fails (an end-of-sequence token, a
-        cancellation) costs nothing but the planning."""
-        if self.waiting or len(batch) != len(self.running):
-            return
+    def _decode_shape(self, owners, ahead: bool):
+        """The shape of the next step if it can only be "each of these requests, which are all
+        that run, decodes one more token" (nobody waits for a place, no prompt is unfinished,
+        nobody reaches its limit of tokens, nobody is at the end of the context or cancelled;
+        `ahead`: and nobody's sampling reads its own earlier tokens), else None."""
+        if self.waiting or len(owners) != len(self.running):
+            return None
         shape = []
-        for (r, toks, want), q in zip(batch, self.running):
-            if r is not q or not want or len(r.feed) != 0 or r.cancelled:
-                return
+        for r, q in zip(owners, self.running):
+            if r is not q or len(r.feed) != 0 or r.cancelled:
+                return None
+            if ahead and self.sampler.needs_history(r.params):
+                return None
             limit = r.params.num_predict
             if limit >= 0 and len(r.generated) + 1 >= limit:
-                return
+                return None
             if self.cache.get(r.request_id).length + 1 > self.num_ctx:
-                return
+                return None
             shape.append((r.request_id, 1, [0]))
-        self.engine.prepare(shape)
+        return shape
+
+    def _plan_ahead(self, owners) -> None:
+        """If the next step is certain but for its tokens, the engine plans it now, while the
+        GPU is busy with this one.  A guess that fails (an end-of-sequence token, a
+        cancellation) costs nothing but the planning."""
+        shape = self._decode_shape(owners, ahead=False)
+        if shape:
+            self.engine.prepare(shape)
+
+    def _launch_ahead(self, owners):
+        """Launches the step after the one whose ids are still on their way, if it is certain
+        but for its tokens: they are taken from the sampler's output on the device.
+        Returns (owners, handle of the ids) or None."""
+        shape = self._decode_shape(owners, ahead=True) if self.look_ahead else None
+        if not shape or not self.engine.prepare(shape):
+            return None                                  # (pages are short: an ordinary step decides what gives)
+        entries = [StepEntry(rid, [0], [0]) for rid, _, _ in shape]
+        self.last_batch = [(rid, 1) for rid, _, _ in shape]
+        logits = self.engine.step(entries, tokens_from=self.sampler.device_ids)
+        # (a request's draw counter moves when its token is read: this step's draw is the one after)
+        rows = [SampleRow(r.params, r.seed, r.draws + 1, r.history, i) for i, r in enumerate(owners)]
+        self.steps_ahead += 1
+        return owners, self.sampler.launch(logits, rows)
 
     # ------------------------------------------------------------------- step
     def step(self) -> list:
         """One pass: admit, batch, run, sample.  Returns the requests that finished."""
         finished: list = []
+        if self._ahead is not None:              # this pass's step runs already
+            launched, self._ahead = self._ahead, None
+            return self._collect(*launched, finished)
+        launched = self._launch(finished)
+        return self._collect(*launched, finished) if launched else finished
 
+    def _launch(self, finished: list):
+        """Admits, batches, runs a step and starts its sampling: (owners of the sampled rows,
+        handle of their ids), or None if no step ran."""
         # cancelled or out of context (runner.go:244-251)
         for r in list(self.running):
             if r.cancelled:
@@ -256,7 +303,7 @@ class Scheduler:
                     self._finish(self.running[0], "length", finished,
                                  "the cache cannot hold this request even alone")
             self.last_batch = []
-            return finished
+            return None
 
         entries = [StepEntry(r.request_id, toks, [len(toks) - 1] if want else []) for r, toks, want in batch]
         self.last_batch = [(r.request_id, len(toks)) for r, toks, _ in batch]
@@ -268,11 +315,20 @@ class Scheduler:
             if want:
                 owners.append(r)
                 rows.append(SampleRow(r.params, r.seed, r.draws, r.history, len(rows)))
-        pending = self.sampler.launch(logits, rows)
-        self._plan_ahead(batch)          # while the GPU runs this step
+        return owners, self.sampler.launch(logits, rows)
+
+    def _collect(self, owners, pending, finished: list) -> list:
+        """Reads the ids of a step that runs (after launching the step behind it, if that one
+        is certain) and gives each request its token."""
+        self._ahead = self._launch_ahead(owners)
+        if self._ahead is None:
+            self._plan_ahead(owners)     # while the GPU runs this step
+        fed_ahead = set(id(r) for r in self._ahead[0]) if self._ahead else ()
         ids = self.sampler.collect(pending)
         now = self.clock()
         for r, token in zip(owners, ids):
+            if r not in self.running:
+                continue                 # it ended at the step before; this token was made for nobody
             if not r.decoding:
                 r.decoding = True
                 if not r.eval_started:
@@ -292,6 +348,8 @@ class Scheduler:
                 self._finish(r, "stop", finished)
             elif r.params.num_predict >= 0 and len(r.generated) >= r.params.num_predict:
                 self._finish(r, "length", finished)
-            else:
-                r.feed = [token]
+            elif id(r) not in fed_ahead:
+                r.feed = [token]         # (else the step that runs already took it on the device)
+        if self._ahead and not any(r in self.running for r in self._ahead[0]):
+            self._ahead = None           # everybody ended: what the step ahead makes is for nobody
         return finished

@@ -49,6 +49,8 @@ class StepPlan:
 class Engine:
     """Model + cache + workspace on one GPU, and step()."""
 
+    takes_device_tokens = True      # step(..., tokens_from=) is there
+
     def __init__(self, model: Model, *, num_pages=None, cache_tokens=None, page_size: int = 16,
                  max_requests: int = 64, max_batch_tokens: int = 2048, num_positions: int | None = None,
                  device="cuda:0", use_graphs: bool = True):
@@ -270,11 +272,11 @@ class Engine:
         self._prepared = (self._signature(shape), plan)
         return True
 
-    def begin(self, entries):
+    def begin(self, entries, tokens_from=None):
         """Checks the entries, takes their pages, sends the step's metadata to the
         device and returns (context, number of wanted rows, key for graph capture or
         None).  step() is begin + the model + commit; tests of single parts call
-        begin() themselves."""
+        begin() themselves.  tokens_from: see step()."""
         entries = list(entries)
         self._check(entries)
         self._reserve(entries)
@@ -287,6 +289,10 @@ class Engine:
             plan = self._plan(shape)
         tokens = entries[0].tokens if len(entries) == 1 else [t for e in entries for t in e.tokens]
         dev = self._upload(plan, tokens)
+        if tokens_from is not None:
+            if tokens_from.dtype != torch.int32 or tokens_from.device != self.device or tokens_from.numel() < plan.n:
+                raise StepError("tokens_from must be int32 on the engine's device, one id a row of the step")
+            dev["token_ids"].copy_(tokens_from[:plan.n])        # on the stream, behind the metadata
         ctx = StepContext(
             n=plan.n, dtype=self.dtype, device=self.device, segments=plan.segments,
             token_ids=dev["token_ids"], positions=dev["positions"], token_segment=dev["token_segment"],
@@ -302,12 +308,18 @@ class Engine:
             self.cache.commit(e.request_id, len(e.tokens))
         self.steps_run += 1
 
-    def step(self, entries) -> torch.Tensor:
+    def step(self, entries, tokens_from=None) -> torch.Tensor:
         """Runs the entries as one batch; returns float32 logits [wanted, vocab] in the
         order of the entries and of each entry's `want` (None if nothing is wanted).
-        The tensor is a view of the workspace: the next step overwrites it."""
+        The tensor is a view of the workspace: the next step overwrites it.
+
+        tokens_from: an int32 tensor on the device that holds the step's token ids, one a
+        row, when the step runs (work queued on the stream before this call may still be
+        writing it); the entries' own tokens then only say how many there are.  For a
+        caller that launches a step before the host has seen the tokens that the step
+        before sampled."""
         entries = list(entries)
-        ctx, w, key = self.begin(entries)
+        ctx, w, key = self.begin(entries, tokens_from)
         n, dev = ctx.n, ctx.extra
         if key is not None:
             graph = self._graphs.get(key)

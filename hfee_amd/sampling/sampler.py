@@ -68,9 +68,23 @@ class Sampler:
     def __init__(self, vocab: int, device, max_rows: int):
         self.vocab, self.device, self.max_rows = vocab, device, max_rows
         self._out = torch.empty(max_rows, dtype=torch.int32, device=device)
-        self._host = torch.empty(max_rows, dtype=torch.int32, pin_memory=True)
-        self._done = torch.cuda.Event()
+        # two places for the ids on the host, taken in turn: a caller may launch the next
+        # sampling before it has collected this one
+        self._slots = [(torch.empty(max_rows, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+                       for _ in range(2)]
+        self._turn = 0
         self._scratch = None
+
+    @property
+    def device_ids(self) -> torch.Tensor:
+        """The ids of the latest launch(), on the device, in the order of its rows: a step that
+        is launched before they are collected can take its tokens from here."""
+        return self._out
+
+    @staticmethod
+    def needs_history(params: SamplingParams) -> bool:
+        """Whether sampling with these options reads the request's earlier tokens."""
+        return params.repeat_penalty != 1 and params.repeat_last_n != 0
 
     def sample(self, logits: torch.Tensor, rows) -> list:
         """logits: float32 [*, vocab] on the device (changed in place by the repeat
@@ -82,11 +96,10 @@ class Sampler:
         do other work on the host between the two while the GPU runs."""
         n = len(rows)
         if n == 0:
-            return 0
+            return (0, 0)
         if n > self.max_rows:
             raise ValueError(f"{n} rows to sample, the sampler was made for {self.max_rows}")
-        plain_greedy = all(r.params.temperature <= 0 and (r.params.repeat_penalty == 1 or r.params.repeat_last_n == 0)
-                           for r in rows)
+        plain_greedy = all(r.params.temperature <= 0 and not self.needs_history(r.params) for r in rows)
         if plain_greedy and [r.logits_row for r in rows] == list(range(logits.shape[0])):
             ops.argmax(self._out, logits)
         else:
@@ -96,13 +109,18 @@ class Sampler:
             dparams = torch.from_numpy(params).to(self.device)
             dhist = torch.from_numpy(hist).to(self.device)
             ops.sample(self._out, logits, dparams, dhist, self._scratch)
-        self._host[:n].copy_(self._out[:n], non_blocking=True)
-        self._done.record()
-        return n
+        slot = self._turn
+        self._turn ^= 1
+        host, done = self._slots[slot]
+        host[:n].copy_(self._out[:n], non_blocking=True)
+        done.record()
+        return (n, slot)
 
-    def collect(self, n: int) -> list:
-        """Waits for the ids of the last launch()."""
+    def collect(self, pending) -> list:
+        """Waits for the ids of a launch() (the latest one or the one before it)."""
+        n, slot = pending
         if n == 0:
             return []
-        self._done.synchronize()
-        return self._host[:n].tolist()
+        host, done = self._slots[slot]
+        done.synchronize()
+        return host[:n].tolist()

@@ -134,3 +134,38 @@ def test_the_command_line_generates_from_token_ids(model_folders):
     p = subprocess.run([sys.executable, os.path.join(root, "bin", "hfee"), "run", folder, "--dtype", "float32"],
                        capture_output=True, text=True, timeout=300, stdin=subprocess.DEVNULL)
     assert p.returncode == 1 and "usage" in p.stderr
+
+
+@pytest.mark.parametrize("dtype,temperature", [("float32", 0.0), ("bfloat16", 0.0), ("float32", 0.7)])
+def test_steps_launched_ahead_give_the_tokens_of_steps_that_wait(model_folders, dtype, temperature):
+    """The scheduler launches a decode step before it has read the ids of the step before
+    (they go from the sampler to the embedding on the device).  With that switched off the
+    same requests give the same tokens and reasons: greedy and seeded sampling, requests of
+    different lengths of which some end early on an end-of-sequence id, so that steps that
+    were launched ahead for them run for nobody."""
+    from hfee_amd import LLM, SamplingParams
+    folder = model_folders[("A", dtype)]
+    prompts = list(tu.make_requests(256, [5, 17, 32, 1], seed=7).values())
+
+    def run(look_ahead, eos=None):
+        llm = LLM(folder, dtype=dtype, num_ctx=128, num_parallel=4, max_batch_tokens=24)
+        assert llm.scheduler.look_ahead
+        llm.scheduler.look_ahead = look_ahead
+        if eos is not None:
+            llm.scheduler.eos = {eos}
+        params = [SamplingParams(temperature=temperature, top_k=0, top_p=1.0, repeat_penalty=1.0, seed=50 + i,
+                                 num_predict=n) for i, n in enumerate([40, 12, 33, 25])]
+        outs = llm.generate(prompts, params)
+        llm.engine.cache.check()
+        assert not llm.engine.cache.requests
+        return [(o.token_ids, o.done_reason) for o in outs], llm.scheduler.steps_ahead
+
+    waited, none_ahead = run(False)
+    assert none_ahead == 0
+    # an id that the longest request samples in its middle: with it as end-of-sequence id that request stops early
+    eos = waited[0][0][20]
+    waited, _ = run(False, eos)
+    assert any(reason == "stop" for _, reason in waited)
+    ahead, launched_ahead = run(True, eos)
+    assert launched_ahead > 10
+    assert ahead == waited

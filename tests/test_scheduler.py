@@ -259,3 +259,110 @@ def test_decode_steps_are_announced_ahead_and_a_wrong_guess_costs_nothing():
     done2 = run_all(s2)
     assert all(done2[k].request.generated == done[k].request.generated for k in "abc")
     assert eng2.batches == eng.batches
+
+
+class DeviceTokenEngine(FakeEngine):
+    """A fake engine that, like the real one, can take a step's tokens from where the sampler
+    left them (here: the sampler's list, read when the step runs)."""
+    takes_device_tokens = True
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.device_fed_steps = 0
+
+    def step(self, entries, tokens_from=None):
+        if tokens_from is not None:
+            assert all(len(e.tokens) == 1 for e in entries) and len(tokens_from) >= len(entries)
+            entries = [type(e)(e.request_id, [tokens_from[i]], e.want) for i, e in enumerate(entries)]
+            self.device_fed_steps += 1
+        return super().step(entries)
+
+
+class DeviceIdsSampler(FakeSampler):
+    """Keeps the ids of its latest launch "on the device"; what a launch returns can be
+    collected after the launch that follows it."""
+
+    def __init__(self):
+        self.device_ids = []
+
+    @staticmethod
+    def needs_history(params):
+        return params.repeat_penalty != 1 and params.repeat_last_n != 0
+
+    def launch(self, logits, rows):
+        out = []
+        for r in rows:
+            seen = logits[r.logits_row]
+            # the host may be one token behind the cache: the token that this step was fed on the device
+            assert list(seen[:len(r.history)]) == list(r.history) and len(seen) - len(r.history) in (0, 1)
+            h = hashlib.sha256(repr((seen, r.seed, r.draw)).encode()).digest()
+            out.append(h[0] % (VOCAB - 1))
+        self.device_ids[:] = out
+        return list(out)
+
+
+def run_staggered(engine, sampler, arrivals, eos=(), **kw):
+    s = Scheduler(engine, sampler, max_num_seqs=kw.get("seqs", 4), max_batch_tokens=kw.get("budget", 32),
+                  num_ctx=kw.get("ctx", 256), eos_token_ids=eos, clock=lambda: 0.0)
+    done, calls = {}, 0
+    while arrivals or s.has_work():
+        for r in arrivals.pop(calls, []):
+            s.add(r)
+        for f in s.step():
+            done[f.request.request_id] = f
+        calls += 1
+        assert calls < 5000
+    return s, done
+
+
+def staggered_requests(params_of):
+    ps = prompts()
+    return {0: [Request(i, ps[i], params_of(i), seed=i) for i in (0, 1)],
+            9: [Request(2, ps[2], params_of(2), seed=2)],
+            30: [Request(4, ps[4], params_of(4), seed=4), Request(5, ps[5], params_of(5), seed=5)]}
+
+
+@pytest.mark.parametrize("pages", [64, 14])
+def test_steps_launched_ahead_give_the_same_tokens_and_reasons(pages):
+    """With an engine that takes tokens from the device, decode steps are launched before the
+    ids of the step before are read.  Tokens, finish reasons and the order of each request's
+    steps are those of the scheduler that waits for every step: also when a request ends on
+    an end-of-sequence id (the token made ahead for it is dropped), when requests arrive in
+    between, when limits of tokens are reached, and when pages are short (then nothing is
+    launched ahead that needs a page that is not there)."""
+    limits = {0: 40, 1: 9, 2: 25, 4: 33, 5: 12}
+    params_of = lambda i: SamplingParams.greedy(num_predict=limits[i])
+    plain_engine = FakeEngine(pages, 4)
+    _, plain = run_staggered(plain_engine, FakeSampler(), staggered_requests(params_of))
+    # an end-of-sequence id that some request meets on its way, so that a step ahead runs for nobody
+    tokens = [t for f in plain.values() for t in f.request.generated[3:-3]]
+    eos = max(set(tokens), key=tokens.count)
+    _, plain = run_staggered(FakeEngine(pages, 4), FakeSampler(), staggered_requests(params_of), eos=[eos])
+    assert any(f.reason == "stop" for f in plain.values())
+    engine = DeviceTokenEngine(pages, 4)
+    sched, ahead = run_staggered(engine, DeviceIdsSampler(), staggered_requests(params_of), eos=[eos])
+    assert sched.steps_ahead > 10 and engine.device_fed_steps == sched.steps_ahead
+    assert set(ahead) == set(plain)
+    for rid in plain:
+        assert ahead[rid].request.generated == plain[rid].request.generated, rid
+        assert ahead[rid].reason == plain[rid].reason
+    assert engine.cache.free_pages() == [pages] and not engine.cache.requests
+    engine.cache.check()
+
+
+def test_nothing_is_launched_ahead_when_sampling_reads_the_history_or_a_request_is_cancelled():
+    ps = prompts()
+    engine = DeviceTokenEngine(64, 4)
+    s = Scheduler(engine, DeviceIdsSampler(), max_num_seqs=4, max_batch_tokens=32, num_ctx=256, clock=lambda: 0.0)
+    s.add(Request(0, ps[0], SamplingParams(temperature=0.0, repeat_penalty=1.1, num_predict=12), seed=0))
+    run_all(s)
+    assert s.steps_ahead == 0          # the penalty needs the token that the host has not seen yet
+    s.add(Request(1, ps[1], SamplingParams.greedy(num_predict=50), seed=1))
+    for _ in range(8):
+        s.step()
+    assert s.steps_ahead > 0
+    s.cancel(1)
+    before = s.steps_ahead
+    done = run_all(s)
+    assert done[1].reason == "cancelled" and s.steps_ahead <= before + 1
+    assert engine.cache.free_pages() == [64]
