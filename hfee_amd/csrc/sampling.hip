@@ -84,7 +84,7 @@ __device__ __forceinline__ MaxIdx better(MaxIdx a, MaxIdx b) {   // greater valu
   return a;
 }
 
-__device__ MaxIdx block_argmax(const float* __restrict__ lg, int V, MaxIdx* scratch) {
+__device__ MaxIdx block_argmax_raw(const float* __restrict__ lg, int V, MaxIdx* scratch) {
   MaxIdx best{-INFINITY, 0x7fffffff};
   const int stride = blockDim.x;
   int j = threadIdx.x;
@@ -111,7 +111,12 @@ __device__ MaxIdx block_argmax(const float* __restrict__ lg, int V, MaxIdx* scra
   __syncthreads();
   MaxIdx r = scratch[0];
   for (int w = 1; w < (int)(blockDim.x + 63) / 64; ++w) r = better(r, scratch[w]);
-  if (r.i == 0x7fffffff) r.i = 0;   // every logit is NaN or -inf
+  return r;                         // id 0x7fffffff: every logit is NaN or -inf
+}
+
+__device__ MaxIdx block_argmax(const float* __restrict__ lg, int V, MaxIdx* scratch) {
+  MaxIdx r = block_argmax_raw(lg, V, scratch);
+  if (r.i == 0x7fffffff) r.i = 0;
   return r;
 }
 
@@ -120,6 +125,53 @@ __global__ __launch_bounds__(THREADS) void argmax_kernel(int* __restrict__ out, 
   __shared__ MaxIdx scratch[16];
   const MaxIdx r = block_argmax(logits + (int64_t)blockIdx.x * ld, V, scratch);
   if (threadIdx.x == 0) out[blockIdx.x] = r.i;
+}
+
+// A row over `parts` workgroups, so that a few rows still use the whole chip: each
+// leaves the first maximum of its stretch in `partial`, counts itself, and the one that
+// arrives last takes the best of them (greater value, then smaller id: the same id whatever
+// the order of arrival) and sets the counter back to zero.
+constexpr int ARGMAX_THREADS = 256;
+
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(int* __restrict__ out,
+                                                                      const float* __restrict__ logits, int64_t ld,
+                                                                      int V, int parts, MaxIdx* __restrict__ partial,
+                                                                      int* __restrict__ counters) {
+  __shared__ MaxIdx scratch[16];
+  __shared__ int last;
+  const int row = blockIdx.x / parts, part = blockIdx.x - row * parts;
+  const int stretch = (V + parts - 1) / parts;
+  const int j0 = min(V, part * stretch), j1 = min(V, j0 + stretch);
+  MaxIdx r = block_argmax_raw(logits + (int64_t)row * ld + j0, j1 - j0, scratch);
+  if (threadIdx.x == 0) {
+    if (r.i != 0x7fffffff) r.i += j0;
+    MaxIdx* mine = partial + (int64_t)row * parts + part;
+    __hip_atomic_store(&mine->v, r.v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&mine->i, r.i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = __hip_atomic_fetch_add(counters + row, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == parts - 1;
+  }
+  __syncthreads();
+  if (!last) return;
+  MaxIdx best{-INFINITY, 0x7fffffff};
+  for (int p = threadIdx.x; p < parts; p += ARGMAX_THREADS) {
+    const MaxIdx* theirs = partial + (int64_t)row * parts + p;
+    MaxIdx o{__hip_atomic_load(&theirs->v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
+             __hip_atomic_load(&theirs->i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)};
+    best = better(best, o);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    MaxIdx o{__shfl_xor(best.v, off, 64), __shfl_xor(best.i, off, 64)};
+    best = better(best, o);
+  }
+  __syncthreads();                                   // (block_argmax_raw's use of scratch is over)
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < ARGMAX_THREADS / 64; ++w) best = better(best, scratch[w]);
+    out[row] = best.i == 0x7fffffff ? 0 : best.i;
+    __hip_atomic_store(counters + row, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, float* __restrict__ logits,
@@ -305,10 +357,23 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
 
 }  // namespace
 
-HFEE_API int hfee_argmax(int* out, const float* logits, int64_t ld, int rows, int V, hipStream_t stream) {
+// partial (rows x 64 pairs of 32-bit words) and counters (rows int32 that are zero, and are
+// zero again afterwards) let a row be spread over up to 64 workgroups; without them one
+// workgroup takes a row.
+HFEE_API int hfee_argmax(int* out, const float* logits, int64_t ld, int rows, int V, void* partial,
+                         int64_t partial_pairs, int* counters, int num_counters, hipStream_t stream) {
   HFEE_REQUIRE(rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d", rows, V);
   if (rows == 0) return 0;
-  argmax_kernel<<<rows, THREADS, 0, stream>>>(out, logits, ld, V);
+  // as many workgroups as fill the chip once, each with at least 2,048 logits
+  int parts = 256 / rows;
+  if (parts > V / 2048) parts = V / 2048;
+  if (parts > 64) parts = 64;
+  if (parts > 1 && partial != nullptr && counters != nullptr && partial_pairs >= (int64_t)rows * parts &&
+      num_counters >= rows) {
+    argmax_parts_kernel<<<rows * parts, ARGMAX_THREADS, 0, stream>>>(out, logits, ld, V, parts, (MaxIdx*)partial, counters);
+  } else {
+    argmax_kernel<<<rows, THREADS, 0, stream>>>(out, logits, ld, V);
+  }
   HFEE_CHECK_LAUNCH("argmax");
   return 0;
 }

@@ -218,13 +218,24 @@ def attention_plain(out, q, cache_layer, positions, token_segment, block_tables,
 
 # ------------------------------------------------------------------- sampling
 
-def argmax(out: torch.Tensor, logits: torch.Tensor):
-    """out[r] = id of the first maximum of logits[r]."""
-    _gpu(out, logits)
+ARGMAX_PARTS = 64
+
+
+def argmax(out: torch.Tensor, logits: torch.Tensor, partial=None, counters=None):
+    """out[r] = id of the first maximum of logits[r].  partial (float32, rows x ARGMAX_PARTS x 2)
+    and counters (int32 zeros, one a row; zero again afterwards) let the kernel spread a row
+    over several workgroups."""
+    _gpu(out, logits, partial, counters)
     rows, V, ld = _rows2d(logits, "argmax logits")
     _check(logits.dtype == torch.float32, "argmax: float32 logits")
     _i32(out, "argmax out", rows)
-    lib.core().call("hfee_argmax", _ptr(out), _ptr(logits), ld, rows, V, _stream())
+    if partial is not None or counters is not None:
+        _check(partial is not None and counters is not None and partial.dtype == torch.float32
+               and partial.is_contiguous() and counters.dtype == torch.int32 and counters.is_contiguous(),
+               "argmax: float32 partial results and int32 counters go together")
+    lib.core().call("hfee_argmax", _ptr(out), _ptr(logits), ld, rows, V, _ptr(partial),
+                    0 if partial is None else partial.numel() // 2, _ptr(counters),
+                    0 if counters is None else counters.numel(), _stream())
 
 
 def sample(out: torch.Tensor, logits: torch.Tensor, params: torch.Tensor, history: torch.Tensor,

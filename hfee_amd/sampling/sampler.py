@@ -74,6 +74,9 @@ class Sampler:
                        for _ in range(2)]
         self._turn = 0
         self._scratch = None
+        # for the argmax over several workgroups a row
+        self._partial = torch.empty(max_rows * ops.ARGMAX_PARTS * 2, dtype=torch.float32, device=device)
+        self._counters = torch.zeros(max_rows, dtype=torch.int32, device=device)
 
     @property
     def device_ids(self) -> torch.Tensor:
@@ -101,7 +104,7 @@ class Sampler:
             raise ValueError(f"{n} rows to sample, the sampler was made for {self.max_rows}")
         plain_greedy = all(r.params.temperature <= 0 and not self.needs_history(r.params) for r in rows)
         if plain_greedy and [r.logits_row for r in rows] == list(range(logits.shape[0])):
-            ops.argmax(self._out, logits)
+            ops.argmax(self._out, logits, self._partial, self._counters)
         else:
             params, hist = pack_rows(rows)
             if self._scratch is None:

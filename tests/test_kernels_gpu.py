@@ -526,6 +526,36 @@ def test_argmax_first_maximum_wins():
     assert out.tolist() == [17, 4999, 0]
 
 
+@pytest.mark.parametrize("rows,V", [(1, 128256), (8, 128256), (3, 5000), (64, 33000), (5, 2048 * 3 + 5), (200, 9000)])
+def test_argmax_over_several_workgroups_a_row(rows, V):
+    """With partial results and counters the kernel spreads a row over workgroups and the last
+    one to arrive takes the best: the first maximum still wins, across the stretches too;
+    twice on the same counters; rows of -inf and NaN give id 0 as with one workgroup."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(rows + V)
+    logits = torch.randn(rows, V, generator=g)
+    top = logits.max().item() + 1
+    for r in range(rows):
+        a, b = sorted(torch.randint(0, V, (2,), generator=g).tolist())
+        logits[r, a] = top
+        logits[r, b] = top               # equal maxima, mostly in different stretches: the first one
+    if rows > 2:
+        logits[1] = float("-inf")
+        logits[2] = float("nan")
+    want = [int(torch.nonzero(row == row.max())[0]) if torch.isfinite(row.max()) else 0 for row in logits]
+    dev = logits.to(DEV)
+    partial = torch.full((rows * ops.ARGMAX_PARTS * 2,), float("nan"), device=DEV)
+    counters = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    single = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    ops.argmax(single, dev)
+    assert single.tolist() == want
+    for _ in range(2):
+        out = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        ops.argmax(out, dev, partial, counters)
+        assert out.tolist() == want
+        assert int(counters.abs().sum()) == 0
+
+
 @pytest.mark.parametrize("H,K,hd,ps,ctx", [(8, 2, 128, 16, 9000), (4, 1, 64, 16, 5000), (8, 2, 128, 32, 6000)])
 def test_attention_over_long_contexts(H, K, hd, ps, ctx):
     """Thousands of keys: the block table no longer fits the 64 entries that a wave holds at
