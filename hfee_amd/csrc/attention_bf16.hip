@@ -538,15 +538,33 @@ __device__ __forceinline__ float read_partial(const float* p) {
   else return *p;
 }
 
+// (The splits' outputs are asked for eight splits at a time, the first eight together with
+// the maxima and sums: a join of up to eight splits costs one latency, not one a split.)
 template <bool COHERENT>
 __device__ __forceinline__ void combine_head(bf16_t* __restrict__ orow, const float* __restrict__ pr, int num_splits) {
+  constexpr int NJ = (HD + 63) / 64, TOGETHER = 8;
   const int lane = threadIdx.x & 63;
   float m = -INFINITY, l = 0.f;
-  float o[(HD + 63) / 64];
+  float o[NJ];
 #pragma unroll
-  for (int j = 0; j < (HD + 63) / 64; ++j) o[j] = 0.f;
+  for (int j = 0; j < NJ; ++j) o[j] = 0.f;
+  auto fetch = [&](float (&part)[TOGETHER][NJ], int first, int last) {     // splits first .. first+7, none beyond `last`
+#pragma unroll
+    for (int u = 0; u < TOGETHER; ++u) {
+      const float* src = pr + (int64_t)min(first + u, last) * (HD + 2);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int d = lane + 64 * j;                      // (no load under a condition: they all go out together)
+        const float v = read_partial<COHERENT>(src + min(d, HD - 1));
+        part[u][j] = d < HD ? v : 0.f;
+      }
+    }
+  };
   for (int s0 = 0; s0 < num_splits; s0 += 64) {          // 64 splits at a time
     const int mine = s0 + lane;
+    const int count = min(64, num_splits - s0);
+    float part[TOGETHER][NJ];
+    fetch(part, s0, s0 + count - 1);
     const float ms = mine < num_splits ? read_partial<COHERENT>(pr + (int64_t)mine * (HD + 2) + HD) : -INFINITY;
     const float ls = mine < num_splits ? read_partial<COHERENT>(pr + (int64_t)mine * (HD + 2) + HD + 1) : 0.f;
     const float m_new = fmaxf(m, wave_max(ms));
@@ -555,21 +573,23 @@ __device__ __forceinline__ void combine_head(bf16_t* __restrict__ orow, const fl
     const float f = exp2f(ms - m_use);                    // this lane's split weight
     l = l * rescale + wave_sum(ls * f);
 #pragma unroll
-    for (int j = 0; j < (HD + 63) / 64; ++j) o[j] *= rescale;
-    const int count = min(64, num_splits - s0);
-    for (int s = 0; s < count; ++s) {
-      const float fs = __shfl(f, s, 64);
+    for (int j = 0; j < NJ; ++j) o[j] *= rescale;
+    for (int c0 = 0; c0 < count; c0 += TOGETHER) {
+      if (c0 > 0) fetch(part, s0 + c0, s0 + count - 1);
 #pragma unroll
-      for (int j = 0; j < (HD + 63) / 64; ++j) {
-        const int d = lane + 64 * j;
-        if (d < HD) o[j] += read_partial<COHERENT>(pr + (int64_t)(s0 + s) * (HD + 2) + d) * fs;
+      for (int u = 0; u < TOGETHER; ++u) {
+        const float fs = __shfl(f, min(c0 + u, 63), 64);
+        if (c0 + u < count) {                             // in the order of the splits
+#pragma unroll
+          for (int j = 0; j < NJ; ++j) o[j] += part[u][j] * fs;
+        }
       }
     }
     m = m_new;
   }
   const float inv = 1.0f / l;
 #pragma unroll
-  for (int j = 0; j < (HD + 63) / 64; ++j) {
+  for (int j = 0; j < NJ; ++j) {
     const int d = lane + 64 * j;
     if (d < HD) orow[d] = float_to_bf16(o[j] * inv);
   }
@@ -595,8 +615,10 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
   const int sidx = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int group = num_heads / lay.kv_heads;
   const int slots = min(group, 32);
-  const int row = seg_rows[sidx], pos = seg_positions[sidx];
-  const int* bt = block_tables + (int64_t)seg_tables[sidx] * bt_stride;
+  // (without seg_rows and seg_tables, segment i is row i with block table i: the block table's
+  // address then waits for no load, and the chain to the first key is one latency shorter)
+  const int row = seg_rows != nullptr ? seg_rows[sidx] : sidx, pos = seg_positions[sidx];
+  const int* bt = block_tables + (int64_t)(seg_tables != nullptr ? seg_tables[sidx] : sidx) * bt_stride;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
 
   // key tiles of this split: a contiguous share of the tiles lo/32 .. pos/32
@@ -700,7 +722,7 @@ __global__ __launch_bounds__(64) void combine_kernel(bf16_t* __restrict__ out, i
                                                      const float* __restrict__ partial, int num_heads,
                                                      int num_splits) {
   const int sidx = blockIdx.x, h = blockIdx.y;
-  combine_head<false>(out + (int64_t)seg_rows[sidx] * ld_out + h * HD,
+  combine_head<false>(out + (int64_t)(seg_rows != nullptr ? seg_rows[sidx] : sidx) * ld_out + h * HD,
                       partial + (int64_t)(sidx * num_heads + h) * num_splits * (HD + 2), num_splits);
 }
 
@@ -768,7 +790,8 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
 }
 
 // seg_rows / seg_positions / seg_tables: per decode segment its row in the batch,
-// its position and its block-table row.  partial: at least
+// its position and its block-table row (seg_rows or seg_tables null: segment i is row i,
+// has block table i).  partial: at least
 // num_segments * num_heads * num_splits * (head_dim + 2) floats when num_splits > 1.
 // counters: null, or at least num_segments * kv_heads int32 that are zero (and are zero
 // again when the kernel has run): the splits are then joined by the workgroup that
@@ -781,6 +804,7 @@ HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q
                                         int* counters, int num_counters, hipStream_t stream) {
   HFEE_REQUIRE(num_segments >= 0, "attention_bf16_decode: bad segment count");
   if (num_segments == 0) return 0;
+  HFEE_REQUIRE(seg_positions != nullptr, "attention_bf16_decode: the segments' positions are missing");
   CacheLayout lay;
   if (check_common("attention_bf16_decode", ld_out, ldq, num_heads, kv_heads, page_size, window, scale, out, q, &lay))
     return 1;

@@ -291,12 +291,20 @@ def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tabl
     shares the keys of one (segment, KV head, split) and joins them in LDS; with
     num_splits > 1 the splits are joined by a second kernel, or, given `counters` (at
     least segments x kv_heads int32 that are zero, and are zero again afterwards), by
-    the workgroup of each (segment, KV head) that finishes last."""
+    the workgroup of each (segment, KV head) that finishes last.  seg_rows or seg_tables
+    None: segment i is row i of q and out, or has row i of block_tables (the kernel then
+    reaches its first keys one load sooner)."""
     n, ldq, ldo = _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size)
-    count = seg_rows.numel()
-    _i32(seg_rows, "attention seg_rows")
+    count = seg_positions.numel()
     _i32(seg_positions, "attention seg_positions", count)
-    _i32(seg_tables, "attention seg_tables", count)
+    if seg_rows is not None:
+        _i32(seg_rows, "attention seg_rows", count)
+    else:
+        _check(count <= n, "attention: more segments than rows")
+    if seg_tables is not None:
+        _i32(seg_tables, "attention seg_tables", count)
+    else:
+        _check(count <= block_tables.shape[0], "attention: more segments than block tables")
     if num_splits > 1:
         _check(partial is not None and partial.dtype == torch.float32 and partial.is_contiguous(),
                "attention: float32 partial buffer expected")

@@ -119,6 +119,8 @@ class Attention(Mixer):
         plan.add("attention.decode_positions", np.asarray(d_pos, dtype=np.int32))
         plan.add("attention.decode_tables", np.asarray(d_tab, dtype=np.int32))
         plan.host["attention.decode_max_position"] = max(d_pos) if d_pos else 0
+        # (a step of decoding requests only: segment i is row i and has block table i)
+        plan.host["attention.decode_in_order"] = d_rows == list(range(len(d_rows))) and d_tab == d_rows
 
     # ---- the layer
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool, then=None):
@@ -183,8 +185,10 @@ class Attention(Mixer):
                 if splits > 1:
                     partial = ctx.workspace.flat("attention.partial", nseg * H * splits * (hd + 2), torch.float32)
                     counters = ctx.workspace.counters("attention.splits", nseg * K)
-                ops.attention_bf16_decode(att, q, cache, rows, ctx.extra["attention.decode_positions"],
-                                          ctx.extra["attention.decode_tables"], tables, H, K, hd,
+                in_order = ctx.host.get("attention.decode_in_order", False)
+                ops.attention_bf16_decode(att, q, cache, None if in_order else rows,
+                                          ctx.extra["attention.decode_positions"],
+                                          None if in_order else ctx.extra["attention.decode_tables"], tables, H, K, hd,
                                           ctx.page_size, self.scale, self.window, partial, splits, _DECODE_WAVES,
                                           counters)
         emit = None

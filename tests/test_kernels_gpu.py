@@ -479,6 +479,31 @@ def _check_attention(H, K, hd, T, window, dtype, ps):
             assert int(counters.abs().sum()) == 0
 
 
+@pytest.mark.parametrize("splits", [1, 5])
+def test_decode_attention_with_segments_in_order(splits):
+    """Without the segments' rows and block-table rows (segment i is row i, has block table i)
+    the decode kernel gives bit for bit what it gives with them spelled out."""
+    from hfee_amd.kernels import ops
+    H, K, hd, ps, B, blocks = 6, 2, 64, 16, 5, 12
+    g = torch.Generator().manual_seed(splits)
+    cache = torch.randn(B * blocks, 2, K, ps * hd, generator=g).to(torch.bfloat16).to(DEV)
+    tables = torch.randperm(B * blocks, generator=g).to(torch.int32).reshape(B, blocks).to(DEV)
+    q = torch.randn(B, H * hd, generator=g).to(torch.bfloat16).to(DEV)
+    pos = torch.tensor([0, 17, 100, 191, 64], dtype=torch.int32, device=DEV)
+    order = torch.arange(B, dtype=torch.int32, device=DEV)
+    outs = []
+    for rows, tabs in ((order, order), (None, None), (None, order), (order, None)):
+        out = torch.zeros(B, H * hd, dtype=torch.bfloat16, device=DEV)
+        partial = torch.zeros(B * H * splits * (hd + 2), dtype=torch.float32, device=DEV)
+        counters = torch.zeros(B * K, dtype=torch.int32, device=DEV)
+        ops.attention_bf16_decode(out, q, cache, rows, pos, tabs, tables, H, K, hd, ps, 0.125, 0, partial, splits,
+                                  counters=counters if splits > 1 else None)
+        outs.append(out)
+    assert float(outs[0].float().abs().sum()) > 0
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+
+
 @pytest.mark.parametrize("pairing", ["half", "interleaved"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rope_cache_write(pairing, dtype):
