@@ -203,7 +203,9 @@ class Scheduler:
         # (a request's draw counter moves when its token is read: this step's draw is the one after)
         rows = [SampleRow(r.params, r.seed, r.draws + 1, r.history, i) for i, r in enumerate(owners)]
         self.steps_ahead += 1
-        return owners, self.sampler.launch(logits, rows)
+        place = getattr(self.engine, "token_place", None) if self.look_ahead else None
+        return owners, (self.sampler.launch(logits, rows, out=place) if place is not None
+                        else self.sampler.launch(logits, rows))
 
     # ------------------------------------------------------------------- step
     def step(self) -> list:
@@ -315,7 +317,9 @@ class Scheduler:
             if want:
                 owners.append(r)
                 rows.append(SampleRow(r.params, r.seed, r.draws, r.history, len(rows)))
-        return owners, self.sampler.launch(logits, rows)
+        place = getattr(self.engine, "token_place", None) if self.look_ahead else None
+        return owners, (self.sampler.launch(logits, rows, out=place) if place is not None
+                        else self.sampler.launch(logits, rows))
 
     def _collect(self, owners, pending, finished: list) -> list:
         """Reads the ids of a step that runs (after launching the step behind it, if that one

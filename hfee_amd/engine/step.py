@@ -180,15 +180,30 @@ class Engine:
             host[offsets[key]:offsets[key] + a.size] = a.reshape(-1)
         plan.packed = (self.steps_run, self._meta_device, pinned, event, total, dev, host[offsets["token_ids"]:])
 
-    def _upload(self, plan: StepPlan, tokens) -> dict:
-        """All planned arrays in one pinned buffer, one copy to the device."""
+    def _upload(self, plan: StepPlan, tokens, tokens_from=None) -> dict:
+        """All planned arrays in one pinned buffer, one copy to the device.  tokens_from: the
+        token ids are (or will be, by the stream's order) on the device: if they lie where the
+        step looks for them, the copy leaves that place alone; else they are copied there."""
         if plan.packed is None or plan.packed[0] != self.steps_run or plan.packed[1] is not self._meta_device:
             self._pack(plan)
         _, _, pinned, event, total, dev, token_place = plan.packed
-        token_place[:len(tokens)] = tokens
-        self._meta_device[:total].copy_(pinned[:total], non_blocking=True)
+        place = dev["token_ids"]
+        first = 0
+        if tokens_from is None:
+            token_place[:len(tokens)] = tokens
+        elif tokens_from.data_ptr() == place.data_ptr():
+            first = (place.numel() + 3) // 4 * 4              # (token_ids is the first array of the layout)
+        self._meta_device[first:total].copy_(pinned[first:total], non_blocking=True)
+        if tokens_from is not None and first == 0:
+            place.copy_(tokens_from[:place.numel()])           # on the stream, behind the metadata
         event.record()
         return dev
+
+    @property
+    def token_place(self):
+        """Where a step of single tokens looks for its token ids on the device (None before
+        the first step): a sampler that leaves its ids here saves the next step a copy."""
+        return None if self._meta_device is None else self._meta_device[:self.max_requests]
 
     def _plan(self, shape) -> StepPlan:
         """The metadata of a step whose entries are `shape`: (request id, number of tokens,
@@ -288,11 +303,10 @@ class Engine:
         else:
             plan = self._plan(shape)
         tokens = entries[0].tokens if len(entries) == 1 else [t for e in entries for t in e.tokens]
-        dev = self._upload(plan, tokens)
-        if tokens_from is not None:
-            if tokens_from.dtype != torch.int32 or tokens_from.device != self.device or tokens_from.numel() < plan.n:
-                raise StepError("tokens_from must be int32 on the engine's device, one id a row of the step")
-            dev["token_ids"].copy_(tokens_from[:plan.n])        # on the stream, behind the metadata
+        if tokens_from is not None and (tokens_from.dtype != torch.int32 or tokens_from.device != self.device
+                                        or tokens_from.numel() < plan.n):
+            raise StepError("tokens_from must be int32 on the engine's device, one id a row of the step")
+        dev = self._upload(plan, tokens, tokens_from)
         ctx = StepContext(
             n=plan.n, dtype=self.dtype, device=self.device, segments=plan.segments,
             token_ids=dev["token_ids"], positions=dev["positions"], token_segment=dev["token_segment"],

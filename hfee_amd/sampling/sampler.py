@@ -68,6 +68,7 @@ class Sampler:
     def __init__(self, vocab: int, device, max_rows: int):
         self.vocab, self.device, self.max_rows = vocab, device, max_rows
         self._out = torch.empty(max_rows, dtype=torch.int32, device=device)
+        self._latest = self._out
         # two places for the ids on the host, taken in turn: a caller may launch the next
         # sampling before it has collected this one
         self._slots = [(torch.empty(max_rows, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
@@ -82,7 +83,7 @@ class Sampler:
     def device_ids(self) -> torch.Tensor:
         """The ids of the latest launch(), on the device, in the order of its rows: a step that
         is launched before they are collected can take its tokens from here."""
-        return self._out
+        return self._latest
 
     @staticmethod
     def needs_history(params: SamplingParams) -> bool:
@@ -94,28 +95,32 @@ class Sampler:
         penalty, as the reference changes them).  Returns one id per row."""
         return self.collect(self.launch(logits, rows))
 
-    def launch(self, logits: torch.Tensor, rows):
+    def launch(self, logits: torch.Tensor, rows, out=None):
         """Starts the sampling of `rows` and returns what collect() takes: the caller may
-        do other work on the host between the two while the GPU runs."""
+        do other work on the host between the two while the GPU runs.  out: an int32
+        tensor on the device that takes the ids in place of the sampler's own (the place
+        where the engine's next step looks for its tokens, say)."""
         n = len(rows)
         if n == 0:
             return (0, 0)
+        dst = self._out if out is None or out.numel() < n else out
+        self._latest = dst
         if n > self.max_rows:
             raise ValueError(f"{n} rows to sample, the sampler was made for {self.max_rows}")
         plain_greedy = all(r.params.temperature <= 0 and not self.needs_history(r.params) for r in rows)
         if plain_greedy and [r.logits_row for r in rows] == list(range(logits.shape[0])):
-            ops.argmax(self._out, logits, self._partial, self._counters)
+            ops.argmax(dst, logits, self._partial, self._counters)
         else:
             params, hist = pack_rows(rows)
             if self._scratch is None:
                 self._scratch = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
             dparams = torch.from_numpy(params).to(self.device)
             dhist = torch.from_numpy(hist).to(self.device)
-            ops.sample(self._out, logits, dparams, dhist, self._scratch)
+            ops.sample(dst, logits, dparams, dhist, self._scratch)
         slot = self._turn
         self._turn ^= 1
         host, done = self._slots[slot]
-        host[:n].copy_(self._out[:n], non_blocking=True)
+        host[:n].copy_(dst[:n], non_blocking=True)
         done.record()
         return (n, slot)
 
