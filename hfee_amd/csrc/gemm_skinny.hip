@@ -2,7 +2,7 @@
 // reading W once from HBM, with the neighbouring small operations folded in so that a
 // decode step of a layer is five launches instead of ten.
 //
-// A workgroup owns 16 weight rows; its eight waves split K in blocks of 64 and
+// A workgroup owns 16 weight rows; its eight waves split K in blocks of 128 and
 // stream their share of W straight from global memory into the A operand of
 // v_mfma_f32_16x16x32_bf16 (lane l: row l%16, eight consecutive k).  The batch rows are
 // the B operand.  Loads are issued one block ahead of the matrix instructions.
@@ -41,9 +41,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_QKV = 4 };
 
-// (a block of 64 columns: with two blocks of a wave in flight, 256 workgroups hold 8 MB of
-// weights in flight, which measured best; with twice that, long rows (K = 14,336) stream 15% slower)
-constexpr int WAVES = 8, ROWS = 16, UNROLL = 2, KBLOCK = 32 * UNROLL;
+constexpr int WAVES = 8, ROWS = 16, UNROLL = 4, KBLOCK = 32 * UNROLL;
 
 union Chunk {
   u32x4 u;
@@ -336,29 +334,26 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_her
 
   const int nfull = a.K / KBLOCK;
   {
-    // Two sets of registers take turns, so that no loaded value is ever copied (a copy
-    // would wait for its load), and no load of the loop stands under a condition (the
-    // wait before a product would then count as if it had not been issued): the
-    // products of a block run while the loads of the next one are in flight.
-    Block b0, b1;
-    XBlock<MT, NORM> x0, x1;
-    const int mine = wave < nfull ? (nfull - 1 - wave) / WAVES + 1 : 0;      // whole blocks of this wave
-    if (mine > 0) load_block<MT, NORM>(b0, x0, w_row, x_rows, a, wave * KBLOCK);
+    // One block ahead, and no further: the next block is asked for, the current one is
+    // multiplied, and the copy into `cur` then waits for the block just asked for.  Forms
+    // of this loop that keep two blocks a wave in flight all the time (two sets of registers
+    // taking turns, in blocks of 128 or of 64 columns) were faster on one matrix in a loop and
+    // slower inside the decode step, where the weights come from memory: 56.9 and 57.4 µs
+    // against 53.5 for q/k/v + output + down of a layer of the 8B shape at batch 8.  (The
+    // block number is kept per lane, as it was when this was measured.)
+    Block cur, nxt;
+    XBlock<MT, NORM> xcur, xnxt;
+    int kb = threadIdx.x >> 6;
+    if (kb < nfull) load_block<MT, NORM>(cur, xcur, w_row, x_rows, a, kb * KBLOCK);
     // (behind the first loads of W, so that it costs no latency of its own)
     if (!NORM && a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
-    int i = 0;
-    for (; mine - i >= 3; i += 2) {
-      load_block<MT, NORM>(b1, x1, w_row, x_rows, a, (wave + (i + 1) * WAVES) * KBLOCK);
-      compute_block<MT, NORM>(acc, ss, b0, x0);
-      load_block<MT, NORM>(b0, x0, w_row, x_rows, a, (wave + (i + 2) * WAVES) * KBLOCK);
-      compute_block<MT, NORM>(acc, ss, b1, x1);
-    }
-    if (mine - i == 2) {
-      load_block<MT, NORM>(b1, x1, w_row, x_rows, a, (wave + (i + 1) * WAVES) * KBLOCK);
-      compute_block<MT, NORM>(acc, ss, b0, x0);
-      compute_block<MT, NORM>(acc, ss, b1, x1);
-    } else if (mine - i == 1) {
-      compute_block<MT, NORM>(acc, ss, b0, x0);
+    while (kb < nfull) {
+      const int kn = kb + WAVES;
+      if (kn < nfull) load_block<MT, NORM>(nxt, xnxt, w_row, x_rows, a, kn * KBLOCK);
+      compute_block<MT, NORM>(acc, ss, cur, xcur);
+      cur = nxt;
+      xcur = xnxt;
+      kb = kn;
     }
   }
   // the last, partial block (K is a multiple of 8: whole chunks are in or out)
