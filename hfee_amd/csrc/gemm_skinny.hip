@@ -468,16 +468,17 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 // weight rows, and that traffic (from L2) outgrows the weights.  Here K is cut into
 // slices of 1,024 columns, each with workgroups of its own.  A workgroup keeps its slice
 // of the batch, all rows, in LDS; each of its waves walks over groups of 16 weight rows
-// on its own: the weights come straight from global memory through a ring of 8 or 16 loads
+// on its own: the weights come straight from global memory through a ring of 4 or 16 loads
 // that runs across group boundaries, the batch operands from LDS; no barrier stands in
 // the loop.  With more than one slice a wave leaves its share of a row group's sums in a
 // scratch buffer and goes on; a second, short kernel (one wave for 16 batch rows of a row
 // group, so that the whole chip takes part) adds the shares in the order of the slices and
 // runs the epilogue.  Nobody waits for anybody, and nothing is counted.
 constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32;
-// loads a wave keeps in flight: with three or four tiles of batch rows a step takes longer,
-// and a shorter ring measured faster (less of the chip's memory queue held by each wave)
-constexpr int mid_ring(int mt) { return mt >= 3 ? 8 : 16; }
+// loads a wave keeps in flight.  Measured inside the decode step at 64 rows (q/k/v, output, down
+// of the 8B shape): 20.3 / 14.2 / 27.2 µs with 8, 15.0 / 13.8 / 27.1 with 4, 19.7 / 15.2 / 30.4 with 2;
+// at 24 and 32 rows 4 and 16 measured alike.
+constexpr int mid_ring(int mt) { return mt >= 3 ? 4 : 16; }
 constexpr int MID_PITCH = MID_KS + 8;        // LDS row pitch of the batch slice in elements: rows 16 bytes askew
 
 constexpr size_t mid_lds_bytes(int mt) { return (size_t)mt * 16 * MID_PITCH * sizeof(bf16_t); }
