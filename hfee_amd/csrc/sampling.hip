@@ -177,6 +177,7 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(int* __res
 __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, float* __restrict__ logits,
                                                          int64_t ld, int V, const SampleParams* __restrict__ params,
                                                          const int* __restrict__ history,
+                                                         const int* latest,
                                                          float* __restrict__ scratch, int64_t ld_scratch) {
   extern __shared__ uint32_t bits[];            // (V + 31) / 32 words, used by the repeat penalty
   __shared__ MaxIdx mscratch[16];
@@ -192,12 +193,20 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
   float* q = scratch + (int64_t)row * ld_scratch;
 
   // ---- repeat penalty (sampler.go:57-74)
-  if (p.repeat_penalty != 1.0f && p.history_length > 0) {
+  // (latest: one more id a row that counts as the newest of its history: the token of the
+  // step before, which lies on the device and which the host has not seen yet when this
+  // sampling is launched.  It may be the very place that `out` names: it is read here,
+  // before anything is written there.)
+  if (p.repeat_penalty != 1.0f && (p.history_length > 0 || latest != nullptr)) {
     const int words = (V + 31) / 32;
     for (int w = tid; w < words; w += THREADS) bits[w] = 0u;
     __syncthreads();
     for (int i = tid; i < p.history_length; i += THREADS) {
       const int id = history[p.history_offset + i];
+      if (id >= 0 && id < V) atomicOr(&bits[id >> 5], 1u << (id & 31));
+    }
+    if (latest != nullptr && tid == 0) {
+      const int id = latest[row];
       if (id >= 0 && id < V) atomicOr(&bits[id >> 5], 1u << (id & 31));
     }
     __syncthreads();
@@ -380,8 +389,11 @@ HFEE_API int hfee_argmax(int* out, const float* logits, int64_t ld, int rows, in
 
 // params: rows x 12 32-bit words (SampleParams).  logits may be changed in place by
 // the repeat penalty, as the reference changes them.  scratch: rows x ld_scratch floats.
+// latest: null, or one id a row that the repeat penalty counts as the newest of the row's
+// history (a row with a window of n ids then brings n - 1 in `history`).
 HFEE_API int hfee_sample(int* out, float* logits, int64_t ld, int rows, int V, const void* params,
-                         const int* history, float* scratch, int64_t ld_scratch, hipStream_t stream) {
+                         const int* history, const int* latest, float* scratch, int64_t ld_scratch,
+                         hipStream_t stream) {
   HFEE_REQUIRE(rows >= 0 && V > 0 && ld >= V && ld_scratch >= V, "sample: bad sizes rows=%d V=%d", rows, V);
   if (rows == 0) return 0;
   const size_t lds = (size_t)((V + 31) / 32) * 4;
@@ -393,7 +405,7 @@ HFEE_API int hfee_sample(int* out, float* logits, int64_t ld, int rows, int V, c
     HFEE_REQUIRE(e == hipSuccess, "sample: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
-  sample_kernel<<<rows, THREADS, lds, stream>>>(out, logits, ld, V, (const SampleParams*)params, history,
+  sample_kernel<<<rows, THREADS, lds, stream>>>(out, logits, ld, V, (const SampleParams*)params, history, latest,
                                                 scratch, ld_scratch);
   HFEE_CHECK_LAUNCH("sample");
   return 0;

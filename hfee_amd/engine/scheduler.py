@@ -36,9 +36,10 @@ without waiting for the host.  If a request turns out to have ended at step t (a
 end-of-sequence token, a stop from its callback), the token that step t+1 made for it
 is dropped; its pages were still its own when that step was queued, and whoever gets
 them next runs after it on the same stream.  Nothing is launched ahead when a request
-waits, a prompt is unfinished, a request is at its limit of tokens or of context, is
-cancelled, samples with a penalty on its own earlier tokens (the host has not seen the
-latest one yet), or when pages are short: then the step is an ordinary one.
+waits, a prompt is unfinished, a request is at its limit of tokens or of context or is
+cancelled, or when pages are short: then the step is an ordinary one.  (A penalty on a
+request's own earlier tokens needs the latest one, which the host has not seen yet: the
+sampler takes it from the device.)
 """
 from __future__ import annotations
 
@@ -161,18 +162,16 @@ class Scheduler:
             self.running.remove(request)
         finished.append(Finished(request, reason, error))
 
-    def _decode_shape(self, owners, ahead: bool):
+    def _decode_shape(self, owners):
         """The shape of the next step if it can only be "each of these requests, which are all
         that run, decodes one more token" (nobody waits for a place, no prompt is unfinished,
-        nobody reaches its limit of tokens, nobody is at the end of the context or cancelled;
-        `ahead`: and nobody's sampling reads its own earlier tokens), else None."""
+        nobody reaches its limit of tokens, nobody is at the end of the context or cancelled),
+        else None."""
         if self.waiting or len(owners) != len(self.running):
             return None
         shape = []
         for r, q in zip(owners, self.running):
             if r is not q or len(r.feed) != 0 or r.cancelled:
-                return None
-            if ahead and self.sampler.needs_history(r.params):
                 return None
             limit = r.params.num_predict
             if limit >= 0 and len(r.generated) + 1 >= limit:
@@ -186,7 +185,7 @@ class Scheduler:
         """If the next step is certain but for its tokens, the engine plans it now, while the
         GPU is busy with this one.  A guess that fails (an end-of-sequence token, a
         cancellation) costs nothing but the planning."""
-        shape = self._decode_shape(owners, ahead=False)
+        shape = self._decode_shape(owners)
         if shape:
             self.engine.prepare(shape)
 
@@ -194,18 +193,19 @@ class Scheduler:
         """Launches the step after the one whose ids are still on their way, if it is certain
         but for its tokens: they are taken from the sampler's output on the device.
         Returns (owners, handle of the ids) or None."""
-        shape = self._decode_shape(owners, ahead=True) if self.look_ahead else None
+        shape = self._decode_shape(owners) if self.look_ahead else None
         if not shape or not self.engine.prepare(shape):
             return None                                  # (pages are short: an ordinary step decides what gives)
         entries = [StepEntry(rid, [0], [0]) for rid, _, _ in shape]
         self.last_batch = [(rid, 1) for rid, _, _ in shape]
         logits = self.engine.step(entries, tokens_from=self.sampler.device_ids)
-        # (a request's draw counter moves when its token is read: this step's draw is the one after)
+        # (a request's draw counter and history move when its token is read: this step's draw is
+        # the one after, and the newest id of every history is the one that the sampler still
+        # holds on the device)
         rows = [SampleRow(r.params, r.seed, r.draws + 1, r.history, i) for i, r in enumerate(owners)]
         self.steps_ahead += 1
-        place = getattr(self.engine, "token_place", None) if self.look_ahead else None
-        return owners, (self.sampler.launch(logits, rows, out=place) if place is not None
-                        else self.sampler.launch(logits, rows))
+        return owners, self.sampler.launch(logits, rows, out=getattr(self.engine, "token_place", None),
+                                           latest=self.sampler.device_ids)
 
     # ------------------------------------------------------------------- step
     def step(self) -> list:

@@ -35,7 +35,7 @@ _CORE_SIGNATURES = {
     "hfee_gemm_skinny": [P, L, P, I, L, P, L, I, I, I, I, P, I, F, P, P, P, P, I, P, P, I, I, P, I, I, I, I,
                          P, I, P, L, P, P, I, F, P, L, I, P],
     "hfee_argmax": [P, P, L, I, I, P, L, P, I, P],
-    "hfee_sample": [P, P, L, I, I, P, P, P, L, P],
+    "hfee_sample": [P, P, L, I, I, P, P, P, P, L, P],
 }
 
 _ATTENTION_SIGNATURES = {

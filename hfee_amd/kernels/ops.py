@@ -239,9 +239,11 @@ def argmax(out: torch.Tensor, logits: torch.Tensor, partial=None, counters=None)
 
 
 def sample(out: torch.Tensor, logits: torch.Tensor, params: torch.Tensor, history: torch.Tensor,
-           scratch: torch.Tensor):
-    """out[r] = sampled id for row r; params is [rows, 12] int32 (see sampling/params.py)."""
-    _gpu(out, logits, params, history, scratch)
+           scratch: torch.Tensor, latest=None):
+    """out[r] = sampled id for row r; params is [rows, 12] int32 (see sampling/params.py).
+    latest: int32 on the device, one id a row that the repeat penalty counts as the newest
+    of the row's history (it may be `out` itself: it is read before `out` is written)."""
+    _gpu(out, logits, params, history, scratch, latest)
     _, V, ld = _rows2d(logits, "sample logits")
     rows = params.shape[0]
     _check(logits.dtype == torch.float32 and scratch.dtype == torch.float32, "sample: float32 logits and scratch")
@@ -251,8 +253,10 @@ def sample(out: torch.Tensor, logits: torch.Tensor, params: torch.Tensor, histor
     _check(rs >= rows and Vs >= V, "sample: scratch too small")
     _i32(out, "sample out", rows)
     _check(history.dtype == torch.int32 and history.is_contiguous(), "sample: history must be int32")
+    if latest is not None:
+        _i32(latest, "sample latest", rows)
     lib.core().call("hfee_sample", _ptr(out), _ptr(logits), ld, rows, V, _ptr(params), _ptr(history),
-                    _ptr(scratch), lds, _stream())
+                    _ptr(latest), _ptr(scratch), lds, _stream())
 
 
 # ------------------------------------------------- matrix-core attention (bfloat16)

@@ -42,8 +42,10 @@ def _f2i(x: float) -> int:
     return struct.unpack("<i", struct.pack("<f", float(x)))[0]
 
 
-def pack_rows(rows) -> tuple:
-    """rows -> ([n, 12] int32 parameter array, flat int32 history)."""
+def pack_rows(rows, one_more: bool = False) -> tuple:
+    """rows -> ([n, 12] int32 parameter array, flat int32 history).  one_more: every row's
+    history has one newer id that is not in `history` (the kernel gets it on the device):
+    the window of the repeat penalty then takes one id fewer from here."""
     params = np.zeros((len(rows), 12), dtype=np.int32)
     hist = []
     for i, r in enumerate(rows):
@@ -51,10 +53,13 @@ def pack_rows(rows) -> tuple:
         recent = []
         if p.repeat_penalty != 1 and p.repeat_last_n != 0:
             recent = list(r.history)
-            if p.repeat_last_n > 0 and len(recent) > p.repeat_last_n:
-                recent = recent[-p.repeat_last_n:]
+            if p.repeat_last_n > 0:
+                keep = p.repeat_last_n - (1 if one_more else 0)
+                recent = recent[-keep:] if keep > 0 else []
         seed, draw = r.seed & _MASK, r.draw & _MASK
-        words = [_f2i(p.temperature), int(p.top_k), _f2i(p.top_p), _f2i(p.min_p), _f2i(p.repeat_penalty),
+        # (a window of 0 ids switches the penalty off: the kernel sees a penalty of 1)
+        words = [_f2i(p.temperature), int(p.top_k), _f2i(p.top_p), _f2i(p.min_p),
+                 _f2i(p.repeat_penalty if p.repeat_last_n != 0 else 1.0),
                  len(hist), len(recent)]
         params[i, :7] = words
         params[i, 7:11] = np.array([seed & 0xffffffff, seed >> 32, draw & 0xffffffff, draw >> 32],
@@ -95,11 +100,14 @@ class Sampler:
         penalty, as the reference changes them).  Returns one id per row."""
         return self.collect(self.launch(logits, rows))
 
-    def launch(self, logits: torch.Tensor, rows, out=None):
+    def launch(self, logits: torch.Tensor, rows, out=None, latest=None):
         """Starts the sampling of `rows` and returns what collect() takes: the caller may
         do other work on the host between the two while the GPU runs.  out: an int32
         tensor on the device that takes the ids in place of the sampler's own (the place
-        where the engine's next step looks for its tokens, say)."""
+        where the engine's next step looks for its tokens, say).  latest: an int32 tensor
+        on the device with one id a row that is newer than the rows' histories (the ids of
+        the sampling before, when this one is launched before they were collected): the
+        repeat penalty counts it in.  It may be the tensor that `out` names."""
         n = len(rows)
         if n == 0:
             return (0, 0)
@@ -111,12 +119,13 @@ class Sampler:
         if plain_greedy and [r.logits_row for r in rows] == list(range(logits.shape[0])):
             ops.argmax(dst, logits, self._partial, self._counters)
         else:
-            params, hist = pack_rows(rows)
+            params, hist = pack_rows(rows, one_more=latest is not None)
             if self._scratch is None:
                 self._scratch = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
             dparams = torch.from_numpy(params).to(self.device)
             dhist = torch.from_numpy(hist).to(self.device)
-            ops.sample(dst, logits, dparams, dhist, self._scratch)
+            ops.sample(dst, logits, dparams, dhist, self._scratch,
+                       latest if any(self.needs_history(r.params) for r in rows) else None)
         slot = self._turn
         self._turn ^= 1
         host, done = self._slots[slot]

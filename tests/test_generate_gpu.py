@@ -136,12 +136,14 @@ def test_the_command_line_generates_from_token_ids(model_folders):
     assert p.returncode == 1 and "usage" in p.stderr
 
 
-@pytest.mark.parametrize("dtype,temperature", [("float32", 0.0), ("bfloat16", 0.0), ("float32", 0.7)])
-def test_steps_launched_ahead_give_the_tokens_of_steps_that_wait(model_folders, dtype, temperature):
+@pytest.mark.parametrize("dtype,temperature,penalty", [("float32", 0.0, 1.0), ("bfloat16", 0.0, 1.0), ("float32", 0.7, 1.0),
+                                                       ("float32", 0.7, 1.3), ("float32", 0.0, 1.5)])
+def test_steps_launched_ahead_give_the_tokens_of_steps_that_wait(model_folders, dtype, temperature, penalty):
     """The scheduler launches a decode step before it has read the ids of the step before
     (they go from the sampler to the embedding on the device).  With that switched off the
-    same requests give the same tokens and reasons: greedy and seeded sampling, requests of
-    different lengths of which some end early on an end-of-sequence id, so that steps that
+    same requests give the same tokens and reasons: greedy and seeded sampling, with and
+    without a penalty on the requests' own earlier tokens (the newest of which the sampler
+    then takes from the device), requests of different lengths of which some end early on an end-of-sequence id, so that steps that
     were launched ahead for them run for nobody."""
     from hfee_amd import LLM, SamplingParams
     folder = model_folders[("A", dtype)]
@@ -153,8 +155,9 @@ def test_steps_launched_ahead_give_the_tokens_of_steps_that_wait(model_folders, 
         llm.scheduler.look_ahead = look_ahead
         if eos is not None:
             llm.scheduler.eos = {eos}
-        params = [SamplingParams(temperature=temperature, top_k=0, top_p=1.0, repeat_penalty=1.0, seed=50 + i,
-                                 num_predict=n) for i, n in enumerate([40, 12, 33, 25])]
+        params = [SamplingParams(temperature=temperature, top_k=0, top_p=1.0, repeat_penalty=penalty,
+                                 repeat_last_n=[64, 5, -1, 1][i], seed=50 + i, num_predict=n)
+                  for i, n in enumerate([40, 12, 33, 25])]
         outs = llm.generate(prompts, params)
         llm.engine.cache.check()
         assert not llm.engine.cache.requests

@@ -464,6 +464,36 @@ def test_sampler_kernel_follows_the_plain_rules():
     assert mixed[2] == alone[0] and mixed[1] == 17
 
 
+def test_sampler_takes_the_newest_id_of_a_history_from_the_device():
+    """The newest id of each row's history may lie on the device only (`latest`: the ids of
+    the sampling before, not yet collected), even in the tensor that takes this sampling's
+    ids: the repeat penalty then sees the same window of ids, and the same ids come out, as
+    with the whole history on the host.  A window of one id is that id alone; a window
+    switched off stays off."""
+    from hfee_amd.sampling import SampleRow, Sampler, SamplingParams
+    V = 700
+    g = torch.Generator().manual_seed(5)
+    base = torch.randn(6, V, generator=g) * 2
+    sampler = Sampler(V, DEV, max_rows=8)
+    histories = [torch.randint(0, V, (n,), generator=g).tolist() for n in (90, 3, 64, 65, 10, 30)]
+    for h, row in zip(histories, base):
+        row[h[-1]] = row.max() + 1.0          # the newest id would win if it were not penalised
+    cases = [SamplingParams(temperature=0.0, repeat_penalty=3.0, repeat_last_n=64),
+             SamplingParams(temperature=0.9, top_k=30, top_p=0.9, repeat_penalty=1.5, repeat_last_n=-1),
+             SamplingParams(temperature=0.0, repeat_penalty=4.0, repeat_last_n=1),
+             SamplingParams(temperature=0.7, top_k=0, top_p=1.0, repeat_penalty=2.0, repeat_last_n=64),
+             SamplingParams(temperature=0.0, repeat_penalty=9.0, repeat_last_n=0),
+             SamplingParams(temperature=0.0, repeat_penalty=1.0)]
+    whole = sampler.sample(base.clone().to(DEV), [SampleRow(p, 11 + i, 4, h, i) for i, (p, h) in enumerate(zip(cases, histories))])
+    place = torch.tensor([h[-1] for h in histories] + [0, 0], dtype=torch.int32, device=DEV)
+    rows = [SampleRow(p, 11 + i, 4, h[:-1], i) for i, (p, h) in enumerate(zip(cases, histories))]
+    ahead = sampler.collect(sampler.launch(base.clone().to(DEV), rows, out=place, latest=place))
+    assert ahead == whole
+    assert place[:6].tolist() == whole
+    assert whole[0] != histories[0][-1] and whole[2] != histories[2][-1]      # the penalty did bite
+    assert whole[4] == histories[4][-1] and whole[5] == histories[5][-1]      # and where it is off, it did not
+
+
 def test_kernels_refuse_what_they_cannot_do():
     from hfee_amd.kernels import KernelError, ops
     with pytest.raises(KernelError, match="GPU tensors"):
