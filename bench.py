@@ -50,6 +50,9 @@ def main() -> int:
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.1-8b")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--sampling", choices=["greedy", "default"], default="greedy",
+                    help="decode with greedy sampling (the default run) or with the reference's default options "
+                         "(temperature 0.8, top-k 40, top-p 0.9, repeat penalty 1.1 over 64 tokens)")
     ap.add_argument("--serving", type=int, default=0, metavar="R",
                     help="instead of the default run: R requests at once under continuous batching, prompts of "
                          "64 to 2,048 tokens, 128 new tokens each, context 4,096; prints its own line")
@@ -106,7 +109,8 @@ def main() -> int:
 
     def decode_run(batch: int, steps: int, warmup: int):
         sched = Scheduler(engine, sampler, max_num_seqs=batch, max_batch_tokens=PREFILL, num_ctx=context)
-        params = SamplingParams.greedy(num_predict=-1, ignore_eos=True)
+        params = (SamplingParams.greedy(num_predict=-1, ignore_eos=True) if args.sampling == "greedy"
+                  else SamplingParams(num_predict=-1, ignore_eos=True, seed=1))
         for i in range(batch):
             prompt = torch.randint(0, V, (PROMPT,), generator=gen).tolist()
             sched.add(Request(("bench", batch, i), prompt, params, seed=i))

@@ -174,6 +174,11 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(int* __res
   }
 }
 
+// The largest top_k whose kept set is gathered into LDS (ids ascending): every rule after
+// top_k then runs over at most this many entries instead of the whole vocabulary.
+constexpr int GATHER_MAX = 1024;
+constexpr int HIST_COPIES = 32, HIST_PITCH = 257;   // counters of a radix pass: one set per lane % 32, a bank apart
+
 __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, float* __restrict__ logits,
                                                          int64_t ld, int V, const SampleParams* __restrict__ params,
                                                          const int* __restrict__ history,
@@ -183,16 +188,23 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
   __shared__ MaxIdx mscratch[16];
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
-  __shared__ int hist[256];
+  __shared__ int hist[HIST_COPIES * HIST_PITCH];
+  __shared__ int bins[256];
   __shared__ uint32_t sh_prefix;
   __shared__ int sh_need;
+  __shared__ float kept_logit[GATHER_MAX];
+  __shared__ float kept_q[GATHER_MAX];
+  __shared__ int kept_id[GATHER_MAX];
+  __shared__ int wave_above[THREADS / 64], wave_ties[THREADS / 64];
 
   const int row = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
   const SampleParams p = params[row];
   float* lg = logits + (int64_t)p.logits_row * ld;
   float* q = scratch + (int64_t)row * ld_scratch;
 
-  // ---- repeat penalty (sampler.go:57-74)
+  // ---- repeat penalty (sampler.go:57-74): each distinct recent id once; the bit set says
+  // which ids have had theirs
   // (latest: one more id a row that counts as the newest of its history: the token of the
   // step before, which lies on the device and which the host has not seen yet when this
   // sampling is launched.  It may be the very place that `out` names: it is read here,
@@ -201,19 +213,15 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     const int words = (V + 31) / 32;
     for (int w = tid; w < words; w += THREADS) bits[w] = 0u;
     __syncthreads();
-    for (int i = tid; i < p.history_length; i += THREADS) {
-      const int id = history[p.history_offset + i];
-      if (id >= 0 && id < V) atomicOr(&bits[id >> 5], 1u << (id & 31));
-    }
-    if (latest != nullptr && tid == 0) {
-      const int id = latest[row];
-      if (id >= 0 && id < V) atomicOr(&bits[id >> 5], 1u << (id & 31));
-    }
-    __syncthreads();
-    for (int j = tid; j < V; j += THREADS) {
-      if (bits[j >> 5] & (1u << (j & 31))) {
-        const float v = lg[j];
-        lg[j] = v > 0.f ? v / p.repeat_penalty : v * p.repeat_penalty;
+    const int count = p.history_length + (latest != nullptr ? 1 : 0);
+    for (int i = tid; i < count; i += THREADS) {
+      const int id = i < p.history_length ? history[p.history_offset + i] : latest[row];
+      if (id >= 0 && id < V) {
+        const uint32_t bit = 1u << (id & 31);
+        if (!(atomicOr(&bits[id >> 5], bit) & bit)) {
+          const float v = lg[id];
+          lg[id] = v > 0.f ? v / p.repeat_penalty : v * p.repeat_penalty;
+        }
       }
     }
     __threadfence_block();
@@ -227,26 +235,38 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     return;
   }
 
-  // ---- top_k: key of the k-th largest and how many of its ties belong (sampler.go:132-151)
+  // ---- top_k: key of the k-th largest and how many of its ties belong (sampler.go:132-151).
+  // A radix select, eight bits a pass.  Logits crowd into a few values of the leading bits, and
+  // 128,000 atomic increments of a handful of LDS words would take milliseconds: every lane % 32
+  // counts in a set of its own, laid out so that equal digits of different lanes fall into
+  // different banks, and the sets are added up after the pass.
   uint32_t t_k = 0u;
   int r_k = 0x7fffffff;
   if (p.top_k > 0 && p.top_k < V) {
     if (tid == 0) { sh_prefix = 0u; sh_need = p.top_k; }
     uint32_t mask = 0u;
+    int* mine = hist + (lane & (HIST_COPIES - 1)) * HIST_PITCH;
     for (int shift = 24; shift >= 0; shift -= 8) {
-      for (int b = tid; b < 256; b += THREADS) hist[b] = 0;
+      for (int b = tid; b < HIST_COPIES * HIST_PITCH; b += THREADS) hist[b] = 0;
       __syncthreads();
       const uint32_t prefix = sh_prefix;
       for (int j = tid; j < V; j += THREADS) {
         const uint32_t key = order_key(lg[j]);
-        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
+        if ((key & mask) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1);
+      }
+      __syncthreads();
+      if (tid < 256) {
+        int sum = 0;
+#pragma unroll 8
+        for (int c = 0; c < HIST_COPIES; ++c) sum += hist[c * HIST_PITCH + tid];
+        bins[tid] = sum;
       }
       __syncthreads();
       if (tid == 0) {
         int need = sh_need, b = 255;
         for (; b > 0; --b) {
-          if (hist[b] >= need) break;
-          need -= hist[b];
+          if (bins[b] >= need) break;
+          need -= bins[b];
         }
         sh_need = need;
         sh_prefix = prefix | ((uint32_t)b << shift);
@@ -258,21 +278,69 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     r_k = sh_need;
   }
 
+  // ---- a small top_k: its set goes to LDS, ids ascending ({key > t_k} and the first r_k
+  // ties), and everything below runs over these few entries.  Wave w takes the w-th
+  // sixteenth of the ids, 64 consecutive ids at a time: first it counts, then, knowing what
+  // the waves before it hold, it places.
+  const bool gathered = p.top_k > 0 && p.top_k < V && p.top_k <= GATHER_MAX;
+  int Vn = V;                                   // entries that the rules below run over
+  const float* lgp = lg;                        // their logits
+  float* qp = q;                                // their unnormalised probabilities
+  if (gathered) {
+    const int span = ((V + THREADS / 64 - 1) / (THREADS / 64) + 63) / 64 * 64;     // ids of a wave, whole groups of 64
+    const int first = min(V, wave * span), last = min(V, first + span);
+    int above = 0, ties = 0;
+    for (int j = first + lane; j - lane < last; j += 64) {
+      const uint32_t key = j < last ? order_key(lg[j]) : 0u;
+      above += __popcll(__ballot(j < last && key > t_k));
+      ties += __popcll(__ballot(j < last && key == t_k));
+    }
+    if (lane == 0) { wave_above[wave] = above; wave_ties[wave] = ties; }
+    __syncthreads();
+    int above_before = 0, ties_before = 0;
+    for (int w = 0; w < wave; ++w) { above_before += wave_above[w]; ties_before += wave_ties[w]; }
+    int at = above_before + min(ties_before, r_k);         // kept entries of the waves before
+    int ties_seen = ties_before;
+    const uint64_t below = (1ull << lane) - 1ull;          // the lanes before this one
+    for (int j = first + lane; j - lane < last; j += 64) {
+      const float v = j < last ? lg[j] : 0.f;
+      const uint32_t key = order_key(v);
+      const bool tie = j < last && key == t_k;
+      const uint64_t tie_mask = __ballot(tie);
+      const bool in = j < last && (key > t_k || (tie && ties_seen + __popcll(tie_mask & below) < r_k));
+      const uint64_t in_mask = __ballot(in);
+      if (in) {
+        const int slot = at + __popcll(in_mask & below);
+        if (slot < GATHER_MAX) { kept_logit[slot] = v; kept_id[slot] = j; }
+      }
+      at += __popcll(in_mask);
+      ties_seen += __popcll(tie_mask);
+    }
+    if (wave == THREADS / 64 - 1 && lane == 0) sh_need = min(at, GATHER_MAX);       // (the last wave has counted them all)
+    __syncthreads();
+    Vn = sh_need;
+    lgp = kept_logit;
+    qp = kept_q;
+    t_k = 0u;                                   // top_k is done: every gathered entry belongs
+    r_k = 0x7fffffff;
+  }
+  auto id_of = [&](int j) { return gathered ? kept_id[j] : j; };
+
   // ---- probabilities of the top_k set, in q (sampler.go:88-96); thread-owned chunks
-  const int chunk = (V + THREADS - 1) / THREADS;
-  const int j0 = min(V, tid * chunk), j1 = min(V, j0 + chunk);
+  const int chunk = (Vn + THREADS - 1) / THREADS;
+  const int j0 = min(Vn, tid * chunk), j1 = min(Vn, j0 + chunk);
   int my_ties = 0;
-  for (int j = j0; j < j1; ++j) my_ties += order_key(lg[j]) == t_k;
+  for (int j = j0; j < j1; ++j) my_ties += order_key(lgp[j]) == t_k;
   int all_ties;
   int tie_rank = block_exclusive_scan<int>(my_ties, iscratch, &all_ties);
   float my_mass = 0.f;
   for (int j = j0; j < j1; ++j) {
-    const float v = lg[j];
+    const float v = lgp[j];
     const uint32_t key = order_key(v);
     bool in = key > t_k;
     if (key == t_k) in = tie_rank++ < r_k;
     const float e = in ? expf((v - top.v) / p.temperature) : 0.f;
-    q[j] = e;
+    qp[j] = e;
     my_mass += e;
   }
   __threadfence_block();
@@ -288,7 +356,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     for (int bit = 31; bit >= 0; --bit) {
       const uint32_t cand = t | (1u << bit);
       float mass = 0.f;
-      for (int j = j0; j < j1; ++j) mass += order_key(lg[j]) >= cand ? q[j] : 0.f;
+      for (int j = j0; j < j1; ++j) mass += order_key(lgp[j]) >= cand ? qp[j] : 0.f;
       float total;
       block_exclusive_scan<float>(mass, fscratch, &total);
       if (total >= target) t = cand;
@@ -296,9 +364,9 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     t_p = t;
     float above = 0.f, tie_p = 0.f;
     for (int j = j0; j < j1; ++j) {
-      const uint32_t key = order_key(lg[j]);
-      if (key > t_p) above += q[j];
-      else if (key == t_p && q[j] > 0.f) tie_p = q[j];
+      const uint32_t key = order_key(lgp[j]);
+      if (key > t_p) above += qp[j];
+      else if (key == t_p && qp[j] > 0.f) tie_p = qp[j];
     }
     float mass_above;
     block_exclusive_scan<float>(above, fscratch, &mass_above);
@@ -308,22 +376,22 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
 
   // ---- min_p and the kept set (sampler.go:109-116), then the draw (sampler.go:118-129)
   int my_pties = 0;
-  for (int j = j0; j < j1; ++j) my_pties += (order_key(lg[j]) == t_p && q[j] > 0.f);
+  for (int j = j0; j < j1; ++j) my_pties += (order_key(lgp[j]) == t_p && qp[j] > 0.f);
   int all_pties;
   int ptie_rank = block_exclusive_scan<int>(my_pties, iscratch, &all_pties);
   float my_keep = 0.f;
   int my_last = -1;
   for (int j = j0; j < j1; ++j) {
-    const uint32_t key = order_key(lg[j]);
-    float w = q[j];
+    const uint32_t key = order_key(lgp[j]);
+    float w = qp[j];
     if (w > 0.f) {
       bool in = key > t_p;
       if (key == t_p) in = ptie_rank++ < r_p;
-      if (p.min_p > 0.f && w < p.min_p && j != top.i) in = false;
+      if (p.min_p > 0.f && w < p.min_p && id_of(j) != top.i) in = false;
       if (!in) w = 0.f;
     }
-    q[j] = w;
-    if (w > 0.f) my_last = j;
+    qp[j] = w;
+    if (w > 0.f) my_last = id_of(j);
     my_keep += w;
   }
   __threadfence_block();
@@ -333,7 +401,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
   const uint64_t draw = ((uint64_t)p.draw_hi << 32) | p.draw_lo;
   const float r = (float)(uniform_from(seed, draw) * (double)total);
 
-    __shared__ int sh_choice;
+  __shared__ int sh_choice;
   if (tid == 0) sh_choice = 0x7fffffff;
   __syncthreads();
   if (my_keep > 0.f && (before < r || r <= 0.f)) {
@@ -341,9 +409,9 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     // reaches r wins, whatever rounding does to the chunk sums
     float run = before;
     for (int j = j0; j < j1; ++j) {
-      if (q[j] <= 0.f) continue;
-      run += q[j];
-      if (run >= r) { atomicMin(&sh_choice, j); break; }
+      if (qp[j] <= 0.f) continue;
+      run += qp[j];
+      if (run >= r) { atomicMin(&sh_choice, id_of(j)); break; }
     }
   }
   __syncthreads();
