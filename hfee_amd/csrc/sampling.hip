@@ -250,7 +250,18 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
       for (int b = tid; b < HIST_COPIES * HIST_PITCH; b += THREADS) hist[b] = 0;
       __syncthreads();
       const uint32_t prefix = sh_prefix;
-      for (int j = tid; j < V; j += THREADS) {
+      int j = tid;
+      for (; j + 7 * THREADS < V; j += 8 * THREADS) {        // eight loads in flight
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = lg[j + u * THREADS];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const uint32_t key = order_key(v[u]);
+          if ((key & mask) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1);
+        }
+      }
+      for (; j < V; j += THREADS) {
         const uint32_t key = order_key(lg[j]);
         if ((key & mask) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1);
       }
@@ -290,10 +301,17 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     const int span = ((V + THREADS / 64 - 1) / (THREADS / 64) + 63) / 64 * 64;     // ids of a wave, whole groups of 64
     const int first = min(V, wave * span), last = min(V, first + span);
     int above = 0, ties = 0;
-    for (int j = first + lane; j - lane < last; j += 64) {
-      const uint32_t key = j < last ? order_key(lg[j]) : 0u;
-      above += __popcll(__ballot(j < last && key > t_k));
-      ties += __popcll(__ballot(j < last && key == t_k));
+    for (int j0 = first + lane; j0 - lane < last; j0 += 8 * 64) {     // eight loads in flight
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = j0 + 64 * u < last ? lg[j0 + 64 * u] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int j = j0 + 64 * u;
+        const uint32_t key = order_key(v[u]);
+        above += __popcll(__ballot(j < last && key > t_k));
+        ties += __popcll(__ballot(j < last && key == t_k));
+      }
     }
     if (lane == 0) { wave_above[wave] = above; wave_ties[wave] = ties; }
     __syncthreads();
@@ -302,19 +320,26 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     int at = above_before + min(ties_before, r_k);         // kept entries of the waves before
     int ties_seen = ties_before;
     const uint64_t below = (1ull << lane) - 1ull;          // the lanes before this one
-    for (int j = first + lane; j - lane < last; j += 64) {
-      const float v = j < last ? lg[j] : 0.f;
-      const uint32_t key = order_key(v);
-      const bool tie = j < last && key == t_k;
-      const uint64_t tie_mask = __ballot(tie);
-      const bool in = j < last && (key > t_k || (tie && ties_seen + __popcll(tie_mask & below) < r_k));
-      const uint64_t in_mask = __ballot(in);
-      if (in) {
-        const int slot = at + __popcll(in_mask & below);
-        if (slot < GATHER_MAX) { kept_logit[slot] = v; kept_id[slot] = j; }
+    for (int j0 = first + lane; j0 - lane < last; j0 += 8 * 64) {
+      float vs[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) vs[u] = j0 + 64 * u < last ? lg[j0 + 64 * u] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {                         // in ascending id
+        const int j = j0 + 64 * u;
+        const float v = vs[u];
+        const uint32_t key = order_key(v);
+        const bool tie = j < last && key == t_k;
+        const uint64_t tie_mask = __ballot(tie);
+        const bool in = j < last && (key > t_k || (tie && ties_seen + __popcll(tie_mask & below) < r_k));
+        const uint64_t in_mask = __ballot(in);
+        if (in) {
+          const int slot = at + __popcll(in_mask & below);
+          if (slot < GATHER_MAX) { kept_logit[slot] = v; kept_id[slot] = j; }
+        }
+        at += __popcll(in_mask);
+        ties_seen += __popcll(tie_mask);
       }
-      at += __popcll(in_mask);
-      ties_seen += __popcll(tie_mask);
     }
     if (wave == THREADS / 64 - 1 && lane == 0) sh_need = min(at, GATHER_MAX);       // (the last wave has counted them all)
     __syncthreads();

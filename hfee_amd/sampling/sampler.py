@@ -80,6 +80,8 @@ class Sampler:
                        for _ in range(2)]
         self._turn = 0
         self._scratch = None
+        self._stage = [None, None]          # pinned buffers for the rows' options, taken in turn with _slots
+        self._options = None                # the same on the device
         # for the argmax over several workgroups a row
         self._partial = torch.empty(max_rows * ops.ARGMAX_PARTS * 2, dtype=torch.float32, device=device)
         self._counters = torch.zeros(max_rows, dtype=torch.int32, device=device)
@@ -122,8 +124,7 @@ class Sampler:
             params, hist = pack_rows(rows, one_more=latest is not None)
             if self._scratch is None:
                 self._scratch = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
-            dparams = torch.from_numpy(params).to(self.device)
-            dhist = torch.from_numpy(hist).to(self.device)
+            dparams, dhist = self._send(params, hist)
             ops.sample(dst, logits, dparams, dhist, self._scratch,
                        latest if any(self.needs_history(r.params) for r in rows) else None)
         slot = self._turn
@@ -132,6 +133,26 @@ class Sampler:
         host[:n].copy_(dst[:n], non_blocking=True)
         done.record()
         return (n, slot)
+
+    def _send(self, params: np.ndarray, hist: np.ndarray):
+        """The rows' options and recent ids to the device through pinned memory, without
+        making the host wait for the stream (a copy from pageable memory would wait for
+        everything queued before it: the whole step)."""
+        need = params.size + hist.size
+        stage = self._stage[self._turn]
+        if stage is None or stage[0].numel() < need:
+            cap = max(2 * need, 12 * self.max_rows + 4096)
+            stage = self._stage[self._turn] = (torch.empty(cap, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+        pinned, sent = stage
+        sent.synchronize()                  # the copy that used this buffer two launches ago
+        if self._options is None or self._options.numel() < need:
+            self._options = torch.empty(max(2 * need, 12 * self.max_rows + 4096), dtype=torch.int32, device=self.device)
+        host = pinned.numpy()
+        host[:params.size] = params.reshape(-1)
+        host[params.size:need] = hist
+        self._options[:need].copy_(pinned[:need], non_blocking=True)
+        sent.record()
+        return self._options[:params.size].view(params.shape), self._options[params.size:need]
 
     def collect(self, pending) -> list:
         """Waits for the ids of a launch() (the latest one or the one before it)."""
