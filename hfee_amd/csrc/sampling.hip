@@ -174,6 +174,160 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(int* __res
   }
 }
 
+// The rules after top_k run either over the whole block (1,024 threads, sums joined through
+// LDS with barriers) or, when top_k has gathered its few entries into LDS, over one wave
+// (64 lanes, sums joined by shuffles, no barrier at all).
+template <typename T, bool WAVE>
+__device__ __forceinline__ T team_exclusive_scan(T v, T* wave_totals, T* total) {
+  if constexpr (!WAVE) {
+    return block_exclusive_scan<T>(v, wave_totals, total);
+  } else {
+    const int lane = threadIdx.x & 63;
+    T incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const T up = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += up;
+    }
+    *total = __shfl(incl, 63, 64);
+    return incl - v;
+  }
+}
+
+template <bool WAVE>
+__device__ __forceinline__ float team_max(float v, float* scratch) {
+  if constexpr (WAVE) return wave_max(v);
+  else return block_max(v, scratch);
+}
+
+// Everything after top_k (sampler.go:88-129) over entries 0 .. Vn-1 with logits lgp and ids
+// `ids` (null: entry j is id j), of which {key > t_k} and the first r_k ties at t_k belong:
+// probabilities into qp, top_p, min_p, the draw.  Every member of the team owns a contiguous
+// chunk of the entries; sums run chunk by chunk and then in a fixed tree.
+template <bool WAVE>
+__device__ __forceinline__ void draw_from_kept(const SampleParams& p, const MaxIdx top, int Vn,
+                                               const float* lgp, float* qp, const int* ids, uint32_t t_k, int r_k,
+                                               int* out_id, float* fscratch, int* iscratch, int* sh_choice) {
+  constexpr int TEAM = WAVE ? 64 : THREADS;
+  const int me = WAVE ? (threadIdx.x & 63) : threadIdx.x;
+  auto id_of = [&](int j) { return ids != nullptr ? ids[j] : j; };
+  const int chunk = (Vn + TEAM - 1) / TEAM;
+  const int j0 = min(Vn, me * chunk), j1 = min(Vn, j0 + chunk);
+  int my_ties = 0;
+  for (int j = j0; j < j1; ++j) my_ties += order_key(lgp[j]) == t_k;
+  int all_ties;
+  int tie_rank = team_exclusive_scan<int, WAVE>(my_ties, iscratch, &all_ties);
+  float my_mass = 0.f;
+  for (int j = j0; j < j1; ++j) {
+    const float v = lgp[j];
+    const uint32_t key = order_key(v);
+    bool in = key > t_k;
+    if (key == t_k) in = tie_rank++ < r_k;
+    const float e = in ? expf((v - top.v) / p.temperature) : 0.f;
+    qp[j] = e;
+    my_mass += e;
+  }
+  if (!WAVE) __threadfence_block();
+  float Z;
+  team_exclusive_scan<float, WAVE>(my_mass, fscratch, &Z);
+
+  // ---- top_p: threshold key and how many of its ties belong (sampler.go:98-108)
+  uint32_t t_p = 0u;
+  int r_p = 0x7fffffff;
+  if (p.top_p > 0.f && p.top_p < 1.f) {
+    const float target = p.top_p * Z;
+    uint32_t t = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t cand = t | (1u << bit);
+      float mass = 0.f;
+      for (int j = j0; j < j1; ++j) mass += order_key(lgp[j]) >= cand ? qp[j] : 0.f;
+      float total;
+      team_exclusive_scan<float, WAVE>(mass, fscratch, &total);
+      if (total >= target) t = cand;
+    }
+    t_p = t;
+    float above = 0.f, tie_p = 0.f;
+    for (int j = j0; j < j1; ++j) {
+      const uint32_t key = order_key(lgp[j]);
+      if (key > t_p) above += qp[j];
+      else if (key == t_p && qp[j] > 0.f) tie_p = qp[j];
+    }
+    float mass_above;
+    team_exclusive_scan<float, WAVE>(above, fscratch, &mass_above);
+    tie_p = team_max<WAVE>(tie_p, fscratch);
+    r_p = tie_p > 0.f ? max(1, (int)ceilf((target - mass_above) / tie_p)) : 1;
+  }
+
+  // ---- min_p and the kept set (sampler.go:109-116), then the draw (sampler.go:118-129)
+  int my_pties = 0;
+  for (int j = j0; j < j1; ++j) my_pties += (order_key(lgp[j]) == t_p && qp[j] > 0.f);
+  int all_pties;
+  int ptie_rank = team_exclusive_scan<int, WAVE>(my_pties, iscratch, &all_pties);
+  float my_keep = 0.f;
+  int my_last = -1;
+  for (int j = j0; j < j1; ++j) {
+    const uint32_t key = order_key(lgp[j]);
+    float w = qp[j];
+    if (w > 0.f) {
+      bool in = key > t_p;
+      if (key == t_p) in = ptie_rank++ < r_p;
+      if (p.min_p > 0.f && w < p.min_p && id_of(j) != top.i) in = false;
+      if (!in) w = 0.f;
+    }
+    qp[j] = w;
+    if (w > 0.f) my_last = id_of(j);
+    my_keep += w;
+  }
+  if (!WAVE) __threadfence_block();
+  float total;
+  const float before = team_exclusive_scan<float, WAVE>(my_keep, fscratch, &total);
+  const uint64_t seed = ((uint64_t)p.seed_hi << 32) | p.seed_lo;
+  const uint64_t draw = ((uint64_t)p.draw_hi << 32) | p.draw_lo;
+  const float r = (float)(uniform_from(seed, draw) * (double)total);
+
+  // every chunk that starts below r walks; the smallest id whose running sum reaches r
+  // wins, whatever rounding does to the chunk sums
+  int mine = 0x7fffffff;
+  if (my_keep > 0.f && (before < r || r <= 0.f)) {
+    float run = before;
+    for (int j = j0; j < j1; ++j) {
+      if (qp[j] <= 0.f) continue;
+      run += qp[j];
+      if (run >= r) { mine = id_of(j); break; }
+    }
+  }
+  if constexpr (WAVE) {
+    int choice = mine, last = my_last;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      choice = min(choice, __shfl_xor(choice, off, 64));
+      last = max(last, __shfl_xor(last, off, 64));
+    }
+    // rounding left r above every running sum: the last kept id (sampler.go:129)
+    if (choice == 0x7fffffff) choice = last < 0 ? top.i : last;
+    if (me == 0) *out_id = choice;
+  } else {
+    if (me == 0) *sh_choice = 0x7fffffff;
+    __syncthreads();
+    if (mine != 0x7fffffff) atomicMin(sh_choice, mine);
+    __syncthreads();
+    if (*sh_choice == 0x7fffffff) {
+      int last = my_last;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off, 64));
+      if ((me & 63) == 0) iscratch[me >> 6] = last;
+      __syncthreads();
+      if (me == 0) {
+        int l = -1;
+        for (int w = 0; w < THREADS / 64; ++w) l = max(l, iscratch[w]);
+        *sh_choice = l < 0 ? top.i : l;
+      }
+      __syncthreads();
+    }
+    if (me == 0) *out_id = *sh_choice;
+  }
+}
+
 // The largest top_k whose kept set is gathered into LDS (ids ascending): every rule after
 // top_k then runs over at most this many entries instead of the whole vocabulary.
 constexpr int GATHER_MAX = 1024;
@@ -273,14 +427,16 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
         bins[tid] = sum;
       }
       __syncthreads();
-      if (tid == 0) {
-        int need = sh_need, b = 255;
-        for (; b > 0; --b) {
-          if (bins[b] >= need) break;
-          need -= bins[b];
-        }
-        sh_need = need;
-        sh_prefix = prefix | ((uint32_t)b << shift);
+      // the digit whose count, with the counts of all larger digits, first reaches what is
+      // still needed: thread t looks at digit 255 - t
+      const int need = sh_need;
+      const int count = tid < 256 ? bins[255 - tid] : 0;
+      int all;
+      const int larger = block_exclusive_scan<int>(count, iscratch, &all);
+      __syncthreads();                                       // (everyone has read sh_need)
+      if (tid < 256 && larger < need && (need <= larger + count || tid == 255)) {
+        sh_need = need - larger;
+        sh_prefix = prefix | ((uint32_t)(255 - tid) << shift);
       }
       mask |= 255u << shift;
       __syncthreads();
@@ -349,112 +505,13 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     t_k = 0u;                                   // top_k is done: every gathered entry belongs
     r_k = 0x7fffffff;
   }
-  auto id_of = [&](int j) { return gathered ? kept_id[j] : j; };
-
-  // ---- probabilities of the top_k set, in q (sampler.go:88-96); thread-owned chunks
-  const int chunk = (Vn + THREADS - 1) / THREADS;
-  const int j0 = min(Vn, tid * chunk), j1 = min(Vn, j0 + chunk);
-  int my_ties = 0;
-  for (int j = j0; j < j1; ++j) my_ties += order_key(lgp[j]) == t_k;
-  int all_ties;
-  int tie_rank = block_exclusive_scan<int>(my_ties, iscratch, &all_ties);
-  float my_mass = 0.f;
-  for (int j = j0; j < j1; ++j) {
-    const float v = lgp[j];
-    const uint32_t key = order_key(v);
-    bool in = key > t_k;
-    if (key == t_k) in = tie_rank++ < r_k;
-    const float e = in ? expf((v - top.v) / p.temperature) : 0.f;
-    qp[j] = e;
-    my_mass += e;
-  }
-  __threadfence_block();
-  float Z;
-  block_exclusive_scan<float>(my_mass, fscratch, &Z);
-
-  // ---- top_p: threshold key and how many of its ties belong (sampler.go:98-108)
-  uint32_t t_p = 0u;
-  int r_p = 0x7fffffff;
-  if (p.top_p > 0.f && p.top_p < 1.f) {
-    const float target = p.top_p * Z;
-    uint32_t t = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = t | (1u << bit);
-      float mass = 0.f;
-      for (int j = j0; j < j1; ++j) mass += order_key(lgp[j]) >= cand ? qp[j] : 0.f;
-      float total;
-      block_exclusive_scan<float>(mass, fscratch, &total);
-      if (total >= target) t = cand;
-    }
-    t_p = t;
-    float above = 0.f, tie_p = 0.f;
-    for (int j = j0; j < j1; ++j) {
-      const uint32_t key = order_key(lgp[j]);
-      if (key > t_p) above += qp[j];
-      else if (key == t_p && qp[j] > 0.f) tie_p = qp[j];
-    }
-    float mass_above;
-    block_exclusive_scan<float>(above, fscratch, &mass_above);
-    tie_p = block_max(tie_p, fscratch);
-    r_p = tie_p > 0.f ? max(1, (int)ceilf((target - mass_above) / tie_p)) : 1;
-  }
-
-  // ---- min_p and the kept set (sampler.go:109-116), then the draw (sampler.go:118-129)
-  int my_pties = 0;
-  for (int j = j0; j < j1; ++j) my_pties += (order_key(lgp[j]) == t_p && qp[j] > 0.f);
-  int all_pties;
-  int ptie_rank = block_exclusive_scan<int>(my_pties, iscratch, &all_pties);
-  float my_keep = 0.f;
-  int my_last = -1;
-  for (int j = j0; j < j1; ++j) {
-    const uint32_t key = order_key(lgp[j]);
-    float w = qp[j];
-    if (w > 0.f) {
-      bool in = key > t_p;
-      if (key == t_p) in = ptie_rank++ < r_p;
-      if (p.min_p > 0.f && w < p.min_p && id_of(j) != top.i) in = false;
-      if (!in) w = 0.f;
-    }
-    qp[j] = w;
-    if (w > 0.f) my_last = id_of(j);
-    my_keep += w;
-  }
-  __threadfence_block();
-  float total;
-  const float before = block_exclusive_scan<float>(my_keep, fscratch, &total);
-  const uint64_t seed = ((uint64_t)p.seed_hi << 32) | p.seed_lo;
-  const uint64_t draw = ((uint64_t)p.draw_hi << 32) | p.draw_lo;
-  const float r = (float)(uniform_from(seed, draw) * (double)total);
-
   __shared__ int sh_choice;
-  if (tid == 0) sh_choice = 0x7fffffff;
-  __syncthreads();
-  if (my_keep > 0.f && (before < r || r <= 0.f)) {
-    // every chunk that starts below r walks; the smallest id whose running sum
-    // reaches r wins, whatever rounding does to the chunk sums
-    float run = before;
-    for (int j = j0; j < j1; ++j) {
-      if (qp[j] <= 0.f) continue;
-      run += qp[j];
-      if (run >= r) { atomicMin(&sh_choice, id_of(j)); break; }
-    }
+  if (gathered) {
+    if (wave == 0)
+      draw_from_kept<true>(p, top, Vn, lgp, qp, kept_id, t_k, r_k, out + row, fscratch, iscratch, &sh_choice);
+  } else {
+    draw_from_kept<false>(p, top, Vn, lgp, qp, nullptr, t_k, r_k, out + row, fscratch, iscratch, &sh_choice);
   }
-  __syncthreads();
-  if (sh_choice == 0x7fffffff) {
-    // rounding left r above every running sum: the last kept id (sampler.go:129)
-    int last = my_last;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off, 64));
-    if ((tid & 63) == 0) iscratch[tid >> 6] = last;
-    __syncthreads();
-    if (tid == 0) {
-      int l = -1;
-      for (int w = 0; w < THREADS / 64; ++w) l = max(l, iscratch[w]);
-      sh_choice = l < 0 ? top.i : l;
-    }
-    __syncthreads();
-  }
-  if (tid == 0) out[row] = sh_choice;
 }
 
 }  // namespace
