@@ -84,22 +84,49 @@ __device__ __forceinline__ MaxIdx better(MaxIdx a, MaxIdx b) {   // greater valu
   return a;
 }
 
+// One pass of the block over lg[0 .. V-1]: see(j, lg[j]) for every j, ascending within a
+// thread.  Rows that are 16-byte aligned are read four logits a load, four loads in flight;
+// others one logit a load, eight in flight.
+template <typename F>
+__device__ __forceinline__ void scan_logits(const float* __restrict__ lg, int V, F see) {
+  const int stride = blockDim.x;
+  if (((uintptr_t)lg & 15) == 0) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const f32x4* lg4 = reinterpret_cast<const f32x4*>(lg);
+    const int quads = V >> 2;
+    int i = threadIdx.x;
+    for (; i + 3 * stride < quads; i += 4 * stride) {
+      f32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = lg4[i + u * stride];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) see(4 * (i + u * stride) + c, v[u][c]);
+    }
+    for (; i < quads; i += stride) {
+      const f32x4 v = lg4[i];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) see(4 * i + c, v[c]);
+    }
+    for (int j = 4 * quads + threadIdx.x; j < V; j += stride) see(j, lg[j]);
+  } else {
+    int j = threadIdx.x;
+    for (; j + 7 * stride < V; j += 8 * stride) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = lg[j + u * stride];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) see(j + u * stride, v[u]);
+    }
+    for (; j < V; j += stride) see(j, lg[j]);
+  }
+}
+
 __device__ MaxIdx block_argmax_raw(const float* __restrict__ lg, int V, MaxIdx* scratch) {
   MaxIdx best{-INFINITY, 0x7fffffff};
-  const int stride = blockDim.x;
-  int j = threadIdx.x;
-  for (; j + 7 * stride < V; j += 8 * stride) {      // eight loads in flight, compared in ascending j
-    float v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = lg[j + u * stride];
-#pragma unroll
-    for (int u = 0; u < 8; ++u)
-      if (v[u] > best.v) best = MaxIdx{v[u], j + u * stride};
-  }
-  for (; j < V; j += stride) {
-    const float v = lg[j];
-    if (v > best.v) best = MaxIdx{v, j};   // ascending j per thread: strict '>' keeps the first
-  }
+  // (ascending j per thread: strict '>' keeps the first)
+  scan_logits(lg, V, [&](int j, float v) { if (v > best.v) best = MaxIdx{v, j}; });
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     MaxIdx o{__shfl_xor(best.v, off, 64), __shfl_xor(best.i, off, 64)};
@@ -404,21 +431,10 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
       for (int b = tid; b < HIST_COPIES * HIST_PITCH; b += THREADS) hist[b] = 0;
       __syncthreads();
       const uint32_t prefix = sh_prefix;
-      int j = tid;
-      for (; j + 7 * THREADS < V; j += 8 * THREADS) {        // eight loads in flight
-        float v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = lg[j + u * THREADS];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const uint32_t key = order_key(v[u]);
-          if ((key & mask) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1);
-        }
-      }
-      for (; j < V; j += THREADS) {
-        const uint32_t key = order_key(lg[j]);
+      scan_logits(lg, V, [&](int, float v) {
+        const uint32_t key = order_key(v);
         if ((key & mask) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1);
-      }
+      });
       __syncthreads();
       if (tid < 256) {
         int sum = 0;
