@@ -531,7 +531,16 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
     const int row = ((it + fill_first) % FILL) * FILL_ROWS + fill_row;
     *reinterpret_cast<u32x4*>(xs + row * MID_PITCH + fill_c * 8) = fill[it];
   }
-  if (slices == 1 && a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
+  if (a.scale_ss != nullptr && (slices == 1 || blockIdx.x == gridDim.x - 1)) {
+    // (with slices, the finishing kernel scales the rows: one workgroup here works the scales
+    // out for it and leaves them behind the shares, so that not every workgroup there adds
+    // up all the shares of every row again)
+    row_scales<MT>(a, row_scale);
+    if (slices > 1) {
+      __syncthreads();
+      if (threadIdx.x < MT * 16) scratch[(int64_t)row_groups * slices * MT * 256 + threadIdx.x] = row_scale[threadIdx.x];
+    }
+  }
   __syncthreads();
 
   const bf16_t* x_lane = xs + r16 * MID_PITCH + g * 8;
@@ -595,16 +604,17 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
 template <int MT, int EPI>
 __global__ __launch_bounds__(WAVES * 64) void mid_finish_kernel(Args a, int row_groups, int slices,
                                                                 const float* __restrict__ scratch) {
-  __shared__ float row_scale[SS_STRIDE];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
   const int unit = blockIdx.x * WAVES + wave;
   const int rg = unit / MT, t = unit - rg * MT;
-  const bool here = rg < row_groups;                       // (whole waves; every wave stays for the barrier below)
+  const bool here = rg < row_groups;                       // (whole waves)
   const int m = t * 16 + r16, n = rg * ROWS + 4 * g;
   const bool live = here && m < a.M && n < a.N;
   const Ahead<EPI> ahead = look_ahead<EPI>(a, m, n, live);
+  // (the rows' scales: left behind the shares by the kernel before)
+  const float scale = a.scale_ss != nullptr ? scratch[(int64_t)row_groups * slices * MT * 256 + m] : 1.f;
   const float* share = scratch + ((int64_t)min(rg, row_groups - 1) * slices * MT + t) * 256 + lane * 4;
   const int64_t step = (int64_t)MT * 256;
   f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -620,9 +630,6 @@ __global__ __launch_bounds__(WAVES * 64) void mid_finish_kernel(Args a, int row_
   }
   float v[4] = {acc[0], acc[1], acc[2], acc[3]};
   if (a.scale_ss != nullptr) {
-    row_scales<MT>(a, row_scale);
-    __syncthreads();
-    const float scale = row_scale[m];
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] *= scale;
   }
@@ -633,7 +640,7 @@ __global__ __launch_bounds__(WAVES * 64) void mid_finish_kernel(Args a, int row_
 template <int MT>
 bool launch_mid_rows(const Args& a, int epi, float* scratch, int64_t scratch_floats, int num_cus, hipStream_t stream) {
   const int row_groups = (a.N + ROWS - 1) / ROWS, slices = a.K / MID_KS;
-  if (slices > 1 && (scratch == nullptr || scratch_floats < (int64_t)row_groups * slices * MT * 256)) return false;
+  if (slices > 1 && (scratch == nullptr || scratch_floats < (int64_t)row_groups * slices * MT * 256 + SS_STRIDE)) return false;
   int per_slice = num_cus / slices;                         // workgroups per slice: eight row groups at a time each
   if (per_slice < 1) per_slice = 1;
   if (per_slice > (row_groups + WAVES - 1) / WAVES) per_slice = (row_groups + WAVES - 1) / WAVES;
@@ -838,7 +845,7 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 // scale_ss: shares left by such a product (scale_blocks x 64 floats) over rows of width K:
 // the finished sums are scaled by 1 / sqrt(sum / K + scale_eps).
 // scratch: for 17 to 64 rows and K a multiple of 1,024, a faster pair of kernels that needs
-// ceil(N / 16) * (K / 1024) * ceil(M / 16) * 256 floats of scratch (none for K = 1,024);
+// ceil(N / 16) * (K / 1024) * ceil(M / 16) * 256 + 64 floats of scratch (none for K = 1,024);
 // without it, or for other sizes, or where it would not pay, the streaming kernel takes
 // the product (force_mid != 0 takes the faster kernels wherever they apply: for tests).
 HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
@@ -904,9 +911,11 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
     HFEE_REQUIRE(!norm && scale_blocks > 0 && scale_eps >= 0.f, "gemm_skinny: a row scale needs its shares and no norm of its own");
     a.scale_ss = scale_ss; a.scale_blocks = scale_blocks; a.scale_eps = scale_eps;
   }
-  // More than 16 rows and very many weight rows (gate/up): the streaming kernel would
-  // read the batch again for every 16 of them; the tiled kernel takes the row scale too.
-  if (scale_ss != nullptr && M > 16 && N >= 16384 && emit_out == nullptr && epi != EPI_QKV && !force_mid)
+  // More than 16 rows and very many weight rows (gate/up) without scratch for the pair of
+  // kernels below: the streaming kernel would read the batch again for every 16 weight rows;
+  // the tiled kernel takes the row scale too.  (With scratch the pair is faster: measured
+  // inside the decode step of the 8B shape, 5,995 -> 6,186 tok/s at batch 32.)
+  if (scale_ss != nullptr && M > 16 && N >= 16384 && emit_out == nullptr && epi != EPI_QKV && !force_mid && scratch == nullptr)
     return hfee_gemm_bf16_scaled(C, epi, ldc, A, lda, W, ldw, M, N, K, scale_ss, scale_blocks, scale_eps, stream);
   const int mt = (M + 15) / 16;
   // Where the kernels with the batch in LDS win, from fits to measured times in microseconds
@@ -914,13 +923,12 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
   // kernel takes the weights' time at 5 TB/s, a launch, and 0.052 a batch row and 1,024
   // columns for reading the batch again with every 16 weight rows (more where the row
   // groups outnumber the CUs); the pair of kernels takes 16.5, or the weights' time at
-  // 4.65 TB/s and 4 where that is more, whatever the number of batch rows.  Not for very
-  // many weight rows (gate/up), where the tiled kernel fills the chip.
+  // 4.65 TB/s and 4 where that is more, whatever the number of batch rows.
   const double weight_mb = 2e-6 * (double)N * (double)K;
   const double rounds = ((N + ROWS - 1) / ROWS) / 256.0;
   const double t_streaming = weight_mb / 5.0 + 3.0 + 0.052 * (K / 1024.0) * (rounds > 1.0 ? rounds : 1.0) * M;
   const double t_pair = weight_mb * 0.215 + 4.0 > 16.5 ? weight_mb * 0.215 + 4.0 : 16.5;
-  const bool mid_pays = t_pair < 0.95 * t_streaming && N < 16384;
+  const bool mid_pays = t_pair < 0.95 * t_streaming;
   if (!norm && mt > 1 && K % MID_KS == 0 && (mid_pays || force_mid)) {
     static int num_cus = 0;
     if (num_cus == 0) {

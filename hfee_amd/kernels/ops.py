@@ -361,7 +361,7 @@ def mid_rows_scratch(n_rows: int, n_weight_rows: int, k: int) -> int:
     (0: it has no use for scratch)."""
     if n_rows <= 16 or n_rows > SKINNY_MAX_ROWS or k % 1024 or k == 1024:
         return 0
-    return ((n_weight_rows + 15) // 16) * (k // 1024) * ((n_rows + 15) // 16) * 256
+    return ((n_weight_rows + 15) // 16) * (k // 1024) * ((n_rows + 15) // 16) * 256 + SS_STRIDE
 
 
 def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0.0, rows=None, m=None, qkv=None,

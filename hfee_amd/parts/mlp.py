@@ -51,7 +51,7 @@ class GatedMLP(FeedForward):
         if halves is None and aligned and few and isinstance(h, LazyNorm) and ops.norm_fusion_pays(*self.w_gate_up.shape):
             norm = h.fusable()
         if halves:        # the norm's first half came with the product before; both projections and the gate
-            ops.linear_fused(act, halves[0], self.w_gate_up, "swiglu", row_scale=halves[1])
+            ops.linear_fused(act, halves[0], self.w_gate_up, "swiglu", row_scale=halves[1], **ctx.workspace.product_scratch(ctx.n, self.w_gate_up))
         elif norm:        # norm, both projections and the gate in one launch
             ops.linear_fused(act, h.x, self.w_gate_up, "swiglu", norm_weight=norm[0], eps=norm[1])
         else:
