@@ -416,10 +416,10 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path):
 
 # -------------------------------------------------------------- the sampler ---
 
-def test_sampler_kernel_follows_the_plain_rules():
+@pytest.mark.parametrize("V", [1000, 1001])
+def test_sampler_kernel_follows_the_plain_rules(V):
     from plain_llama import plain_repeat_penalty, plain_sampling_distribution
     from hfee_amd.sampling import SampleRow, Sampler, SamplingParams, uniform
-    V = 1000
     g = torch.Generator().manual_seed(0)
     base = torch.randn(V, generator=g) * 2
     base[17] = base[400] = base.max() + 0.5          # tied maxima
@@ -464,15 +464,15 @@ def test_sampler_kernel_follows_the_plain_rules():
     assert mixed[2] == alone[0] and mixed[1] == 17
 
 
-def test_sampler_takes_the_newest_id_of_a_history_from_the_device():
+@pytest.mark.parametrize("V", [700, 1003, 4099])
+def test_sampler_takes_the_newest_id_of_a_history_from_the_device(V):
     """The newest id of each row's history may lie on the device only (`latest`: the ids of
     the sampling before, not yet collected), even in the tensor that takes this sampling's
     ids: the repeat penalty then sees the same window of ids, and the same ids come out, as
     with the whole history on the host.  A window of one id is that id alone; a window
     switched off stays off."""
     from hfee_amd.sampling import SampleRow, Sampler, SamplingParams
-    V = 700
-    g = torch.Generator().manual_seed(5)
+    g = torch.Generator().manual_seed(5)             # (a vocabulary that is no multiple of 4: rows that are not 16-byte aligned)
     base = torch.randn(6, V, generator=g) * 2
     sampler = Sampler(V, DEV, max_rows=8)
     histories = [torch.randint(0, V, (n,), generator=g).tolist() for n in (90, 3, 64, 65, 10, 30)]
