@@ -464,6 +464,25 @@ def test_sampler_kernel_follows_the_plain_rules(V):
     assert mixed[2] == alone[0] and mixed[1] == 17
 
 
+def test_sampler_with_a_top_k_too_large_to_gather():
+    """A top_k above 1,024 is not gathered into LDS: the radix select's threshold then
+    serves the rules that run over the whole vocabulary.  Draws match the inverse CDF of
+    the plain distribution."""
+    from plain_llama import plain_sampling_distribution
+    from hfee_amd.sampling import SampleRow, Sampler, SamplingParams, uniform
+    V = 3001
+    g = torch.Generator().manual_seed(9)
+    base = torch.randn(V, generator=g) * 3
+    p = SamplingParams(temperature=1.1, top_k=1500, top_p=0.95, min_p=0.0, repeat_penalty=1.0)
+    dist = plain_sampling_distribution(base, p.temperature, p.top_k, p.top_p, p.min_p)
+    cum = torch.cumsum(dist, 0)
+    sampler = Sampler(V, DEV, max_rows=64)
+    rows = [SampleRow(p, seed=5, draw=r, history=[], logits_row=r) for r in range(64)]
+    ids = sampler.sample(base.repeat(64, 1).to(DEV), rows)
+    exact = sum(int(i == int((cum >= uniform(5, r)).nonzero()[0])) for r, i in enumerate(ids))
+    assert all(dist[i] > 0 for i in ids) and exact >= 62, exact
+
+
 @pytest.mark.parametrize("V", [700, 1003, 4099])
 def test_sampler_takes_the_newest_id_of_a_history_from_the_device(V):
     """The newest id of each row's history may lie on the device only (`latest`: the ids of
