@@ -25,10 +25,38 @@ __global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ tabl
   for (int j = threadIdx.x; j < d; j += blockDim.x) out[(int64_t)row * d + j] = to_float<T>(table[src + j]);
 }
 
+// bfloat16 rows of a width that is a multiple of 8, 16-byte aligned: eight elements a
+// thread, a row over several workgroups (a decode step's few rows then take one round of
+// loads, not sixteen one after the other)
+__global__ __launch_bounds__(256) void embed_bf16_wide_kernel(float* __restrict__ out, const bf16_t* __restrict__ table,
+                                                              const int* __restrict__ ids, int d) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  const int row = blockIdx.x, j = 8 * (blockIdx.y * 256 + threadIdx.x);
+  if (j >= d) return;
+  const u32x4 v = *reinterpret_cast<const u32x4*>(table + (int64_t)ids[row] * d + j);
+  float* o = out + (int64_t)row * d + j;
+  f32x4 lo, hi;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    lo[2 * i] = __uint_as_float(v[i] << 16);
+    lo[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+    hi[2 * i] = __uint_as_float(v[2 + i] << 16);
+    hi[2 * i + 1] = __uint_as_float(v[2 + i] & 0xffff0000u);
+  }
+  *reinterpret_cast<f32x4*>(o) = lo;
+  *reinterpret_cast<f32x4*>(o + 4) = hi;
+}
+
 HFEE_API int hfee_embed(float* out, const void* table, int table_dtype, const int* ids,
                         int n, int d, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && d > 0, "embed: bad sizes n=%d d=%d", n, d);
   if (n == 0) return 0;
+  if (table_dtype == DT_BF16 && d % 8 == 0 && (uintptr_t)table % 16 == 0 && (uintptr_t)out % 16 == 0 && n <= 65535) {
+    embed_bf16_wide_kernel<<<dim3(n, (d + 2047) / 2048), 256, 0, stream>>>(out, (const bf16_t*)table, ids, d);
+    HFEE_CHECK_LAUNCH("embed");
+    return 0;
+  }
   if (table_dtype == DT_F32)
     embed_kernel<float><<<n, 256, 0, stream>>>(out, (const float*)table, ids, d);
   else if (table_dtype == DT_BF16)

@@ -393,13 +393,14 @@ def test_swiglu_and_add(dtype):
     close(xd, x.double() + out.double().cpu(), 1e-6)
 
 
+@pytest.mark.parametrize("d", [97, 104, 2048 + 8, 4096])      # odd; a multiple of 8 (eight elements a thread); several workgroups a row
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_embed(dtype):
+def test_embed(dtype, d):
     from hfee_amd.kernels import ops
     g = torch.Generator().manual_seed(4)
-    table = torch.randn(321, 97, generator=g).to(dtype)
+    table = torch.randn(321, d, generator=g).to(dtype)
     ids = torch.tensor([0, 320, 5, 5, 17], dtype=torch.int32)
-    out = torch.empty(5, 97, dtype=torch.float32, device=DEV)
+    out = torch.empty(5, d, dtype=torch.float32, device=DEV)
     ops.embed(out, table.to(DEV), ids.to(DEV))
     assert torch.equal(out.cpu(), table[ids.long()].float())
 
