@@ -603,7 +603,8 @@ __device__ __forceinline__ void combine_head(bf16_t* __restrict__ orow, const fl
 // (segment, head, split): the unnormalised output, the maximum, the sum.
 constexpr int DECODE_MAX_WAVES = 4;      // each wave holds two tiles' operands: registers allow no more
 
-__global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
+template <bool AHEAD>
+__global__ __launch_bounds__(DECODE_MAX_WAVES * 64, AHEAD ? 1 : 2) void decode_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, CacheLayout lay, const int* __restrict__ seg_rows,
     const int* __restrict__ seg_positions, const int* __restrict__ seg_tables,
@@ -635,7 +636,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64) void decode_kernel(
     load_query(q_op, q + (int64_t)row * ldq + h * HD, slot_ok);
     Tile st;
     init_tile(st);
-    attend_tiles<true>(st, q_op, cache, lay, bt, bt_stride, off, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
+    attend_tiles<AHEAD>(st, q_op, cache, lay, bt, bt_stride, off, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
                  scale_log2, lo, pos);
 
     // this wave's state into LDS
@@ -826,15 +827,33 @@ HFEE_API int hfee_attention_bf16_decode(void* out, int64_t ld_out, const void* q
   const size_t lds = waves * per_wave;
   static bool raised = false;
   if (lds > 48 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)decode_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)(DECODE_MAX_WAVES * 32 * (HD + 2) * sizeof(float) < 160 * 1024
-                                                 ? DECODE_MAX_WAVES * 32 * (HD + 2) * sizeof(float) : 160 * 1024));
+    const int most = (int)(DECODE_MAX_WAVES * 32 * (HD + 2) * sizeof(float) < 160 * 1024
+                               ? DECODE_MAX_WAVES * 32 * (HD + 2) * sizeof(float) : 160 * 1024);
+    hipError_t e = hipFuncSetAttribute((const void*)decode_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, most);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)decode_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, most);
     HFEE_REQUIRE(e == hipSuccess, "attention_bf16_decode: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
-  decode_kernel<<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
-                                         seg_rows, seg_positions, seg_tables, block_tables, bt_stride, num_heads,
-                                         scale * LOG2E, window, partial, num_splits, in_kernel_join ? counters : nullptr);
+  // With more workgroups than CUs, the form that holds one tile's operands (two workgroups
+  // fit a CU and hide each other's loads); else the form that asks for the next tile while it
+  // multiplies this one (one workgroup a CU, and nobody else to hide its loads).
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    num_cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+               prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+  }
+  const bool ahead = (int64_t)num_segments * kv_heads * num_splits <= num_cus;
+  if (ahead)
+    decode_kernel<true><<<grid, waves * 64, lds, stream>>>(
+        (bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, seg_rows, seg_positions, seg_tables,
+        block_tables, bt_stride, num_heads, scale * LOG2E, window, partial, num_splits, in_kernel_join ? counters : nullptr);
+  else
+    decode_kernel<false><<<grid, waves * 64, lds, stream>>>(
+        (bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, seg_rows, seg_positions, seg_tables,
+        block_tables, bt_stride, num_heads, scale * LOG2E, window, partial, num_splits, in_kernel_join ? counters : nullptr);
   HFEE_CHECK_LAUNCH("attention_bf16_decode");
   if (num_splits > 1 && !in_kernel_join) {
     dim3 cgrid(num_segments, num_heads);

@@ -480,6 +480,32 @@ def _check_attention(H, K, hd, T, window, dtype, ps):
             assert int(counters.abs().sum()) == 0
 
 
+@pytest.mark.parametrize("B,splits", [(40, 1), (70, 2), (12, 3)])
+def test_decode_attention_with_more_workgroups_than_cus(B, splits):
+    """With more (segment, KV head, split) workgroups than the chip has CUs the decode kernel
+    runs in the form that holds one tile's operands, two workgroups a CU; with fewer, in the
+    form that loads one tile ahead.  Both against the plain attention kernel."""
+    from hfee_amd.kernels import ops
+    H, K, hd, ps, blocks = 16, 8, 64, 16, 20
+    g = torch.Generator().manual_seed(B)
+    cache = (torch.randn(B * blocks, 2, K, ps * hd, generator=g) * 0.5).to(torch.bfloat16).to(DEV)
+    tables = torch.randperm(B * blocks, generator=g).to(torch.int32).reshape(B, blocks).to(DEV)
+    q = torch.randn(B, H * hd, generator=g).to(torch.bfloat16).to(DEV)
+    pos = torch.randint(0, blocks * ps, (B,), generator=g).to(torch.int32)
+    pos[0], pos[1] = 0, blocks * ps - 1
+    pos = pos.to(DEV)
+    order = torch.arange(B, dtype=torch.int32, device=DEV)
+    want = torch.zeros(B, H * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention_plain(want, q, cache, pos, order, tables, H, K, hd, ps, 0.125, 0)
+    out = torch.zeros(B, H * hd, dtype=torch.bfloat16, device=DEV)
+    partial = torch.zeros(B * H * splits * (hd + 2), dtype=torch.float32, device=DEV)
+    counters = torch.zeros(B * K, dtype=torch.int32, device=DEV)
+    ops.attention_bf16_decode(out, q, cache, order, pos, order, tables, H, K, hd, ps, 0.125, 0, partial, splits,
+                              counters=counters if splits > 1 else None)
+    close(out, want, 2e-2)
+    assert int(counters.abs().sum()) == 0
+
+
 @pytest.mark.parametrize("splits", [1, 5])
 def test_decode_attention_with_segments_in_order(splits):
     """Without the segments' rows and block-table rows (segment i is row i, has block table i)
