@@ -274,14 +274,64 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
                                         const int* __restrict__ positions, const int* __restrict__ token_segment,
                                         const int* __restrict__ block_tables, int bt_stride,
                                         const float* __restrict__ cos_table, const float* __restrict__ sin_table,
-                                        int half, bf16_t* __restrict__ cache, CacheLayout lay, int num_heads) {
+                                        int half, bf16_t* __restrict__ cache, CacheLayout lay, int num_heads,
+                                        int n, int values_by_groups) {
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   union Eight {
     u32x4 u;
     bf16_t e[8];
   };
-  const int t = blockIdx.x;
+  // Some workgroups take the values of 16 consecutive tokens each.  The cache keeps values
+  // transposed (a column of a head holds the page's slots side by side), so a token alone
+  // writes two bytes here and two bytes there; 16 tokens that fill 16 slots in a row of one
+  // page (a prompt's portion that starts on a page's edge) write 32 bytes a column at once.
+  // (the groups' workgroups, which run longer than a token's, come first: none is left over at the end)
+  const int groups = values_by_groups ? (n + 15) / 16 : 0;
+  if ((int)blockIdx.x < groups) {
+    extern __shared__ __attribute__((aligned(16))) bf16_t group_values[];      // [16][kv_heads * head_dim]
+    __shared__ int g_pos[16], g_page[16];
+    const int t0 = 16 * (int)blockIdx.x, count = min(16, n - t0);
+    const int width = lay.kv_heads * lay.head_dim, chunks = width / 8;
+    const int pieces = count * chunks;
+    for (int first = threadIdx.x; first < pieces; first += 8 * blockDim.x) {      // eight loads in flight
+      u32x4 piece[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int idx = min(first + u * (int)blockDim.x, pieces - 1), j = idx / chunks, c = idx - j * chunks;
+        piece[u] = *reinterpret_cast<const u32x4*>(v + (int64_t)(t0 + j) * ldv + 8 * c);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int idx = first + u * (int)blockDim.x, j = idx / chunks, c = idx - j * chunks;
+        if (idx < pieces) *reinterpret_cast<u32x4*>(group_values + j * width + 8 * c) = piece[u];
+      }
+    }
+    if (threadIdx.x < count) {
+      const int p = positions[t0 + threadIdx.x];
+      g_pos[threadIdx.x] = p;
+      g_page[threadIdx.x] = block_tables[(int64_t)token_segment[t0 + threadIdx.x] * bt_stride + (p >> lay.page_shift)];
+    }
+    __syncthreads();
+    bool in_a_row = count == 16 && (g_pos[0] & 15) == 0;
+    for (int j = 1; j < count; ++j) in_a_row = in_a_row && g_pos[j] == g_pos[0] + j && g_page[j] == g_page[0];
+    for (int col = threadIdx.x; col < width; col += blockDim.x) {
+      const int h = col / lay.head_dim, d = col - h * lay.head_dim;
+      if (in_a_row) {
+        union { u32x4 u[2]; bf16_t e[16]; } row;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) row.e[CacheLayout::value_slot(j)] = group_values[j * width + col];
+        u32x4* dst = reinterpret_cast<u32x4*>(cache + lay.value_column(g_page[0], h, d) + (g_pos[0] & (lay.page_size - 1)));
+        dst[0] = row.u[0];
+        dst[1] = row.u[1];
+      } else {
+        for (int j = 0; j < count; ++j)
+          cache[lay.value_offset(g_page[j], h, g_pos[j] & (lay.page_size - 1), d)] = group_values[j * width + col];
+      }
+    }
+    return;
+  }
+  const int t = (int)blockIdx.x - groups;
   const int pos = positions[t];
   const int hd = lay.head_dim, per_head = hd / 8;
   const float* cs = cos_table ? cos_table + (int64_t)pos * half : nullptr;
@@ -317,9 +367,10 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
     const int h = w / per_head, d = (w - h * per_head) * 8;
     Eight x, y;
     x.u = *reinterpret_cast<const u32x4*>(kt + w * 8);
-    y.u = *reinterpret_cast<const u32x4*>(vt + w * 8);
+    if (!values_by_groups) y.u = *reinterpret_cast<const u32x4*>(vt + w * 8);
     rotate(x, d);
     *reinterpret_cast<u32x4*>(cache + lay.key_offset(page, h, slot, d)) = x.u;
+    if (values_by_groups) continue;                                    // (other workgroups write the values)
     bf16_t* vc = cache + lay.value_offset(page, h, slot, d);          // column d of the head; the next is page_size on
 #pragma unroll
     for (int c = 0; c < 8; ++c) vc[(int64_t)c * lay.page_size] = y.e[c];
@@ -355,8 +406,14 @@ HFEE_API int hfee_rope_cache_write(void* q, int64_t ldq, const void* k, int64_t 
            (q == nullptr || (ldq % 8 == 0 && (uintptr_t)q % 16 == 0)) &&
            (k == nullptr || (ldk % 8 == 0 && ldv % 8 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0)) &&
            (uintptr_t)cos_table % 16 == 0 && (uintptr_t)sin_table % 16 == 0 && (uintptr_t)cache % 16 == 0)
-    rope_cache_pairs_kernel<<<n, 256, 0, stream>>>((bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv,
-        positions, token_segment, block_tables, bt_stride, cos_table, sin_table, half, (bf16_t*)cache, lay, num_heads);
+  {
+    // (the values of 16 tokens through LDS, if a workgroup's share of it fits and there is more than one group)
+    const size_t group_bytes = (size_t)32 * kv_heads * head_dim;
+    const int by_groups = k != nullptr && cache != nullptr && n >= 32 && group_bytes <= 48 * 1024;
+    rope_cache_pairs_kernel<<<n + (by_groups ? (n + 15) / 16 : 0), 256, by_groups ? group_bytes : 0, stream>>>(
+        (bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv, positions, token_segment, block_tables, bt_stride,
+        cos_table, sin_table, half, (bf16_t*)cache, lay, num_heads, n, by_groups);
+  }
   else if (dtype == DT_BF16)
     rope_cache_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv,
         positions, token_segment, block_tables, bt_stride, cos_table, sin_table, half, pairing,

@@ -565,6 +565,47 @@ def test_rope_cache_write(pairing, dtype):
             assert torch.equal(lay[page, 1, h].view(hd, ps)[:, vslot(slot)], v[t].view(K, hd)[h])
 
 
+@pytest.mark.parametrize("ps", [16, 32])
+def test_rope_cache_write_of_long_portions(ps):
+    """From 32 tokens on the values of 16 consecutive tokens are written together: whole
+    32-byte runs of the transposed value layout where the 16 tokens fill 16 slots in a row of
+    one page, element by element where they do not (a portion that starts inside a page, a
+    group that spans two requests, the last, partial group).  Two requests with their own
+    block tables; every key and value is found where the layout says."""
+    from hfee_amd.kernels import ops
+    from hfee_amd.parts.rotary import Rotary
+    from hfee_amd.config.specs import PositionSpec, params
+    H, K, hd = 3, 2, 32
+    rot = Rotary(PositionSpec("rope", params(head_dim=hd, rotary_dim=hd, theta=10000.0, scaling=None, pairing="interleaved")))
+    rot.prepare(256, DEV)
+    # request 0: positions 32 .. 84 (starts on a page's edge); request 1: positions 5 .. 58 (does not)
+    pos = torch.tensor(list(range(32, 85)) + list(range(5, 59)), dtype=torch.int32)
+    seg = torch.tensor([0] * 53 + [1] * 54, dtype=torch.int32)
+    T = pos.numel()
+    g = torch.Generator().manual_seed(ps)
+    q = torch.randn(T, H * hd, generator=g).to(torch.bfloat16)
+    k = torch.randn(T, K * hd, generator=g).to(torch.bfloat16)
+    v = torch.randn(T, K * hd, generator=g).to(torch.bfloat16)
+    blocks = 96 // ps
+    tables = torch.randperm(2 * blocks, generator=g).to(torch.int32).reshape(2, blocks)
+    layer = torch.zeros(2 * blocks, 2, K, ps * hd, dtype=torch.bfloat16, device=DEV)
+    one_by_one = torch.zeros_like(layer)
+    args = (rot.cos, rot.sin, rot.pairing)
+    ops.rope_cache_write(q.clone().to(DEV), k.to(DEV), v.to(DEV), pos.to(DEV), seg.to(DEV), tables.to(DEV), *args,
+                         layer, H, K, hd, ps, int(pos.max()))
+    for t in range(T):          # the same, a token a call: the path for short batches
+        ops.rope_cache_write(q[t:t + 1].clone().to(DEV), k[t:t + 1].to(DEV), v[t:t + 1].to(DEV), pos[t:t + 1].to(DEV),
+                             torch.zeros(1, dtype=torch.int32, device=DEV), tables[int(seg[t]):int(seg[t]) + 1].to(DEV),
+                             *args, one_by_one, H, K, hd, ps, int(pos.max()))
+    assert torch.equal(layer, one_by_one)
+    lay = layer.cpu()
+    for t in range(T):
+        p = int(pos[t])
+        page, slot = int(tables[int(seg[t]), p // ps]), p % ps
+        for h in range(K):
+            assert torch.equal(lay[page, 1, h].view(hd, ps)[:, vslot(slot)], v[t].view(K, hd)[h])
+
+
 def test_argmax_first_maximum_wins():
     from hfee_amd.kernels import ops
     logits = torch.zeros(3, 5000)
