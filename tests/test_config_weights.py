@@ -165,3 +165,17 @@ def test_schedule_and_cache_groups_are_data():
     assert kinds["full"].cache_layers == (0, 2) and kinds["window"].cache_layers == (1,) and kinds["window"].window == 32
     with pytest.raises(ValueError, match="which no layer writes"):
         Model(replace(spec, schedule=(ScheduleEntry(0, 0), ScheduleEntry(1, 5, False))), torch.float32).cache_groups()
+
+
+def test_the_benchmark_refuses_more_than_one_gpu():
+    """`bench.py --gpus N` for N > 1 prints one line that says so and exits with 2, before
+    anything touches a GPU."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    done = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "4", "--steps", "2", "--warmup", "1"],
+                          capture_output=True, text=True, timeout=120)
+    assert done.returncode == 2
+    lines = [l for l in (done.stdout + done.stderr).splitlines() if l.strip()]
+    assert len(lines) == 1 and "one GPU" in lines[0]
