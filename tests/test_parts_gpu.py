@@ -464,6 +464,32 @@ def test_sampler_kernel_follows_the_plain_rules(V):
     assert mixed[2] == alone[0] and mixed[1] == 17
 
 
+@pytest.mark.parametrize("top_k", [40, 700, 1500])
+def test_sampler_takes_the_first_ties_at_the_top_k_threshold(top_k):
+    """Thousands of equal logits at the top_k threshold, spread over the whole vocabulary (so
+    over all the waves that gather the kept set): the ones with the smallest ids belong, as
+    many as top_k leaves room for after the larger logits (sampler.go:132-151)."""
+    from plain_llama import plain_sampling_distribution
+    from hfee_amd.sampling import SampleRow, Sampler, SamplingParams
+    V = 9001
+    g = torch.Generator().manual_seed(top_k)
+    base = torch.full((V,), -2.0)
+    tied = torch.randperm(V, generator=g)[:4000]
+    base[tied] = 1.0
+    larger = torch.randperm(V, generator=g)[:10]
+    base[larger] = 1.5
+    p = SamplingParams(temperature=1.0, top_k=top_k, top_p=1.0, min_p=0.0, repeat_penalty=1.0)
+    support = set(plain_sampling_distribution(base, p.temperature, p.top_k, p.top_p, p.min_p).nonzero().flatten().tolist())
+    assert len(support) == top_k
+    sampler = Sampler(V, DEV, max_rows=64)
+    seen = set()
+    for c in range(12):
+        rows = [SampleRow(p, seed=3, draw=64 * c + r, history=[], logits_row=r) for r in range(64)]
+        seen |= set(sampler.sample(base.repeat(64, 1).to(DEV), rows))
+    assert seen <= support, sorted(seen - support)[:5]
+    assert len(seen) >= min(top_k, 300) // 2            # and the draws do spread over it
+
+
 def test_sampler_with_a_top_k_too_large_to_gather():
     """A top_k above 1,024 is not gathered into LDS: the radix select's threshold then
     serves the rules that run over the whole vocabulary.  Draws match the inverse CDF of
