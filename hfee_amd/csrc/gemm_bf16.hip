@@ -377,9 +377,20 @@ template <int MODE, int TM, int TN, int STAGES>
 __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restrict__ C, int64_t ldc,
                                                                   const bf16_t* __restrict__ A, int64_t lda,
                                                                   const bf16_t* __restrict__ W, int64_t ldw,
-                                                                  int M, int N, int K, QkvArgs qkv, RowScale rs) {
+                                                                  int M, int N, int K, QkvArgs qkv, RowScale rs,
+                                                                  int k_split, int64_t c_split) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
   extern __shared__ __attribute__((aligned(16))) bf16_t lds_tiles[];
+  // K cut over workgroups (k_split > 0): workgroup row blockIdx.y takes columns
+  // y * k_split .. of A and W and leaves its product in a matrix of its own, c_split elements
+  // after the one before; a second kernel adds them up.
+  if (k_split > 0) {
+    const int z = blockIdx.y;
+    A += (int64_t)z * k_split;
+    W += (int64_t)z * k_split;
+    K = min(k_split, K - z * k_split);
+    C = (void*)((float*)C + (int64_t)z * c_split);
+  }
   auto a_tile = [&](int buf) { return lds_tiles + buf * (BM * PPITCH); };
   auto w_tile = [&](int buf) { return lds_tiles + 2 * BM * PPITCH + buf * (BN * PPITCH); };
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -528,24 +539,102 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
   }
 }
 
+// Scratch that a caller may bring for products with few tiles (see launch_pipelined).
+struct Partial {
+  float* at = nullptr;
+  int64_t floats = 0;
+};
+
+// The second kernel of a product whose K was cut over workgroups: adds the `splits`
+// partial products (each M x N float32, one after the other) in their order and stores
+// the sum the way MODE says.  Four columns a thread; N is a multiple of 4 and the rows of C
+// are aligned for it.
 template <int MODE>
-int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                     int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, const RowScale& rs = RowScale{}) {
-  // 128 x 128 tiles, two workgroups per CU.  (128 x 256 tiles halve the LDS reads per
-  // matrix instruction but leave one wave per SIMD, and measured 20 % slower.)
-  constexpr int TM = 2, TN = 2, STAGES = 3;
-  const size_t lds = (size_t)2 * (64 * TM + 64 * TN) * PPITCH * sizeof(bf16_t);
+__global__ __launch_bounds__(256) void gemm_split_finish_kernel(void* __restrict__ C, int64_t ldc,
+                                                                const float* __restrict__ partial, int splits,
+                                                                int M, int N) {
+  const int quads = N >> 2;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * quads) return;
+  const int m = (int)(idx / quads), n = 4 * (int)(idx - (int64_t)m * quads);
+  constexpr int MOST = 8;
+  f32x4 part[MOST];
+#pragma unroll
+  for (int z = 0; z < MOST; ++z)        // all asked for together; past the last one: a repeat that is not added
+    part[z] = *reinterpret_cast<const f32x4*>(partial + ((int64_t)min(z, splits - 1) * M + m) * N + n);
+  f32x4 sum = part[0];
+#pragma unroll
+  for (int z = 1; z < MOST; ++z)
+    if (z < splits) sum += part[z];
+  if constexpr (MODE == OUT_BF16) {
+    u32x2 o;
+    o[0] = (uint32_t)float_to_bf16(sum[0]) | ((uint32_t)float_to_bf16(sum[1]) << 16);
+    o[1] = (uint32_t)float_to_bf16(sum[2]) | ((uint32_t)float_to_bf16(sum[3]) << 16);
+    *reinterpret_cast<u32x2*>((bf16_t*)C + (int64_t)m * ldc + n) = o;
+  } else {
+    f32x4* c = reinterpret_cast<f32x4*>((float*)C + (int64_t)m * ldc + n);
+    if constexpr (MODE == OUT_ADD_F32) sum += *c;
+    *c = sum;
+  }
+}
+
+template <int MODE>
+int raise_pipelined_lds(size_t lds) {
   static bool raised = false;
   if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_pipelined_kernel<MODE, 2, 2, 3>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail("gemm_bf16: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
+  return 0;
+}
+
+// How many ways K is cut for M x N x K through 128 x 128 tiles (1: not at all): with fewer
+// than 256 tiles a part of the chip stands idle while a few workgroups walk the whole of K
+// (the output and down products of a prompt of 128 tokens: 32 tiles); the cut makes up to
+// 512 workgroups of them, each with at least 512 columns.
+inline int pipelined_splits(int M, int N, int K) {
+  const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
+  if (M <= 64 || tiles >= 256 || K < 2048 || N % 4 != 0) return 1;
+  // (two workgroups of this kernel fit a CU; measured, a prompt of 128 tokens is faster with one a CU
+  // and fewer partial products, one of 512 tokens with two)
+  int splits = (int)((tiles < 128 ? 256 : 512) / tiles);
+  if (splits > 8) splits = 8;
+  if (splits > K / 512) splits = K / 512;
+  if (splits < 2) return 1;
+  const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+  return (K + k_split - 1) / k_split;
+}
+
+template <int MODE>
+int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
+                     int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, const RowScale& rs = RowScale{},
+                     const Partial& partial = Partial{}) {
+  // 128 x 128 tiles, two workgroups per CU.  (128 x 256 tiles halve the LDS reads per
+  // matrix instruction but leave one wave per SIMD, and measured 20 % slower.)
+  constexpr int TM = 2, TN = 2, STAGES = 3;
+  const size_t lds = (size_t)2 * (64 * TM + 64 * TN) * PPITCH * sizeof(bf16_t);
+  if (raise_pipelined_lds<MODE>(lds)) return 1;
   const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
   if (tiles > (1 << 30)) return fail("gemm_bf16: too many tiles");
   dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
-  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv, rs);
+  if constexpr (MODE == OUT_BF16 || MODE == OUT_F32 || MODE == OUT_ADD_F32) {
+    const int splits = pipelined_splits(M, N, K);
+    const bool rows_fit = MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0) : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
+    if (splits > 1 && rs.shares == nullptr && rows_fit && partial.at != nullptr && (uintptr_t)partial.at % 16 == 0 &&
+        partial.floats >= (int64_t)splits * M * N) {
+      if (raise_pipelined_lds<OUT_F32>(lds)) return 1;
+      const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+      grid.y = splits;
+      gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
+          partial.at, N, A, lda, W, ldw, M, N, K, qkv, rs, k_split, (int64_t)M * N);
+      const int64_t threads = (int64_t)M * (N / 4);
+      gemm_split_finish_kernel<MODE><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(C, ldc, partial.at, splits, M, N);
+      return 0;
+    }
+  }
+  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv, rs, 0, 0);
   return 0;
 }
 
@@ -1068,23 +1157,24 @@ inline TiledPlan plan_tiled(int M, int N, int K, bool large_ok, bool may_split) 
 
 template <int MODE>
 int launch_tiled_kernel(int choice, void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                        int M, int N, int K, hipStream_t stream, const QkvArgs& qkv) {
+                        int M, int N, int K, hipStream_t stream, const QkvArgs& qkv, const Partial& partial = Partial{}) {
   if (choice == 6) return launch_direct<MODE, 4, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
-  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream, RowScale{}, partial);
 }
 
 template <int MODE>
 int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                   int M, int N, int K, int force_kernel, hipStream_t stream, const QkvArgs& qkv = QkvArgs{}) {
+                   int M, int N, int K, int force_kernel, hipStream_t stream, const QkvArgs& qkv = QkvArgs{},
+                   const Partial& partial = Partial{}) {
   const bool large_ok = large_fits(lda, ldw, M, N, K);
   if (force_kernel == 2 || (force_kernel >= 4 && force_kernel <= 6))
     return launch_tiled_kernel<MODE>(force_kernel >= 4 && !large_ok ? 2 : force_kernel, C, ldc, A, lda, W, ldw, M, N, K,
-                                     stream, qkv);
+                                     stream, qkv, partial);
   // (the q/k/v epilogue finds a column's head by its number: those products stay whole)
   const TiledPlan plan = plan_tiled(M, N, K, large_ok, MODE != OUT_QKV);
-  if (int rc = launch_tiled_kernel<MODE>(plan.first, C, ldc, A, lda, W, ldw, M, plan.n1, K, stream, qkv)) return rc;
+  if (int rc = launch_tiled_kernel<MODE>(plan.first, C, ldc, A, lda, W, ldw, M, plan.n1, K, stream, qkv, partial)) return rc;
   if (plan.second == 0) return 0;
   const int64_t skip = MODE == OUT_SWIGLU ? plan.n1 / 2 : plan.n1;         // output columns of the first part
   void* c2 = (MODE == OUT_BF16 || MODE == OUT_SWIGLU) ? (void*)((bf16_t*)C + skip) : (void*)((float*)C + skip);
@@ -1099,7 +1189,7 @@ inline bool skinny_pays(int M, int N) { return M <= 16 || (M <= 64 && N < 16384)
 
 template <int MODE, bool VEC>
 int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-           int M, int N, int K, int force_kernel, hipStream_t stream) {
+           int M, int N, int K, int force_kernel, hipStream_t stream, const Partial& partial) {
   const bool skinny = force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N));
   if (skinny) {
     const int mt = (M + 15) / 16;
@@ -1119,7 +1209,7 @@ int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, 
     dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM);
     if (grid.y > 65535) return fail("gemm_bf16: too many rows (%d)", M);
     if (VEC && force_kernel != 3)
-      return launch_aligned<MODE>(C, ldc, A, lda, W, ldw, M, N, K, force_kernel, stream);
+      return launch_aligned<MODE>(C, ldc, A, lda, W, ldw, M, N, K, force_kernel, stream, QkvArgs{}, partial);
     gemm_bf16_tiled_kernel<MODE, VEC><<<grid, 256, 0, stream>>>(C, ldc, A, lda, W, ldw, M, N, K);
   }
   return 0;
@@ -1171,8 +1261,21 @@ HFEE_API int hfee_gemm_bf16_plan(int M, int N, int K, int* first, int* n1, int* 
 // force_kernel: 0 choose by the sizes, 1 skinny, 2 tiled 128 x 128, 3 the simple tiled
 // kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192 (for tests of each
 // kernel alone; 4 to 6 fall back to 2 where they do not apply).
+// float32 words of scratch that hfee_gemm_bf16 can use for M x N x K (0: none): products with
+// too few tiles for the chip are cut along K over more workgroups, which leave their partial
+// products there for a second kernel to add up.
+HFEE_API int hfee_gemm_bf16_scratch(int M, int N, int K) {
+  const int splits = pipelined_splits(M, N, K);          // (fewer than 256 tiles of 128 x 128, at most 8 cuts: it fits an int)
+  return splits > 1 ? splits * M * N : 0;
+}
+
+// scratch: null, or hfee_gemm_bf16_scratch(M, N, K) float32 words, 16-byte aligned.
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
-                            int64_t ldw, int M, int N, int K, int force_kernel, hipStream_t stream) {
+                            int64_t ldw, int M, int N, int K, int force_kernel, float* scratch,
+                            int64_t scratch_floats, hipStream_t stream) {
+  Partial partial;
+  partial.at = scratch;
+  partial.floats = scratch != nullptr ? scratch_floats : 0;
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16: a leading dimension is shorter than its row");
   HFEE_REQUIRE(out_mode >= 0 && out_mode <= 3, "gemm_bf16: unknown output mode %d", out_mode);
@@ -1197,8 +1300,8 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
   const bf16_t* w = (const bf16_t*)W;
   int rc;
 #define GO(MODE)                                                                                  \
-  rc = vec ? launch<MODE, true>(C, ldc, a, lda, w, ldw, M, N, K, force_kernel, stream)             \
-           : launch<MODE, false>(C, ldc, a, lda, w, ldw, M, N, K, force_kernel, stream)
+  rc = vec ? launch<MODE, true>(C, ldc, a, lda, w, ldw, M, N, K, force_kernel, stream, partial)    \
+           : launch<MODE, false>(C, ldc, a, lda, w, ldw, M, N, K, force_kernel, stream, partial)
   if (out_mode == OUT_BF16) GO(OUT_BF16);
   else if (out_mode == OUT_F32) GO(OUT_F32);
   else GO(OUT_ADD_F32);

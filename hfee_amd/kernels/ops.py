@@ -102,9 +102,17 @@ def residual_add(x: torch.Tensor, y: torch.Tensor):
 
 # ---------------------------------------------------------------- matrix product
 
+def linear_scratch(m: int, n: int, k: int) -> int:
+    """float32 words of scratch that `linear` can use for a bfloat16 product of m rows with an
+    [n, k] weight (0: none): with too few tiles for the chip, K is cut over more workgroups,
+    which leave their partial products there for a second kernel to add up."""
+    return int(lib.core().raw("hfee_gemm_bf16_scratch")(int(m), int(n), int(k)))
+
+
 def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate: bool = False, kernel: int = 0,
-           gate: bool = False):
+           gate: bool = False, scratch=None):
     """out (+)= x @ weight.T, weight stored [out_features, in_features].
+    scratch (bfloat16 products): float32, `linear_scratch(M, N, K)` words, or None.
 
     float32 x and weight: the true 32-bit product, out float32.
     bfloat16 x and weight: matrix cores with float32 accumulation; out bfloat16, or
@@ -122,7 +130,8 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
     if gate:
         _check(x.dtype == weight.dtype == out.dtype == torch.bfloat16 and not accumulate and N % 2 == 0,
                "linear: the gate epilogue takes bfloat16 operands and an even number of weight rows")
-        lib.core().call("hfee_gemm_bf16", _ptr(out), 3, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K, kernel, _stream())
+        lib.core().call("hfee_gemm_bf16", _ptr(out), 3, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K, kernel,
+                        None, 0, _stream())
         return
     _check(x.dtype == weight.dtype, "linear: x and weight dtypes differ")
     if x.dtype == torch.float32:
@@ -136,8 +145,11 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
         else:
             mode = 0 if out.dtype == torch.bfloat16 else 1
             _check(out.dtype in (torch.bfloat16, torch.float32), "linear: out dtype")
+        if scratch is not None:
+            _gpu(scratch)
+            _check(scratch.dtype == torch.float32 and scratch.is_contiguous(), "linear: float32 scratch expected")
         lib.core().call("hfee_gemm_bf16", _ptr(out), mode, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K,
-                        kernel, _stream())
+                        kernel, _ptr(scratch), 0 if scratch is None else scratch.numel(), _stream())
     else:
         raise KernelError(f"linear: unsupported dtype {x.dtype}")
 

@@ -154,7 +154,7 @@ class Attention(Mixer):
         else:
             hn = h.tensor() if isinstance(h, LazyNorm) else h
             if writes_cache:
-                ops.linear(qkv, hn, self.w_qkv)
+                ops.linear(qkv, hn, self.w_qkv, **ctx.workspace.split_scratch(n, self.w_qkv))
                 k = qkv[:, self.q_width:self.q_width + self.kv_width]
                 v = qkv[:, self.q_width + self.kv_width:]
             else:   # this run of the layer reads keys and values that another run wrote
@@ -198,4 +198,4 @@ class Attention(Mixer):
         if emit:       # the output projection adds into x and begins the norm that follows
             ops.linear_fused(x, att, self.w_o, "add", emit=emit, **ctx.workspace.product_scratch(n, self.w_o))
         else:
-            ops.linear(x, att, self.w_o, accumulate=True)
+            ops.linear(x, att, self.w_o, accumulate=True, **ctx.workspace.split_scratch(n, self.w_o))

@@ -217,6 +217,15 @@ class Workspace:
             return {}
         return dict(scratch=self.flat("product.partial", words, torch.float32))
 
+    def split_scratch(self, n_rows: int, weight: torch.Tensor) -> dict:
+        """The `scratch` argument of `ops.linear` for a bfloat16 product of n_rows rows with
+        this weight (empty where it has no use for it)."""
+        from ..kernels import ops
+        if weight.dtype != torch.bfloat16:
+            return {}
+        words = ops.linear_scratch(n_rows, weight.shape[0], weight.shape[1])
+        return dict(scratch=self.flat("product.partial", words, torch.float32)) if words else {}
+
     def counters(self, name: str, count: int) -> torch.Tensor:
         """`count` int32 that are zero, for kernels whose workgroups count themselves
         (the one that finishes last does a final piece of work and sets the counter

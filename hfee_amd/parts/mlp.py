@@ -69,4 +69,4 @@ class GatedMLP(FeedForward):
         elif aligned and ops.FUSED_NORM_MAX_ROWS < n <= ops.SKINNY_MAX_ROWS:
             ops.linear_fused(x, act, self.w_down, "add", **ctx.workspace.product_scratch(n, self.w_down))
         else:
-            ops.linear(x, act, self.w_down, accumulate=True)
+            ops.linear(x, act, self.w_down, accumulate=True, **ctx.workspace.split_scratch(n, self.w_down))

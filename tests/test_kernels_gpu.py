@@ -100,6 +100,40 @@ def test_gemm_bf16(M, N, K, kernel, mode):
     assert (err <= tol * (1 + mag)).all(), float((err / (1 + mag)).max())
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 640, 2112),
+                                   (100, 2048, 2048)])
+@pytest.mark.parametrize("mode", ["bf16", "f32", "add"])
+def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
+    """Products with too few 128 x 128 tiles for the chip: given scratch, K is cut over up to
+    eight times as many workgroups and a second kernel adds the partial products (K that is
+    no multiple of the cut, M and N that are no multiples of a tile); the same numbers as
+    without scratch up to the order of the sums."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(M + 3 * N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    ref = x.double() @ w.double().t()
+    mag = x.abs().double() @ w.abs().double().t()
+    words = ops.linear_scratch(M, N, K)
+    assert words >= 2 * M * N and words % (M * N) == 0
+    scratch = torch.full((words,), float("nan"), dtype=torch.float32, device=DEV)
+    c0 = torch.randn(M, N, generator=g)
+    outs = []
+    for kw in (dict(scratch=scratch), dict()):
+        if mode == "add":
+            out = c0.clone().to(DEV)
+            ops.linear(out, x.to(DEV), w.to(DEV), accumulate=True, **kw)
+            want, tol = ref + c0.double(), 1e-5
+        else:
+            out = torch.zeros(M, N, dtype=torch.bfloat16 if mode == "bf16" else torch.float32, device=DEV)
+            ops.linear(out, x.to(DEV), w.to(DEV), **kw)
+            want, tol = ref, 1e-2 if mode == "bf16" else 1e-5
+        err = (out.double().cpu() - want).abs()
+        assert (err <= tol * (1 + mag + want.abs())).all(), float((err / (1 + mag)).max())
+        outs.append(out)
+    assert ops.linear_scratch(64, N, K) == 0 and ops.linear_scratch(2048, 4096, K) == 0
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 128, 32), (300, 200, 520), (2048, 512, 1024), (129, 258, 72), (65, 130, 200),
                                    (257, 384, 64), (1000, 96, 4096), (600, 520, 192), (256, 512, 64),
                                    (513, 258, 320)])
