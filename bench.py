@@ -61,6 +61,8 @@ def main() -> int:
                          "steps at that context with --batch requests; prints its own line")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own short line")
+    ap.add_argument("--prefill-tokens", type=int, default=0, metavar="T",
+                    help="with --prefill-only: a prompt of T tokens (65 to 2,048) in place of 2,048")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -135,16 +137,16 @@ def main() -> int:
             sched.step()
         return dt, mean_ctx
 
-    def prefill_run():
+    def prefill_run(tokens: int = PREFILL):
         best = None
         for i in range(3):
-            prompt = torch.randint(0, V, (PREFILL,), generator=gen).tolist()
+            prompt = torch.randint(0, V, (tokens,), generator=gen).tolist()
             from hfee_amd.engine import StepEntry
             rid = ("prefill", i)
             engine.admit(rid)
             torch.cuda.synchronize()
             t = time.perf_counter()
-            logits = engine.step([StepEntry(rid, prompt, [PREFILL - 1])])
+            logits = engine.step([StepEntry(rid, prompt, [tokens - 1])])
             del logits
             torch.cuda.synchronize()
             dt = time.perf_counter() - t
@@ -235,8 +237,13 @@ def main() -> int:
         return 0
 
     if args.prefill_only:
-        pt = prefill_run()
-        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": PREFILL, "layers": L}), flush=True)
+        tokens = args.prefill_tokens or PREFILL
+        if not 1 <= tokens <= PREFILL:
+            print(f"bench.py: --prefill-tokens takes 1 to {PREFILL}")
+            return 2
+        pt = prefill_run(tokens)
+        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": tokens, "layers": L,
+                          "us_per_layer": round(pt * 1e6 / L, 1)}), flush=True)
         return 0
 
     dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
