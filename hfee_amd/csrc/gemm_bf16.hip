@@ -591,18 +591,19 @@ int raise_pipelined_lds(size_t lds) {
 }
 
 // How many ways K is cut for M x N x K through 128 x 128 tiles (1: not at all): with fewer
-// than 256 tiles a part of the chip stands idle while a few workgroups walk the whole of K
+// than 256 tiles (384 where K is long) a part of the chip stands idle while a few workgroups walk the whole of K
 // (the output and down products of a prompt of 128 tokens: 32 tiles); the cut makes up to
 // 512 workgroups of them, each with at least 512 columns.
 inline int pipelined_splits(int M, int N, int K) {
   const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
-  if (M <= 64 || tiles >= 256 || K < 2048 || N % 4 != 0) return 1;
+  const bool long_k = K >= 8192;
+  if (M <= 64 || tiles >= (long_k ? 384 : 256) || K < 2048 || N % 4 != 0) return 1;
   // (two workgroups of this kernel fit a CU; measured, a prompt of 128 tokens is faster with one a CU
-  // and fewer partial products, one of 512 tokens with two)
-  int splits = (int)((tiles < 128 ? 256 : 512) / tiles);
+  // and fewer partial products, one of 512 tokens with two; two cuts only pay where K is long)
+  int splits = tiles < 128 ? (int)(256 / tiles) : tiles < 256 ? (int)(512 / tiles) : 2;
   if (splits > 8) splits = 8;
   if (splits > K / 512) splits = K / 512;
-  if (splits < 2) return 1;
+  if (splits < 2 || (splits == 2 && !long_k)) return 1;
   const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
   return (K + k_split - 1) / k_split;
 }
