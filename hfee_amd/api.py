@@ -9,9 +9,7 @@ and the reason it ended.
 from __future__ import annotations
 
 import os
-from dataclasses import dataclass, field
-
-import torch
+from dataclasses import dataclass
 
 from .engine import Engine, load_model, random_model
 from .engine.scheduler import Request, Scheduler, Stats

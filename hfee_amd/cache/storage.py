@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import torch
 
-from .manager import CacheGroupSpec, CacheError
+from .manager import CacheError
 
 
 class CacheStorage:

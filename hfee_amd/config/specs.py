@@ -8,7 +8,7 @@ part classes in `hfee_amd.parts` are chosen by the `kind` strings, layer by laye
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Any, Optional
 
 

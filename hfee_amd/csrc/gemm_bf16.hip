@@ -1193,7 +1193,6 @@ int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, 
            int M, int N, int K, int force_kernel, hipStream_t stream, const Partial& partial) {
   const bool skinny = force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N));
   if (skinny) {
-    const int mt = (M + 15) / 16;
     dim3 grid((N + SK_ROWS - 1) / SK_ROWS);
     for (int m0 = 0; m0 < M; m0 += 64) {   // M > 64 only when the kernel was forced
       const int rows = M - m0 < 64 ? M - m0 : 64;
@@ -1205,7 +1204,6 @@ int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, 
       else if (g == 3) gemm_bf16_skinny_kernel<MODE, VEC, 3><<<grid, SK_WAVES * 64, 0, stream>>>(c, ldc, a, lda, W, ldw, rows, N, K);
       else gemm_bf16_skinny_kernel<MODE, VEC, 4><<<grid, SK_WAVES * 64, 0, stream>>>(c, ldc, a, lda, W, ldw, rows, N, K);
     }
-    (void)mt;
   } else {
     dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM);
     if (grid.y > 65535) return fail("gemm_bf16: too many rows (%d)", M);
@@ -1257,11 +1255,6 @@ HFEE_API int hfee_gemm_bf16_plan(int M, int N, int K, int* first, int* n1, int* 
   return 0;
 }
 
-// out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate (the
-// rows of W alternate gate/up; C is [M, N/2] bfloat16; aligned operands and M > 64 only).
-// force_kernel: 0 choose by the sizes, 1 skinny, 2 tiled 128 x 128, 3 the simple tiled
-// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192 (for tests of each
-// kernel alone; 4 to 6 fall back to 2 where they do not apply).
 // float32 words of scratch that hfee_gemm_bf16 can use for M x N x K (0: none): products with
 // too few tiles for the chip are cut along K over more workgroups, which leave their partial
 // products there for a second kernel to add up.
@@ -1270,6 +1263,12 @@ HFEE_API int hfee_gemm_bf16_scratch(int M, int N, int K) {
   return splits > 1 ? splits * M * N : 0;
 }
 
+// C = A W^T for bfloat16 A [M, K] and W [N, K].
+// out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate (the
+// rows of W alternate gate/up; C is [M, N/2] bfloat16; aligned operands only).
+// force_kernel: 0 choose by the sizes, 1 skinny, 2 tiled 128 x 128, 3 the simple tiled
+// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192 (for tests of each
+// kernel alone; 4 to 6 fall back to 2 where they do not apply).
 // scratch: null, or hfee_gemm_bf16_scratch(M, N, K) float32 words, 16-byte aligned.
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
                             int64_t ldw, int M, int N, int K, int force_kernel, float* scratch,
@@ -1288,15 +1287,13 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
   if (out_mode == 3) {
     HFEE_REQUIRE(N % 2 == 0 && vec, "gemm_bf16: the SiLU gate needs an even N and aligned operands");
     if (skinny_pays(M, N))
-      return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, 3, nullptr, 0, 0.f, nullptr, nullptr, nullptr, nullptr,
-                              0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, nullptr, 0, 0, stream);
+      return hfee_gemm_skinny_plain(C, ldc, A, lda, W, ldw, M, N, K, OUT_SWIGLU, stream);
     if (launch_aligned<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, force_kernel, stream)) return 1;
     HFEE_CHECK_LAUNCH("gemm_bf16");
     return 0;
   }
   if (vec && M <= 64 && (force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N))))   // gemm_skinny.hip
-    return hfee_gemm_skinny(C, ldc, A, 0, lda, W, ldw, M, N, K, out_mode, nullptr, 0, 0.f, nullptr, nullptr, nullptr,
-                            nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0, 0, 0, 0, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0.f, nullptr, 0, 0, stream);
+    return hfee_gemm_skinny_plain(C, ldc, A, lda, W, ldw, M, N, K, out_mode, stream);
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   int rc;

@@ -47,7 +47,6 @@ import time
 from collections import deque
 from dataclasses import dataclass, field
 
-from ..cache import OutOfPages
 from ..sampling import SampleRow, SamplingParams
 from .step import StepEntry
 

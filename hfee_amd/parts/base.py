@@ -18,11 +18,10 @@ bind(tensors) (take your tensors out of the dict by full name).
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Callable, Optional
+from typing import Optional
 
 import torch
 
-from ..weights.spec import TensorSpec
 
 _REGISTRIES: dict[str, dict] = {"norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}}
 

@@ -7,9 +7,9 @@ import torch
 
 import hfee_amd  # noqa: F401
 from conftest import TINY_A, TINY_B, make_model_folder
-from hfee_amd.config import ConfigError, LlamaConfig, config_from_dict, config_from_folder, model_spec_of
+from hfee_amd.config import ConfigError, config_from_dict, config_from_folder, model_spec_of
 from hfee_amd.engine.model import Model, declared_tensors
-from hfee_amd.weights import (Checkpoint, SafetensorsError, WeightsError, check_tensors, convert_for_engine,
+from hfee_amd.weights import (Checkpoint, SafetensorsError, WeightsError, convert_for_engine,
                               load_tensors, random_tensors, write_safetensors)
 
 

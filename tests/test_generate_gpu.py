@@ -1,9 +1,7 @@
 """Generation through the entry point: greedy and seeded sampling, scheduler on the GPU."""
 import pytest
-import torch
 
 import trace_util as tu
-from conftest import TINY
 
 pytestmark = pytest.mark.gpu
 

@@ -2,7 +2,6 @@
 import pytest
 import torch
 
-from conftest import TINY
 
 pytestmark = pytest.mark.gpu
 

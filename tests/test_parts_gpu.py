@@ -3,7 +3,6 @@ data (a layer run twice, a layer reading another's cache, a windowed layer); and
 toy mixer with state of its own, defined here, registered, built and stepped
 without touching the framework's files."""
 import math
-import os
 from dataclasses import dataclass, replace
 
 import numpy as np
@@ -11,7 +10,7 @@ import pytest
 import torch
 
 import trace_util as tu
-from conftest import TINY, TINY_A, make_model_folder
+from conftest import TINY_A
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"

@@ -3,7 +3,6 @@ that reduce to a library routine, invariants, and the vectors that the reference
 own tests hold.  Each is chosen so that a plausible mistake fails it."""
 import math
 
-import pytest
 import torch
 import torch.nn.functional as F
 
