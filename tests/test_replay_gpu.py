@@ -134,3 +134,54 @@ def test_trace_run_program(model_folders, tmp_path, dtype):
     assert rel(s0[0], la[0]) < tol and rel(s0[1], la[9]) < tol
     assert rel(s1[0], lb[8]) < tol
     assert rel(s2[0], la[20]) < tol and rel(s2[1], la[12]) < tol
+
+
+def random_configuration(rng):
+    """A small configuration of the architecture with every size drawn: head sizes in steps of
+    16 up to 256, any number of heads and groups, widths that are multiples of 8, 4 or 2,
+    any feed-forward width and vocabulary."""
+    kv_heads = rng.randint(1, 4)
+    scaling = None
+    if rng.random() < 0.4:
+        scaling = {"rope_type": "llama3", "factor": rng.choice([2.0, 8.0, 32.0]), "low_freq_factor": 1.0,
+                   "high_freq_factor": rng.choice([2.0, 4.0]),
+                   "original_max_position_embeddings": rng.choice([32, 64, 128])}
+    return {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": rng.randint(1, 4),
+            "hidden_size": rng.choice([8, 8, 8, 4, 2]) * rng.randint(5, 40),
+            "num_attention_heads": kv_heads * rng.choice([1, 1, 2, 3, 4, 5, 7, 8]), "num_key_value_heads": kv_heads,
+            "head_dim": 16 * rng.randint(1, 16), "intermediate_size": rng.choice([8, 8, 4, 2, 1]) * rng.randint(9, 70),
+            "vocab_size": rng.randint(50, 3000), "max_position_embeddings": 512,
+            "rope_theta": rng.choice([10000.0, 500000.0, 1e6]), "rope_scaling": scaling,
+            "rms_norm_eps": rng.choice([1e-5, 1e-6, 3e-4]), "tie_word_embeddings": rng.random() < 0.5,
+            "hidden_act": "silu"}
+
+
+@pytest.mark.parametrize("seed", [7, 10, 18, 22, 30, 37])
+def test_drawn_configurations_match_the_plain_implementation(tmp_path, seed):
+    """Six configurations with sizes drawn at random, whole and mixed, in both types.  These seeds
+    draw widths of 36, 58 and 68, head sizes from 80 to 224, 15 heads in 3 groups, 32 in 4,
+    feed-forward widths of 9, 11 and 37, a vocabulary of 66, and the scaled rotation thrice."""
+    import random
+
+    from conftest import make_model_folder
+    from plain_llama import PlainLlama
+    from hfee_amd.replay import Replayer
+    rng = random.Random(4000 + seed)
+    cj = random_configuration(rng)
+    lengths = [rng.randint(1, 200) for _ in range(4)]
+    reqs = tu.make_requests(cj["vocab_size"], lengths, seed=seed)
+    mixed_steps, peak = tu.mixed(reqs, seed=seed)
+    for dtype in ("float32", "bfloat16"):
+        folder = make_model_folder(tmp_path / dtype, cj, seed=seed, dtype=dtype, std=0.05, norm_init="one_plus_normal")
+        plain = PlainLlama(folder)
+        want = {}
+        for rid, toks in reqs.items():
+            lg = plain.forward(toks)
+            for p in range(len(toks)):
+                want[(rid, p)] = lg[p].numpy()
+        rep = Replayer(folder, dtype, max_tokens=max(peak, 256))
+        for what, steps in (("whole", tu.whole(reqs)), ("mixed", mixed_steps)):
+            sizes = {k: cj[k] for k in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim",
+                                        "intermediate_size", "vocab_size", "num_hidden_layers")}
+            check(tu.run(rep, steps), want, TOL[dtype], f"{sizes} {dtype} {what}")
+            rep.engine.cache.check()
