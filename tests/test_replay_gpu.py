@@ -185,3 +185,50 @@ def test_drawn_configurations_match_the_plain_implementation(tmp_path, seed):
                                         "intermediate_size", "vocab_size", "num_hidden_layers")}
             check(tu.run(rep, steps), want, TOL[dtype], f"{sizes} {dtype} {what}")
             rep.engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_requests_decoding_together(tmp_path, dtype):
+    """72, then 40, 20, 10 and 3 requests decode in one step each, in a changing order: products
+    and decode attention of more than 64, of 17 to 64 and of fewer rows inside the whole model
+    (the other replays hold four requests at most); the prompts come seven requests a step."""
+    import random
+
+    from conftest import make_model_folder
+    from plain_llama import PlainLlama
+    from hfee_amd.replay import Replayer
+    cj = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 2, "hidden_size": 512,
+          "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 1000,
+          "vocab_size": 777, "max_position_embeddings": 256, "rope_theta": 10000.0, "rope_scaling": None,
+          "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "hidden_act": "silu"}
+    rng = random.Random(5)
+    count, tail = 72, 12
+    lengths = [rng.randint(tail + 2, 90) for _ in range(count)]
+    folder = make_model_folder(tmp_path / "m", cj, seed=5, dtype=dtype, std=0.03, norm_init="one_plus_normal")
+    plain = PlainLlama(folder)
+    reqs = tu.make_requests(cj["vocab_size"], lengths, seed=5)
+    ids = list(reqs)
+    rep = Replayer(folder, dtype, max_tokens=sum((n + 63) // 64 * 64 for n in lengths), max_requests=count)
+    steps = []
+    for i in range(0, count, 7):
+        steps.append({"entries": [(r, reqs[r][:-tail], [len(reqs[r]) - tail - 1]) for r in ids[i:i + 7]], "end": []})
+    live, fed = list(ids), {r: len(reqs[r]) - tail for r in ids}
+    for t in range(tail):
+        live = live[:{3: 40, 6: 20, 8: 10, 10: 3}.get(t, len(live))]
+        order = list(live)
+        rng.shuffle(order)
+        steps.append({"entries": [(r, [reqs[r][fed[r]]], [0]) for r in order], "end": []})
+        for r in order:
+            fed[r] += 1
+    steps[-1]["end"] = ids
+    got = tu.run(rep, steps)
+    want = {}
+    for rid, toks in reqs.items():
+        lg = plain.forward(toks)
+        for (r, p) in got:
+            if r == rid:
+                want[(r, p)] = lg[p].numpy()
+    assert len(got) == count + 3 * 72 + 3 * 40 + 2 * 20 + 2 * 10 + 2 * 3
+    check(got, want, TOL[dtype], f"many live requests, {dtype}")
+    rep.engine.cache.check()
+    assert not rep.engine.cache.requests
