@@ -3,6 +3,7 @@ of changing size and mixed with other requests on a small page pool, in 32-bit a
 in bfloat16, all compared with the plain implementation."""
 import json
 import os
+import shutil
 import subprocess
 import sys
 
@@ -232,3 +233,54 @@ def test_many_requests_decoding_together(tmp_path, dtype):
     check(got, want, TOL[dtype], f"many live requests, {dtype}")
     rep.engine.cache.check()
     assert not rep.engine.cache.requests
+
+
+def test_layers_of_a_production_size_match_the_plain_implementation(tmp_path):
+    """Two layers with the sizes of Llama-3.1-8B (width 4,096, 32 heads in 8 groups, feed-forward
+    14,336, vocabulary 128,256, scaled rotation) in bfloat16: the kernels that only such sizes
+    choose (tiles of 256 rows, K cut over workgroups, the pair of kernels for 17 to 64 rows, the
+    streaming kernels with their fused norms) inside the whole model.  Prompts of 1,024, 300, 130
+    and 70 rows, 40 short ones eight a step, then 44, 30, 17, 8 and 2 requests decoding together."""
+    import random
+
+    from conftest import make_model_folder
+    from plain_llama import PlainLlama
+    from hfee_amd.replay import Replayer
+    cj = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 2, "hidden_size": 4096,
+          "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 14336,
+          "vocab_size": 128256, "max_position_embeddings": 8192, "rope_theta": 500000.0,
+          "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                           "original_max_position_embeddings": 8192},
+          "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "hidden_act": "silu"}
+    rng = random.Random(0)
+    tail = 10
+    lengths = [1024 + tail, 300 + tail, 130 + tail, 70 + tail] + [rng.randint(tail + 2, 40) for _ in range(40)]
+    folder = make_model_folder(tmp_path / "m", cj, seed=1, dtype="bfloat16", std=0.02, norm_init="one_plus_normal")
+    reqs = tu.make_requests(cj["vocab_size"], lengths, seed=1)
+    ids = list(reqs)
+    rep = Replayer(folder, "bfloat16", max_tokens=sum((n + 63) // 64 * 64 for n in lengths), max_requests=64)
+    steps = [{"entries": [(r, reqs[r][:-tail], [0, len(reqs[r]) - tail - 1])], "end": []} for r in ids[:4]]
+    for i in range(4, len(ids), 8):
+        steps.append({"entries": [(r, reqs[r][:-tail], [len(reqs[r]) - tail - 1]) for r in ids[i:i + 8]], "end": []})
+    live, fed = list(ids), {r: len(reqs[r]) - tail for r in ids}
+    for t in range(tail):
+        live = live[:{3: 30, 5: 17, 7: 8, 9: 2}.get(t, len(live))]
+        order = list(live)
+        rng.shuffle(order)
+        steps.append({"entries": [(r, [reqs[r][fed[r]]], [0]) for r in order], "end": []})
+        for r in order:
+            fed[r] += 1
+    steps[-1]["end"] = ids
+    got = tu.run(rep, steps)
+    rep.engine.cache.check()
+    del rep
+    plain = PlainLlama(folder)
+    want = {}
+    for rid, toks in reqs.items():
+        lg = plain.forward(toks)
+        for (r, p) in got:
+            if r == rid:
+                want[(r, p)] = lg[p].numpy()
+    del plain
+    shutil.rmtree(folder, ignore_errors=True)          # (3 GB of weights)
+    check(got, want, TOL["bfloat16"], "two layers of the 8B sizes")
