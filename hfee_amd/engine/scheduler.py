@@ -241,15 +241,13 @@ class Scheduler:
                 break
             rc = self.cache.requests[r.request_id]
             if any(len(t) * ps <= rc.length for t in rc.tables):      # its next token starts a new page
-                while self._room(r) < 1:
-                    victim = self.running[-1]
-                    if victim is r:
-                        others = [x for x in self.running if x is not r]
-                        if not others:
-                            break
-                        victim = others[-1]
+                while self._room(r) < 1 and self.running[-1] is not r:
+                    victim = self.running[-1]          # always younger than r
                     batch = [b for b in batch if b[0] is not victim]
                     self._preempt(victim)
+                if self._room(r) < 1 and len(self.running) > 1:
+                    self._preempt(r)                   # r is the youngest itself: nobody older gives way to it
+                    continue
                 if self._room(r) < 1:
                     self._finish(r, "length", finished, "the cache cannot hold this request even alone")
                     continue
@@ -257,6 +255,19 @@ class Scheduler:
             batch.append((r, r.feed[:1], True))
             budget -= 1
         budget = self.max_batch_tokens - sum(len(t) for _, t, _ in batch)
+
+        # prompt portions of requests admitted earlier, oldest first: they come before anybody
+        # new is let in, so that pages which a preemption has freed go to those who waited
+        # for them and not back to the request that gave them up
+        for r in self.running:
+            if r.decoding or budget == 0:
+                continue
+            n = min(len(r.feed), budget, self._room(r))
+            if n < 1:
+                continue
+            self.cache.reserve(r.request_id, n)
+            batch.append((r, r.feed[:n], n == len(r.feed)))
+            budget -= n
 
         # admit waiting requests while there is a slot, a place and pages for a first portion
         while self.waiting and len(self.running) < self.max_num_seqs and self.cache.num_free_slots > 0 and budget > 0:
@@ -282,18 +293,6 @@ class Scheduler:
                 self.cache.reserve(r.request_id, n)
                 batch.append((r, r.feed[:n], n == len(r.feed)))
                 budget -= n
-
-        # prompt portions of requests admitted earlier
-        in_batch = {id(b[0]) for b in batch}
-        for r in self.running:
-            if r.decoding or id(r) in in_batch or budget == 0:
-                continue
-            n = min(len(r.feed), budget, self._room(r))
-            if n < 1:
-                continue
-            self.cache.reserve(r.request_id, n)
-            batch.append((r, r.feed[:n], n == len(r.feed)))
-            budget -= n
 
         if not batch:
             if self.running and not finished:

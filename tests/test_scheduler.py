@@ -161,6 +161,52 @@ def test_scarce_pages_preempt_the_youngest_and_give_the_same_tokens():
     assert eng.cache.free_pages() == [12]
 
 
+def test_the_youngest_request_gives_way_when_it_is_the_one_that_needs_a_page():
+    """Two pages of 16 tokens; A (8 tokens, admitted first) and B (15 tokens).  B reaches
+    the edge of its page first: it is the younger one, so it is B that is preempted, never
+    A, and both produce what they produce alone."""
+    eng, s = make(num_pages=2, seqs=2, budget=64)
+    a, b = list(range(8)), list(range(20, 35))
+    s.add(Request(0, a, SamplingParams.greedy(num_predict=8), seed=0))
+    s.add(Request(1, b, SamplingParams.greedy(num_predict=4), seed=1))
+    done = run_all(s)
+    assert done[0].request.stats.preemptions == 0, "an older request was preempted for a younger one"
+    assert done[1].request.stats.preemptions >= 1
+    assert done[0].request.generated == solo(a, 0, 8) and done[0].reason == "length"
+    assert done[1].request.generated == solo(b, 1, 4) and done[1].reason == "length"
+    eng.cache.check()
+    assert eng.cache.free_pages() == [2]
+
+
+def test_random_arrivals_under_scarce_pages_never_preempt_an_older_request_for_a_younger():
+    import random
+    rng = random.Random(11)
+    for trial in range(30):
+        pages = rng.randint(3, 9)
+        eng, s = make(num_pages=pages, seqs=rng.randint(2, 4), budget=rng.choice([8, 24, 64]))
+        want = {}
+        for i in range(rng.randint(2, 6)):
+            p = [rng.randrange(VOCAB - 1) for _ in range(rng.randint(1, 30))]
+            n = rng.randint(1, 20)
+            want[i] = (p, n)
+            s.add(Request(i, p, SamplingParams.greedy(num_predict=n), seed=i))
+        order = {}
+        original = s._preempt
+
+        def spy(victim, s=s, order=order):
+            older = [r for r in s.running if r.admitted_order < victim.admitted_order]
+            younger = [r for r in s.running if r.admitted_order > victim.admitted_order]
+            assert not younger, "a request was preempted while a younger one kept running"
+            original(victim)
+        s._preempt = spy
+        done = run_all(s)
+        for i, (p, n) in want.items():
+            if done[i].error is None:
+                assert done[i].request.generated == solo(p, i, n), (trial, i)
+        eng.cache.check()
+        assert eng.cache.free_pages() == [pages]
+
+
 def test_a_request_too_large_for_the_cache_ends_with_length():
     eng, s = make(num_pages=2, seqs=2, budget=64)
     s.add(Request("big", list(range(40)), SamplingParams.greedy(num_predict=5), seed=1))
