@@ -18,6 +18,9 @@
 // The random number is counter based: splitmix64 of (seed, draw index), one stream
 // per request, independent of what else is sampled in the same call.
 #include "common.h"
+#include "no_alloc_entry.h"
+
+#include <atomic>
 
 using namespace hfee;
 
@@ -550,6 +553,59 @@ HFEE_API int hfee_argmax(int* out, const float* logits, int64_t ld, int rows, in
     argmax_kernel<<<rows, THREADS, 0, stream>>>(out, logits, ld, V);
   }
   HFEE_CHECK_LAUNCH("argmax");
+  return 0;
+}
+
+// ---- the same without a buffer from the caller (see no_alloc_entry.h) ----------------
+// The partial results and the counters live in this array.  In host code its name is only a
+// handle for hipGetSymbolAddress: every GPU has its own copy at its own address, looked up
+// once per device (with that device current) and kept in argmax_static_address; host code
+// hands that address on, never the name.
+static __device__ __align__(256) unsigned char argmax_static_scratch[HFEE_ARGMAX_STATIC_BYTES];
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> argmax_static_address[MAX_DEVICES];
+
+// (a fill kernel and not hipMemsetAsync: a caller may be capturing a graph)
+__global__ void clear_counters_kernel(int* __restrict__ counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0;
+}
+
+}  // namespace
+
+HFEE_API int hfee_argmax_static(int* out, const float* logits, int64_t ld, int rows, int V, hipStream_t stream) {
+  HFEE_REQUIRE(rows >= 0 && V > 0 && ld >= V, "argmax_static: bad sizes rows=%d V=%d", rows, V);
+  HFEE_REQUIRE(rows <= HFEE_ARGMAX_STATIC_MAX_ROWS, "argmax_static: %d rows in one call, the library's buffer holds %d",
+               rows, HFEE_ARGMAX_STATIC_MAX_ROWS);
+  HFEE_REQUIRE(out != nullptr && logits != nullptr, "argmax_static: null pointer");
+  if (rows == 0) return 0;
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  HFEE_REQUIRE(e == hipSuccess && device >= 0 && device < MAX_DEVICES, "argmax_static: no current device (%s)",
+               hipGetErrorString(e));
+  void* base = argmax_static_address[device].load(std::memory_order_acquire);
+  if (base == nullptr) {        // first call on this device (two threads at once find the same address)
+    e = hipGetSymbolAddress(&base, HIP_SYMBOL(argmax_static_scratch));
+    HFEE_REQUIRE(e == hipSuccess && base != nullptr, "argmax_static: cannot find the library's buffer on device %d: %s",
+                 device, hipGetErrorString(e));
+    argmax_static_address[device].store(base, std::memory_order_release);
+  }
+  MaxIdx* partial = (MaxIdx*)base;
+  int* counters = (int*)((unsigned char*)base + (size_t)HFEE_ARGMAX_STATIC_MAX_ROWS * HFEE_ARGMAX_STATIC_PARTS * sizeof(MaxIdx));
+  int parts = 256 / rows;                                   // as hfee_argmax chooses
+  if (parts > V / 2048) parts = V / 2048;
+  if (parts > HFEE_ARGMAX_STATIC_PARTS) parts = HFEE_ARGMAX_STATIC_PARTS;
+  if (parts > 1) {
+    // the counters must be zero; a call that was cut short may have left them otherwise
+    clear_counters_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(counters, rows);
+    argmax_parts_kernel<<<rows * parts, ARGMAX_THREADS, 0, stream>>>(out, logits, ld, V, parts, partial, counters);
+  } else {
+    argmax_kernel<<<rows, THREADS, 0, stream>>>(out, logits, ld, V);
+  }
+  HFEE_CHECK_LAUNCH("argmax_static");
   return 0;
 }
 

@@ -37,6 +37,7 @@ _CORE_SIGNATURES = {
                          P, I, P, L, P, P, I, F, P, L, I, P],
     "hfee_argmax": [P, P, L, I, I, P, L, P, I, P],
     "hfee_sample": [P, P, L, I, I, P, P, P, P, L, P],
+    "hfee_argmax_static": [P, P, L, I, I, P],
 }
 
 _ATTENTION_SIGNATURES = {
