@@ -41,8 +41,8 @@ PROMPT = 1024
 PREFILL = 2048
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="bench.py")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
@@ -63,7 +63,7 @@ def main() -> int:
                     help="run only the 2,048-token prefill (for profiling); prints its own short line")
     ap.add_argument("--prefill-tokens", type=int, default=0, metavar="T",
                     help="with --prefill-only: a prompt of T tokens (65 to 2,048) in place of 2,048")
-    args = ap.parse_args()
+    args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2

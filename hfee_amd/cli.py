@@ -23,6 +23,7 @@ Usage:
 Commands:
   run <model> [prompt]   Generate from a model folder (config.json + model.safetensors)
   replay ...             Feed token ids step by step and write logits (see bin/trace_run)
+  bench ...              Decode and prefill throughput (the options of bench.py)
   version                Print the version
 
 Environment:
@@ -181,6 +182,19 @@ def interactive(llm, params, verbose: bool, load: float) -> int:
             print()
 
 
+def bench(argv) -> int:
+    """`hfee bench ...`: the measurement program that lies beside the package, with its own options."""
+    import importlib.util
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")
+    if not os.path.isfile(path):
+        print(f"hfee bench: {path} is not there (the measurement program ships with the source tree)", file=sys.stderr)
+        return 1
+    spec = importlib.util.spec_from_file_location("hfee_bench", path)
+    module = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(module)
+    return module.main(argv)
+
+
 def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
     if not argv:
@@ -192,6 +206,8 @@ def main(argv=None) -> int:
     if cmd == "replay":
         from .replay import main as replay_main
         return replay_main(rest)
+    if cmd == "bench":
+        return bench(rest)
     if cmd in ("version", "--version", "-v"):
         print(f"hfee version {VERSION}")
         return 0

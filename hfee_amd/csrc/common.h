@@ -58,6 +58,30 @@ __device__ __forceinline__ bf16_t float_to_bf16(float f) {
   return __builtin_bit_cast(bf16_t, (__bf16)f);
 }
 
+// ---- what goes into the cache is finite ------------------------------------------
+// The matrix-core attention multiplies keys and values that a query must not see by a
+// weight of zero instead of skipping them, and such keys may lie in a page that belonged
+// to another request before.  Zero times infinity is NaN, so an infinity or NaN that one
+// request's numbers overflowed to must never reach the cache, or it would turn up in the
+// output of whoever gets the page next: every write to the cache goes through these (an
+// infinity becomes the largest finite number of its sign, a NaN a finite number).
+constexpr float kBf16Max = 3.3895313892515355e38f;      // 0x7F7F: the largest finite bfloat16
+constexpr float kF32Max = 3.4028234663852886e38f;
+
+__device__ __forceinline__ float finite_for_bf16(float v) { return fminf(fmaxf(v, -kBf16Max), kBf16Max); }
+
+__device__ __forceinline__ bf16_t finite_bf16(bf16_t b) {
+  return (b & 0x7F80) == 0x7F80 ? (bf16_t)((b & 0x8000) | 0x7F7F) : b;
+}
+
+__device__ __forceinline__ uint32_t finite_bf16x2(uint32_t w) {
+  return (uint32_t)finite_bf16((bf16_t)(w & 0xffff)) | ((uint32_t)finite_bf16((bf16_t)(w >> 16)) << 16);
+}
+
+template <typename T> __device__ __forceinline__ T finite_for_cache(T v);
+template <> __device__ __forceinline__ float finite_for_cache<float>(float v) { return fminf(fmaxf(v, -kF32Max), kF32Max); }
+template <> __device__ __forceinline__ bf16_t finite_for_cache<bf16_t>(bf16_t v) { return finite_bf16(v); }
+
 template <typename T> __device__ __forceinline__ float to_float(T v);
 template <> __device__ __forceinline__ float to_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ float to_float<bf16_t>(bf16_t v) { return bf16_to_float(v); }

@@ -262,8 +262,8 @@ __global__ void rope_cache_kernel(T* __restrict__ q, int64_t ldq, const T* __res
     } else {
       val = to_float<T>(kt[h * hd + dd]);
     }
-    cache[lay.key_offset(page, h, slot, dd)] = from_float<T>(val);
-    cache[lay.value_offset(page, h, slot, dd)] = vt[h * hd + dd];
+    cache[lay.key_offset(page, h, slot, dd)] = finite_for_cache<T>(from_float<T>(val));
+    cache[lay.value_offset(page, h, slot, dd)] = finite_for_cache<T>(vt[h * hd + dd]);
   }
 }
 
@@ -320,13 +320,13 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
       if (in_a_row) {
         union { u32x4 u[2]; bf16_t e[16]; } row;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) row.e[CacheLayout::value_slot(j)] = group_values[j * width + col];
+        for (int j = 0; j < 16; ++j) row.e[CacheLayout::value_slot(j)] = finite_bf16(group_values[j * width + col]);
         u32x4* dst = reinterpret_cast<u32x4*>(cache + lay.value_column(g_page[0], h, d) + (g_pos[0] & (lay.page_size - 1)));
         dst[0] = row.u[0];
         dst[1] = row.u[1];
       } else {
         for (int j = 0; j < count; ++j)
-          cache[lay.value_offset(g_page[j], h, g_pos[j] & (lay.page_size - 1), d)] = group_values[j * width + col];
+          cache[lay.value_offset(g_page[j], h, g_pos[j] & (lay.page_size - 1), d)] = finite_bf16(group_values[j * width + col]);
       }
     }
     return;
@@ -369,11 +369,13 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
     x.u = *reinterpret_cast<const u32x4*>(kt + w * 8);
     if (!values_by_groups) y.u = *reinterpret_cast<const u32x4*>(vt + w * 8);
     rotate(x, d);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) x.u[c] = finite_bf16x2(x.u[c]);       // only finite values go into the cache
     *reinterpret_cast<u32x4*>(cache + lay.key_offset(page, h, slot, d)) = x.u;
     if (values_by_groups) continue;                                    // (other workgroups write the values)
     bf16_t* vc = cache + lay.value_offset(page, h, slot, d);          // column d of the head; the next is page_size on
 #pragma unroll
-    for (int c = 0; c < 8; ++c) vc[(int64_t)c * lay.page_size] = y.e[c];
+    for (int c = 0; c < 8; ++c) vc[(int64_t)c * lay.page_size] = finite_bf16(y.e[c]);
   }
 }
 

@@ -328,6 +328,10 @@ __device__ __forceinline__ void store_wave_qkv(void* C, int64_t ldc, int M, int 
             v[3] = x2 * s1 + x3 * c1;
           }
         }
+        if (!is_q) {                                           // only finite values go into the cache
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = finite_for_bf16(v[e]);
+        }
         u32x2 o;
         o[0] = (uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16);
         o[1] = (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16);

@@ -32,6 +32,7 @@ struct QkvPlace {
   bool rotate[2];
   bf16_t* dst;           // null: nothing to store
   int step;              // elements between the four values at dst (1: one 8-byte store)
+  bool cached;           // dst lies in the cache: only finite values go there
 };
 
 __device__ __forceinline__ QkvPlace qkv_place(const QkvArgs& q, void* C, int64_t ldc, int m, int n) {
@@ -49,6 +50,7 @@ __device__ __forceinline__ QkvPlace qkv_place(const QkvArgs& q, void* C, int64_t
   }
   w.dst = nullptr;
   w.step = 1;
+  w.cached = head >= q.num_heads;
   if (head < q.num_heads) {
     w.dst = (bf16_t*)C + (int64_t)m * ldc + n;
   } else if (q.cache != nullptr) {
@@ -76,7 +78,7 @@ __device__ __forceinline__ void qkv_put(const QkvPlace& w, float* v) {
   }
   bf16_t o[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) o[i] = float_to_bf16(v[i]);
+  for (int i = 0; i < 4; ++i) o[i] = float_to_bf16(w.cached ? finite_for_bf16(v[i]) : v[i]);
   if (w.dst == nullptr) return;
   if (w.step == 1) {
     *reinterpret_cast<qkv_u32x2*>(w.dst) = *reinterpret_cast<const qkv_u32x2*>(o);

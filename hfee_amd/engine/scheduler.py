@@ -18,13 +18,18 @@ decides the same way here:
 The reference reserves a whole context per slot up front, so pages never run out
 there.  Here they can, and this is what happens:
 
-  1. a waiting request is admitted only if a state slot is free and the free pages
-     cover its first portion on top of what the running requests need this step;
+  1. requests that run come before requests that wait: decoding requests first, then the
+     prompts that are still being read, oldest first, and only then is a waiting request
+     admitted, if a state slot is free and the free pages cover its first portion (so the
+     pages that a preemption frees go to those who needed them, not back to the request
+     that gave them up);
   2. a prompt portion is shortened to what the free pages hold (or waits a step);
-  3. if a decoding request cannot get the page its next token needs, the request
-     admitted last is preempted: its pages go back, and it returns to the front of
-     the waiting line with prompt + generated tokens as its new prompt (its sampler
-     stream goes on where it was, so the tokens it produces are the same);
+  3. if a decoding request cannot get the page its next token needs, requests younger than
+     it are preempted, youngest first: their pages go back, and they return to the front
+     of the waiting line with prompt + generated tokens as their new prompt (the sampler
+     stream goes on where it was, so the tokens they produce are the same); if it is the
+     youngest itself, it is the one that is preempted.  Nobody is ever preempted for the
+     sake of a younger request;
   4. a request that is alone and still cannot get a page finishes with "length".
 The request admitted first is never preempted, so every step makes progress.
 

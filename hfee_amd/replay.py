@@ -7,6 +7,7 @@ returns the last logits (/root/reference/internal/llm/forward.go:36-39).
 
 Input: one JSON object per line,
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+`want` may also be "all" (every token of the entry) or "last".
 Output: for a step in which something is wanted, <out>/<step>.f32 holds the logits
 at the wanted places as little-endian float32 [wanted, vocab], in the order of the
 entries and of `want`.  After every step a line `done <step>` is printed.
@@ -40,15 +41,41 @@ def _split(entries, limit):
     return steps
 
 
+def wanted_places(want, count: int) -> list:
+    """`want` of a trace entry as a list of places among the entry's tokens: a list is
+    taken as it is, "all" is every token, "last" the last one."""
+    if want is None:
+        return []
+    if isinstance(want, str):
+        if want == "all":
+            return list(range(count))
+        if want == "last":
+            return [count - 1]
+        raise ValueError(f'want must be a list of places, "all" or "last", not {want!r}')
+    return [int(w) for w in want]
+
+
 class Replayer:
+    """max_tokens: the most tokens that live requests hold at any time, each request's count
+    rounded up to a multiple of 64 (to a whole page where pages are larger: then every live
+    request may leave one more page partly empty, and the pool has one for each).  The page
+    pool is made for exactly that, so that pages are given back and used again.
+    batch_limit: the most tokens one engine step takes (larger steps of a trace are cut)."""
+
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16,
-                 max_requests: int = 8, device: str = "cuda:0"):
-        from .engine import Engine, load_model
-        model, _ = load_model(model_dir, dtype, device)
+                 max_requests: int = 64, device: str = "cuda:0", batch_limit: int | None = None,
+                 random_weights: bool = False, seed: int = 0):
+        from .engine import Engine, load_model, random_model
+        from .config.registry import config_from_folder
+        if random_weights:
+            model = random_model(config_from_folder(model_dir), seed, dtype, device)
+        else:
+            model, _ = load_model(model_dir, dtype, device)
         page = page_size
         tokens = max(max_tokens, 64)
-        self.batch_limit = min(tokens, 8192)
-        self.engine = Engine(model, num_pages=(tokens + page - 1) // page, page_size=page,
+        pages = (tokens + page - 1) // page + (max_requests if page > 64 else 0)
+        self.batch_limit = max(1, min(tokens, 8192) if batch_limit is None else batch_limit)
+        self.engine = Engine(model, num_pages=pages, page_size=page,
                              max_requests=max_requests, max_batch_tokens=self.batch_limit,
                              num_positions=min(tokens, model.spec.max_positions), device=device)
 
@@ -60,7 +87,7 @@ class Replayer:
         for rid, tokens, want in entries:
             if not self.engine.is_live(rid):
                 self.engine.admit(rid)
-            ents.append(StepEntry(rid, list(tokens), list(want)))
+            ents.append(StepEntry(rid, list(tokens), wanted_places(want, len(tokens))))
         total = sum(len(e.tokens) for e in ents)
         if total <= self.batch_limit:
             logits = self.engine.step(ents)
@@ -99,9 +126,14 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens that live requests hold at any time (the cache pool is made for it)")
     ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--max-requests", type=int, default=64, help="most requests that are live at a time")
+    ap.add_argument("--random-weights", action="store_true",
+                    help="read config.json only; the weights are seeded random ones")
+    ap.add_argument("--seed", type=int, default=0, help="seed of the random weights")
     args = ap.parse_args(argv)
     os.makedirs(args.out, exist_ok=True)
-    rep = Replayer(args.model, args.dtype, args.max_tokens, page_size=args.page_size)
+    rep = Replayer(args.model, args.dtype, args.max_tokens, page_size=args.page_size,
+                   max_requests=args.max_requests, random_weights=args.random_weights, seed=args.seed)
     for line in sys.stdin:
         line = line.strip()
         if not line:

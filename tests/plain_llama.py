@@ -151,9 +151,10 @@ class PlainLlama:
             for name in f.keys():
                 self.w[name] = f.get_tensor(name).to(F64)
 
-    def forward(self, tokens, schedule=None, windows=None) -> torch.Tensor:
+    def forward(self, tokens, schedule=None, windows=None, rows=None) -> torch.Tensor:
         """/root/reference/internal/llm/forward.go:51-142 for one sequence from
-        position 0, logits at every position.  schedule: [(layer, cache, writes)] in
+        position 0, logits at every position (or at the positions `rows` only: the
+        reference runs its final norm and head for the wanted rows, forward.go:117-130).  schedule: [(layer, cache, writes)] in
         running order (default: every layer once, its own cache); an entry that does
         not write reads the keys and values that the entry which wrote `cache` made.
         windows: {layer: keys kept} for layers with a window."""
@@ -181,6 +182,8 @@ class PlainLlama:
             h = plain_swiglu(plain_matmul(xb, w[p + "mlp.gate_proj.weight"]),
                              plain_matmul(xb, w[p + "mlp.up_proj.weight"]))            # forward.go:110-112
             x = x + plain_matmul(h, w[p + "mlp.down_proj.weight"])                     # forward.go:113-114
+        if rows is not None:
+            x = x[torch.as_tensor(list(rows), dtype=torch.long)]
         x = plain_rmsnorm(x, w["model.norm.weight"], self.eps)                         # forward.go:124-128
         head = w["model.embed_tokens.weight"] if self.tied else w["lm_head.weight"]    # model.go:118-121
         return plain_matmul(x, head)                                                   # forward.go:132-141

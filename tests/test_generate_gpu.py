@@ -23,21 +23,54 @@ def test_greedy_generation_matches_the_plain_implementation(model_folders):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_seeded_sampling_does_not_depend_on_the_batch(model_folders, dtype):
     """Tiny B's workload: prompts of 40, 3 and 100 tokens, portions of 16, 24 tokens at
-    temperature 0.8 with a fixed seed: together and alone give the same tokens."""
+    temperature 0.8 with a fixed seed.  In 32-bit, together, alone and in another order give
+    the same tokens (the bits of a row do not depend on the batch).  In bfloat16 the kernels
+    differ with the number of rows, and a draw from a flat distribution turns on the last
+    bits: there the requests run together in the opposite order with a budget that takes all
+    prompts in one step, which changes which row of the batch and of the sampler each one is
+    and nothing else, and the tokens must be the same."""
     from hfee_amd import LLM, SamplingParams
     folder = model_folders[("B", dtype)]
     prompts = list(tu.make_requests(320, [40, 3, 100], seed=2).values())
     params = [SamplingParams(temperature=0.8, seed=100 + i, num_predict=24) for i in range(3)]
-    llm = LLM(folder, dtype=dtype, num_ctx=256, num_parallel=3, max_batch_tokens=16)
-    together = llm.generate(prompts, params)
-    for p, sp, o in zip(prompts, params, together):
-        alone = llm.generate([p], sp)[0]
-        assert len(o.token_ids) == 24
-        if dtype == "float32":
-            assert alone.token_ids == o.token_ids
-        else:       # rounding differs between batch shapes in bfloat16: most tokens still agree
-            same = sum(a == b for a, b in zip(alone.token_ids, o.token_ids))
-            assert alone.token_ids[0] == o.token_ids[0] and same >= 1
+    if dtype == "float32":
+        llm = LLM(folder, dtype=dtype, num_ctx=256, num_parallel=3, max_batch_tokens=16)
+        together = llm.generate(prompts, params)
+        assert len({tuple(o.token_ids) for o in together}) == 3, "three requests, three streams"
+        for p, sp, o in zip(prompts, params, together):
+            assert len(o.token_ids) == 24 and llm.generate([p], sp)[0].token_ids == o.token_ids
+        order = [2, 0, 1]
+        again = llm.generate([prompts[i] for i in order], [params[i] for i in order])
+        assert [o.token_ids for o in again] == [together[i].token_ids for i in order]
+    wide = LLM(folder, dtype=dtype, num_ctx=256, num_parallel=3, max_batch_tokens=256)
+    a = wide.generate(prompts, params)
+    b = wide.generate(list(reversed(prompts)), list(reversed(params)))
+    assert all(len(o.token_ids) == 24 for o in a) and len({tuple(o.token_ids) for o in a}) == 3
+    assert [o.token_ids for o in a] == [o.token_ids for o in reversed(b)]
+
+
+def test_greedy_bfloat16_does_not_depend_on_the_batch(model_folders):
+    """bfloat16, greedy: each request alone, all together, and the plain implementation
+    agree on every token up to the first choice that is a near tie in the plain
+    implementation's logits (there a last bit may decide, and what follows is another
+    sequence)."""
+    from plain_llama import PlainLlama
+    from hfee_amd import LLM, SamplingParams
+    checked = 0
+    for name, vocab, lengths in (("A", 256, [5, 17, 32, 1]), ("B", 320, [40, 3, 100])):
+        folder = model_folders[(name, "bfloat16")]
+        plain = PlainLlama(folder)
+        prompts = list(tu.make_requests(vocab, lengths, seed=12).values())
+        sp = SamplingParams.greedy(num_predict=20)
+        llm = LLM(folder, dtype="bfloat16", num_ctx=128, num_parallel=4, max_batch_tokens=24)
+        together = llm.generate(prompts, sp)
+        for p, o in zip(prompts, together):
+            want = plain.greedy(p, 20)
+            margins = tu.greedy_margins(plain, p, want)
+            alone = llm.generate([p], sp)[0]
+            checked += tu.agree_until_a_near_tie(o.token_ids, want, margins, f"{name} together")
+            tu.agree_until_a_near_tie(alone.token_ids, want, margins, f"{name} alone")
+    assert checked >= 40, f"only {checked} tokens could be compared: the test has lost its teeth"
 
 
 def test_scarce_pages_preempt_and_still_give_the_same_tokens(model_folders):
@@ -51,6 +84,30 @@ def test_scarce_pages_preempt_and_still_give_the_same_tokens(model_folders):
     outs = tight.generate(prompts, sp)
     assert [o.token_ids for o in outs] == want
     assert sum(o.stats.preemptions for o in outs) > 0
+    assert outs[0].stats.preemptions == 0, "the request admitted first is never preempted"
+    tight.engine.cache.check()
+    assert not tight.engine.cache.requests
+
+
+def test_scarce_pages_preempt_in_bfloat16(model_folders):
+    """The same on the bfloat16 kernels: a preempted request reads its own tokens again as a
+    prompt (other kernels than the single steps that made them), so its tokens are compared
+    with the plain implementation's up to the first near tie."""
+    from plain_llama import PlainLlama
+    from hfee_amd import LLM, SamplingParams
+    folder = model_folders[("A", "bfloat16")]
+    plain = PlainLlama(folder)
+    prompts = list(tu.make_requests(256, [30, 28, 26, 31], seed=4).values())
+    sp = SamplingParams.greedy(num_predict=40)
+    tight = LLM(folder, dtype="bfloat16", num_ctx=128, num_parallel=4, num_pages=10)
+    outs = tight.generate(prompts, sp)
+    assert sum(o.stats.preemptions for o in outs) > 0 and outs[0].stats.preemptions == 0
+    assert all(len(o.token_ids) == 40 and o.done_reason == "length" for o in outs)
+    checked = 0
+    for p, o in zip(prompts, outs):
+        want = plain.greedy(p, 40)
+        checked += tu.agree_until_a_near_tie(o.token_ids, want, tu.greedy_margins(plain, p, want), "preempted")
+    assert checked >= 30, f"only {checked} tokens could be compared"
     tight.engine.cache.check()
     assert not tight.engine.cache.requests
 

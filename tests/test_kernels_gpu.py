@@ -130,7 +130,11 @@ def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
             want, tol = ref, 1e-2 if mode == "bf16" else 1e-5
         err = (out.double().cpu() - want).abs()
         assert (err <= tol * (1 + mag + want.abs())).all(), float((err / (1 + mag)).max())
-        outs.append(out)
+        outs.append(out.double().cpu())
+    # with and without the cut: the same sums in another order
+    cut_err = (outs[0] - outs[1]).abs()
+    order_tol = 1e-2 if mode == "bf16" else 2e-6
+    assert (cut_err <= order_tol * (1 + mag + outs[1].abs())).all(), float((cut_err / (1 + mag)).max())
     assert ops.linear_scratch(64, N, K) == 0 and ops.linear_scratch(2048, 4096, K) == 0
 
 
@@ -728,3 +732,111 @@ def test_attention_over_long_contexts(H, K, hd, ps, ctx):
         assert int(counters.abs().sum()) == 0
     # the far key carries weight: without it the result would be another
     assert ref.float().abs().max() > 0.2
+
+
+@pytest.mark.parametrize("H,K,hd", [(32, 8, 128), (32, 8, 64), (6, 1, 48)])
+def test_split_key_join_on_buffers_that_are_used_again(H, K, hd):
+    """The engine hands every layer and every step the same buffer for the splits' partial
+    results and the same counters.  Three hundred calls in a row on one such pair, each with
+    new queries, positions, page tables, batch sizes and split counts (both forms of the
+    kernel: a tile ahead with up to one workgroup a CU, tile by tile beyond; splits that find
+    no key at all), none waited for before the next is queued: every call's output is bit for
+    bit the output of the same call with the splits joined by a second launch on buffers of
+    its own, and the counters are zero after every batch of calls."""
+    import random
+    from hfee_amd.kernels import ops
+    ps, blocks, b_max, s_max = 16, 80, 40, 8
+    rng = random.Random(hd + K)
+    g = torch.Generator(device=DEV).manual_seed(hd)
+    cache = (torch.randn(b_max * blocks, 2, K, ps * hd, generator=g, device=DEV) * 0.5).to(torch.bfloat16)
+    shared_partial = torch.full((b_max * H * s_max * (hd + 2),), 3.0e30, dtype=torch.float32, device=DEV)
+    shared_counters = torch.zeros(b_max * K, dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(hd)
+    done = 0
+    while done < 300:
+        group = []
+        for _ in range(10):
+            B = rng.choice([1, 1, 2, 3, 8, 8, 20, 40])
+            splits = rng.randint(2, s_max)
+            tables = torch.randperm(b_max * blocks, generator=g, device=DEV)[:B * blocks].to(torch.int32).reshape(B, blocks)
+            q = torch.randn(B, H * hd, generator=g, device=DEV).to(torch.bfloat16)
+            pos = torch.tensor([rng.choice([0, 5, 31, 32, 100, rng.randrange(blocks * ps), blocks * ps - 1])
+                                for _ in range(B)], dtype=torch.int32, device=DEV)
+            out = torch.zeros(B, H * hd, dtype=torch.bfloat16, device=DEV)
+            ops.attention_bf16_decode(out, q, cache, None, pos, None, tables, H, K, hd, ps, scale, 0,
+                                      shared_partial[:B * H * splits * (hd + 2)], splits,
+                                      counters=shared_counters[:B * K])
+            group.append((B, splits, tables, q, pos, out))
+        assert int(shared_counters.abs().sum()) == 0, f"the counters are not back at zero after call {done + 10}"
+        for B, splits, tables, q, pos, out in group:
+            want = torch.zeros(B, H * hd, dtype=torch.bfloat16, device=DEV)
+            partial = torch.zeros(B * H * splits * (hd + 2), dtype=torch.float32, device=DEV)
+            ops.attention_bf16_decode(want, q, cache, None, pos, None, tables, H, K, hd, ps, scale, 0, partial, splits,
+                                      counters=None)
+            assert torch.equal(out, want), f"call {done}: batch {B}, {splits} splits, positions {pos.tolist()}"
+            done += 1
+    # and the join is the right one: against the plain kernel
+    B, splits, tables, q, pos, out = group[-1]
+    ref = torch.zeros_like(out)
+    ops.attention_plain(ref, q, cache, pos, torch.arange(B, dtype=torch.int32, device=DEV), tables, H, K, hd, ps, scale, 0)
+    close(out, ref, 2e-2)
+
+
+def _poison():
+    """Numbers that overflow: rows of 1e38 against weights of +-10."""
+    return 1.0e38
+
+
+@pytest.mark.parametrize("M", [1, 9, 40, 100, 300])
+def test_only_finite_numbers_reach_the_cache(M):
+    """Keys and values that overflow to infinity or NaN (here: projections of rows of 1e38) are
+    written to the cache as finite numbers, by every kernel that writes there: the products
+    with the q/k/v epilogue (streaming, batch in LDS, tiled) and the rotation kernels (a token
+    a workgroup; values of 16 tokens together).  The attention kernels multiply keys that a
+    query must not see by zero, and zero times infinity would be NaN for the page's next owner."""
+    from hfee_amd.kernels import ops
+    H, K, hd, half, d, ps = 4, 2, 32, 16, 1024, 16
+    g = torch.Generator().manual_seed(M)
+    N = (H + 2 * K) * hd
+    w = (torch.randn(N, d, generator=g) * 10).to(torch.bfloat16).to(DEV)
+    x = torch.randn(M, d, generator=g)
+    x[::2] = _poison()
+    x = x.to(torch.bfloat16).to(DEV)
+    pos = torch.arange(M, dtype=torch.int32, device=DEV)
+    seg = torch.zeros(M, dtype=torch.int32, device=DEV)
+    nblocks = (M + ps - 1) // ps
+    tables = torch.arange(nblocks, dtype=torch.int32, device=DEV).reshape(1, nblocks)
+    ang = torch.arange(M + 1, dtype=torch.float64)[:, None] * (1.0 / 10000.0 ** (torch.arange(half) / half))[None, :]
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    plain_y = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(plain_y, x, w)
+    assert not torch.isfinite(plain_y.float()).all(), "the test's inputs must overflow"
+
+    def fresh():
+        return torch.zeros(nblocks, 2, K, ps * hd, dtype=torch.bfloat16, device=DEV)
+
+    def check(layer, what):
+        assert torch.isfinite(layer.float()).all(), f"{what}: a number that is not finite reached the cache"
+        assert float(layer.float().abs().max()) > 1e37, f"{what}: the overflowing rows were not written at all"
+    qkv = dict(positions=pos, token_segment=seg, block_tables=tables, cos=cos, sin=sin, num_heads=H, kv_heads=K,
+               head_dim=hd, page_size=ps)
+    q_out = torch.zeros(M, H * hd, dtype=torch.bfloat16, device=DEV)
+    layer = fresh()
+    ops.linear_fused(q_out, x, w, "qkv", qkv=dict(qkv, cache_layer=layer))      # streaming up to 64 rows, tiled beyond
+    check(layer, "q/k/v epilogue")
+    if 16 < M <= 64:
+        layer = fresh()
+        scratch = torch.zeros(ops.mid_rows_scratch(M, N, d), dtype=torch.float32, device=DEV)
+        ops.linear_fused(q_out, x, w, "qkv", qkv=dict(qkv, cache_layer=layer), scratch=scratch, force_mid_rows=True)
+        check(layer, "q/k/v epilogue with the batch in LDS")
+    y = plain_y.clone()
+    for pairing in (1, 0):          # the kernel for adjacent pairs (values of 16 tokens together from 32 rows on); the general one
+        layer = fresh()
+        ops.rope_cache_write(y[:, :H * hd], y[:, H * hd:(H + K) * hd], y[:, (H + K) * hd:], pos, seg, tables, cos, sin,
+                             pairing, layer, H, K, hd, ps, M - 1)
+        check(layer, f"rotation kernel, pairing {pairing}")
+    y32 = plain_y.float()
+    layer = torch.zeros(nblocks, 2, K, ps * hd, dtype=torch.float32, device=DEV)
+    ops.rope_cache_write(y32[:, :H * hd], y32[:, H * hd:(H + K) * hd], y32[:, (H + K) * hd:], pos, seg, tables, cos, sin,
+                         0, layer, H, K, hd, ps, M - 1)
+    check(layer, "rotation kernel, 32-bit")

@@ -508,6 +508,40 @@ def test_sampler_with_a_top_k_too_large_to_gather():
     assert all(dist[i] > 0 for i in ids) and exact >= 62, exact
 
 
+@pytest.mark.parametrize("top_k", [40, 0, 1024, 1025, 5000])
+def test_sampler_at_the_vocabulary_of_the_real_models(top_k):
+    """128,256 logits a row (32 sets of radix counters, the gather of up to 1,024 ids and the
+    path beyond it, a penalty bit set of 16 KB), with the reference's default options
+    (/root/reference/internal/llm/sampler.go:23-34: temperature 0.8, top_p 0.9, a penalty of 1.1
+    on the last 64 ids) and top_k as given: at least 99 in 100 draws are exactly the inverse
+    CDF of the plain distribution at the request's own random number, none is outside the kept set."""
+    from plain_llama import plain_repeat_penalty, plain_sampling_distribution
+    from hfee_amd.sampling import SampleRow, Sampler, SamplingParams, uniform
+    V = 128256
+    g = torch.Generator().manual_seed(top_k + 1)
+    base = torch.randn(V, generator=g) * 2.5
+    base[100000] = base[77] = base.max() + 0.25                  # tied maxima far apart
+    p = SamplingParams(top_k=top_k)
+    assert (p.temperature, p.top_p, p.repeat_penalty, p.repeat_last_n, p.min_p) == (0.8, 0.9, 1.1, 64, 0.0)
+    history = torch.randint(0, V, (90,), generator=g).tolist() + [77]
+    pen = plain_repeat_penalty(base, history, p.repeat_penalty, p.repeat_last_n)
+    dist = plain_sampling_distribution(pen, p.temperature, p.top_k, p.top_p, p.min_p)
+    cum = torch.cumsum(dist, 0)
+    kept = int((dist > 0).sum())
+    assert kept >= 2 and (top_k == 0 or kept <= top_k)
+    sampler = Sampler(V, DEV, max_rows=64)
+    exact = draws = 0
+    for c in range(3):
+        logits = base.repeat(64, 1).to(DEV)
+        rows = [SampleRow(p, seed=1234, draw=c * 64 + r, history=history, logits_row=r) for r in range(64)]
+        for r, i in enumerate(sampler.sample(logits, rows)):
+            assert dist[i] > 0, f"id {i} is outside the kept set of {kept}"
+            want = int(torch.searchsorted(cum, torch.tensor(uniform(1234, c * 64 + r), dtype=cum.dtype)))
+            exact += int(i == want)
+            draws += 1
+    assert exact >= 0.99 * draws, f"top_k {top_k}: only {exact} of {draws} draws match the inverse CDF ({kept} ids kept)"
+
+
 @pytest.mark.parametrize("V", [700, 1003, 4099])
 def test_sampler_takes_the_newest_id_of_a_history_from_the_device(V):
     """The newest id of each row's history may lie on the device only (`latest`: the ids of

@@ -115,26 +115,89 @@ def test_trace_run_program(model_folders, tmp_path, dtype):
         {"step": 0, "entries": [{"id": "a", "tokens": toks["r0"][:10], "want": [0, 9]}], "end": []},
         {"step": 1, "entries": [{"id": "a", "tokens": toks["r0"][10:12], "want": []},
                                 {"id": "b", "tokens": toks["r1"], "want": [8]}], "end": ["b"]},
-        {"step": 2, "entries": [{"id": "a", "tokens": toks["r0"][12:], "want": [8, 0]}], "end": ["a"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks["r0"][12:19], "want": []}], "end": []},
+        {"step": 3, "entries": [{"id": "a", "tokens": toks["r0"][19:], "want": [1, 0]}], "end": ["a"]},
+        {"step": 4, "entries": [{"id": "b", "tokens": toks["r1"][:4], "want": "last"}], "end": []},
+        {"step": 5, "entries": [{"id": "b", "tokens": toks["r1"][4:], "want": "all"}], "end": ["b"]},
     ]
     out = tmp_path / "out"
     p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
                         "--out", str(out), "--max-tokens", "128"],
                        input="\n".join(json.dumps(l) for l in lines) + "\n", capture_output=True, text=True, timeout=300)
     assert p.returncode == 0, p.stderr[-2000:]
-    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
-    assert not (out / "1.f32").exists() or True
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(6)]
+    assert not (out / "2.f32").exists(), "a step in which nothing is wanted writes no file"
+    assert sorted(f.name for f in out.iterdir()) == ["0.f32", "1.f32", "3.f32", "4.f32", "5.f32"]
     plain = PlainLlama(folder)
     la, lb = plain.forward(toks["r0"]), plain.forward(toks["r1"])
     V = 256
     s0 = np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V)
     s1 = np.fromfile(out / "1.f32", dtype="<f4").reshape(-1, V)
-    s2 = np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V)
-    assert s0.shape[0] == 2 and s1.shape[0] == 1 and s2.shape[0] == 2
+    s3 = np.fromfile(out / "3.f32", dtype="<f4").reshape(-1, V)
+    s4 = np.fromfile(out / "4.f32", dtype="<f4").reshape(-1, V)
+    s5 = np.fromfile(out / "5.f32", dtype="<f4").reshape(-1, V)
+    assert s0.shape[0] == 2 and s1.shape[0] == 1 and s3.shape[0] == 2 and s4.shape[0] == 1 and s5.shape[0] == 5
     tol = TOL[dtype]
     assert rel(s0[0], la[0]) < tol and rel(s0[1], la[9]) < tol
     assert rel(s1[0], lb[8]) < tol
-    assert rel(s2[0], la[20]) < tol and rel(s2[1], la[12]) < tol
+    assert rel(s3[0], la[20]) < tol and rel(s3[1], la[19]) < tol          # in the order of `want`
+    assert rel(s4[0], lb[3]) < tol and all(rel(s5[i], lb[4 + i]) < tol for i in range(5))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_short_requests_just_fit_the_pool(model_folders, dtype):
+    """Ten live requests of 3 to 64 tokens under max_tokens = 10 x 64: every page of the pool is
+    taken at the end (a request's count rounds up to 64), more requests are live than the
+    four of the other traces, and all of them decode in one step."""
+    from plain_llama import PlainLlama
+    from hfee_amd.replay import Replayer
+    folder = model_folders[("A", dtype)]
+    lengths = [64, 3, 17, 64, 33, 50, 64, 16, 48, 61]
+    reqs = tu.make_requests(256, lengths, seed=21)
+    rep = Replayer(folder, dtype, max_tokens=64 * len(lengths))
+    assert rep.engine.cache.pools[0].num_pages == 4 * len(lengths)
+    steps = [{"entries": [(r, t[:-2], [len(t) - 3]) for r, t in reqs.items()], "end": []},
+             {"entries": [(r, t[-2:-1], [0]) for r, t in reqs.items()], "end": []},
+             {"entries": [(r, t[-1:], [0]) for r, t in reversed(list(reqs.items()))], "end": list(reqs)}]
+    got = tu.run(rep, steps)
+    plain = PlainLlama(folder)
+    want = {}
+    for rid, t in reqs.items():
+        lg = plain.forward(t)
+        for (r, p) in got:
+            if r == rid:
+                want[(r, p)] = lg[p].numpy()
+    check(got, want, TOL[dtype], f"ten live requests, {dtype}")
+    rep.engine.cache.check()
+    assert not rep.engine.cache.requests
+    with pytest.raises(Exception, match="pages"):        # one token more than the pool holds is refused, loudly
+        rep.step([(f"x{i}", [1] * 64, []) for i in range(len(lengths))] + [("y", [1], [])])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_larger_than_the_engine_takes_is_cut(model_folders, plain_logits, dtype):
+    """A replayer whose engine takes 40 tokens a step runs steps of up to 300: they are cut into
+    consecutive engine steps (an entry may be cut in the middle), the wanted rows come back in
+    the order of the entries and of `want`.  Same numbers as the uncut steps (in 32-bit the same bits)."""
+    from hfee_amd.replay import Replayer
+    reqs, want = plain_logits("C", dtype)
+    folder = model_folders[("C", dtype)]
+    ids = list(reqs)
+    steps = [{"entries": [(ids[0], reqs[ids[0]][:100], [99, 0, 50]), (ids[1], reqs[ids[1]], [69, 3]),
+                          (ids[3], reqs[ids[3]], list(range(41)))], "end": [ids[1], ids[3]]},
+             {"entries": [(ids[0], reqs[ids[0]][100:], [49, 7]), (ids[2], reqs[ids[2]], [299, 39, 40, 0])],
+              "end": [ids[0], ids[2]]}]
+    results = {}
+    for limit in (40, None):
+        rep = Replayer(folder, dtype, max_tokens=1024, batch_limit=limit)
+        results[limit] = tu.run(rep, steps)
+        assert not rep.engine.cache.requests
+        assert set(results[limit]) == {(ids[0], p) for p in (99, 0, 50, 149, 107)} | {(ids[1], 69), (ids[1], 3)} | \
+            {(ids[3], p) for p in range(41)} | {(ids[2], p) for p in (299, 39, 40, 0)}
+        check(results[limit], {k: want[k] for k in results[limit]}, TOL[dtype], f"C {dtype} steps cut at {limit}")
+    if dtype == "float32":
+        for k, row in results[None].items():
+            assert np.array_equal(row, results[40][k]), f"bits differ at {k}"
 
 
 def random_configuration(rng):
@@ -233,6 +296,60 @@ def test_many_requests_decoding_together(tmp_path, dtype):
     check(got, want, TOL[dtype], f"many live requests, {dtype}")
     rep.engine.cache.check()
     assert not rep.engine.cache.requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_context_of_thousands_of_tokens_inside_the_whole_model(tmp_path, dtype):
+    """One request read in portions of 2,048 tokens up to position 4,600 and then decoded for
+    eight steps, beside a short request that decodes in the same steps, with the head shape of
+    the large models (heads of 128 in groups of four, scaled rotation): block tables of hundreds
+    of pages (the attention kernels hold 64 entries at a time), portions that start deep in the
+    context, decode steps that split thousands of keys.  The query and key projections are
+    scaled up so that attention is sharp (a few far keys carry most of the weight): a page that
+    is skipped, read twice or taken from the wrong request would show.  Logits at the edges of
+    every portion, at the places where the kernels' window of the block table moves, and at
+    every decoded token, against the plain implementation."""
+    import safetensors.torch
+    from conftest import make_model_folder
+    from plain_llama import PlainLlama
+    from hfee_amd.replay import Replayer
+    cj = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 2, "hidden_size": 1024,
+          "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 128, "intermediate_size": 2048,
+          "vocab_size": 3000, "max_position_embeddings": 8192, "rope_theta": 500000.0,
+          "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                           "original_max_position_embeddings": 2048},
+          "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "hidden_act": "silu"}
+    folder = make_model_folder(tmp_path / "m", cj, seed=3, dtype=dtype, std=0.03, norm_init="one_plus_normal")
+    path = os.path.join(folder, "model.safetensors")
+    tensors = safetensors.torch.load_file(path)
+    for name in tensors:
+        if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
+            tensors[name] = (tensors[name].float() * 1.6).to(tensors[name].dtype)
+    safetensors.torch.save_file(tensors, path)
+    long_len, tail = 4600, 8
+    reqs = tu.make_requests(cj["vocab_size"], [long_len + tail, 40 + 2 + tail], seed=17)
+    big, small = reqs["r0"], reqs["r1"]
+    rep = Replayer(folder, dtype, max_tokens=4672 + 64)
+    edges = [0, 1, 1023, 1024, 2046, 2047]
+    steps = [{"entries": [("big", big[:2048], edges), ("small", small[:40], [39])], "end": []},
+             {"entries": [("small", small[40:41], [0]), ("big", big[2048:4096], [0, 1, 1023, 1024, 2047])], "end": []},
+             {"entries": [("big", big[4096:long_len], [0, 1, 503]), ("small", small[41:42], [0])], "end": []}]
+    for i in range(tail):
+        steps.append({"entries": [("big", [big[long_len + i]], [0]), ("small", [small[42 + i]], [0])], "end": []})
+    steps[-1]["end"] = ["big", "small"]
+    got = tu.run(rep, steps)
+    rep.engine.cache.check()
+    assert not rep.engine.cache.requests
+    del rep
+    plain = PlainLlama(folder)
+    want = {}
+    for rid, toks in (("big", big), ("small", small)):
+        rows = sorted(p for (r, p) in got if r == rid)
+        lg = plain.forward(toks, rows=rows)
+        for i, p in enumerate(rows):
+            want[(rid, p)] = lg[i].numpy()
+    assert len(got) == 6 + 1 + 1 + 5 + 3 + 1 + 2 * tail
+    check(got, want, TOL[dtype], f"a context of {long_len + tail} tokens, {dtype}")
 
 
 def test_layers_of_a_production_size_match_the_plain_implementation(tmp_path):

@@ -93,3 +93,36 @@ def run(replayer, steps):
 def make_requests(vocab, lengths, seed):
     rng = np.random.default_rng(seed)
     return {f"r{i}": rng.integers(0, vocab, size=n).tolist() for i, n in enumerate(lengths)}
+
+
+# A greedy token can only be compared across precisions where the choice is clear.  The
+# margin of a choice is (largest logit - second largest) / max |logit| in the plain
+# implementation; bfloat16 logits are within a few thousandths of max |logit| of it, so a
+# choice with a margin above NEAR_TIE is the same in every precision and every batch.
+NEAR_TIE = 3e-2
+
+
+def greedy_margins(plain, prompt, tokens):
+    """The margin of every greedy choice along prompt + tokens (teacher-forced)."""
+    import torch
+    seq = list(prompt) + list(tokens)
+    logits = plain.forward(seq[:-1]) if len(seq) > 1 else None
+    out = []
+    for i in range(len(tokens)):
+        row = logits[len(prompt) - 1 + i]
+        top = torch.topk(row, 2).values
+        out.append(float((top[0] - top[1]) / row.abs().max()))
+    return out
+
+
+def agree_until_a_near_tie(got, want, margins, what=""):
+    """Asserts that `got` equals `want` token by token; they may part only at a choice whose
+    margin is below NEAR_TIE (after that the two are different sequences and nothing more
+    can be compared).  Returns how many tokens agreed."""
+    n = 0
+    for g, w, m in zip(got, want, margins):
+        if g != w:
+            assert m < NEAR_TIE, f"{what}: token {n} is {g}, expected {w} (margin {m:.3f}); got {got}, want {want}"
+            break
+        n += 1
+    return n
