@@ -81,6 +81,13 @@ def test_llama3_frequency_scaling():
     # Tiny B: frequencies 0 and 1 are kept, 2 is blended, 3..15 are divided by exactly 8
     assert ratio[0] == 1.0 and ratio[1] == 1.0 and 1.0 < ratio[2] < 8.0
     assert all(abs(r - 8.0) < 1e-12 for r in ratio[3:])
+    # The blended one, worked by hand: inv_freq[2] = 500000^(-4/32) = 0.193923, wavelength
+    # 2 pi / 0.193923 = 32.4005; s = (64 / 32.4005 - 1) / (4 - 1) = 0.325094; the frequency becomes
+    # (1 - s) f / 8 + s f = 0.409457 f, so base / scaled = 2.44226.  A blend that is linear in the
+    # wavelength instead of in N0 / wavelength ((32.40 - 16) / (64 - 16) of the way to f / 8) would
+    # give 1.4265, and s put on the divided frequency instead of the kept one 1.3975.
+    assert abs(float(base[2]) - 0.193923) < 1e-6
+    assert abs(ratio[2] - 2.44226) < 1e-4
     assert all(a >= b for a, b in zip(sc.tolist(), sc.tolist()[1:])), "monotone"
     # continuous at both edges of the band: a wavelength just inside matches just outside
     n0, lo, hi, f = 64.0, 1.0, 4.0, 8.0
