@@ -31,17 +31,29 @@ class CacheError(RuntimeError):
 
 @dataclass(frozen=True)
 class CacheGroupSpec:
+    """Cache layers with the same needs.  token_shape: the elements one token adds to one
+    layer (attention: (2, kv_heads, head_dim)); the manager needs only its size, the
+    arrangement inside a page (`layout`) is the business of the parts that use the layers."""
     kind: str                 # "full" or "window"
-    kv_heads: int
-    head_dim: int
+    token_shape: tuple
     cache_layers: tuple       # ids of the cache layers in this group
     window: int = 0           # keys kept per token for kind == "window"
+    layout: str = ""
 
     def __post_init__(self):
         if self.kind not in ("full", "window"):
             raise CacheError(f"unknown cache group kind {self.kind!r}")
         if self.kind == "window" and self.window <= 0:
             raise CacheError("a window group needs a positive window")
+        if not self.token_shape or any(int(n) < 1 for n in self.token_shape):
+            raise CacheError(f"a token must add at least one element to a cache layer, got {self.token_shape!r}")
+
+    @property
+    def token_elements(self) -> int:
+        n = 1
+        for k in self.token_shape:
+            n *= int(k)
+        return n
 
 
 class PagePool:

@@ -49,6 +49,37 @@ class FeedForwardSpec:
 
 
 @dataclass(frozen=True)
+class EmbeddingSpec:
+    kind: str = "lookup"      # key in the embedding registry
+    params: tuple = ()
+
+    def get(self, name: str, default: Any = None):
+        return dict(self.params).get(name, default)
+
+
+@dataclass(frozen=True)
+class HeadSpec:
+    kind: str = "norm_linear"   # key in the head registry: final norm, then the vocabulary product
+    params: tuple = ()
+
+    def get(self, name: str, default: Any = None):
+        return dict(self.params).get(name, default)
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """What one cache layer of a part needs of the paged cache.  token_shape: the elements
+    that a token adds to the layer (keys and values of attention: (2, kv_heads, head_dim); a
+    latent vector: (width,)); how they are arranged inside a page is the part's own affair
+    (`layout` names it: two parts may share a cache layer only if they agree on it).  Cache
+    layers with equal needs share a group of pages."""
+    kind: str                 # "full": every token is kept; "window": the last `window` tokens
+    token_shape: tuple
+    window: int = 0
+    layout: str = ""
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One block: how norm, mixer, feed-forward and the residual stream are arranged."""
     arrangement: str     # key in the block registry, e.g. "prenorm"
@@ -89,6 +120,8 @@ class ModelSpec:
     eos_token_ids: tuple = ()
     bos_token_id: Optional[int] = None
     ignored_tensor_suffixes: tuple = ()   # names in a checkpoint that are not weights
+    embedding: EmbeddingSpec = EmbeddingSpec()
+    head: HeadSpec = HeadSpec()
 
 
 def params(**kw) -> tuple:

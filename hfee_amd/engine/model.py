@@ -15,7 +15,7 @@ import torch
 from ..cache.manager import CacheGroupSpec
 from ..config.registry import config_from_folder, model_spec_of
 from ..config.specs import ModelSpec
-from ..parts import Embedding, Head, lookup
+from ..parts import lookup
 from ..weights.loader import bind_tensors, engine_dtype, load_tensors
 from ..weights.random_init import random_tensors
 
@@ -34,10 +34,12 @@ class EngineInfo:
 class Model:
     def __init__(self, spec: ModelSpec, dtype: torch.dtype):
         self.spec, self.dtype = spec, dtype
-        self.embedding = Embedding(spec.embedding_name, spec.vocab, spec.hidden)
+        self.embedding = lookup("embedding", spec.embedding.kind)(spec.embedding, spec.embedding_name, spec.vocab,
+                                                                  spec.hidden, dtype)
         self.blocks = [lookup("block", ls.arrangement)(ls, dtype) for ls in spec.layers]
         final_norm = lookup("norm", spec.final_norm.kind)(spec.final_norm, spec.final_norm_name)
-        self.head = Head(final_norm, spec.head_name, spec.vocab, spec.hidden, self.embedding, dtype)
+        self.head = lookup("head", spec.head.kind)(spec.head, final_norm, spec.head_name, spec.vocab, spec.hidden,
+                                                   self.embedding, dtype)
         self.schedule = tuple(spec.schedule)
         for e in self.schedule:
             if not 0 <= e.layer < len(self.blocks):
@@ -59,42 +61,66 @@ class Model:
         self.head.bind(tensors)
         self.bound = True
 
+    # ---- parts
+    def parts(self):
+        """Every part of the model once, in running order: the embedding, each layer's
+        parts, the head's.  Whatever a part asks of the engine (state, preparation, a
+        step's metadata, graph capture) is collected over this list."""
+        out, seen = [], set()
+        for owner in [self.embedding, *self.blocks, self.head]:
+            for p in owner.parts():
+                if id(p) not in seen:
+                    seen.add(id(p))
+                    out.append(p)
+        return out
+
     # ---- cache
     def cache_groups(self):
-        """Cache layers with the same needs share a group.  A cache layer's needs
-        are those of the mixer that writes it."""
+        """Cache layers with the same needs share a group.  A cache layer's needs are
+        those of the block that writes it (a block answers for the part of it that uses
+        the cache)."""
         needs: dict = {}
         for e in self.schedule:
-            spec = self.blocks[e.layer].mixer.cache_spec()
-            if spec is None:
+            need = self.blocks[e.layer].cache_spec()
+            if need is None:
                 continue
             if e.writes_cache:
-                if e.cache in needs and needs[e.cache] != spec:
-                    raise ValueError(f"cache layer {e.cache} is written by mixers with different needs")
-                needs[e.cache] = spec
+                if e.cache in needs and needs[e.cache] != need:
+                    raise ValueError(f"cache layer {e.cache} is written by layers with different needs")
+                needs[e.cache] = need
         for e in self.schedule:
-            spec = self.blocks[e.layer].mixer.cache_spec()
-            if spec is not None and not e.writes_cache:
+            need = self.blocks[e.layer].cache_spec()
+            if need is not None and not e.writes_cache:
                 if e.cache not in needs:
                     raise ValueError(f"layer {e.layer} reads cache layer {e.cache}, which no layer writes")
                 writer = next(w for w in self.schedule if w.cache == e.cache and w.writes_cache)
-                mine = getattr(self.blocks[e.layer].mixer, "key_layout", lambda: None)()
-                theirs = getattr(self.blocks[writer.layer].mixer, "key_layout", lambda: None)()
-                if needs[e.cache][1:3] != spec[1:3] or mine != theirs:
+                mine = getattr(self.blocks[e.layer], "key_layout", lambda: None)()
+                theirs = getattr(self.blocks[writer.layer], "key_layout", lambda: None)()
+                theirs_need = needs[e.cache]
+                if (theirs_need.token_shape, theirs_need.layout) != (need.token_shape, need.layout) or mine != theirs:
                     raise ValueError(f"layer {e.layer} cannot read cache layer {e.cache}: its keys are laid out "
                                      f"differently from those that layer {writer.layer} writes")
         by_need: dict = {}
-        for layer, spec in sorted(needs.items()):
-            by_need.setdefault(spec, []).append(layer)
-        return [CacheGroupSpec(kind=k, kv_heads=kv, head_dim=hd, window=w, cache_layers=tuple(layers))
-                for (k, kv, hd, w), layers in by_need.items()]
+        for layer, need in sorted(needs.items()):
+            by_need.setdefault(need, []).append(layer)
+        return [CacheGroupSpec(kind=n.kind, token_shape=tuple(n.token_shape), window=n.window, layout=n.layout,
+                               cache_layers=tuple(layers))
+                for n, layers in by_need.items()]
 
-    def mixers(self):
-        return [b.mixer for b in self.blocks]
+    def state_specs(self):
+        return [s for p in self.parts() for s in p.state_specs()]
 
     def prepare(self, info: EngineInfo):
-        for m in self.mixers():
-            m.prepare(info)
+        for p in self.parts():
+            p.prepare(info)
+
+    def plan(self, plan):
+        for p in self.parts():
+            p.plan(plan)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in self.parts())
 
 
 def declared_tensors(config):

@@ -74,9 +74,8 @@ class Engine:
         self.storage = CacheStorage(self.groups, page_size, num_pages, max_requests, self.dtype, self.device)
         self.workspace = Workspace(max_batch_tokens, self.device)
         info = EngineInfo(self.num_positions, self.device, self.dtype, page_size, max_requests, self.storage)
-        for m in model.mixers():
-            for name, shape, dt in m.state_specs():
-                self.storage.add_state(name, shape, dt)
+        for name, shape, dt in model.state_specs():
+            self.storage.add_state(name, shape, dt)
         model.prepare(info)
         self._meta_capacity = 0
         self._meta_views: dict = {}        # layout of a step's metadata -> (offsets, views of the device buffer)
@@ -86,8 +85,7 @@ class Engine:
         # decode-only steps are replayed as captured HIP graphs, one per
         # (batch size, block-table width, wanted rows): launch gaps would otherwise
         # cost more than the kernels at small batches
-        self.use_graphs = use_graphs and all(
-            p.graph_safe for b in model.blocks for p in (b.parts() if hasattr(b, "parts") else [b]))
+        self.use_graphs = use_graphs and model.graph_safe
         self._graphs: dict = {}
         self.graph_replays = 0
 
@@ -246,12 +244,7 @@ class Engine:
             plan.add(f"block_tables.{g}", bt)
         if decode_only:
             plan.host["graph.max_context"] = max(widths) * self.page_size
-        seen = set()
-        for entry in self.model.schedule:
-            mixer = self.model.blocks[entry.layer].mixer
-            if id(mixer) not in seen:
-                seen.add(id(mixer))
-                mixer.plan(plan)
+        self.model.plan(plan)
         plan.n, plan.wanted, plan.max_position = n, len(logit_rows), int(positions.max())
         plan.graph_key = None
         if decode_only:

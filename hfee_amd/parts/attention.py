@@ -23,7 +23,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from ..config.specs import MixerSpec
+from ..config.specs import CacheNeed, MixerSpec
 from ..kernels import ops
 from ..weights.spec import TensorSpec
 from .base import LazyNorm, Mixer, lookup, register_mixer
@@ -96,7 +96,13 @@ class Attention(Mixer):
 
     # ---- cache
     def cache_spec(self):
-        return ("window" if self.window > 0 else "full", self.kv_heads, self.head_dim, self.window)
+        # keys of a (page, head) as [slot][head_dim], values transposed: csrc/common.h's CacheLayout
+        return CacheNeed("window" if self.window > 0 else "full", (2, self.kv_heads, self.head_dim), self.window,
+                         layout="keys by slot, values by dimension")
+
+    def _cache_layer(self, ctx, cache_layer):
+        """The cache layer as the kernels take it: [pages, 2, kv_heads, page_size * head_dim]."""
+        return ctx.storage.layer(cache_layer, (2, self.kv_heads, ctx.page_size * self.head_dim))
 
     def prepare(self, info):
         if self.position is not None:
@@ -127,7 +133,7 @@ class Attention(Mixer):
         H, K, hd = self.num_heads, self.kv_heads, self.head_dim
         n = ctx.n
         group = ctx.storage.group_of(cache_layer)
-        cache = ctx.storage.layer(cache_layer)
+        cache = self._cache_layer(ctx, cache_layer)
         tables = ctx.block_tables[group]
         pos = self.position
         cos, sin = (pos.cos, pos.sin) if pos else (None, None)

@@ -2,14 +2,21 @@
 and what a step hands it.
 
 A part gets all its sizes and constants through its spec; it never learns which
-model it is in.  Five kinds, each with a registry from the spec's `kind` string to
+model it is in.  Seven kinds, each with a registry from the spec's `kind` string to
 a class:
 
+  embedding       forward(ctx, x): the residual stream's first value from the token ids
   norm            forward(ctx, out, x, rows=None)
   position        prepare(num_positions, device); applied by the mixer that owns it
   mixer           forward_add(ctx, x, h, cache_layer, writes_cache): x += mix(h)
   feed_forward    forward_add(ctx, x, h):                            x += ffn(h)
   block           forward(ctx, x, entry): one layer's arrangement of the above
+  head            forward(ctx, logits, x, rows): logits of the wanted rows
+
+Every part, whatever its kind, may also ask for per-request state of fixed size
+(state_specs), prepare itself before the first step (prepare), add int32 metadata to
+every step (plan), and, through its block, for a layer of the paged cache (cache_spec):
+the engine collects these from all parts of the model alike.
 
 `x` is the residual stream, float32 [n, hidden]; `h` is a normed copy in the
 engine's dtype.  Every part also has tensor_specs() -> [TensorSpec] and
@@ -23,7 +30,8 @@ from typing import Optional
 import torch
 
 
-_REGISTRIES: dict[str, dict] = {"norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}}
+_REGISTRIES: dict[str, dict] = {"norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {},
+                                "embedding": {}, "head": {}}
 
 
 def _register(family: str, kind: str, cls):
@@ -49,6 +57,14 @@ def register_feed_forward(kind: str, cls=None):
 
 def register_block(kind: str, cls=None):
     return _register("block", kind, cls) if cls else (lambda c: _register("block", kind, c))
+
+
+def register_embedding(kind: str, cls=None):
+    return _register("embedding", kind, cls) if cls else (lambda c: _register("embedding", kind, c))
+
+
+def register_head(kind: str, cls=None):
+    return _register("head", kind, cls) if cls else (lambda c: _register("head", kind, c))
 
 
 def lookup(family: str, kind: str):
@@ -81,17 +97,21 @@ class Part:
     def bind(self, tensors: dict) -> None:
         pass
 
-
-class Mixer(Part):
-    """Mixes information between the tokens of a sequence."""
+    def parts(self) -> list:
+        """The parts this one is made of, itself included if it has hooks of its own (a
+        block lists its norms, mixer and feed-forward)."""
+        return [self]
 
     def cache_spec(self):
-        """None, or (kind, kv_heads, head_dim, window): the growing memory one
-        cache layer of this mixer needs ("full" or "window")."""
+        """None, or a CacheNeed: the growing memory that one cache layer of this part
+        needs.  The engine asks a layer's block, which answers for the part of it that
+        reads and writes the cache layer named by the schedule."""
         return None
 
     def state_specs(self) -> list:
-        """Per-request states of fixed size: [(name, shape, dtype)]."""
+        """Per-request states of fixed size: [(name, shape, dtype)].  The engine keeps
+        one tensor [max_requests, *shape] per name (info.storage.states[name], indexed
+        by a request's slot) and clears a slot when a request is admitted."""
         return []
 
     def prepare(self, engine_info) -> None:
@@ -99,7 +119,12 @@ class Mixer(Part):
 
     def plan(self, plan) -> None:
         """Called once per step before the metadata goes to the device; may add
-        int32 arrays with plan.add(key, array) (shared by parts that use one key)."""
+        int32 arrays with plan.add(key, array) (they arrive as ctx.extra[key]) and
+        host values with plan.host[key] = value."""
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a sequence."""
 
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool) -> None:
         raise NotImplementedError

@@ -27,6 +27,13 @@ class PreNormBlock(Part):
     def parts(self):
         return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
 
+    # the layer of the paged cache that a run of this block is given belongs to its mixer
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def key_layout(self):
+        return getattr(self.mixer, "key_layout", lambda: None)()
+
     def tensor_specs(self):
         return [s for p in self.parts() for s in p.tensor_specs()]
 

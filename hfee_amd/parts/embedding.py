@@ -10,13 +10,19 @@ from __future__ import annotations
 
 import torch
 
+from ..config.specs import EmbeddingSpec, HeadSpec
 from ..kernels import ops
 from ..weights.spec import TensorSpec
-from .base import Part
+from .base import Part, register_embedding, register_head
 
 
+@register_embedding("lookup")
 class Embedding(Part):
-    def __init__(self, name: str, vocab: int, hidden: int):
+    """constructor of every embedding kind: (spec, tensor name, vocabulary, width, engine dtype);
+    `table` is what a head without a matrix of its own shares."""
+    graph_safe = True
+
+    def __init__(self, spec: EmbeddingSpec, name: str, vocab: int, hidden: int, dtype: torch.dtype = None):
         self.name, self.vocab, self.hidden = name, vocab, hidden
         self.table = None
 
@@ -30,11 +36,19 @@ class Embedding(Part):
         ops.embed(x, self.table, ctx.token_ids)
 
 
+@register_head("norm_linear")
 class Head(Part):
-    def __init__(self, norm, name, vocab: int, hidden: int, embedding: Embedding, dtype: torch.dtype):
+    """constructor of every head kind: (spec, the final norm part, tensor name or None to share
+    the embedding's table, vocabulary, width, the embedding part, engine dtype)."""
+    graph_safe = True
+
+    def __init__(self, spec: HeadSpec, norm, name, vocab: int, hidden: int, embedding, dtype: torch.dtype):
         self.norm, self.name, self.vocab, self.hidden = norm, name, vocab, hidden
         self.embedding, self.dtype = embedding, dtype
         self.weight = None
+
+    def parts(self):
+        return [self.norm, self]
 
     def tensor_specs(self):
         specs = self.norm.tensor_specs()

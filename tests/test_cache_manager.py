@@ -6,8 +6,8 @@ import pytest
 
 from hfee_amd.cache import CacheError, CacheGroupSpec, CacheManager, OutOfPages, PagePool
 
-FULL = CacheGroupSpec("full", kv_heads=2, head_dim=16, cache_layers=(0, 1))
-WIN = CacheGroupSpec("window", kv_heads=2, head_dim=16, cache_layers=(2,), window=40)
+FULL = CacheGroupSpec("full", (2, 2, 16), cache_layers=(0, 1))
+WIN = CacheGroupSpec("window", (2, 2, 16), cache_layers=(2,), window=40)
 
 
 def test_pool_refuses_double_free_and_foreign_free():

@@ -690,3 +690,204 @@ def test_attention_window_edge():
                         outs[f"decode{splits}"] = out[T - 1]
                 for name, o in outs.items():
                     assert torch.allclose(o.float().cpu(), want, atol=3e-2), (dtype, T, W, inside, name)
+
+
+def test_toy_parts_of_every_kind_without_a_change_to_the_framework(tmp_path):
+    """A toy architecture in which nothing is the built-in kind: an embedding with a scale,
+    a mixer whose growing memory is one latent vector a token (not keys and values), a
+    feed-forward that keeps per-request state and plans per-step metadata, a block
+    arrangement without a mixer, and a head that scales its logits.  All are defined and
+    registered here; the engine collects their cache needs, state, preparation and step
+    metadata like anybody's, runs them in portions beside another request, and the result is
+    the plain computation's."""
+    import numpy as np
+    import hfee_amd  # noqa: F401
+    from hfee_amd.config import (CacheNeed, EmbeddingSpec, FeedForwardSpec, HeadSpec, LayerSpec, MixerSpec, ModelSpec,
+                                 NormSpec, ScheduleEntry, params, register_architecture)
+    from hfee_amd.config.base import KeyReader
+    from hfee_amd.engine import Engine, StepEntry, load_model
+    from hfee_amd.parts import (FeedForward, Mixer, Part, lookup, register_block, register_embedding,
+                                register_feed_forward, register_head, register_mixer)
+    from hfee_amd.weights import Checkpoint, TensorSpec, write_model_folder
+    from plain_llama import plain_rmsnorm
+
+    @register_embedding("toy_scaled_lookup")
+    class ScaledLookup(Part):
+        def __init__(self, spec, name, vocab, hidden, dtype):
+            self.name, self.vocab, self.hidden, self.scale = name, vocab, hidden, float(spec.get("scale"))
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name, (self.vocab, self.hidden))]
+
+        def bind(self, tensors):
+            self.table = tensors[self.name]
+
+        def forward(self, ctx, x):
+            x.copy_(self.table[ctx.token_ids.long()].float() * self.scale)
+
+    @register_mixer("toy_latent_mean")
+    class LatentMean(Mixer):
+        """x += W mean(h of the sequence so far); the h are kept in the paged cache, one vector a token."""
+
+        def __init__(self, spec, prefix, dtype):
+            self.width, self.prefix = spec.get("hidden"), prefix
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + "w.weight", (self.width, self.width))]
+
+        def bind(self, tensors):
+            self.w = tensors.pop(self.prefix + "w.weight")
+
+        def cache_spec(self):
+            return CacheNeed("full", (self.width,), layout="a latent vector a slot")
+
+        def forward_add(self, ctx, x, h, cache_layer, writes_cache):
+            ps = ctx.page_size
+            pages = ctx.storage.layer(cache_layer, (ps, self.width))
+            tables = ctx.block_tables[ctx.storage.group_of(cache_layer)].cpu()
+            for i, seg in enumerate(ctx.segments):
+                for j in range(seg.length):
+                    p = seg.start + j
+                    pages[int(tables[i, p // ps]), p % ps] = h[seg.row0 + j].to(pages.dtype)
+                held = torch.stack([pages[int(tables[i, p // ps]), p % ps] for p in range(seg.start + seg.length)]).float()
+                sums = held.cumsum(0)
+                for j in range(seg.length):
+                    p = seg.start + j
+                    x[seg.row0 + j] += self.w.float() @ (sums[p] / (p + 1))
+
+    @register_feed_forward("toy_counting")
+    class Counting(FeedForward):
+        """x[t] += (W h[t]) * (1 + t % 2) + t / 100: the parity comes with the step's metadata, the
+        count of tokens that the request has run before lives in its state slot."""
+
+        def __init__(self, spec, prefix, dtype):
+            self.width, self.prefix = spec.get("hidden"), prefix
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + "w.weight", (self.width, self.width))]
+
+        def bind(self, tensors):
+            self.w = tensors.pop(self.prefix + "w.weight")
+
+        def state_specs(self):
+            return [(self.prefix + "seen", (1,), torch.float32)]
+
+        def prepare(self, info):
+            self.seen = info.storage.states[self.prefix + "seen"]
+
+        def plan(self, plan):
+            if "toy.parity" not in plan.arrays:          # (the layers' feed-forwards share it)
+                plan.add("toy.parity", np.concatenate([np.arange(s.start, s.start + s.length) % 2 for s in plan.segments]))
+
+        def forward_add(self, ctx, x, h):
+            x += (h.float() @ self.w.float().t()) * (1 + ctx.extra["toy.parity"].float())[:, None]
+            for seg in ctx.segments:
+                rows = slice(seg.row0, seg.row0 + seg.length)
+                x[rows] += 0.01 * (self.seen[seg.slot] + torch.arange(seg.length, device=x.device))[:, None]
+                self.seen[seg.slot] += seg.length
+
+    @register_block("toy_feed_forward_only")
+    class FeedForwardOnly(Part):
+        def __init__(self, spec, dtype):
+            self.norm = lookup("norm", spec.feed_forward_norm.kind)(spec.feed_forward_norm, spec.prefix + "norm.weight")
+            self.ffn = lookup("feed_forward", spec.feed_forward.kind)(spec.feed_forward, spec.prefix + "ffn.", dtype)
+            self.hidden = spec.hidden
+
+        def parts(self):
+            return [self.norm, self.ffn]
+
+        def tensor_specs(self):
+            return self.norm.tensor_specs() + self.ffn.tensor_specs()
+
+        def bind(self, tensors):
+            self.norm.bind(tensors)
+            self.ffn.bind(tensors)
+
+        def forward(self, ctx, x, entry):
+            h = ctx.rows("toy.normed", self.hidden)
+            self.norm.forward(ctx, h, x)
+            self.ffn.forward_add(ctx, x, h)
+
+    @register_head("toy_scaled_head")
+    class ScaledHead(Part):
+        def __init__(self, spec, norm, name, vocab, hidden, embedding, dtype):
+            self.norm, self.embedding, self.hidden, self.scale = norm, embedding, hidden, float(spec.get("logit_scale"))
+
+        def parts(self):
+            return [self.norm, self]
+
+        def tensor_specs(self):
+            return self.norm.tensor_specs()
+
+        def bind(self, tensors):
+            self.norm.bind(tensors)
+
+        def forward(self, ctx, logits, x, rows):
+            h = ctx.rows("toy.head", self.hidden, n=logits.shape[0])
+            self.norm.forward(ctx, h, x, rows)
+            logits.copy_((h.float() @ self.embedding.table.float().t()) * self.scale)
+
+    @dataclass(frozen=True)
+    class EveryConfig:
+        architecture: str
+        hidden: int
+        vocab: int
+
+        @staticmethod
+        def from_dict(d, where="config.json"):
+            r = KeyReader(d, where)
+            c = EveryConfig("ToyEveryKindForCausalLM", r.int("e_hidden"), r.int("e_vocab"))
+            r.finish()
+            return c
+
+        def to_dict(self):
+            return {"architectures": ["ToyEveryKindForCausalLM"], "e_hidden": self.hidden, "e_vocab": self.vocab}
+
+    def every_spec(c):
+        norm = NormSpec("rmsnorm", c.hidden, 1e-5)
+        ffn = FeedForwardSpec("toy_counting", params(hidden=c.hidden))
+        latent = MixerSpec("toy_latent_mean", params(hidden=c.hidden))
+        layers = (LayerSpec("prenorm", c.hidden, latent, ffn, norm, norm, "e.0."),
+                  LayerSpec("toy_feed_forward_only", c.hidden, MixerSpec("none"), ffn, norm, norm, "e.1."))
+        return ModelSpec("ToyEveryKindForCausalLM", c.hidden, c.vocab, layers, (ScheduleEntry(0, 0), ScheduleEntry(1, 1)),
+                         norm, "e.embed.weight", "e.norm.weight", None, max_positions=256,
+                         embedding=EmbeddingSpec("toy_scaled_lookup", params(scale=3.0)),
+                         head=HeadSpec("toy_scaled_head", params(logit_scale=0.5)))
+
+    register_architecture("ToyEveryKindForCausalLM", EveryConfig, every_spec)
+    cfg = EveryConfig("ToyEveryKindForCausalLM", 24, 60)
+    folder = write_model_folder(str(tmp_path / "every"), cfg, seed=2, std=0.2)
+    model, _ = load_model(folder, "float32")
+    eng = Engine(model, num_pages=8, page_size=16, max_requests=2, max_batch_tokens=64)
+    assert not eng.use_graphs
+    assert [(g.kind, g.token_shape, g.cache_layers) for g in eng.groups] == [("full", (24,), (0,))]
+    assert eng.storage.pages[0].shape == (1, 8, 16 * 24)
+    assert set(eng.storage.states) == {"e.0.feed_forward.seen", "e.1.ffn.seen"}
+
+    toks = tu.make_requests(60, [50, 30], seed=4)
+    eng.admit("other")
+    eng.admit("a")
+    got, i, oi = [], 0, 0
+    for n in [9, 1, 22, 2, 16]:
+        entries = [StepEntry("a", toks["r0"][i:i + n], list(range(n)))]
+        if oi < 30:
+            entries.insert(0, StepEntry("other", toks["r1"][oi:oi + 7], []))
+            oi += 7
+        got.append(eng.step(entries).double().cpu())
+        i += n
+    got = torch.cat(got)
+    assert float(eng.storage.states["e.1.ffn.seen"][eng.cache.get("a").slot]) == 50
+    eng.cache.check()
+
+    ck = Checkpoint(folder)
+    t = {n: ck.tensor(n).double() for n in ck.names()}
+    T = 50
+    x = t["e.embed.weight"][toks["r0"]] * 3.0
+    at = torch.arange(T, dtype=torch.float64)
+    h = plain_rmsnorm(x, t["e.0.mixer_norm.weight"], 1e-5)
+    x = x + (h.cumsum(0) / (at + 1)[:, None]) @ t["e.0.mixer.w.weight"].t()
+    for norm_name, w_name in (("e.0.feed_forward_norm.weight", "e.0.feed_forward.w.weight"), ("e.1.norm.weight", "e.1.ffn.w.weight")):
+        h = plain_rmsnorm(x, t[norm_name], 1e-5)
+        x = x + (h @ t[w_name].t()) * (1 + at % 2)[:, None] + 0.01 * at[:, None]
+    want = plain_rmsnorm(x, t["e.norm.weight"], 1e-5) @ t["e.embed.weight"].t() * 0.5
+    assert torch.allclose(got, want, atol=2e-4, rtol=2e-4), float((got - want).abs().max())

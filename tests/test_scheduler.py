@@ -15,7 +15,7 @@ EOS = 49
 
 class FakeEngine:
     def __init__(self, num_pages, max_requests, page_size=16):
-        self.cache = CacheManager([CacheGroupSpec("full", 1, 16, (0,))], page_size, num_pages, max_requests)
+        self.cache = CacheManager([CacheGroupSpec("full", (2, 1, 16), (0,))], page_size, num_pages, max_requests)
         self.fed = {}          # request -> tokens in its cache
         self.batches = []      # per step: [(request, n tokens, wants logits)]
         self.prepared = None   # the shape that the scheduler announced for the next step
