@@ -106,6 +106,7 @@ __device__ __forceinline__ LaneOffsets lane_offsets(const CacheLayout& lay, int 
 // cache never holds anything but finite numbers).  The tile lies in at most two pages;
 // their numbers are scalars out of the page window, and a lane's address is one of two
 // bases plus what lane_offsets worked out once.
+template <bool STREAMED>
 __device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict__ cache, const CacheLayout& lay,
                                           const LaneOffsets& off, const int* __restrict__ bt, int bt_stride,
                                           PageWindow& pages, int k0, int kv_first, int kv_last) {
@@ -120,12 +121,18 @@ __device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict
   const int in_page = k0 & (lay.page_size - 1);
   const bf16_t* krow = (r32 < 16 ? base_a : base_b) + off.key + in_page * lay.head_dim;
 #pragma unroll
-  for (int c = 0; c < NC; ++c) ops.k[c].u = *reinterpret_cast<const u32x4*>(krow + c * 16);
+  for (int c = 0; c < NC; ++c) {
+    if constexpr (STREAMED) ops.k[c].u = load_streamed(reinterpret_cast<const u32x4*>(krow + c * 16));
+    else ops.k[c].u = *reinterpret_cast<const u32x4*>(krow + c * 16);
+  }
   const bf16_t* vbase[2] = {base_a + in_page, base_b + ((k0 + 16) & (lay.page_size - 1))};
 #pragma unroll
   for (int u = 0; u < 2; ++u)
 #pragma unroll
-    for (int t = 0; t < NDT; ++t) ops.v[u][t].u = *reinterpret_cast<const u32x4*>(vbase[u] + off.value[t]);
+    for (int t = 0; t < NDT; ++t) {
+      if constexpr (STREAMED) ops.v[u][t].u = load_streamed(reinterpret_cast<const u32x4*>(vbase[u] + off.value[t]));
+      else ops.v[u][t].u = *reinterpret_cast<const u32x4*>(vbase[u] + off.value[t]);
+    }
 }
 
 // Adds the keys k0 .. k0+31 to the running state.  q_op: this slot's query, pre-loaded
@@ -214,8 +221,9 @@ __device__ __forceinline__ void compute_tile(Tile& st, const Op* q_op, const Til
 // are issued while the tile before it is computed (two tiles' operands in registers:
 // for kernels that run one wave per SIMD anyway); otherwise tile by tile.
 // all_first..all_last: the keys that every slot in use sees (a tile inside this range
-// needs no mask).
-template <bool AHEAD>
+// needs no mask).  STREAMED: nobody else reads these keys in this launch (a decode step: one
+// workgroup per sequence, KV head and stretch of keys), so they are loaded as a stream.
+template <bool AHEAD, bool STREAMED>
 __device__ __forceinline__ void attend_tiles(Tile& st, const Op* q_op, const bf16_t* __restrict__ cache,
                                              const CacheLayout& lay, const int* __restrict__ bt, int bt_stride,
                                              const LaneOffsets& off, int first, int end, int step, int kv_first, int kv_last,
@@ -225,17 +233,17 @@ __device__ __forceinline__ void attend_tiles(Tile& st, const Op* q_op, const bf1
   pages.base = -1;
   if constexpr (AHEAD) {
     TileOps cur, nxt;
-    load_tile(cur, cache, lay, off, bt, bt_stride, pages, first * 32, kv_first, kv_last);
+    load_tile<STREAMED>(cur, cache, lay, off, bt, bt_stride, pages, first * 32, kv_first, kv_last);
     for (int t = first; t < end; t += step) {
       const int tn = t + step;
-      if (tn < end) load_tile(nxt, cache, lay, off, bt, bt_stride, pages, tn * 32, kv_first, kv_last);
+      if (tn < end) load_tile<STREAMED>(nxt, cache, lay, off, bt, bt_stride, pages, tn * 32, kv_first, kv_last);
       compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2, t * 32 >= all_first && t * 32 + 31 <= all_last);
       cur = nxt;
     }
   } else {
     for (int t = first; t < end; t += step) {
       TileOps cur;
-      load_tile(cur, cache, lay, off, bt, bt_stride, pages, t * 32, kv_first, kv_last);
+      load_tile<STREAMED>(cur, cache, lay, off, bt, bt_stride, pages, t * 32, kv_first, kv_last);
       compute_tile(st, q_op, cur, t * 32, pos, lo, scale_log2, t * 32 >= all_first && t * 32 + 31 <= all_last);
     }
   }
@@ -302,7 +310,7 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
   const int kv_last = pos0 + rows - 1;
   const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
   // every row in use sees the keys from the last row's window start to the first row's position
-  attend_tiles<false>(st, q_op, cache, lay, bt, bt_stride, lane_offsets(lay, kvh), kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
+  attend_tiles<false, false>(st, q_op, cache, lay, bt, bt_stride, lane_offsets(lay, kvh), kv_first >> 5, (kv_last >> 5) + 1, 1, kv_first, kv_last, pos, lo,
                scale_log2, window > 0 ? max(0, kv_last - window + 1) : 0, pos0);
 
   const float l_slot = finish_sum(st);
@@ -636,7 +644,7 @@ __global__ __launch_bounds__(DECODE_MAX_WAVES * 64, AHEAD ? 1 : 2) void decode_k
     load_query(q_op, q + (int64_t)row * ldq + h * HD, slot_ok);
     Tile st;
     init_tile(st);
-    attend_tiles<AHEAD>(st, q_op, cache, lay, bt, bt_stride, off, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
+    attend_tiles<AHEAD, false>(st, q_op, cache, lay, bt, bt_stride, off, t_begin + wave, t_end, waves, lo, pos, slot_ok ? pos : -1, lo,
                  scale_log2, lo, pos);
 
     // this wave's state into LDS

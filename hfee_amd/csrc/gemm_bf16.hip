@@ -1290,14 +1290,10 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
                    ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
   if (out_mode == 3) {
     HFEE_REQUIRE(N % 2 == 0 && vec, "gemm_bf16: the SiLU gate needs an even N and aligned operands");
-    if (skinny_pays(M, N))
-      return hfee_gemm_skinny_plain(C, ldc, A, lda, W, ldw, M, N, K, OUT_SWIGLU, stream);
     if (launch_aligned<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, force_kernel, stream)) return 1;
     HFEE_CHECK_LAUNCH("gemm_bf16");
     return 0;
   }
-  if (vec && M <= 64 && (force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N))))   // gemm_skinny.hip
-    return hfee_gemm_skinny_plain(C, ldc, A, lda, W, ldw, M, N, K, out_mode, stream);
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   int rc;

@@ -6,7 +6,7 @@
 #include "qkv_epilogue.h"
 
 HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
-                              int64_t ldw, int M, int N, int K, int epi,
+                              int64_t w_stride, int M, int N, int K, int epi,
                               const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
                               const int* positions, const int* token_segment, const int* block_tables,
                               int bt_stride, const float* cos_table, const float* sin_table, int half,
@@ -15,20 +15,6 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                               int64_t ld_emit, float* emit_ss, const float* scale_ss, int scale_blocks,
                               float scale_eps, float* scratch, int64_t scratch_floats, int force_mid,
                               hipStream_t stream);
-
-// The product alone through the streaming kernels: bfloat16 A, no norm, no rotation, nothing
-// emitted or scaled, no workspace.
-inline int hfee_gemm_skinny_plain(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int64_t ldw, int M,
-                                  int N, int K, int epi, hipStream_t stream) {
-  return hfee_gemm_skinny(C, ldc, A, /*a_is_f32=*/0, lda, W, ldw, M, N, K, epi,
-                          /*norm_weight=*/nullptr, 0, /*eps=*/0.f, /*rows=*/nullptr, /*positions=*/nullptr,
-                          /*token_segment=*/nullptr, /*block_tables=*/nullptr, /*bt_stride=*/0,
-                          /*cos_table=*/nullptr, /*sin_table=*/nullptr, /*half=*/0, /*table_positions=*/0,
-                          /*cache=*/nullptr, /*num_heads=*/0, /*kv_heads=*/0, /*head_dim=*/0, /*page_size=*/0,
-                          /*emit_weight=*/nullptr, 0, /*emit_out=*/nullptr, /*ld_emit=*/0, /*emit_ss=*/nullptr,
-                          /*scale_ss=*/nullptr, /*scale_blocks=*/0, /*scale_eps=*/0.f,
-                          /*scratch=*/nullptr, /*scratch_floats=*/0, /*force_mid=*/0, stream);
-}
 
 HFEE_API int hfee_gemm_bf16_qkv(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int64_t ldw, int M,
                                 int N, int K, const hfee::QkvArgs* qkv, int force_kernel, hipStream_t stream);

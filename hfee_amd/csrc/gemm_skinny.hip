@@ -8,6 +8,13 @@
 // the B operand.  Loads are issued one block ahead of the matrix instructions.
 // Partial sums meet in LDS and are added in wave order (a fixed order).
 //
+// W comes in tiles (see WeightTiles in common.h): 16 rows x 32 columns are one kilobyte in
+// the order in which a wave's lanes hold them as an operand, so that a load instruction of a
+// wave reads one contiguous kilobyte, whole 128-byte lines that nobody else touches, and
+// can carry the non-temporal hint.  With rows of W as they lie in a checkpoint the same
+// instruction reads sixteen half lines, each of which a second instruction asks for again:
+// a read-only stream of that pattern measures 5.9 TB/s on this GPU, the kilobytes 6.5.
+//
 // Folded in:
 //   NORM   the RMSNorm in front of the product
 //          (/root/reference/internal/ggml/ops.go:124-134): A is the float32 residual
@@ -41,7 +48,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_QKV = 4 };
 
-constexpr int WAVES = 8, ROWS = 16, UNROLL = 4, KBLOCK = 32 * UNROLL;
+constexpr int WAVES = 8, ROWS = 16;
 
 union Chunk {
   u32x4 u;
@@ -54,8 +61,8 @@ struct Args {
   int64_t ldc;
   const void* A;              // bfloat16 [M, K], or float32 rows when NORM
   int64_t lda;
-  const bf16_t* W;
-  int64_t ldw;
+  const bf16_t* W;            // in tiles of 16 rows x 32 columns
+  int64_t w_stride;           // elements from one row of tiles to the next
   int M, N, K;
   const void* norm_weight;    // NORM: [K]
   int norm_weight_is_f32;
@@ -76,42 +83,47 @@ struct Args {
 
 constexpr int SS_STRIDE = 64;   // rows of a product of this file
 
+// A K block is U steps of 32 columns: what a wave asks for at once and keeps in flight while
+// it multiplies the block before.
+template <int U>
 struct Block {                // one wave's operands for one K block
-  Chunk w[UNROLL];
+  Chunk w[U];
 };
 
-template <int MT, bool NORM>
+template <int MT, bool NORM, int U>
 struct XBlock;
 
-template <int MT>
-struct XBlock<MT, false> {
-  Chunk x[MT][UNROLL];
+template <int MT, int U>
+struct XBlock<MT, false, U> {
+  Chunk x[MT][U];
 };
 
-template <int MT>
-struct XBlock<MT, true> {     // raw float32 activations and the norm weight
-  f32x4 x[MT][UNROLL][2];
-  f32x4 nw[UNROLL][2];
+template <int MT, int U>
+struct XBlock<MT, true, U> {     // raw float32 activations and the norm weight
+  f32x4 x[MT][U][2];
+  f32x4 nw[U][2];
 };
 
 __device__ __forceinline__ f32x4 load_f4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 
-template <int MT, bool NORM>
-__device__ __forceinline__ void load_block(Block& b, XBlock<MT, NORM>& xb, const bf16_t* __restrict__ w_row,
+template <int MT, bool NORM, int U>
+__device__ __forceinline__ void load_block(Block<U>& b, XBlock<MT, NORM, U>& xb, const bf16_t* __restrict__ w_row,
                                            const void* const* x_rows, const Args& a, int k) {
-  // w_row and x_rows already point at this lane's eight-element column group
+  // w_row points at this lane's place in the first tile of its row of tiles, x_rows at its
+  // eight-element column group; 32 columns on is the next tile
 #pragma unroll
-  for (int s = 0; s < UNROLL; ++s) b.w[s].u = *reinterpret_cast<const u32x4*>(w_row + k + 32 * s);
+  for (int s = 0; s < U; ++s)
+    b.w[s].u = load_streamed(reinterpret_cast<const u32x4*>(w_row + (int64_t)(k + 32 * s) * WeightTiles::PER_COLUMN));
   if constexpr (!NORM) {
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int s = 0; s < UNROLL; ++s)
+      for (int s = 0; s < U; ++s)
         xb.x[t][s].u = *reinterpret_cast<const u32x4*>((const bf16_t*)x_rows[t] + k + 32 * s);
   } else {
     const int kg = k + 8 * ((threadIdx.x & 63) >> 4);
 #pragma unroll
-    for (int s = 0; s < UNROLL; ++s) {
+    for (int s = 0; s < U; ++s) {
       if (a.norm_weight_is_f32) {
         xb.nw[s][0] = load_f4((const float*)a.norm_weight + kg + 32 * s);
         xb.nw[s][1] = load_f4((const float*)a.norm_weight + kg + 32 * s + 4);
@@ -133,12 +145,12 @@ __device__ __forceinline__ void load_block(Block& b, XBlock<MT, NORM>& xb, const
   }
 }
 
-template <int MT, bool NORM>
-__device__ __forceinline__ void compute_block(f32x4* acc, float* ss, const Block& b, const XBlock<MT, NORM>& xb) {
+template <int MT, bool NORM, int U>
+__device__ __forceinline__ void compute_block(f32x4* acc, float* ss, const Block<U>& b, const XBlock<MT, NORM, U>& xb) {
 #pragma unroll
   for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int s = 0; s < UNROLL; ++s) {
+    for (int s = 0; s < U; ++s) {
       if constexpr (!NORM) {
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.w[s].v, xb.x[t][s].v, acc[t], 0, 0, 0);
       } else {
@@ -298,18 +310,21 @@ __device__ __forceinline__ void finish_rows_ahead(const Args& a, const Ahead<EPI
 }
 
 template <int MT, bool NORM, int EPI>
-__global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_here) {
+__global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
+  // (two kilobytes of weights a wave and step of the loop for up to 16 batch rows, one beyond:
+  // with 8 waves a CU and a block in flight that is 64 KB a CU on its way, what the memory's
+  // latency takes at the CU's share of the bandwidth)
+  constexpr int U = MT == 1 ? 8 : 4, KBLOCK = 32 * U;
   __shared__ float partial[WAVES][MT][64][4];
   __shared__ float ss_part[WAVES][MT][16];
   __shared__ float row_scale[SS_STRIDE];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
-  // rows_here (16, or 12 where that fills the chip more evenly): the weight rows of this
-  // workgroup; with 12, the matrix instruction's last four rows repeat the twelfth and are dropped
-  const int n0 = blockIdx.x * rows_here;
-  // rows beyond N or M read a valid row; what they produce is never stored
-  const bf16_t* w_row = a.W + (int64_t)min(n0 + min(r16, rows_here - 1), a.N - 1) * a.ldw + g * 8;
+  const int n0 = blockIdx.x * ROWS;
+  // rows beyond N lie in the last row of tiles (zeros), rows beyond M read a valid row; what
+  // they produce is never stored
+  const bf16_t* w_row = WeightTiles::lane_place(a.W, a.w_stride, n0 + r16, g);
   const void* x_rows[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -329,7 +344,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_her
   // the threads that will finish the sums (the first MT waves, four sums each) ask now for
   // what they will need then
   const int f_t = threadIdx.x >> 6, f_m = f_t * 16 + (lane & 15), f_n = n0 + 4 * (lane >> 4);
-  const bool f_live = f_t < MT && f_m < a.M && f_n < a.N && 4 * (lane >> 4) < rows_here;
+  const bool f_live = f_t < MT && f_m < a.M && f_n < a.N;
   const Ahead<EPI> ahead = look_ahead<EPI>(a, f_m, f_n, f_live);
 
   const int nfull = a.K / KBLOCK;
@@ -341,16 +356,16 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_her
     // slower inside the decode step, where the weights come from memory: 56.9 and 57.4 µs
     // against 53.5 for q/k/v + output + down of a layer of the 8B shape at batch 8.  (The
     // block number is kept per lane, as it was when this was measured.)
-    Block cur, nxt;
-    XBlock<MT, NORM> xcur, xnxt;
+    Block<U> cur, nxt;
+    XBlock<MT, NORM, U> xcur, xnxt;
     int kb = threadIdx.x >> 6;
-    if (kb < nfull) load_block<MT, NORM>(cur, xcur, w_row, x_rows, a, kb * KBLOCK);
+    if (kb < nfull) load_block<MT, NORM, U>(cur, xcur, w_row, x_rows, a, kb * KBLOCK);
     // (behind the first loads of W, so that it costs no latency of its own)
     if (!NORM && a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
     while (kb < nfull) {
       const int kn = kb + WAVES;
-      if (kn < nfull) load_block<MT, NORM>(nxt, xnxt, w_row, x_rows, a, kn * KBLOCK);
-      compute_block<MT, NORM>(acc, ss, cur, xcur);
+      if (kn < nfull) load_block<MT, NORM, U>(nxt, xnxt, w_row, x_rows, a, kn * KBLOCK);
+      compute_block<MT, NORM, U>(acc, ss, cur, xcur);
       cur = nxt;
       xcur = xnxt;
       kb = kn;
@@ -360,13 +375,13 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_her
   if (a.K % KBLOCK != 0 && wave == nfull % WAVES) {
     const int k0 = nfull * KBLOCK;
 #pragma unroll
-    for (int s = 0; s < UNROLL; ++s) {
+    for (int s = 0; s < U; ++s) {
       const int k = k0 + 32 * s + g * 8;      // this lane's first element of the chunk
       if (k0 + 32 * s >= a.K) break;          // uniform: the whole step is beyond K
       const bool in = k < a.K;
       Chunk w;
       w.u = u32x4{0u, 0u, 0u, 0u};
-      if (in) w.u = *reinterpret_cast<const u32x4*>(w_row + k0 + 32 * s);
+      if (in) w.u = load_streamed(reinterpret_cast<const u32x4*>(w_row + (int64_t)(k0 + 32 * s) * WeightTiles::PER_COLUMN));
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         Chunk c;
@@ -410,7 +425,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_her
     const int t = idx >> 6, l = idx & 63;
     const int m = t * 16 + (l & 15);
     const int n = n0 + 4 * (l >> 4);
-    const bool live = m < a.M && n < a.N && 4 * (l >> 4) < rows_here;
+    const bool live = m < a.M && n < a.N;
     float v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -438,20 +453,11 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a, int rows_her
 
 template <int MT, bool NORM>
 void launch_epi(const Args& a, int epi, hipStream_t stream) {
-  // Twelve rows a workgroup where that takes fewer rounds of rows over the chip than
-  // sixteen (6,144 rows on 256 CUs: two workgroups a CU of 12 rows each instead of one or
-  // two of 16).  Not with EMIT: its shares are counted in groups of 16 rows.
-  static int num_cus = 0;
-  if (num_cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    num_cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-               prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
-  }
-  auto rounds = [&](int rows) { return (((a.N + rows - 1) / rows + num_cus - 1) / num_cus) * rows; };
-  const int rows_here = (a.emit_out == nullptr && rounds(12) < rounds(ROWS)) ? 12 : ROWS;
-  dim3 grid((a.N + rows_here - 1) / rows_here);
-#define GO(E) skinny_kernel<MT, NORM, E><<<grid, WAVES * 64, 0, stream>>>(a, rows_here)
+  // (a workgroup takes a whole row of tiles: with 8 or 12 rows a workgroup, which spread 6,144
+  // rows more evenly over 256 CUs, a wave's load is no longer a whole kilobyte, and that costs
+  // more than the uneven rounds: q/k/v of the 8B shape 16.6 us against 12.7)
+  dim3 grid((a.N + ROWS - 1) / ROWS);
+#define GO(E) skinny_kernel<MT, NORM, E><<<grid, WAVES * 64, 0, stream>>>(a)
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
@@ -514,8 +520,8 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   // ---- then the first weights: behind every wave's requests for the batch, also in the
   // queue of loads that the waves of a CU share (the barrier waits for the issue, not the data)
   __syncthreads();
-  auto row_ptr = [&](int rg) {       // rows beyond N read the last row; what they produce is never stored
-    return a.W + (int64_t)min(rg * ROWS + r16, a.N - 1) * a.ldw + k0 + g * 8;
+  auto row_ptr = [&](int rg) {       // rows beyond N are zeros of the last row of tiles; what they produce is never stored
+    return WeightTiles::lane_place(a.W, a.w_stride, rg * ROWS + r16, g) + (int64_t)k0 * WeightTiles::PER_COLUMN;
   };
   // (row groups are dealt out so that every workgroup of a slice gets as many, within one)
   const int per_slice = gridDim.x / slices;
@@ -524,7 +530,7 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   constexpr int MID_RING = mid_ring(MT);
   Chunk ring[MID_RING];
 #pragma unroll
-  for (int st = 0; st < MID_RING; ++st) ring[st].u = *reinterpret_cast<const u32x4*>(w_cur + st * 32);
+  for (int st = 0; st < MID_RING; ++st) ring[st].u = load_streamed(reinterpret_cast<const u32x4*>(w_cur + st * WeightTiles::TILE));
 
 #pragma unroll
   for (int it = 0; it < FILL; ++it) {
@@ -558,8 +564,8 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st % MID_RING].v, b, acc[t], 0, 0, 0);
       }
       const int ahead = st + MID_RING;
-      ring[st % MID_RING].u = ahead < MID_STEPS ? *reinterpret_cast<const u32x4*>(w_cur + ahead * 32)
-                                                : *reinterpret_cast<const u32x4*>(w_next + (ahead - MID_STEPS) * 32);
+      ring[st % MID_RING].u = ahead < MID_STEPS ? load_streamed(reinterpret_cast<const u32x4*>(w_cur + ahead * WeightTiles::TILE))
+                                                : load_streamed(reinterpret_cast<const u32x4*>(w_next + (ahead - MID_STEPS) * WeightTiles::TILE));
     }
     // The order of issue, spelled out (groups: 0x008 matrix, 0x100 LDS read, 0x020 global
     // load): the batch operands of a step are read under the products of the step before,
@@ -740,12 +746,12 @@ __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups
   }
 
   // ---- stream W ---------------------------------------------------------------------
-  auto row_ptr = [&](int rg) { return a.W + (int64_t)min(rg * ROWS + r16, a.N - 1) * a.ldw + g * 8; };
+  auto row_ptr = [&](int rg) { return WeightTiles::lane_place(a.W, a.w_stride, rg * ROWS + r16, g); };
   int rg = blockIdx.x;                       // the host launches at most row_groups workgroups
   const bf16_t* w_cur = row_ptr(rg);
   Chunk ring[RING];
 #pragma unroll
-  for (int s = 0; s < RING; ++s) ring[s].u = *reinterpret_cast<const u32x4*>(w_cur + koff(s));
+  for (int s = 0; s < RING; ++s) ring[s].u = load_streamed(reinterpret_cast<const u32x4*>(w_cur + koff(s) * WeightTiles::PER_COLUMN));
   if (!NORM && a.scale_ss != nullptr) {      // (behind the first loads of W: it costs no latency of its own)
     __shared__ float row_scale[SS_STRIDE];
     row_scales<1>(a, row_scale);
@@ -762,8 +768,8 @@ __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups
     for (int s = 0; s < STEPS; ++s) {
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % RING].v, b[s].v, acc, 0, 0, 0);
       const int ahead = s + RING;          // refill the slot RING steps ahead
-      ring[s % RING].u = ahead < STEPS ? *reinterpret_cast<const u32x4*>(w_cur + koff(ahead))
-                                       : *reinterpret_cast<const u32x4*>(w_next + koff(ahead - STEPS));
+      ring[s % RING].u = ahead < STEPS ? load_streamed(reinterpret_cast<const u32x4*>(w_cur + koff(ahead) * WeightTiles::PER_COLUMN))
+                                       : load_streamed(reinterpret_cast<const u32x4*>(w_next + koff(ahead - STEPS) * WeightTiles::PER_COLUMN));
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) partial[wave][lane][i] = acc[i];
@@ -849,7 +855,7 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 // without it, or for other sizes, or where it would not pay, the streaming kernel takes
 // the product (force_mid != 0 takes the faster kernels wherever they apply: for tests).
 HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
-                              int64_t ldw, int M, int N, int K, int epi,
+                              int64_t w_stride, int M, int N, int K, int epi,
                               const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
                               const int* positions, const int* token_segment, const int* block_tables,
                               int bt_stride, const float* cos_table, const float* sin_table, int half,
@@ -861,10 +867,13 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
   HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
   if (M == 0) return 0;
   HFEE_REQUIRE(epi >= 0 && epi <= 4, "gemm_skinny: unknown epilogue %d", epi);
-  HFEE_REQUIRE(M <= 64 || epi == EPI_QKV, "gemm_skinny: at most 64 rows (more for q/k/v only), got %d", M);
-  HFEE_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0,
-               "gemm_skinny: K and the leading dimensions must be multiples of 8 and the operands 16-byte aligned");
-  HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_skinny: a leading dimension is shorter than its row");
+  HFEE_REQUIRE(M <= 64, "gemm_skinny: at most 64 rows, got %d", M);
+  HFEE_REQUIRE(K % 8 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0,
+               "gemm_skinny: K and lda must be multiples of 8 and the operands 16-byte aligned");
+  HFEE_REQUIRE(lda >= K, "gemm_skinny: lda is shorter than a row");
+  HFEE_REQUIRE(w_stride == WeightTiles::row_stride(K),
+               "gemm_skinny: the weight must come in tiles of 16 x 32 (%lld elements a row of tiles for K = %d, got %lld)",
+               (long long)WeightTiles::row_stride(K), K, (long long)w_stride);
   const bool norm = a_is_f32 != 0;
   if (norm) {
     HFEE_REQUIRE(M <= 16, "gemm_skinny: the fused norm takes at most 16 rows, got %d", M);
@@ -874,7 +883,7 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
     HFEE_REQUIRE(rows == nullptr, "gemm_skinny: a row gather needs the fused norm");
   }
   Args a{};
-  a.C = C; a.ldc = ldc; a.A = A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw;
+  a.C = C; a.ldc = ldc; a.A = A; a.lda = lda; a.W = (const bf16_t*)W; a.w_stride = w_stride;
   a.M = M; a.N = N; a.K = K;
   a.norm_weight = norm_weight; a.norm_weight_is_f32 = norm_weight_is_f32; a.eps = eps; a.rows = rows;
   if (epi == EPI_SWIGLU) {
@@ -893,11 +902,6 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
     a.qkv.positions = positions; a.qkv.token_segment = token_segment; a.qkv.block_tables = block_tables;
     a.qkv.bt_stride = bt_stride; a.qkv.cos_table = cos_table; a.qkv.sin_table = sin_table; a.qkv.half = half;
     a.qkv.cache = cache; a.qkv.num_heads = num_heads;
-    if (M > 64) {       // a prefill portion: the tiled kernels, with the same epilogue
-      HFEE_REQUIRE(!norm && emit_out == nullptr && scale_ss == nullptr,
-                   "gemm_skinny: more than 64 rows take neither a fused norm nor a row scale");
-      return hfee_gemm_bf16_qkv(C, ldc, A, lda, W, ldw, M, N, K, &a.qkv, 0, stream);
-    }
   } else {
     HFEE_REQUIRE(ldc >= N, "gemm_skinny: ldc is shorter than a row");
   }
@@ -911,12 +915,6 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
     HFEE_REQUIRE(!norm && scale_blocks > 0 && scale_eps >= 0.f, "gemm_skinny: a row scale needs its shares and no norm of its own");
     a.scale_ss = scale_ss; a.scale_blocks = scale_blocks; a.scale_eps = scale_eps;
   }
-  // More than 16 rows and very many weight rows (gate/up) without scratch for the pair of
-  // kernels below: the streaming kernel would read the batch again for every 16 weight rows;
-  // the tiled kernel takes the row scale too.  (With scratch the pair is faster: measured
-  // inside the decode step of the 8B shape, 5,995 -> 6,186 tok/s at batch 32.)
-  if (scale_ss != nullptr && M > 16 && N >= 16384 && emit_out == nullptr && epi != EPI_QKV && !force_mid && scratch == nullptr)
-    return hfee_gemm_bf16_scaled(C, epi, ldc, A, lda, W, ldw, M, N, K, scale_ss, scale_blocks, scale_eps, stream);
   const int mt = (M + 15) / 16;
   // Where the kernels with the batch in LDS win, from fits to measured times in microseconds
   // (1,024 to 15,360 weight rows, K from 2,048 to 14,336, 17 to 64 batch rows): the streaming
@@ -956,4 +954,30 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
   else launch_epi<4, false>(a, epi, stream);
   HFEE_CHECK_LAUNCH("gemm_skinny");
   return 0;
+}
+
+// The q/k/v product of more than 64 rows (a prompt's portion) with the same epilogue, through
+// the tiled kernels: W as rows [N, K] with leading dimension ldw, not in tiles.
+HFEE_API int hfee_gemm_qkv_rows(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int64_t ldw, int M,
+                                int N, int K, const int* positions, const int* token_segment, const int* block_tables,
+                                int bt_stride, const float* cos_table, const float* sin_table, int half,
+                                int table_positions, void* cache, int num_heads, int kv_heads, int head_dim,
+                                int page_size, hipStream_t stream) {
+  HFEE_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_qkv_rows: bad sizes M=%d N=%d K=%d", M, N, K);
+  HFEE_REQUIRE(head_dim > 0 && head_dim % 4 == 0 && num_heads > 0 && kv_heads > 0 &&
+               N == (num_heads + 2 * kv_heads) * head_dim, "gemm_qkv_rows: q/k/v rows do not match the heads");
+  HFEE_REQUIRE(ldc >= (int64_t)num_heads * head_dim && ldc % 4 == 0 && (uintptr_t)C % 8 == 0,
+               "gemm_qkv_rows: the q output is too narrow or not 8-byte aligned");
+  HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_qkv_rows: a leading dimension is shorter than its row");
+  HFEE_REQUIRE(positions != nullptr, "gemm_qkv_rows: q/k/v needs positions");
+  HFEE_REQUIRE(half >= 0 && 2 * half <= head_dim, "gemm_qkv_rows: rotary width exceeds the head");
+  HFEE_REQUIRE(cos_table == nullptr || table_positions > 0, "gemm_qkv_rows: empty rotation table");
+  QkvArgs q{};
+  if (make_cache_layout(&q.lay, kv_heads, head_dim, page_size)) return 1;
+  HFEE_REQUIRE(cache == nullptr || (token_segment != nullptr && block_tables != nullptr),
+               "gemm_qkv_rows: writing the cache needs block tables");
+  q.positions = positions; q.token_segment = token_segment; q.block_tables = block_tables;
+  q.bt_stride = bt_stride; q.cos_table = cos_table; q.sin_table = sin_table; q.half = half;
+  q.cache = cache; q.num_heads = num_heads;
+  return hfee_gemm_bf16_qkv(C, ldc, A, lda, W, ldw, M, N, K, &q, 0, stream);
 }

@@ -4,9 +4,12 @@ Two kinds of library:
   * `core`: every kernel whose sizes are run-time arguments;
   * `attention_bf16_hd<N>`: the matrix-core attention kernels, compiled for one head
     size each, on demand (a model compiles only the head size it has).
-Libraries are built in-tree (hfee_amd/_lib); if that folder cannot be written, in
-$HFEE_BUILD_DIR or a per-user folder under the system's temporary directory.
-A library is rebuilt when its sources or flags no longer match the stamp beside it.
+Libraries are built in-tree (hfee_amd/_lib); if that folder cannot be written, in a
+per-user folder under the system's temporary directory; $HFEE_BUILD_DIR, if set, comes
+before both.  A library is rebuilt when its sources or flags no longer match the stamp
+beside it.  $HFEE_EXTRA_FLAGS adds compiler flags (they are part of the stamp): together
+with $HFEE_BUILD_DIR that builds a variant beside the in-tree libraries, to measure one
+against the other.
 """
 from __future__ import annotations
 
@@ -28,7 +31,7 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fvisibility=h
          "-Wno-unused-command-line-argument"]
 
 CORE_SOURCES = ["elementwise.hip", "gemm_f32.hip", "attention_ref.hip", "gemm_bf16.hip", "gemm_skinny.hip",
-                "sampling.hip"]
+                "sampling.hip", "yardstick.hip"]
 ATTENTION_SOURCE = "attention_bf16.hip"
 HEAD_DIMS = tuple(range(16, 257, 16))
 
@@ -63,18 +66,23 @@ def _writable(path: str) -> bool:
         pass
 
 
+def extra_flags() -> list:
+    return os.environ.get("HFEE_EXTRA_FLAGS", "").split()
+
+
 def build_dirs() -> list:
     """Folders a library may live in, in the order they are searched."""
-    dirs = [IN_TREE]
+    dirs = []
     if os.environ.get("HFEE_BUILD_DIR"):
-        dirs.append(os.environ["HFEE_BUILD_DIR"])
+        dirs.append(os.path.abspath(os.environ["HFEE_BUILD_DIR"]))
+    dirs.append(IN_TREE)
     dirs.append(os.path.join(tempfile.gettempdir(), f"hfee_amd-{os.getuid()}", "_lib"))
     return dirs
 
 
 def _stamp(sources, defines) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS + sorted(defines)).encode())
+    h.update(" ".join(FLAGS + extra_flags() + sorted(defines)).encode())
     for name in sorted(set(sources) | {"common.h"} | {f for f in os.listdir(CSRC) if f.endswith(".h")}):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(name.encode() + b"\0" + f.read())
@@ -150,7 +158,7 @@ def build_library(name: str, force: bool = False) -> str:
     for src in sources:
         obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
         objs.append(obj)
-        cmds.append((src, [cc, *FLAGS, *defines, "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]))
+        cmds.append((src, [cc, *FLAGS, *extra_flags(), *defines, "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]))
     _run_with_heartbeat(cmds, name)
     so = os.path.join(out_dir, f"libhfee_{name}.so")
     tmp = so + f".{os.getpid()}.tmp"

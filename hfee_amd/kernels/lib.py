@@ -35,9 +35,12 @@ _CORE_SIGNATURES = {
     "hfee_gemm_bf16_plan": [I, I, I, P, P, P],
     "hfee_gemm_skinny": [P, L, P, I, L, P, L, I, I, I, I, P, I, F, P, P, P, P, I, P, P, I, I, P, I, I, I, I,
                          P, I, P, L, P, P, I, F, P, L, I, P],
+    "hfee_gemm_qkv_rows": [P, L, P, L, P, L, I, I, I, P, P, P, I, P, P, I, I, P, I, I, I, I, P],
     "hfee_argmax": [P, P, L, I, I, P, L, P, I, P],
     "hfee_sample": [P, P, L, I, I, P, P, P, P, L, P],
     "hfee_argmax_static": [P, P, L, I, I, P],
+    "hfee_read_stream": [P, L, P, I, I, P],
+    "hfee_mfma_loop": [P, I, I, P],
 }
 
 _ATTENTION_SIGNATURES = {

@@ -100,6 +100,23 @@ def residual_add(x: torch.Tensor, y: torch.Tensor):
     lib.core().call("hfee_residual_add", _ptr(x), _ptr(y), _dt(y), x.numel(), _stream())
 
 
+def read_stream(t: torch.Tensor, workgroups: int = 2048, keep_out_of_l2: bool = False):
+    """Reads every byte of t once and keeps nothing: the read-only yardstick of the memory,
+    and a prefetch (what is read stays in the memory-side cache for the kernel that comes
+    for it next; keep_out_of_l2 for a prefetch that runs beside another kernel)."""
+    _gpu(t)
+    _check(t.is_contiguous(), "read_stream: a contiguous tensor expected")
+    nbytes = t.numel() * t.element_size()
+    _check(nbytes % 16 == 0 and t.data_ptr() % 16 == 0, "read_stream: 16-byte alignment expected")
+    lib.core().call("hfee_read_stream", _ptr(t), nbytes, None, int(workgroups), int(keep_out_of_l2), _stream())
+
+
+def mfma_loop(iterations: int, workgroups: int) -> float:
+    """Launches a loop of nothing but bfloat16 matrix instructions; returns the flops it does."""
+    lib.core().call("hfee_mfma_loop", None, int(iterations), int(workgroups), _stream())
+    return float(workgroups) * 4 * iterations * 8 * 2 * 32 * 32 * 16
+
+
 # ---------------------------------------------------------------- matrix product
 
 def linear_scratch(m: int, n: int, k: int) -> int:
@@ -357,12 +374,37 @@ def norm_fusion_pays(n_rows: int, k: int) -> bool:
 _EPI = {"bf16": 0, "f32": 1, "add": 2, "swiglu": 3, "qkv": 4}
 
 
-def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether the streaming kernel takes this product (bfloat16 weight, aligned shapes)."""
-    K = weight.shape[1]
-    return (weight.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and K % 8 == 0
-            and weight.stride(0) % 8 == 0 and x.stride(0) % 8 == 0
-            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+class TiledWeight:
+    """A bfloat16 weight [n, k] in tiles of 16 rows x 32 columns, the form that the products of
+    up to 64 rows stream (`linear_fused`): a tile is a kilobyte in the order in which a wave
+    holds it as a matrix operand ([column group of 8][row][8 columns]), the tiles of 16 rows
+    follow one another along k, and n and k are filled up with zeros to whole tiles."""
+
+    def __init__(self, tiles: torch.Tensor, n: int, k: int):
+        self.tiles, self.n, self.k = tiles, n, k
+        self.row_stride = ((k + 31) // 32) * 512          # elements from one row of tiles to the next
+
+    @property
+    def shape(self):
+        return (self.n, self.k)
+
+    def rows(self) -> torch.Tensor:
+        """The weight as rows again, [n, k] (for tests)."""
+        nt, kt = self.tiles.shape[0], self.tiles.shape[1]
+        return self.tiles.view(nt, kt, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nt * 16, kt * 32)[:self.n, :self.k]
+
+
+def tile_weight(weight: torch.Tensor) -> TiledWeight:
+    """weight [n, k] bfloat16 (rows as they lie in a checkpoint) -> the same in tiles."""
+    _check(weight.dim() == 2 and weight.dtype == torch.bfloat16, "tile_weight: a 2-D bfloat16 weight expected")
+    n, k = weight.shape
+    nt, kt = (n + 15) // 16, (k + 31) // 32
+    if nt * 16 != n or kt * 32 != k:
+        padded = torch.zeros((nt * 16, kt * 32), dtype=weight.dtype, device=weight.device)
+        padded[:n, :k] = weight
+        weight = padded
+    tiles = weight.view(nt, 16, kt, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(nt, kt, 512)
+    return TiledWeight(tiles, n, k)
 
 
 SS_STRIDE = 64     # rows of a table of sum-of-squares shares (one row of the table per 16 weight rows)
@@ -378,8 +420,9 @@ def mid_rows_scratch(n_rows: int, n_weight_rows: int, k: int) -> int:
 
 def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0.0, rows=None, m=None, qkv=None,
                  emit=None, row_scale=None, scratch=None, force_mid_rows=False):
-    """out = epilogue(norm(x) @ weight.T) in one launch, for at most 64 rows ("qkv": any
-    number of rows; more than 64 take the tiled kernels with the same epilogue).
+    """out = epilogue(norm(x) @ weight.T) in one launch, for at most 64 rows; weight: a
+    `TiledWeight`.  ("qkv" with a weight as rows [N, K]: any number of rows, through the tiled
+    kernels with the same epilogue; nothing else is fused there.)
 
     emit (with "add"): dict(weight, out, shares): the norm that follows the residual add, in
     two halves: this product also writes bfloat16(out_new * weight) to emit["out"] [M, N] and
@@ -397,12 +440,18 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
     alternate gate/up; out [M, N/2]) | "qkv" (rotation + cache write; see
     parts/attention.py; qkv = dict(positions, token_segment, block_tables, cos, sin,
     cache_layer, num_heads, kv_heads, head_dim, page_size))."""
-    _gpu(out, x, weight, norm_weight, rows)
-    N, K, ldw = _rows2d(weight, "linear_fused weight")
+    if not isinstance(weight, TiledWeight):
+        _check(epilogue == "qkv" and norm_weight is None and emit is None and row_scale is None,
+               "linear_fused: the weight must be a TiledWeight (ops.tile_weight); only the plain q/k/v product "
+               "takes a weight as rows")
+        return _qkv_rows(out, x, weight, qkv)
+    _gpu(out, x, weight.tiles, norm_weight, rows)
+    N, K, ldw = weight.n, weight.k, weight.row_stride
     Mx, Kx, lda = _rows2d(x, "linear_fused x")
     M = Mx if m is None else m
     _check(Kx == K, "linear_fused: inner sizes differ")
-    _check(weight.dtype == torch.bfloat16, "linear_fused: bfloat16 weight expected")
+    _check(M <= SKINNY_MAX_ROWS, f"linear_fused: at most {SKINNY_MAX_ROWS} rows, got {M}")
+    weight = weight.tiles
     fused_norm = norm_weight is not None
     if fused_norm:
         _check(x.dtype == torch.float32 and M <= FUSED_NORM_MAX_ROWS, "linear_fused: the fused norm takes <= 16 float32 rows")
@@ -467,3 +516,29 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
     lib.core().call("hfee_gemm_skinny", _ptr(out), ldc, _ptr(x), int(fused_norm), lda, _ptr(weight), ldw, M, N, K, epi,
                     _ptr(norm_weight), int(fused_norm and norm_weight.dtype == torch.float32), float(eps), _ptr(rows),
                     None, None, None, 0, None, None, 0, 0, None, 0, 0, 0, 0, *e_args, *s_args, *w_args, _stream())
+
+
+def _qkv_rows(out, x, weight, q):
+    """The q/k/v product with rotation and cache write for a weight as rows [N, K]."""
+    _gpu(out, x, weight)
+    N, K, ldw = _rows2d(weight, "linear_fused weight")
+    M, Kx, lda = _rows2d(x, "linear_fused x")
+    Mo, No, ldc = _rows2d(out, "linear_fused out")
+    _check(Kx == K and Mo >= M, "linear_fused: shapes")
+    _check(x.dtype == weight.dtype == out.dtype == torch.bfloat16, "linear_fused: bfloat16 tensors expected")
+    H, KV, hd, ps = q["num_heads"], q["kv_heads"], q["head_dim"], q["page_size"]
+    _check(N == (H + 2 * KV) * hd and No == H * hd, "linear_fused: q/k/v shapes")
+    cache = q.get("cache_layer")
+    if cache is not None:
+        _check(cache.is_contiguous() and tuple(cache.shape[1:]) == (2, KV, ps * hd) and cache.dtype == torch.bfloat16,
+               "linear_fused: cache layer shape")
+        _i32(q["token_segment"], "linear_fused token_segment", M)
+        bt = q["block_tables"]
+        _check(bt.dtype == torch.int32 and bt.dim() == 2 and bt.stride(1) == 1, "linear_fused: block tables")
+    _i32(q["positions"], "linear_fused positions", M)
+    cos, sin = q.get("cos"), q.get("sin")
+    half, table_positions = (cos.shape[1], cos.shape[0]) if cos is not None else (0, 0)
+    bt = q.get("block_tables")
+    lib.core().call("hfee_gemm_qkv_rows", _ptr(out), ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K,
+                    _ptr(q["positions"]), _ptr(q.get("token_segment")), _ptr(bt), 0 if bt is None else bt.stride(0),
+                    _ptr(cos), _ptr(sin), half, table_positions, _ptr(cache), H, KV, hd, ps, _stream())

@@ -88,6 +88,11 @@ class Attention(Mixer):
         self.w_qkv = torch.cat([wq, wk, tensors.pop(p + "v_proj.weight")], dim=0).contiguous()
         self.w_o = tensors.pop(p + "o_proj.weight").contiguous()
         self.pairing = 1          # pairs are (2i, 2i + 1) from here on
+        # a second copy in tiles for steps of up to 64 rows, whose products stream the weights
+        # (as rows they serve the tiled products of longer portions)
+        self.streams = self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.q_width % 8 == 0
+        self.w_qkv_tiles = ops.tile_weight(self.w_qkv) if self.streams else None
+        self.w_o_tiles = ops.tile_weight(self.w_o) if self.streams else None
 
     def key_layout(self):
         """What two layers must share to read one cache layer."""
@@ -141,7 +146,7 @@ class Attention(Mixer):
         # as a kernel of its own, spread over the whole chip, measured faster than as the
         # tail of 256 x 256 tiles with one wave a SIMD: 135 us against 156 us a layer at
         # 2,048 rows)
-        fused = self.dtype == torch.bfloat16 and n <= ops.SKINNY_MAX_ROWS and self.hidden % 8 == 0
+        fused = self.streams and n <= ops.SKINNY_MAX_ROWS
         qkv = ctx.rows("attention.qkv", self.q_width + 2 * self.kv_width)
         q = qkv[:, :self.q_width]
         if fused:
@@ -151,12 +156,12 @@ class Attention(Mixer):
             norm = h.fusable() if (halves is None and few and isinstance(h, LazyNorm)
                                    and ops.norm_fusion_pays(*self.w_qkv.shape)) else None
             a = halves[0] if halves else h.x if norm else (h.tensor() if isinstance(h, LazyNorm) else h)
-            ops.linear_fused(q, a, self.w_qkv, "qkv", norm_weight=norm[0] if norm else None,
+            ops.linear_fused(q, a, self.w_qkv_tiles, "qkv", norm_weight=norm[0] if norm else None,
                              eps=norm[1] if norm else 0.0, row_scale=halves[1] if halves else None,
                              qkv=dict(positions=ctx.positions, token_segment=ctx.token_segment, block_tables=tables,
                                       cos=cos, sin=sin, cache_layer=cache if writes_cache else None,
                                       num_heads=H, kv_heads=K, head_dim=hd, page_size=ctx.page_size),
-                             **ctx.workspace.product_scratch(n, self.w_qkv))
+                             **ctx.workspace.product_scratch(n, self.w_qkv_tiles))
         else:
             hn = h.tensor() if isinstance(h, LazyNorm) else h
             if writes_cache:
@@ -197,11 +202,8 @@ class Attention(Mixer):
                                           None if in_order else ctx.extra["attention.decode_tables"], tables, H, K, hd,
                                           ctx.page_size, self.scale, self.window, partial, splits, _DECODE_WAVES,
                                           counters)
-        emit = None
-        if then is not None and self.dtype == torch.bfloat16 and n <= ops.SKINNY_MAX_ROWS \
-                and self.hidden % 8 == 0 and self.q_width % 8 == 0:
-            emit = then.offer()
-        if emit:       # the output projection adds into x and begins the norm that follows
-            ops.linear_fused(x, att, self.w_o, "add", emit=emit, **ctx.workspace.product_scratch(n, self.w_o))
+        if fused:      # the output projection adds into x and, if asked, begins the norm that follows
+            emit = then.offer() if then is not None else None
+            ops.linear_fused(x, att, self.w_o_tiles, "add", emit=emit, **ctx.workspace.product_scratch(n, self.w_o_tiles))
         else:
             ops.linear(x, att, self.w_o, accumulate=True, **ctx.workspace.split_scratch(n, self.w_o))

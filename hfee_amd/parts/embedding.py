@@ -59,14 +59,21 @@ class Head(Part):
     def bind(self, tensors):
         self.norm.bind(tensors)
         self.weight = tensors[self.name].contiguous() if self.name is not None else self.embedding.table
+        # a second copy in tiles for up to 64 wanted rows, whose product streams the weights
+        self.streams = self.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.hidden % 8 == 0
+        self.weight_tiles = ops.tile_weight(self.weight) if self.streams else None
 
     def forward(self, ctx, logits, x, rows):
         """logits[i] = head(norm(x[rows[i]])); logits float32 [len(rows), vocab]."""
         w = logits.shape[0]
         fused = getattr(self.norm, "fused_form", lambda: None)()
-        if (fused and self.dtype == torch.bfloat16 and w <= ops.FUSED_NORM_MAX_ROWS and self.hidden % 8 == 0
-                and self.weight.dtype == torch.bfloat16 and ops.norm_fusion_pays(self.vocab, self.hidden)):
-            ops.linear_fused(logits, x, self.weight, "f32", norm_weight=fused[0], eps=fused[1], rows=rows, m=w)
+        if self.streams and w <= ops.SKINNY_MAX_ROWS:
+            if fused and w <= ops.FUSED_NORM_MAX_ROWS and ops.norm_fusion_pays(self.vocab, self.hidden):
+                ops.linear_fused(logits, x, self.weight_tiles, "f32", norm_weight=fused[0], eps=fused[1], rows=rows, m=w)
+                return
+            normed = ctx.rows("head.normed", self.hidden, n=w)
+            self.norm.forward(ctx, normed, x, rows)
+            ops.linear_fused(logits, normed, self.weight_tiles, "f32", **ctx.workspace.product_scratch(w, self.weight_tiles))
             return
         normed = ctx.rows("head.normed", self.hidden, n=w)
         self.norm.forward(ctx, normed, x, rows)

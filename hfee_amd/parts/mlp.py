@@ -40,33 +40,38 @@ class GatedMLP(FeedForward):
         self.w_gate_up = torch.stack([tensors.pop(p + "gate_proj.weight"), tensors.pop(p + "up_proj.weight")],
                                      dim=1).reshape(2 * self.intermediate, self.hidden).contiguous()
         self.w_down = tensors.pop(p + "down_proj.weight").contiguous()
+        # a second copy in tiles for steps of up to 64 rows, whose products stream the weights
+        self.streams = self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.intermediate % 8 == 0
+        self.w_gate_up_tiles = ops.tile_weight(self.w_gate_up) if self.streams else None
+        self.w_down_tiles = ops.tile_weight(self.w_down) if self.streams else None
 
     def forward_add(self, ctx, x, h, then=None):
-        F = self.intermediate
+        F, n = self.intermediate, ctx.n
         act = ctx.rows("mlp.act", F)
-        aligned = self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and F % 8 == 0
-        few = ctx.n <= ops.FUSED_NORM_MAX_ROWS
-        halves = h.row_scale() if (aligned and isinstance(h, LazyNorm)) else None      # (offered for few rows only)
-        norm = None
-        if halves is None and aligned and few and isinstance(h, LazyNorm) and ops.norm_fusion_pays(*self.w_gate_up.shape):
-            norm = h.fusable()
-        if halves:        # the norm's first half came with the product before; both projections and the gate
-            ops.linear_fused(act, halves[0], self.w_gate_up, "swiglu", row_scale=halves[1], **ctx.workspace.product_scratch(ctx.n, self.w_gate_up))
-        elif norm:        # norm, both projections and the gate in one launch
-            ops.linear_fused(act, h.x, self.w_gate_up, "swiglu", norm_weight=norm[0], eps=norm[1])
-        else:
-            hn = h.tensor() if isinstance(h, LazyNorm) else h
-            if aligned:   # the gate in the product's epilogue
-                ops.linear(act, hn, self.w_gate_up, gate=True)
+        aligned = self.streams
+        lazy = isinstance(h, LazyNorm)
+        if aligned and n <= ops.SKINNY_MAX_ROWS:        # both products stream the weights' tiles
+            w = self.w_gate_up_tiles
+            halves = h.row_scale() if lazy else None     # (offered for few rows only)
+            norm = None
+            if halves is None and lazy and n <= ops.FUSED_NORM_MAX_ROWS and ops.norm_fusion_pays(*w.shape):
+                norm = h.fusable()
+            if halves:        # the norm's first half came with the product before; both projections and the gate
+                ops.linear_fused(act, halves[0], w, "swiglu", row_scale=halves[1], **ctx.workspace.product_scratch(n, w))
+            elif norm:        # norm, both projections and the gate in one launch
+                ops.linear_fused(act, h.x, w, "swiglu", norm_weight=norm[0], eps=norm[1])
             else:
-                gate_up = ctx.rows("mlp.gate_up", 2 * F)
-                ops.linear(gate_up, hn, self.w_gate_up)
-                ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
-        n = ctx.n
-        emit = then.offer() if (then is not None and aligned and n <= ops.SKINNY_MAX_ROWS) else None
-        if emit:          # the down projection adds into x and begins the norm that follows
-            ops.linear_fused(x, act, self.w_down, "add", emit=emit, **ctx.workspace.product_scratch(n, self.w_down))
-        elif aligned and ops.FUSED_NORM_MAX_ROWS < n <= ops.SKINNY_MAX_ROWS:
-            ops.linear_fused(x, act, self.w_down, "add", **ctx.workspace.product_scratch(n, self.w_down))
+                ops.linear_fused(act, h.tensor() if lazy else h, w, "swiglu", **ctx.workspace.product_scratch(n, w))
+            # the down projection adds into x and, if asked, begins the norm that follows
+            emit = then.offer() if then is not None else None
+            ops.linear_fused(x, act, self.w_down_tiles, "add", emit=emit,
+                             **ctx.workspace.product_scratch(n, self.w_down_tiles))
+            return
+        hn = h.tensor() if lazy else h
+        if aligned:   # the gate in the product's epilogue
+            ops.linear(act, hn, self.w_gate_up, gate=True)
         else:
-            ops.linear(x, act, self.w_down, accumulate=True, **ctx.workspace.split_scratch(n, self.w_down))
+            gate_up = ctx.rows("mlp.gate_up", 2 * F)
+            ops.linear(gate_up, hn, self.w_gate_up)
+            ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
+        ops.linear(x, act, self.w_down, accumulate=True, **ctx.workspace.split_scratch(n, self.w_down))

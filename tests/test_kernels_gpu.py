@@ -201,8 +201,27 @@ def test_gemm_bf16_over_two_launches():
     assert ops.tiled_plan(2048, 4096, 4096)[2] == 0 and ops.tiled_plan(2048, 4096, 14336)[2] == 0
 
 
+def test_weights_in_tiles():
+    """tile_weight lays [n, k] out in kilobytes of 16 rows x 32 columns, each in the order
+    [column group of 8][row][8 columns], the tiles of 16 rows one after the other along k; n
+    and k are filled up with zeros; rows() gives the weight back."""
+    from hfee_amd.kernels import ops
+    for n, k in ((16, 32), (48, 96), (50, 40), (7, 8), (33, 200)):
+        w = torch.arange(n * k, dtype=torch.float32).reshape(n, k).to(torch.bfloat16).to(DEV)
+        t = ops.tile_weight(w)
+        nt, kt = (n + 15) // 16, (k + 31) // 32
+        assert t.tiles.shape == (nt, kt, 512) and t.shape == (n, k) and t.row_stride == kt * 512
+        assert torch.equal(t.rows(), w)
+        flat = t.tiles.cpu()
+        for row, col in ((0, 0), (n - 1, k - 1), (n // 2, k // 3), (min(17, n - 1), min(33, k - 1))):
+            lane = 16 * ((col % 32) // 8) + row % 16              # the lane that holds it, and where in its 16 bytes
+            assert flat[row // 16, col // 32, lane * 8 + col % 8] == w[row, col].cpu()
+        assert float(flat.float().abs().sum()) == float(w.float().abs().sum())      # the filling is zeros
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (8, 344, 96), (16, 100, 256), (3, 16400, 1024), (16, 16500, 2048),
-                                   (5, 17000, 4096), (2, 16390, 3072), (33, 200, 128), (64, 52, 1024)])
+                                   (5, 17000, 4096), (2, 16390, 3072), (33, 200, 128), (64, 52, 1024),
+                                   (7, 50, 40), (12, 107, 200), (4, 20, 8), (9, 6144, 512)])
 @pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu"])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_decode_products(M, N, K, epilogue, norm):
@@ -237,9 +256,9 @@ def test_fused_decode_products(M, N, K, epilogue, norm):
     else:
         out = torch.zeros(M, N, dtype=torch.bfloat16 if epilogue == "bf16" else torch.float32, device=DEV)
     if norm:
-        ops.linear_fused(out, xs.to(DEV), w.to(DEV), epilogue, norm_weight=nw.to(DEV), eps=1e-5, rows=rows.to(DEV), m=M)
+        ops.linear_fused(out, xs.to(DEV), ops.tile_weight(w.to(DEV)), epilogue, norm_weight=nw.to(DEV), eps=1e-5, rows=rows.to(DEV), m=M)
     else:
-        ops.linear_fused(out, x.to(DEV), w.to(DEV), epilogue)
+        ops.linear_fused(out, x.to(DEV), ops.tile_weight(w.to(DEV)), epilogue)
     tol = 2e-2 if epilogue in ("bf16", "swiglu") or norm else 1e-5
     err = (out.double().cpu() - ref).abs()
     assert (err <= tol * (1 + mag)).all(), float((err / (1 + mag)).max())
@@ -270,7 +289,7 @@ def test_products_of_17_to_64_rows(M, N, K, epilogue):
             want = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
             bound = 2e-2 * (mag[:, 0::2] + 1) * (mag[:, 1::2] + 1)
             out = torch.zeros(M, N // 2, dtype=torch.bfloat16, device=DEV)
-            ops.linear_fused(out, x.to(DEV), w.to(DEV), "swiglu", **kw)
+            ops.linear_fused(out, x.to(DEV), ops.tile_weight(w.to(DEV)), "swiglu", **kw)
         elif epilogue in ("add", "emit"):
             want, bound = ref + c0.double(), 1e-5 * (1 + mag + c0.abs().double())
             out = c0.clone().to(DEV)
@@ -280,7 +299,7 @@ def test_products_of_17_to_64_rows(M, N, K, epilogue):
                 emitted = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
                 shares = torch.zeros(((N + 15) // 16) * 64, dtype=torch.float32, device=DEV)
                 emit = dict(weight=nw.to(DEV), out=emitted, shares=shares)
-            ops.linear_fused(out, x.to(DEV), w.to(DEV), "add", emit=emit, **kw)
+            ops.linear_fused(out, x.to(DEV), ops.tile_weight(w.to(DEV)), "add", emit=emit, **kw)
             if emit:
                 close(emitted, want * nw.double(), 1e-2)
                 got = shares.view(-1, 64)[:, :M].double().sum(0).cpu()
@@ -292,11 +311,11 @@ def test_products_of_17_to_64_rows(M, N, K, epilogue):
             scale = 1 / torch.sqrt(shares.view(blocks, 64)[:, :M].double().sum(0) / K + 1e-5)
             want, bound = ref * scale[:, None], 2e-2 * (1 + mag * scale[:, None])
             out = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
-            ops.linear_fused(out, x.to(DEV), w.to(DEV), "bf16", row_scale=dict(shares=shares.to(DEV), blocks=blocks, eps=1e-5), **kw)
+            ops.linear_fused(out, x.to(DEV), ops.tile_weight(w.to(DEV)), "bf16", row_scale=dict(shares=shares.to(DEV), blocks=blocks, eps=1e-5), **kw)
         else:
             want, bound = ref, (2e-2 if epilogue == "bf16" else 1e-5) * (1 + mag)
             out = torch.zeros(M, N, dtype=torch.bfloat16 if epilogue == "bf16" else torch.float32, device=DEV)
-            ops.linear_fused(out, x.to(DEV), w.to(DEV), epilogue, **kw)
+            ops.linear_fused(out, x.to(DEV), ops.tile_weight(w.to(DEV)), epilogue, **kw)
         err = (out.double().cpu() - want).abs()
         assert (err <= bound).all(), float((err / bound).max())
 
@@ -326,7 +345,7 @@ def test_norm_in_two_halves(M, N, K, N2, epilogue2):
     emitted = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
     blocks = (N + 15) // 16
     shares = torch.full((blocks * 64,), float("nan"), dtype=torch.float32, device=DEV)
-    ops.linear_fused(x, a.to(DEV), w1.to(DEV), "add", emit=dict(weight=nw.to(DEV), out=emitted, shares=shares))
+    ops.linear_fused(x, a.to(DEV), ops.tile_weight(w1.to(DEV)), "add", emit=dict(weight=nw.to(DEV), out=emitted, shares=shares))
     err = (x.double().cpu() - x1).abs()
     assert (err <= 1e-5 * (1 + x0.abs().double() + a.abs().double() @ w1.abs().double().t())).all()
     got_ss = shares.view(blocks, 64)[:, :M].double().sum(0).cpu()
@@ -344,7 +363,7 @@ def test_norm_in_two_halves(M, N, K, N2, epilogue2):
         ref = ref + c0.double()
     else:
         out = torch.zeros(M, N2, dtype=torch.bfloat16, device=DEV)
-    ops.linear_fused(out, emitted, w2.to(DEV), epilogue2, row_scale=scale)
+    ops.linear_fused(out, emitted, ops.tile_weight(w2.to(DEV)), epilogue2, row_scale=scale)
     err = (out.double().cpu() - ref).abs()
     assert (err <= 2e-2 * (1 + mag)).all(), float((err / (1 + mag)).max())
 
@@ -398,7 +417,7 @@ def _check_fused_qkv(H, K, hd, half, M, norm, d, **kw):
     k_ref[..., :2 * half] = plain_rope(k_ref[..., :2 * half], pos.tolist(), inv, "interleaved")
     layer = torch.zeros(M * 4, 2, K, ps * hd, dtype=torch.bfloat16, device=DEV)
     q_out = torch.zeros(M, H * hd, dtype=torch.bfloat16, device=DEV)
-    ops.linear_fused(q_out, x.to(DEV), w.to(DEV), "qkv", norm_weight=nw.to(DEV) if norm else None, eps=1e-6,
+    ops.linear_fused(q_out, x.to(DEV), ops.tile_weight(w.to(DEV)) if M <= 64 else w.to(DEV), "qkv", norm_weight=nw.to(DEV) if norm else None, eps=1e-6,
                      qkv=dict(positions=pos.to(DEV), token_segment=seg.to(DEV), block_tables=tables.to(DEV), cos=cos, sin=sin,
                               cache_layer=layer, num_heads=H, kv_heads=K, head_dim=hd, page_size=ps), **kw)
     close(q_out, q_ref.reshape(M, H * hd), 2e-2)
@@ -822,12 +841,12 @@ def test_only_finite_numbers_reach_the_cache(M):
                head_dim=hd, page_size=ps)
     q_out = torch.zeros(M, H * hd, dtype=torch.bfloat16, device=DEV)
     layer = fresh()
-    ops.linear_fused(q_out, x, w, "qkv", qkv=dict(qkv, cache_layer=layer))      # streaming up to 64 rows, tiled beyond
+    ops.linear_fused(q_out, x, ops.tile_weight(w) if M <= 64 else w, "qkv", qkv=dict(qkv, cache_layer=layer))      # streaming up to 64 rows, tiled beyond
     check(layer, "q/k/v epilogue")
     if 16 < M <= 64:
         layer = fresh()
         scratch = torch.zeros(ops.mid_rows_scratch(M, N, d), dtype=torch.float32, device=DEV)
-        ops.linear_fused(q_out, x, w, "qkv", qkv=dict(qkv, cache_layer=layer), scratch=scratch, force_mid_rows=True)
+        ops.linear_fused(q_out, x, ops.tile_weight(w), "qkv", qkv=dict(qkv, cache_layer=layer), scratch=scratch, force_mid_rows=True)
         check(layer, "q/k/v epilogue with the batch in LDS")
     y = plain_y.clone()
     for pairing in (1, 0):          # the kernel for adjacent pairs (values of 16 tokens together from 32 rows on); the general one
