@@ -145,11 +145,24 @@ __device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyO
   const int lane = threadIdx.x & 63, G = lane >> 5;
 
   // ---- S^T = K Q^T ------------------------------------------------------------
+  // All key operands are asked for before the first product, and all value operands behind
+  // them, before the exponentials: where they come from LDS, a read takes a hundred cycles
+  // and more to arrive, and read two at a time between the products, as the compiler
+  // orders them on its own, every pair's latency stood in the chain.
   f32x16 s;
 #pragma unroll
   for (int r = 0; r < 16; ++r) s[r] = 0.f;
+  bf16x8 k_ops[NC];
 #pragma unroll
-  for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(key_op(c), q_op[c].v, s, 0, 0, 0);
+  for (int c = 0; c < NC; ++c) k_ops[c] = key_op(c);
+  bf16x8 v_ops[2][NDT];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int t = 0; t < NDT; ++t) v_ops[u][t] = value_op(u, t);
+  __builtin_amdgcn_sched_barrier(0);          // (the reads stay in front of the products)
+#pragma unroll
+  for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_ops[c], q_op[c].v, s, 0, 0, 0);
 
   // ---- mask, running maximum and sum ------------------------------------------
   // all_visible (the same for the whole wave): every key of the tile is visible to every
@@ -208,7 +221,7 @@ __device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyO
   for (int u = 0; u < 2; ++u)
 #pragma unroll
     for (int t = 0; t < NDT; ++t)
-      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(value_op(u, t), p[u].v, st.o[t], 0, 0, 0);
+      st.o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_ops[u][t], p[u].v, st.o[t], 0, 0, 0);
 }
 
 __device__ __forceinline__ void compute_tile(Tile& st, const Op* q_op, const TileOps& ops, int k0, int pos, int lo,
@@ -344,6 +357,11 @@ __global__ __launch_bounds__(64) void prefill_kernel(bf16_t* __restrict__ out, i
 // but finite numbers, so a masked value times zero is zero).
 constexpr int KV_BLOCKS = NC + 2 * NDT;           // 1 KB blocks of one key tile: keys, then values
 constexpr int SHARED_WAVES = 4;
+// key tiles of LDS where loads are waited for by count: four (three of them on their way) where
+// two workgroups of four tiles fit a CU's 160 KB (head sizes up to 128: 16 KB a tile), else three
+// (prefill attention of the 8B shape, 2,048 tokens: 67.6 us a layer with three, 65.0 with four)
+constexpr int SHARED_TILES = HD <= 128 ? 4 : 3;
+static_assert(SHARED_TILES == 3 || SHARED_TILES == 4, "the waits are written for three or four tiles");
 
 __device__ __forceinline__ void request_tile(char* __restrict__ tile_lds, const bf16_t* __restrict__ cache,
                                              const CacheLayout& lay, const LaneOffsets& off,
@@ -422,11 +440,15 @@ __device__ __forceinline__ WaveBlocks<WAVES> wave_blocks(const CacheLayout& lay,
   return w;
 }
 
-template <int WAVES>
+// BUFFER: the loads are buffer loads over the whole cache layer (which must be smaller than
+// 4 GB: a lane's place is 32 bits from the layer's start).  The compiler does not connect
+// them with the reads of the LDS that follow, as it does the global loads into LDS, before
+// which it waits for every load in flight: the caller waits by count (and must).
+template <int WAVES, bool BUFFER>
 __device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds, const bf16_t* __restrict__ cache,
-                                                    const CacheLayout& lay, const WaveBlocks<WAVES>& w,
-                                                    const int* __restrict__ bt, int bt_stride, PageWindow& pages,
-                                                    int k0, int kv_first, int kv_last, int wave) {
+                                                    __amdgpu_buffer_rsrc_t rsrc, const CacheLayout& lay,
+                                                    const WaveBlocks<WAVES>& w, const int* __restrict__ bt, int bt_stride,
+                                                    PageWindow& pages, int k0, int kv_first, int kv_last, int wave) {
   typedef __attribute__((address_space(3))) void* lds_ptr;
   typedef const __attribute__((address_space(1))) void* global_ptr;
   const int block_a = k0 >> lay.page_shift, block_b = (k0 + 16) >> lay.page_shift;
@@ -447,19 +469,37 @@ __device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds,
 #pragma unroll
   for (int j = 0; j < WaveBlocks<WAVES>::J; ++j) {
     if (KV_BLOCKS % WAVES == 0 || j < w.count) {
-      const uint64_t page_bytes = ((uint64_t)(w.second[j] ? b_hi : a_hi) << 32) | (w.second[j] ? b_lo : a_lo);
-      const char* src = (const char*)cache + page_bytes + (w.lane_off[j] + (w.kind[j] == 0 ? add[0] : w.kind[j] == 1 ? add[1] : add[2]));
-      __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)(tile_lds + (wave + WAVES * j) * 1024), 16, 0, 0);
+      const uint32_t in_layer = w.lane_off[j] + (w.kind[j] == 0 ? add[0] : w.kind[j] == 1 ? add[1] : add[2]);
+      if constexpr (BUFFER) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr)(tile_lds + (wave + WAVES * j) * 1024), 16,
+                                                 (w.second[j] ? b_lo : a_lo) + in_layer, 0, 0, 0);
+      } else {
+        const uint64_t page_bytes = ((uint64_t)(w.second[j] ? b_hi : a_hi) << 32) | (w.second[j] ? b_lo : a_lo);
+        const char* src = (const char*)cache + page_bytes + in_layer;
+        __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)(tile_lds + (wave + WAVES * j) * 1024), 16, 0, 0);
+      }
     }
   }
 }
 
+// The operand of s_waitcnt that waits until at most n vector memory operations are outstanding
+// and for nothing else (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
+constexpr int vmcnt_only(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+
 // work: per row tile 4 ints (first row, rows <= 32, first position, block-table row).
 // WAVES: the waves of a workgroup if they are SHARED_WAVES, 0 for any other number.
-template <int WAVES>
-__global__ __launch_bounds__(SHARED_WAVES * 64) void prefill_shared_kernel(
+// RING: key tiles come through buffer loads (layer_bytes < 4 GB) into a ring of SHARED_TILES
+// tiles of LDS and are waited for by count (WAVES must divide a tile's blocks).
+// (At most 256 registers a lane, so that two workgroups share a CU and take turns at the
+// matrix pipe; without the second number the compiler took 262 with the accumulators in the
+// other half of the register file, one workgroup a CU and a hundred moves between the halves
+// a step.  History of this kernel at the 8B shape, 2,048 tokens, us a layer: 85 with one tile
+// ahead behind a fence; 81.5 with the ring; 71.5 within 256 registers; 67.6 with a tile's
+// sixteen operand reads in front of its products; 65.0 with four tiles.)
+template <int WAVES, bool RING>
+__global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
-    const bf16_t* __restrict__ cache, CacheLayout lay, const int* __restrict__ work, int num_tiles,
+    const bf16_t* __restrict__ cache, uint32_t layer_bytes, CacheLayout lay, const int* __restrict__ work, int num_tiles,
     const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2, int window) {
   extern __shared__ __attribute__((aligned(1024))) char kv_lds[];     // two tiles of KV_BLOCKS KB
   const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
@@ -500,21 +540,67 @@ __global__ __launch_bounds__(SHARED_WAVES * 64) void prefill_shared_kernel(
   constexpr int TILE_BYTES = KV_BLOCKS * 1024;
   const LaneOffsets off = lane_offsets(lay, kvh);
   const WaveBlocks<WAVES == 0 ? 1 : WAVES> mine = wave_blocks<WAVES == 0 ? 1 : WAVES>(lay, kvh, wave);
-  auto request = [&](int t) {
-    char* dst = kv_lds + ((t - t_first) & 1) * TILE_BYTES;
-    if constexpr (WAVES != 0) request_wave_blocks<WAVES>(dst, cache, lay, mine, bt, bt_stride, pages, t * 32, kv_first, kv_last, wave);
-    else request_tile(dst, cache, lay, off, bt, bt_stride, pages, t * 32, kv_first, kv_last, wave, waves);
-  };
-  request(t_first);
-  __syncthreads();               // waits for the loads too
-  for (int t = t_first; t < t_end; ++t) {
-    const char* cur = kv_lds + ((t - t_first) & 1) * TILE_BYTES + lane * 16;
-    if (t + 1 < t_end) request(t + 1);
+  // (a raw buffer of 32-bit data over the layer; only the ring's loads go through it)
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cache, 0, (int)layer_bytes, 0x00020000);
+  auto compute = [&](int t, const char* tile_at) {
+    const char* cur = tile_at + lane * 16;
     compute_tile_with(
         st, q_op, [&](int c) { return *reinterpret_cast<const bf16x8*>(cur + c * 1024); },
         [&](int u, int tt) { return *reinterpret_cast<const bf16x8*>(cur + (NC + u * NDT + tt) * 1024); }, t * 32, pos, lo,
         scale_log2, t * 32 >= all_first && t * 32 + 31 <= pos0);
-    __syncthreads();             // the next tile has landed; nobody reads this one any more
+  };
+  if constexpr (RING) {
+    // Every wave brings the same number of blocks of a tile, so a wave can wait for its loads by
+    // count: SHARED_TILES tiles of LDS, all but one of them on their way.  The keys come from the
+    // L2, whose latency is as long as a tile takes to multiply.  (With global loads into LDS the
+    // compiler puts a wait for every load in flight in front of the first read of LDS that
+    // follows them, so that every step waited for the tile it had just asked for.)
+    static_assert(WAVES != 0 && KV_BLOCKS % (WAVES == 0 ? 1 : WAVES) == 0, "a wave's loads of a tile must be a fixed number");
+    constexpr int W = WAVES == 0 ? 1 : WAVES, MINE = KV_BLOCKS / W;     // loads a wave issues for a tile
+    auto request = [&](int t) {
+      request_wave_blocks<W, true>(kv_lds + ((t - t_first) % SHARED_TILES) * TILE_BYTES, cache, rsrc, lay, mine, bt, bt_stride,
+                                   pages, t * 32, kv_first, kv_last, wave);
+    };
+    // Nothing is on its way when the loop begins but what the loop itself asks for: the compiler
+    // keeps count of the loads whose registers it knows (the queries'), and one of those in
+    // flight across the loop's edge makes it wait, in front of every product, until only the
+    // loads of that very step are outstanding, which is one tile ahead again and no more.
+    request(t_first);
+    if (t_first + 1 < t_end) request(t_first + 1);
+    if (SHARED_TILES == 4 && t_first + 2 < t_end) request(t_first + 2);
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    for (int t = t_first; t < t_end; ++t) {
+      // this wave's blocks of tile t have landed (those of the tiles after it may still be on their way) ...
+      const int behind = min(SHARED_TILES - 2, t_end - 1 - t);          // tiles asked for after tile t
+      // (the wait is the compiler's own builtin, not text it cannot read: it then knows that
+      // the loads of before the loop, the queries, have arrived, and does not wait for them,
+      // and with them for every load behind them, in front of every product)
+      if (behind >= 2) __builtin_amdgcn_s_waitcnt(vmcnt_only(2 * MINE));
+      else if (behind == 1) __builtin_amdgcn_s_waitcnt(vmcnt_only(MINE));
+      else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+      // ... and after the barrier everybody's have, and nobody reads tile t - 1 any more, whose
+      // place the next request takes.  (No fence: it would wait for every load in flight.)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (t + SHARED_TILES - 1 < t_end) request(t + SHARED_TILES - 1);
+      compute(t, kv_lds + ((t - t_first) % SHARED_TILES) * TILE_BYTES);
+    }
+  } else {
+    auto request = [&](int t) {
+      char* dst = kv_lds + ((t - t_first) & 1) * TILE_BYTES;
+      if constexpr (WAVES != 0)
+        request_wave_blocks<WAVES, false>(dst, cache, rsrc, lay, mine, bt, bt_stride, pages, t * 32,
+                                          kv_first, kv_last, wave);
+      else request_tile(dst, cache, lay, off, bt, bt_stride, pages, t * 32, kv_first, kv_last, wave, waves);
+    };
+    request(t_first);
+    __syncthreads();               // waits for the loads too
+    for (int t = t_first; t < t_end; ++t) {
+      if (t + 1 < t_end) request(t + 1);
+      compute(t, kv_lds + ((t - t_first) & 1) * TILE_BYTES);
+      __syncthreads();             // the next tile has landed; nobody reads this one any more
+    }
   }
 
   const float l_slot = finish_sum(st);
@@ -756,11 +842,12 @@ static int check_common(const char* name, int64_t ld_out, int64_t ldq, int num_h
 // variant: 0 choose, 1 one wave per (tile, head), 2 key tiles shared in LDS by the heads
 // of a KV head (for tests of each kernel alone).
 HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* q, int64_t ldq,
-                                         const void* cache, const int* work, int num_tiles,
+                                         const void* cache, int cache_pages, const int* work, int num_tiles,
                                          const int* block_tables, int bt_stride, int num_heads, int kv_heads,
                                          int page_size, float scale, int window, int variant, hipStream_t stream) {
   HFEE_REQUIRE(num_tiles >= 0, "attention_bf16_prefill: bad tile count");
   HFEE_REQUIRE(variant >= 0 && variant <= 2, "attention_bf16_prefill: unknown kernel choice %d", variant);
+  HFEE_REQUIRE(cache_pages > 0, "attention_bf16_prefill: a cache layer of %d pages", cache_pages);
   if (num_tiles == 0) return 0;
   CacheLayout lay;
   if (check_common("attention_bf16_prefill", ld_out, ldq, num_heads, kv_heads, page_size, window, scale, out, q, &lay))
@@ -773,26 +860,35 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
                                             work, num_tiles, block_tables, bt_stride, num_heads, scale * LOG2E, window);
   } else {
     const int waves = group < SHARED_WAVES ? group : SHARED_WAVES, chunks = (group + waves - 1) / waves;
-    const size_t lds = (size_t)2 * KV_BLOCKS * 1024;
+    // the ring of tiles with loads waited for by count: four waves that bring equal shares of a
+    // tile, and a layer that 32 bits address
+    const int64_t layer_bytes = (int64_t)cache_pages * lay.page_stride * 2;
+    const bool ring = waves == SHARED_WAVES && KV_BLOCKS % SHARED_WAVES == 0 && layer_bytes < (1ll << 32);
+    const size_t lds = (size_t)(ring ? SHARED_TILES : 2) * KV_BLOCKS * 1024;
     static bool raised = false;
-    if (lds > 48 * 1024 && !raised) {
-      hipError_t e = hipFuncSetAttribute((const void*)prefill_shared_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds);
+    if (!raised) {
+      const int most = SHARED_TILES * KV_BLOCKS * 1024;
+      hipError_t e = hipFuncSetAttribute((const void*)prefill_shared_kernel<0, false>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, most);
       if (e == hipSuccess)
-        e = hipFuncSetAttribute((const void*)prefill_shared_kernel<SHARED_WAVES>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute((const void*)prefill_shared_kernel<SHARED_WAVES, false>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, most);
+      if (e == hipSuccess && KV_BLOCKS % SHARED_WAVES == 0)
+        e = hipFuncSetAttribute((const void*)prefill_shared_kernel<SHARED_WAVES, KV_BLOCKS % SHARED_WAVES == 0>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, most);
       HFEE_REQUIRE(e == hipSuccess, "attention_bf16_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
       raised = true;
     }
     dim3 grid((unsigned)(((int64_t)num_tiles * kv_heads * chunks + 7) / 8 * 8));
-    if (waves == SHARED_WAVES)
-      prefill_shared_kernel<SHARED_WAVES><<<grid, waves * 64, lds, stream>>>(
-          (bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, work, num_tiles, block_tables, bt_stride,
-          num_heads, scale * LOG2E, window);
-    else
-      prefill_shared_kernel<0><<<grid, waves * 64, lds, stream>>>(
-          (bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, work, num_tiles, block_tables, bt_stride,
-          num_heads, scale * LOG2E, window);
+#define GO(W, R)                                                                                                    \
+  prefill_shared_kernel<W, R><<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,         \
+                                                                (const bf16_t*)cache, (uint32_t)(ring ? layer_bytes : 0),  \
+                                                                lay, work, num_tiles, block_tables, bt_stride, num_heads, \
+                                                                scale * LOG2E, window)
+    if (ring) GO(SHARED_WAVES, (KV_BLOCKS % SHARED_WAVES == 0));
+    else if (waves == SHARED_WAVES) GO(SHARED_WAVES, false);
+    else GO(0, false);
+#undef GO
   }
   HFEE_CHECK_LAUNCH("attention_bf16_prefill");
   return 0;

@@ -312,7 +312,7 @@ def attention_bf16_prefill(out, q, cache_layer, tiles, block_tables, num_heads: 
     _check(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
            "attention: tiles must be [num_tiles, 4] int32")
     lib.attention_bf16(head_dim).call(
-        "hfee_attention_bf16_prefill", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(tiles),
+        "hfee_attention_bf16_prefill", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), cache_layer.shape[0], _ptr(tiles),
         tiles.shape[0], _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, page_size,
         float(scale), int(window), int(kernel), _stream())
 
