@@ -11,7 +11,11 @@ the scheduler (one new token for every request).  W untimed steps, then exactly 
 timed steps between two synchronisations.  One JSON line is printed: decoded
 tokens per second, the step's achieved fraction of the HBM roofline (every weight
 read once plus the cache of the live requests), a 2,048-token prefill with its
-fraction of the bf16 matrix peak, and decode at batch 1 and 64.
+fraction of the bf16 matrix peak, and under `points` decode at batch 1 and 64, the
+same measurements at the 1B and 13B shapes of the architecture, and prefill and
+decode at a context of 8,192 tokens.  Beside the published peaks the line gives what
+the simplest kernels reach on the GPU it ran on (`measured_peak`: a read-only stream
+over 4 GiB, a loop of nothing but matrix instructions; `--yardsticks` prints them alone).
 """
 import argparse
 import json
@@ -41,7 +45,7 @@ PROMPT = 1024
 PREFILL = 2048
 
 
-def main(argv=None) -> int:
+def parse(argv=None):
     ap = argparse.ArgumentParser(prog="bench.py")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
@@ -63,11 +67,91 @@ def main(argv=None) -> int:
                     help="run only the 2,048-token prefill (for profiling); prints its own short line")
     ap.add_argument("--prefill-tokens", type=int, default=0, metavar="T",
                     help="with --prefill-only: a prompt of T tokens (65 to 2,048) in place of 2,048")
-    args = ap.parse_args(argv)
+    ap.add_argument("--yardsticks", action="store_true",
+                    help="only measure what the simplest kernels get from this GPU: a read-only stream over 4 GiB "
+                         "and a loop of nothing but bfloat16 matrix instructions; prints its own line")
+    ap.add_argument("--no-extra-points", action="store_true",
+                    help="skip the other shapes and the longer context that the default run adds under `points`")
+    return ap.parse_args(argv)
+
+
+def yardsticks():
+    """What the simplest possible kernels reach on this GPU: (GB/s of a read-only stream over
+    4 GiB of device memory, TFLOP/s of a loop of nothing but bfloat16 matrix instructions)."""
+    import torch
+    from hfee_amd.kernels import ops
+    buf = torch.empty(4 << 30, dtype=torch.uint8, device="cuda:0")
+    buf.fill_(1)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def best(fn, reps=5):
+        fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(reps):
+            start.record()
+            fn()
+            stop.record()
+            torch.cuda.synchronize()
+            times.append(start.elapsed_time(stop) * 1e-3)
+        return min(times)
+    read_s = best(lambda: ops.read_stream(buf, 2048, True))
+    flops = ops.mfma_loop(1, 1)
+    mfma_s = best(lambda: ops.mfma_loop(2000, 2048))
+    flops = flops * 2000 * 2048
+    del buf
+    torch.cuda.empty_cache()
+    return (4 << 30) / read_s / 1e9, flops / mfma_s / 1e12
+
+
+def main(argv=None) -> int:
+    args = parse(argv)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.yardsticks:
+        import hfee_amd  # noqa: F401
+        gbs, tflops = yardsticks()
+        print(json.dumps({"read_stream_gb_per_s": round(gbs, 1), "hbm_published_gb_per_s": HBM_PEAK / 1e9,
+                          "mfma_loop_tflop_per_s": round(tflops, 1), "bf16_published_tflop_per_s": BF16_PEAK / 1e12}),
+              flush=True)
+        return 0
+    line = run(args)
+    if isinstance(line, int):
+        return line
+    if "points" in line and not args.no_extra_points and args.shape == "llama-3.1-8b" and not args.layers:
+        import copy
+        import torch
+        torch.cuda.empty_cache()
+        # the same measurements at the other shapes of the architecture and at a longer context
+        for shape in ("llama-3.2-1b", "llama-2-13b"):
+            other = copy.copy(args)
+            other.shape, other.no_points, other.steps, other.warmup = shape, False, min(args.steps, 32), min(args.warmup, 4)
+            other.only_prefill_point = True
+            got = run(other)
+            torch.cuda.empty_cache()
+            line["points"][f"decode_b8_{shape}"] = got["value"]
+            line["points"][f"decode_b8_hbm_frac_{shape}"] = got["roofline"]["frac"]
+            line["points"][f"prefill_2048_{shape}"] = got["prefill"]["value"]
+            line["points"][f"prefill_2048_frac_{shape}"] = got["prefill"]["frac"]
+        longer = copy.copy(args)
+        longer.context, longer.steps, longer.warmup = 8192, min(args.steps, 16), 2
+        got = run(longer)
+        torch.cuda.empty_cache()
+        line["points"]["prefill_8192"] = got["prefill"]["value"]
+        line["points"]["prefill_8192_frac"] = got["prefill"]["frac"]
+        line["points"]["decode_b8_ctx8192"] = got["decode"]["value"]
+        line["points"]["decode_b8_ctx8192_hbm_frac"] = got["decode"]["hbm_frac"]
+        gbs, tflops = yardsticks()
+        line["roofline"]["measured_peak"] = round(gbs, 1)
+        line["roofline"]["frac_of_measured"] = round(line["roofline"]["achieved"] / gbs, 4)
+        line["prefill"]["measured_peak_tflops"] = round(tflops, 1)
+    print(json.dumps(line), flush=True)
+    return 0
 
+
+def run(args):
+    """One measurement as the arguments say; returns the record to print (or an exit code)."""
     import torch
 
     import hfee_amd  # noqa: F401
@@ -175,15 +259,14 @@ def main(argv=None) -> int:
     if args.serving:
         serving_run(min(args.serving, 8))        # (compiles nothing, but captures graphs and sizes buffers)
         dt, prompt_tokens, made, steps = serving_run(args.serving)
-        print(json.dumps({
+        return ({
             "metric": "continuous batching, generated tok/s (%s bf16)" % SHAPE_NAMES[args.shape],
             "value": round(made / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "seconds": round(dt, 3),
             "all_tokens_per_s": round((prompt_tokens + made) / dt, 1), "dtype": "bf16",
             "data": "synthetic (seeded uniform random token ids, random N(0,0.02) weights)",
             "config": {"model": SHAPE_NAMES[args.shape] + "-shaped", "layers": L, "requests": args.serving,
                        "prompt_tokens_total": prompt_tokens, "generated_total": made, "seq_len": context,
-                       "max_batch_tokens": PREFILL, "page_size": page_size}}), flush=True)
-        return 0
+                       "max_batch_tokens": PREFILL, "page_size": page_size}})
 
     def context_run(batch: int, tokens: int, steps: int, warmup: int):
         """Prompts of `tokens` tokens, the first one timed alone (portions of 2,048 tokens
@@ -226,15 +309,14 @@ def main(argv=None) -> int:
         T = args.context
         flops = 2.0 * T * (L * layer_params) + 2.0 * V * d + L * 4.0 * hd * H * T * (T + 1) / 2
         step_bytes = weight_bytes + args.batch * (T + args.warmup + args.steps / 2) * kv_bytes_per_token
-        print(json.dumps({
+        return ({
             "metric": "prefill and decode at a context of %d tokens (%s bf16)" % (T, SHAPE_NAMES[args.shape]),
             "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 2),
                         "frac": round(flops / prefill_s / BF16_PEAK, 4)},
             "decode": {"value": round(args.batch * args.steps / dt, 1), "batch": args.batch,
                        "ms_per_step": round(dt / args.steps * 1e3, 3),
                        "hbm_frac": round(step_bytes / (dt / args.steps) / HBM_PEAK, 4)},
-            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": L}), flush=True)
-        return 0
+            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": L})
 
     if args.prefill_only:
         tokens = args.prefill_tokens or PREFILL
@@ -242,9 +324,7 @@ def main(argv=None) -> int:
             print(f"bench.py: --prefill-tokens takes 1 to {PREFILL}")
             return 2
         pt = prefill_run(tokens)
-        print(json.dumps({"prefill_ms": round(pt * 1e3, 3), "tokens": tokens, "layers": L,
-                          "us_per_layer": round(pt * 1e6 / L, 1)}), flush=True)
-        return 0
+        return {"prefill_ms": round(pt * 1e3, 3), "tokens": tokens, "layers": L, "us_per_layer": round(pt * 1e6 / L, 1)}
 
     dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
@@ -272,13 +352,12 @@ def main(argv=None) -> int:
         line["prefill"] = {"value": round(PREFILL / pt, 1), "tokens": PREFILL, "ms": round(pt * 1e3, 3),
                            "frac": round(flops / pt / BF16_PEAK, 4)}
         points = {}
-        for b in (1, 64):
+        for b in (() if getattr(args, "only_prefill_point", False) else (1, 64)):
             steps = max(8, min(args.steps, 64))
             dtb, _ = decode_run(b, steps, min(args.warmup, 4))
             points[f"decode_b{b}"] = round(b * steps / dtb, 2)
         line["points"] = points
-    print(json.dumps(line), flush=True)
-    return 0
+    return line
 
 
 if __name__ == "__main__":

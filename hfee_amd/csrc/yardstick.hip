@@ -47,9 +47,10 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(float* __restrict__ sink
   f32x16 acc[8];
   bf16x8 a, b;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    a[e] = (__bf16)(float)((threadIdx.x + e) & 3);
-    b[e] = (__bf16)(float)((threadIdx.x * 3 + e) & 1);
+  for (int e = 0; e < 8; ++e) {       // operands with every bit in use, as real ones have: the power they draw sets the clock
+    const uint32_t h = (threadIdx.x * 8u + e + 1u) * 2654435761u;
+    a[e] = (__bf16)((float)(int)((h >> 8) & 0xffff) * (1.0f / 65536.0f) - 0.5f);
+    b[e] = (__bf16)((float)(int)((h >> 12) & 0xffff) * (1.0f / 65536.0f) - 0.5f);
   }
 #pragma unroll
   for (int k = 0; k < 8; ++k)
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(float* __restrict__ sink
   for (int k = 0; k < 8; ++k)
 #pragma unroll
     for (int r = 0; r < 16; ++r) total += acc[k][r];
-  if (total == -1.0f && sink != nullptr) sink[0] = total;        // (never: the sums are not negative)
+  if (total == 12345.678f && sink != nullptr) sink[0] = total;   // (never, for all practical purposes)
 }
 
 }  // namespace
