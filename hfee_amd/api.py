@@ -83,7 +83,7 @@ class LLM:
             self._next_id += 1
             req = Request(rid, ids, p, seed=p.resolved_seed())
             helpers[rid] = {"index": i, "utf8": Utf8Buffer(), "stop": Stopper(list(p.stop)), "text": [],
-                            "first": True}
+                            "first": True, "hit": False}
             req.on_token = self._make_emit(helpers[rid], on_token)
             requests.append(req)
         outputs: dict = {}
@@ -96,7 +96,7 @@ class LLM:
                     text = None
                     if self.tokenizer is not None:
                         tail = h["stop"].flush() + h["utf8"].flush()
-                        if tail and fin.reason != "stop-string":
+                        if tail and not h["hit"]:
                             h["text"].append(tail)
                         text = "".join(h["text"])
                     outputs[fin.request.request_id] = Output(list(fin.request.generated), text, fin.request.stats,
@@ -123,6 +123,7 @@ class LLM:
                     piece = piece.lstrip(" ")      # runner.go:296-299
                     h["first"] = piece == ""
                 text, hit = h["stop"].push(piece)
+                h["hit"] = hit
                 if text:
                     h["text"].append(text)
             if on_token is not None:

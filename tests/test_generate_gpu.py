@@ -141,6 +141,40 @@ def test_stop_on_eos_and_context_limit(model_folders, tmp_path):
         small.generate([list(range(20))], SamplingParams.greedy())
 
 
+def test_a_prompt_given_as_text(model_folders, tmp_path):
+    """A folder with a tokenizer.json takes text: the prompt's ids (after the begin-of-sequence
+    id the configuration names) are the tokenizer's, the tokens are the plain implementation's,
+    the text is their bytes joined (leading spaces of the answer dropped), and a stop string
+    ends the answer in front of it."""
+    import json, shutil
+    from plain_llama import PlainLlama
+    from test_text import MERGES, byte_level_folder
+    from hfee_amd import LLM, SamplingParams
+    from hfee_amd.text import FolderTokenizer
+    dst = tmp_path / "with_text"
+    shutil.copytree(model_folders[("B", "float32")], dst)
+    path, vocab = byte_level_folder(dst, MERGES, added=[("<|eot|>", True)])
+    cj = json.load(open(dst / "config.json"))
+    cj["bos_token_id"] = len(vocab)
+    json.dump(cj, open(dst / "config.json", "w"))
+    tok = FolderTokenizer(path)
+    prompt = "hello world 123<|eot|>hello"
+    ids = [len(vocab)] + tok.encode(prompt)
+    assert ids[1] == vocab["hello"] and ids.count(len(vocab)) == 2 and len(ids) < len(prompt)
+    want = PlainLlama(str(dst)).greedy(ids, 24)
+    text = b"".join(tok.piece(t) for t in want).decode("utf-8", errors="replace").lstrip(" ")
+    assert len(text) >= 8            # tokens beyond the tokenizer's vocabulary print nothing
+    llm = LLM(str(dst), dtype="float32", num_ctx=128, num_parallel=2)
+    assert llm.encode(prompt) == ids
+    seen = []
+    o = llm.generate([prompt], SamplingParams.greedy(num_predict=24), on_token=lambda i, t, piece: seen.append(piece))[0]
+    assert o.token_ids == want and o.text == text and "".join(seen) + o.text[len("".join(seen)):] == text
+    stop = text[5:7]
+    o = llm.generate([prompt], SamplingParams.greedy(num_predict=24, stop=(stop,)))[0]
+    assert o.text == text[:text.index(stop)] and o.done_reason == "stop"
+    assert len(o.token_ids) < len(want) and o.token_ids == want[:len(o.token_ids)]
+
+
 def test_an_interrupted_call_leaves_nothing_behind(model_folders):
     """An error from the caller's on_token ends the call; its requests are cancelled and
     their pages freed, and the next call gives the usual tokens."""

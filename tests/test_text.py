@@ -1,0 +1,185 @@
+"""The tokenizer over a model folder's tokenizer.json: the reference's own vectors for the
+word rules and the merges, and small vocabularies made here for everything around them."""
+import json
+import random
+
+import pytest
+
+from hfee_amd.text import (FolderTokenizer, Utf8Buffer, _BYTE_TO_CHAR, merge_pieces, split_gpt2,
+                           split_llama3)
+
+LLAMA3_PATTERN = ("(?i:'s|'t|'re|'ve|'m|'ll|'d)|[^\\r\\n\\p{L}\\p{N}]?\\p{L}+|\\p{N}{1,3}| ?[^\\s\\p{L}\\p{N}]+[\\r\\n]*"
+                  "|\\s*[\\r\\n]+|\\s+(?!\\S)|\\s+")
+
+
+def test_the_reference_vectors_for_the_llama3_rule():
+    """/root/reference/internal/tokenizer/pretokenize_test.go:8-24"""
+    assert split_llama3("Hello world") == ["Hello", " world"]
+    assert split_llama3("It's 12345!") == ["It", "'s", " ", "123", "45", "!"]
+    assert split_llama3("a  b\n\n  c") == ["a", " ", " b", "\n\n", " ", " c"]
+    assert split_llama3("x  ") == ["x", "  "]
+
+
+def test_the_reference_vector_for_the_gpt2_rule():
+    """/root/reference/internal/tokenizer/pretokenize_test.go:26-32"""
+    assert split_gpt2("I'm here  now") == ["I", "'m", " here", " ", " now"]
+
+
+def test_the_reference_vector_for_the_merges():
+    """/root/reference/internal/tokenizer/pretokenize_test.go:34-45: ranks decide, not the order
+    in the word: "b c" is there from the start but "a b" (rank 0) goes first."""
+    ranks = {"a b": 0, "ab c": 1, "b c": 2}
+    assert merge_pieces(["a", "b", "c", "b", "c"], lambda l, r: ranks.get(l + " " + r)) == ["abc", "bc"]
+
+
+def test_the_leftmost_pair_goes_first_among_equal_ranks():
+    assert merge_pieces(["a", "a", "a"], lambda l, r: 0 if (l, r) == ("a", "a") else None) == ["aa", "a"]
+
+
+def test_what_the_rules_differ_in():
+    assert split_llama3("I'M") == ["I", "'M"] and split_gpt2("I'M") == ["I", "'", "M"]            # case of a contraction
+    assert split_llama3("x1234") == ["x", "123", "4"] and split_llama3("x1234", 1) == ["x", "1", "2", "3", "4"]
+    assert split_gpt2("x1234 56") == ["x", "1234", " 56"]
+    assert split_llama3("-foo") == ["-foo"] and split_gpt2("-foo") == ["-", "foo"]                # a symbol leads a word
+    assert split_llama3("a!?\n\nb") == ["a", "!?\n\n", "b"] and split_gpt2("a!?\n\nb") == ["a", "!?", "\n", "\n", "b"]
+    assert split_llama3("a \n \n  b") == ["a", " \n \n", " ", " b"]                               # up to the last newline
+    assert split_llama3("été 中文") == ["été", " 中文"]       # letters of any script
+    assert split_llama3("a  b") == ["a", " ", " b"]                           # a no-break space is a space
+
+
+def test_every_rule_loses_no_character():
+    rng = random.Random(0)
+    alphabet = "ab Z'’s\n\r\t 19!?.é中 -_'re'LL"
+    for _ in range(300):
+        text = "".join(rng.choice(alphabet) for _ in range(rng.randint(0, 40)))
+        for rule in (split_llama3, lambda t: split_llama3(t, 1), split_gpt2):
+            words = rule(text)
+            assert "".join(words) == text and all(words)
+
+
+def byte_level_folder(tmp_path, merges, added=(), pattern=LLAMA3_PATTERN):
+    vocab = {_BYTE_TO_CHAR[b]: b for b in range(256)}
+    for left, right in merges:
+        vocab[left + right] = len(vocab)
+    spec = {
+        "version": "1.0", "truncation": None, "padding": None, "normalizer": None, "post_processor": None,
+        "added_tokens": [{"id": len(vocab) + i, "content": c, "special": special, "single_word": False, "lstrip": False,
+                          "rstrip": False, "normalized": False} for i, (c, special) in enumerate(added)],
+        "pre_tokenizer": {"type": "Sequence", "pretokenizers": [
+            {"type": "Split", "pattern": {"Regex": pattern}, "behavior": "Isolated", "invert": False},
+            {"type": "ByteLevel", "add_prefix_space": False, "trim_offsets": True, "use_regex": False}]},
+        "decoder": {"type": "ByteLevel", "add_prefix_space": True, "trim_offsets": True, "use_regex": True},
+        "model": {"type": "BPE", "dropout": None, "unk_token": None, "continuing_subword_prefix": None,
+                  "end_of_word_suffix": None, "fuse_unk": False, "byte_fallback": False,
+                  "vocab": vocab, "merges": [f"{l} {r}" for l, r in merges]},
+    }
+    path = tmp_path / "tokenizer.json"
+    path.write_text(json.dumps(spec), encoding="utf-8")
+    return str(path), vocab
+
+
+G = _BYTE_TO_CHAR[ord(" ")]
+MERGES = [("l", "l"), ("h", "e"), ("he", "ll"), (G, "w"), ("o", "r"), (G + "w", "or"), ("hell", "o"),
+          (_BYTE_TO_CHAR[0xE2], _BYTE_TO_CHAR[0x82]), ("1", "2"), ("12", "3")]
+
+
+def test_a_byte_level_vocabulary(tmp_path):
+    path, vocab = byte_level_folder(tmp_path, MERGES, added=[("<|eot|>", True), ("<|eot|>x", False)])
+    tok = FolderTokenizer(path)
+    assert tok.byte_level and tok.llama3_rule and tok.max_digits == 3
+    ids = tok.encode("hello world")
+    assert ids == [vocab["hello"], vocab[G + "wor"], ord("l"), ord("d")]
+    assert tok.encode("12345") == [vocab["123"], ord("4"), ord("5")]          # digits in threes, then the merges
+    # the euro sign's three bytes: the first two have a merge, the third stays alone;
+    # the text comes back whole only once all its bytes have been joined
+    ids = tok.encode("€")
+    assert ids == [vocab[_BYTE_TO_CHAR[0xE2] + _BYTE_TO_CHAR[0x82]], 0xAC]
+    buf = Utf8Buffer()
+    assert [buf.add(tok.piece(i)) for i in ids] == ["", "€"]
+    # special tokens stay one id, the longest one at a place wins, and the text between them
+    # is cut as if it stood alone
+    eot, eotx = len(vocab), len(vocab) + 1
+    assert tok.encode("hello<|eot|>hello<|eot|>x") == [vocab["hello"], eot, vocab["hello"], eotx]
+    assert tok.piece(eot) == b"" and tok.piece(eotx) == b"<|eot|>x"           # a control token prints nothing
+    assert tok.encode("") == [] and tok.encode("<|eot|>") == [eot]
+
+
+def test_text_comes_back_byte_for_byte(tmp_path):
+    path, _ = byte_level_folder(tmp_path, MERGES)
+    tok = FolderTokenizer(path)
+    rng = random.Random(1)
+    alphabet = "helo wrd123 \n\t'sLL€é中\U0001f600!?"
+    for _ in range(200):
+        text = "".join(rng.choice(alphabet) for _ in range(rng.randint(1, 60)))
+        assert b"".join(tok.piece(i) for i in tok.encode(text)) == text.encode("utf-8"), text
+
+
+def test_the_rule_is_read_from_the_file(tmp_path):
+    gpt2 = "'s|'t|'re|'ve|'m|'ll|'d| ?\\p{L}+| ?\\p{N}+| ?[^\\s\\p{L}\\p{N}]+|\\s+(?!\\S)|\\s+"
+    path, vocab = byte_level_folder(tmp_path, MERGES, pattern=gpt2)
+    tok = FolderTokenizer(path)
+    assert not tok.llama3_rule
+    assert tok.encode("12345") == [vocab["123"], ord("4"), ord("5")]          # all digits one word: merges decide
+    assert tok.encode("-hello") == [ord("-"), vocab["hello"]]
+    one_digit = LLAMA3_PATTERN.replace("{1,3}", "")
+    path, vocab = byte_level_folder(tmp_path, MERGES, pattern=one_digit)
+    tok = FolderTokenizer(path)
+    assert tok.llama3_rule and tok.max_digits == 1
+    assert tok.encode("123") == [ord("1"), ord("2"), ord("3")]                # no merge reaches across words
+
+
+def sentencepiece_folder(tmp_path):
+    pieces = ["<unk>", "<s>", "</s>"] + [f"<0x{b:02X}>" for b in range(256)]
+    pieces += ["▁", "h", "e", "l", "o", "w", "he", "ll", "hell", "hello", "▁hello", "▁w"]
+    vocab = {p: i for i, p in enumerate(pieces)}
+    merges = [("h", "e"), ("l", "l"), ("he", "ll"), ("hell", "o"), ("▁", "hello"), ("▁", "w")]
+    spec = {
+        "added_tokens": [{"id": 0, "content": "<unk>", "special": True}, {"id": 1, "content": "<s>", "special": True},
+                         {"id": 2, "content": "</s>", "special": True}],
+        "normalizer": {"type": "Sequence", "normalizers": [{"type": "Prepend", "prepend": "▁"},
+                                                           {"type": "Replace", "pattern": {"String": " "}, "content": "▁"}]},
+        "pre_tokenizer": None,
+        "decoder": {"type": "Sequence", "decoders": [{"type": "Replace", "pattern": {"String": "▁"}, "content": " "},
+                                                     {"type": "ByteFallback"}, {"type": "Fuse"}]},
+        "model": {"type": "BPE", "vocab": vocab, "merges": [f"{l} {r}" for l, r in merges], "byte_fallback": True},
+    }
+    path = tmp_path / "tokenizer.json"
+    path.write_text(json.dumps(spec), encoding="utf-8")
+    return str(path), vocab
+
+
+def test_a_vocabulary_of_the_sentencepiece_kind(tmp_path):
+    """/root/reference/internal/tokenizer/tokenizer.go:187-218, 242-262: a space before the text
+    that follows a special token (or the start), spaces as U+2581, bytes for what has no piece."""
+    path, vocab = sentencepiece_folder(tmp_path)
+    tok = FolderTokenizer(path)
+    assert not tok.byte_level and tok.space_prefix
+    assert tok.encode("hello w") == [vocab["▁hello"], vocab["▁w"]]
+    euro = [vocab["<0xE2>"], vocab["<0x82>"], vocab["<0xAC>"]]
+    assert tok.encode("€") == [vocab["▁"]] + euro
+    assert tok.encode("<s>hello</s>") == [1, vocab["▁hello"], 2]
+    buf = Utf8Buffer()
+    assert "".join(buf.add(tok.piece(i)) for i in tok.encode("hello €")) == " hello €"
+    assert tok.piece(vocab["<0xE2>"]) == b"\xe2" and tok.piece(1) == b"" and tok.piece(10 ** 6) == b""
+
+
+def test_other_kinds_of_tokenizer_are_refused(tmp_path):
+    path = tmp_path / "tokenizer.json"
+    path.write_text(json.dumps({"model": {"type": "Unigram", "vocab": [["a", 0.0]]}}))
+    with pytest.raises(ValueError, match="type BPE"):
+        FolderTokenizer(str(path))
+
+
+def test_the_same_ids_as_the_tokenizers_package(tmp_path):
+    """A second reading of the same file where one is installed: byte-level words, merges and
+    special tokens give the same ids."""
+    tokenizers = pytest.importorskip("tokenizers")
+    path, _ = byte_level_folder(tmp_path, MERGES, added=[("<|eot|>", True)])
+    theirs = tokenizers.Tokenizer.from_file(path)
+    ours = FolderTokenizer(path)
+    rng = random.Random(2)
+    alphabet = "helo wrd123 \n\r\t'sLL€é中!?-"
+    texts = ["hello world", "It's 12345!", "a  b\n\n  c", "x  ", "hello<|eot|>hello world", "I'M we'Re  \n "]
+    texts += ["".join(rng.choice(alphabet) for _ in range(rng.randint(1, 50))) for _ in range(200)]
+    for text in texts:
+        assert ours.encode(text) == theirs.encode(text, add_special_tokens=False).ids, repr(text)
