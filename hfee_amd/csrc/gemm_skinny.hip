@@ -675,6 +675,146 @@ bool launch_mid_rows(const Args& a, int epi, float* scratch, int64_t scratch_flo
   return true;
 }
 
+// ------------------------------------------- 17 to 64 rows, many weight rows ---
+// Where the weight rows alone fill the chip (gate/up, the vocabulary head) nothing has to be
+// cut along K, and the shares, their buffer and the second kernel fall away: a product of
+// 28,672 weight rows and 64 batch rows in four slices writes and reads a quarter of the
+// weights' bytes again as shares.  Here a wave owns a group of 16 weight rows over the whole
+// of K and a workgroup's eight waves walk K together, 512 columns at a time: the batch's
+// columns of the moment lie in LDS, twice, so that the next 512 are brought (through
+// registers, from L2) under the products of these; one barrier a slice.  The weights come as
+// above, through a ring of loads that runs on across slices and row groups.
+constexpr int WIDE_KS = 512, WIDE_STEPS = WIDE_KS / 32, WIDE_PITCH = WIDE_KS + 8;
+
+constexpr int WIDE_MIN_GROUPS_A_CU = 6;       // of eight: below, the kernels above with their slices of K spread better
+
+constexpr size_t mid_wide_lds_bytes(int mt) { return (size_t)2 * mt * 16 * WIDE_PITCH * sizeof(bf16_t); }
+
+template <int MT, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_groups) {
+  extern __shared__ __attribute__((aligned(16))) char wide_lds[];
+  bf16_t* xs = (bf16_t*)wide_lds;                                    // [2][MT * 16][WIDE_PITCH]
+  __shared__ float row_scale[SS_STRIDE];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r16 = lane & 15, g = lane >> 4;
+  const int slices = a.K / WIDE_KS, tiles = a.K / 32;
+
+  // a slice of the batch: MT * 16 rows of 64 chunks of 16 bytes, a row a wave and round
+  constexpr int FILL = MT * 16 / WAVES;
+  auto ask = [&](u32x4* fill, int slice) {
+#pragma unroll
+    for (int it = 0; it < FILL; ++it) {
+      const int row = it * WAVES + wave;
+      fill[it] = u32x4{0u, 0u, 0u, 0u};                              // rows beyond M are zeros
+      if (row < a.M) fill[it] = *reinterpret_cast<const u32x4*>((const bf16_t*)a.A + (int64_t)row * a.lda + slice * WIDE_KS + lane * 8);
+    }
+  };
+  auto put = [&](const u32x4* fill, int buf) {
+#pragma unroll
+    for (int it = 0; it < FILL; ++it)
+      *reinterpret_cast<u32x4*>(xs + ((buf * MT * 16) + it * WAVES + wave) * WIDE_PITCH + lane * 8) = fill[it];
+  };
+  auto row_ptr = [&](int rg) {       // rows beyond N are zeros of the last row of tiles; what they produce is never stored
+    return WeightTiles::lane_place(a.W, a.w_stride, min(rg, row_groups - 1) * ROWS + r16, g);
+  };
+
+  // the batch first (from L2: it must not wait in line behind weights from memory), then the ring
+  u32x4 fill[FILL];
+  ask(fill, 0);
+  const int stride = gridDim.x * WAVES;
+  const bf16_t* w_cur = row_ptr(blockIdx.x * WAVES + wave);
+  constexpr int RING = mid_ring(MT);
+  static_assert(WIDE_STEPS % RING == 0, "a ring slot must mean the same step in every slice");
+  Chunk ring[RING];
+#pragma unroll
+  for (int st = 0; st < RING; ++st) ring[st].u = load_streamed(reinterpret_cast<const u32x4*>(w_cur + st * WeightTiles::TILE));
+  put(fill, 0);
+  if (a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
+  __syncthreads();
+
+  int buf = 0;
+  for (int first = blockIdx.x * WAVES; first < row_groups; first += stride) {      // (the same for all waves: barriers inside)
+    const int rg = first + wave;
+    const bf16_t* w_next = row_ptr(rg + stride);                     // past the end: a repeat that nobody uses
+    f32x4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < slices; ++s) {
+      ask(fill, s + 1 < slices ? s + 1 : 0);
+      const bf16_t* x_lane = xs + (buf * MT * 16 + r16) * WIDE_PITCH + g * 8;
+#pragma unroll
+      for (int st = 0; st < WIDE_STEPS; ++st) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const bf16x8 b = *reinterpret_cast<const bf16x8*>(x_lane + t * 16 * WIDE_PITCH + st * 32);
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st % RING].v, b, acc[t], 0, 0, 0);
+        }
+        const int ahead = s * WIDE_STEPS + st + RING;
+        const bf16_t* src = ahead < tiles ? w_cur + (int64_t)ahead * WeightTiles::TILE : w_next + (int64_t)(ahead - tiles) * WeightTiles::TILE;
+        ring[st % RING].u = load_streamed(reinterpret_cast<const u32x4*>(src));
+      }
+      // (the order of issue as in the kernel above: LDS reads of a step under the products of the
+      // step before, a ring slot refilled as soon as its step has been multiplied)
+      __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+#pragma unroll
+      for (int st = 0; st < WIDE_STEPS; ++st) {
+        if (st + 1 < WIDE_STEPS) __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      put(fill, buf ^ 1);          // read last in the slice before this one: everybody has passed that barrier
+      __syncthreads();
+      buf ^= 1;
+    }
+    if (rg < row_groups) {
+      const int n = rg * ROWS + 4 * g;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + r16;
+        float v[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        if (a.scale_ss != nullptr) {
+          const float scale = row_scale[m];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] *= scale;
+        }
+        const bool live = m < a.M && n < a.N;
+        finish_rows_ahead<EPI>(a, look_ahead<EPI>(a, m, n, live), m, n, live, v, rg, lane);
+      }
+    }
+    w_cur = w_next;
+  }
+}
+
+// Returns true if the kernel for 17 to 64 rows and many weight rows took the product.
+template <int MT>
+bool launch_mid_wide(const Args& a, int epi, int num_cus, hipStream_t stream) {
+  const int row_groups = (a.N + ROWS - 1) / ROWS, groups = (row_groups + WAVES - 1) / WAVES;
+  const int per = (groups + num_cus - 1) / num_cus;                  // rounds of a workgroup, all but equal
+  const int grid = (groups + per - 1) / per;
+  const size_t lds = mid_wide_lds_bytes(MT);
+#define GO(E)                                                                                                  \
+  do {                                                                                                         \
+    static bool raised = false;                                                                                \
+    if (!raised) {                                                                                             \
+      if (hipFuncSetAttribute((const void*)mid_wide_kernel<MT, E>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                              (int)lds) != hipSuccess)                                                        \
+        return false;                                                                                          \
+      raised = true;                                                                                           \
+    }                                                                                                          \
+    mid_wide_kernel<MT, E><<<grid, WAVES * 64, lds, stream>>>(a, row_groups);                                  \
+  } while (0)
+  switch (epi) {
+    case EPI_BF16: GO(EPI_BF16); break;
+    case EPI_F32: GO(EPI_F32); break;
+    case EPI_ADD: GO(EPI_ADD); break;
+    case EPI_SWIGLU: GO(EPI_SWIGLU); break;
+    default: GO(EPI_QKV); break;
+  }
+#undef GO
+  return true;
+}
+
 // ------------------------------------------------------------ wide products ---
 // For products with many weight rows (gate/up, the vocabulary head) and at most 16
 // batch rows.  Workgroups are persistent: each walks several groups of 16 weight
@@ -853,7 +993,8 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 // scratch: for 17 to 64 rows and K a multiple of 1,024, a faster pair of kernels that needs
 // ceil(N / 16) * (K / 1024) * ceil(M / 16) * 256 + 64 floats of scratch (none for K = 1,024);
 // without it, or for other sizes, or where it would not pay, the streaming kernel takes
-// the product (force_mid != 0 takes the faster kernels wherever they apply: for tests).
+// the product (force_mid: 1 takes the pair of kernels with slices of K wherever it applies,
+// 2 the kernel for many weight rows: for tests).
 HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32, int64_t lda, const void* W,
                               int64_t w_stride, int M, int N, int K, int epi,
                               const void* norm_weight, int norm_weight_is_f32, float eps, const int* rows,
@@ -927,14 +1068,25 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
   const double t_streaming = weight_mb / 5.0 + 3.0 + 0.052 * (K / 1024.0) * (rounds > 1.0 ? rounds : 1.0) * M;
   const double t_pair = weight_mb * 0.215 + 4.0 > 16.5 ? weight_mb * 0.215 + 4.0 : 16.5;
   const bool mid_pays = t_pair < 0.95 * t_streaming;
-  if (!norm && mt > 1 && K % MID_KS == 0 && (mid_pays || force_mid)) {
-    static int num_cus = 0;
-    if (num_cus == 0) {
-      int dev = 0;
-      hipDeviceProp_t prop;
-      num_cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-                 prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    num_cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+               prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+  }
+  // weight rows enough for most of the CUs to have eight row groups each: nothing is cut along K
+  const bool wide_rows = (N + ROWS - 1) / ROWS >= WIDE_MIN_GROUPS_A_CU * num_cus;
+  if (!norm && mt > 1 && K % WIDE_KS == 0 && (force_mid == 2 || (force_mid == 0 && wide_rows))) {
+    const bool took = mt == 2 ? launch_mid_wide<2>(a, epi, num_cus, stream)
+                    : mt == 3 ? launch_mid_wide<3>(a, epi, num_cus, stream)
+                              : launch_mid_wide<4>(a, epi, num_cus, stream);
+    if (took) {
+      HFEE_CHECK_LAUNCH("gemm_skinny(17 to 64 rows, many weight rows)");
+      return 0;
     }
+  }
+  if (!norm && mt > 1 && K % MID_KS == 0 && (mid_pays || force_mid == 1)) {
     const bool took = mt == 2 ? launch_mid_rows<2>(a, epi, scratch, scratch_floats, num_cus, stream)
                     : mt == 3 ? launch_mid_rows<3>(a, epi, scratch, scratch_floats, num_cus, stream)
                               : launch_mid_rows<4>(a, epi, scratch, scratch_floats, num_cus, stream);

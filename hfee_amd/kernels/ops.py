@@ -431,8 +431,9 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
     emitted tensor, and the finished sums are scaled by 1 / sqrt(sum of shares / K + eps).
     scratch (float32, `mid_rows_scratch` words): lets products of 17 to 64 rows over
     K % 1024 == 0 take a kernel that keeps the batch in LDS and cuts K over workgroups, and a
-    second one that adds the slices up, where that pays (force_mid_rows: wherever it applies,
-    for tests).
+    second one that adds the slices up, where that pays.  Products with weight rows enough to
+    fill the chip take a kernel that cuts nothing and needs no scratch.  (force_mid_rows, for
+    tests: 1 takes the first wherever it applies, 2 the second.)
 
     x: bfloat16 [M, K]; or, with norm_weight, the float32 residual stream (at most 16
     rows; `rows` optionally gathers them, then `m` is their number).

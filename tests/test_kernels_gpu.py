@@ -271,6 +271,20 @@ def test_products_of_17_to_64_rows(M, N, K, epilogue):
     """The kernel that keeps the batch in LDS and cuts K over workgroups (17 to 64 rows,
     K a multiple of 1,024) and the kernel that adds its slices up, with every epilogue, twice
     in a row on the same scratch, against the unfused formulas."""
+    _products_of_17_to_64_rows(M, N, K, epilogue, 1)
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 48, 512), (33, 200, 1536), (64, 4100, 2048), (40, 6150, 4096), (64, 100, 1024),
+                                   (50, 33000, 512), (24, 130, 2560)])
+@pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu", "emit", "scaled"])
+def test_products_of_17_to_64_rows_and_many_weight_rows(M, N, K, epilogue):
+    """The kernel whose waves own 16 weight rows each over the whole of K (a multiple of 512),
+    the batch passing through LDS 512 columns at a time: one round of a workgroup, several, and
+    fewer row groups than a workgroup has waves; every epilogue; against the unfused formulas."""
+    _products_of_17_to_64_rows(M, N, K, epilogue, 2)
+
+
+def _products_of_17_to_64_rows(M, N, K, epilogue, kernel):
     from hfee_amd.kernels import ops
     if epilogue == "swiglu" and N % 2:
         N += 1
@@ -279,10 +293,10 @@ def test_products_of_17_to_64_rows(M, N, K, epilogue):
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
     ref = x.double() @ w.double().t()
     mag = x.double().abs() @ w.double().abs().t()
-    words = ops.mid_rows_scratch(M, N, K)
-    assert (words > 0) == (K > 1024)
+    words = ops.mid_rows_scratch(M, N, K) if kernel == 1 else 0
+    assert kernel == 2 or (words > 0) == (K > 1024)
     scratch = torch.full((max(words, 1),), float("nan"), dtype=torch.float32, device=DEV)
-    kw = dict(scratch=scratch, force_mid_rows=True)
+    kw = dict(scratch=scratch, force_mid_rows=kernel)
     c0 = torch.randn(M, N, generator=g)
     for _ in range(2):
         if epilogue == "swiglu":
@@ -379,13 +393,15 @@ def test_fused_qkv_rotation_and_cache_write(H, K, hd, half, M, norm):
     _check_fused_qkv(H, K, hd, half, M, norm, 96)
 
 
+@pytest.mark.parametrize("kernel", [1, 2])
 @pytest.mark.parametrize("H,K,hd,half,M,d", [(4, 2, 16, 8, 17, 2048), (5, 1, 64, 32, 64, 1024), (6, 3, 48, 8, 40, 3072)])
-def test_fused_qkv_with_the_batch_in_lds(H, K, hd, half, M, d):
-    """The same through the kernel for 17 to 64 rows that cuts K over workgroups."""
+def test_fused_qkv_with_the_batch_in_lds(H, K, hd, half, M, d, kernel):
+    """The same through the kernels for 17 to 64 rows: the one that cuts K over workgroups and
+    the one for many weight rows."""
     from hfee_amd.kernels import ops
     N = (H + 2 * K) * hd
     scratch = torch.full((max(ops.mid_rows_scratch(M, N, d), 1),), float("nan"), dtype=torch.float32, device=DEV)
-    _check_fused_qkv(H, K, hd, half, M, False, d, scratch=scratch, force_mid_rows=True)
+    _check_fused_qkv(H, K, hd, half, M, False, d, scratch=scratch, force_mid_rows=kernel)
 
 
 def _check_fused_qkv(H, K, hd, half, M, norm, d, **kw):
