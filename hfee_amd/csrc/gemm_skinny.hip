@@ -472,7 +472,7 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 // ------------------------------------------------------------ 17 to 64 rows ---
 // With more than 16 batch rows the streaming kernel reads the batch again for every 16
 // weight rows, and that traffic (from L2) outgrows the weights.  Here K is cut into
-// slices of 1,024 columns, each with workgroups of its own.  A workgroup keeps its slice
+// slices of 1,024 columns (the last one may be half a slice), each with workgroups of its own.  A workgroup keeps its slice
 // of the batch, all rows, in LDS; each of its waves walks over groups of 16 weight rows
 // on its own: the weights come straight from global memory through a ring of 4 or 16 loads
 // that runs across group boundaries, the batch operands from LDS; no barrier stands in
@@ -480,7 +480,7 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 // scratch buffer and goes on; a second, short kernel (one wave for 16 batch rows of a row
 // group, so that the whole chip takes part) adds the shares in the order of the slices and
 // runs the epilogue.  Nobody waits for anybody, and nothing is counted.
-constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32;
+constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32, MID_HALF = MID_STEPS / 2;
 // loads a wave keeps in flight.  Measured inside the decode step at 64 rows (q/k/v, output, down
 // of the 8B shape): 20.3 / 14.2 / 27.2 µs with 8, 15.0 / 13.8 / 27.1 with 4, 19.7 / 15.2 / 30.4 with 2;
 // at 24 and 32 rows 4 and 16 measured alike.
@@ -514,7 +514,8 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   for (int it = 0; it < FILL; ++it) {
     const int row = ((it + fill_first) % FILL) * FILL_ROWS + fill_row;
     fill[it] = u32x4{0u, 0u, 0u, 0u};                             // rows beyond M are zeros
-    if (row < a.M) fill[it] = *reinterpret_cast<const u32x4*>((const bf16_t*)a.A + (int64_t)row * a.lda + k0 + fill_c * 8);
+    if (row < a.M && k0 + fill_c * 8 < a.K)                       // (the last slice may be half a slice)
+      fill[it] = *reinterpret_cast<const u32x4*>((const bf16_t*)a.A + (int64_t)row * a.lda + k0 + fill_c * 8);
   }
 
   // ---- then the first weights: behind every wave's requests for the batch, also in the
@@ -550,32 +551,36 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   __syncthreads();
 
   const bf16_t* x_lane = xs + r16 * MID_PITCH + g * 8;
+  const int steps = min(MID_STEPS, (a.K - k0) / 32);      // of this slice: 32, or 16 in a last half slice
   while (rg < row_groups) {
     const int rg_next = rg + stride;
     const bf16_t* w_next = row_ptr(rg_next < row_groups ? rg_next : rg);    // past the end: a repeat that nobody uses
     f32x4 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < steps; h += MID_HALF) {
 #pragma unroll
-    for (int st = 0; st < MID_STEPS; ++st) {
+      for (int s = 0; s < MID_HALF; ++s) {
+        const int st = h + s;
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        const bf16x8 b = *reinterpret_cast<const bf16x8*>(x_lane + t * 16 * MID_PITCH + st * 32);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st % MID_RING].v, b, acc[t], 0, 0, 0);
+        for (int t = 0; t < MT; ++t) {
+          const bf16x8 b = *reinterpret_cast<const bf16x8*>(x_lane + t * 16 * MID_PITCH + st * 32);
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[s % MID_RING].v, b, acc[t], 0, 0, 0);
+        }
+        const int ahead = st + MID_RING;
+        const bf16_t* src = ahead < steps ? w_cur + ahead * WeightTiles::TILE : w_next + (ahead - steps) * WeightTiles::TILE;
+        ring[s % MID_RING].u = load_streamed(reinterpret_cast<const u32x4*>(src));
       }
-      const int ahead = st + MID_RING;
-      ring[st % MID_RING].u = ahead < MID_STEPS ? load_streamed(reinterpret_cast<const u32x4*>(w_cur + ahead * WeightTiles::TILE))
-                                                : load_streamed(reinterpret_cast<const u32x4*>(w_next + (ahead - MID_STEPS) * WeightTiles::TILE));
-    }
-    // The order of issue, spelled out (groups: 0x008 matrix, 0x100 LDS read, 0x020 global
-    // load): the batch operands of a step are read under the products of the step before,
-    // and a ring slot is refilled as soon as its step has been multiplied.
-    __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+      // The order of issue, spelled out (groups: 0x008 matrix, 0x100 LDS read, 0x020 global
+      // load): the batch operands of a step are read under the products of the step before,
+      // and a ring slot is refilled as soon as its step has been multiplied.
+      __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
 #pragma unroll
-    for (int st = 0; st < MID_STEPS; ++st) {
-      if (st + 1 < MID_STEPS) __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      for (int s = 0; s < MID_HALF; ++s) {
+        if (s + 1 < MID_HALF) __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
     }
 
     const int n = rg * ROWS + 4 * g;
@@ -645,7 +650,7 @@ __global__ __launch_bounds__(WAVES * 64) void mid_finish_kernel(Args a, int row_
 // Returns true if the kernels for 17 to 64 rows took the product.
 template <int MT>
 bool launch_mid_rows(const Args& a, int epi, float* scratch, int64_t scratch_floats, int num_cus, hipStream_t stream) {
-  const int row_groups = (a.N + ROWS - 1) / ROWS, slices = a.K / MID_KS;
+  const int row_groups = (a.N + ROWS - 1) / ROWS, slices = (a.K + MID_KS - 1) / MID_KS;
   if (slices > 1 && (scratch == nullptr || scratch_floats < (int64_t)row_groups * slices * MT * 256 + SS_STRIDE)) return false;
   int per_slice = num_cus / slices;                         // workgroups per slice: eight row groups at a time each
   if (per_slice < 1) per_slice = 1;
@@ -990,8 +995,8 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 // product's shares of the rows' sums of squares to emit_ss (ceil(N / 16) x 64 floats).
 // scale_ss: shares left by such a product (scale_blocks x 64 floats) over rows of width K:
 // the finished sums are scaled by 1 / sqrt(sum / K + scale_eps).
-// scratch: for 17 to 64 rows and K a multiple of 1,024, a faster pair of kernels that needs
-// ceil(N / 16) * (K / 1024) * ceil(M / 16) * 256 + 64 floats of scratch (none for K = 1,024);
+// scratch: for 17 to 64 rows and K a multiple of 512, a faster pair of kernels that needs
+// ceil(N / 16) * ceil(K / 1024) * ceil(M / 16) * 256 + 64 floats of scratch (none for K <= 1,024);
 // without it, or for other sizes, or where it would not pay, the streaming kernel takes
 // the product (force_mid: 1 takes the pair of kernels with slices of K wherever it applies,
 // 2 the kernel for many weight rows: for tests).
@@ -1086,7 +1091,7 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
       return 0;
     }
   }
-  if (!norm && mt > 1 && K % MID_KS == 0 && (mid_pays || force_mid == 1)) {
+  if (!norm && mt > 1 && K % (MID_KS / 2) == 0 && (mid_pays || force_mid == 1)) {
     const bool took = mt == 2 ? launch_mid_rows<2>(a, epi, scratch, scratch_floats, num_cus, stream)
                     : mt == 3 ? launch_mid_rows<3>(a, epi, scratch, scratch_floats, num_cus, stream)
                               : launch_mid_rows<4>(a, epi, scratch, scratch_floats, num_cus, stream);
