@@ -729,7 +729,7 @@ __global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_gr
   ask(fill, 0);
   const int stride = gridDim.x * WAVES;
   const bf16_t* w_cur = row_ptr(blockIdx.x * WAVES + wave);
-  constexpr int RING = mid_ring(MT);
+  constexpr int RING = mid_ring(MT);          // (8 or 16 loads a wave in flight at 64 rows: the step within 1 %)
   static_assert(WIDE_STEPS % RING == 0, "a ring slot must mean the same step in every slice");
   Chunk ring[RING];
 #pragma unroll
