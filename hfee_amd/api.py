@@ -30,14 +30,17 @@ class LLM:
     def __init__(self, model=None, *, config=None, random_weights: bool = False, seed: int = 0,
                  dtype: str = "bfloat16", num_ctx: int = 4096, num_parallel: int = 4,
                  max_batch_tokens: int = 2048, page_size: int = 16, num_pages: int | None = None,
-                 device: str = "cuda:0", weight_std: float = 0.02):
+                 device: str = "cuda:0", weight_std: float = 0.02, keep_prefixes: bool = True):
         """model: a folder with config.json and model.safetensors.  With
         random_weights=True (or config=... and no folder) the weights are seeded
         random numbers made on the device.  num_ctx is the context window of one
         request, num_parallel the number of requests served at once (the
         reference's HFEE_NUM_CTX and HFEE_NUM_PARALLEL,
         /root/reference/internal/server/server.go:46-57), max_batch_tokens the token
-        budget of a step (256 in the reference, /root/reference/internal/llm/runner.go:11)."""
+        budget of a step (256 in the reference, /root/reference/internal/llm/runner.go:11).
+        keep_prefixes: a finished request's full pages stay in the cache, and a prompt that
+        begins with the same tokens does not run them again (the reference reuses the longest
+        common prefix of a free slot's tokens, runner.go:198-229)."""
         from .config import config_from_folder
         if model is not None and not random_weights:
             self.model, self.config = load_model(model, dtype, device)
@@ -50,6 +53,7 @@ class LLM:
         if num_pages is None:
             num_pages = num_parallel * ((self.num_ctx + page_size - 1) // page_size)
         self.engine = Engine(self.model, num_pages=num_pages, page_size=page_size, max_requests=num_parallel,
+                             keep_prefixes=keep_prefixes,
                              max_batch_tokens=max_batch_tokens, num_positions=self.num_ctx, device=device)
         self.sampler = Sampler(spec.vocab, self.engine.device, max_rows=num_parallel)
         self.scheduler = Scheduler(self.engine, self.sampler, max_num_seqs=num_parallel,

@@ -12,10 +12,24 @@ key; a "window" group keeps the last `window` keys, and pages that the window ha
 passed go back to the pool at commit time.  Pages come back when a request is
 released and are handed out again at once (last freed, first reused).
 
+Prefixes kept between requests.  The reference leaves a finished request's cache in its
+slot and puts the next request into the slot whose tokens share the longest prefix with
+it, so that only the rest of the prompt is run, and always at least one token
+(/root/reference/internal/llm/runner.go:198-229).  With pages the same thing is done page
+by page (`keep_prefixes`): the full pages of a released request stay behind, each under a
+digest of all tokens up to its end; a new request takes over, from the first page on, the
+kept pages whose digests its own prompt produces, as its own (a page is never shared:
+it is free, kept, or owned by one request), and runs what is left.  Kept pages count as
+free: when the free list is empty the oldest kept page is taken, the deepest page of a
+chain before the pages in front of it.  Only models whose groups all keep every token can
+do this (a window group has given pages back; fixed-size state cannot be cut back).
+
 This file is bookkeeping only (no tensors); storage.py holds the device memory.
 """
 from __future__ import annotations
 
+import hashlib
+from collections import OrderedDict
 from dataclasses import dataclass, field
 
 import numpy as np
@@ -56,9 +70,12 @@ class CacheGroupSpec:
         return n
 
 
+KEPT = ("kept prefix",)      # the owner of pages that wait for a request with the same prefix
+
+
 class PagePool:
     """The pages of one group.  LIFO free list; every page is free or owned by
-    exactly one request."""
+    exactly one owner (a request, or KEPT)."""
 
     def __init__(self, num_pages: int):
         if num_pages < 1:
@@ -66,12 +83,17 @@ class PagePool:
         self.num_pages = num_pages
         self._free = list(range(num_pages - 1, -1, -1))   # pop() hands out 0 first
         self._owner: list = [None] * num_pages
+        self.reclaimable = lambda: 0        # pages that `reclaim` can still bring back
+        self.reclaim = lambda: None         # brings at least one page back to the free list
 
     @property
     def num_free(self) -> int:
-        return len(self._free)
+        """Pages that can be taken: the free ones and those a kept prefix would give up."""
+        return len(self._free) + self.reclaimable()
 
     def take(self, owner) -> int:
+        if not self._free and self.reclaimable():
+            self.reclaim()
         if not self._free:
             raise OutOfPages("no free page")
         page = self._free.pop()
@@ -92,12 +114,18 @@ class PagePool:
     def owner_of(self, page: int):
         return self._owner[page]
 
+    def hand_over(self, page: int, owner, new_owner) -> None:
+        if self._owner[page] != owner or owner is None or new_owner is None:
+            raise CacheError(f"page {page} belongs to {self._owner[page]!r}, not {owner!r}")
+        self._owner[page] = new_owner
+
 
 @dataclass
 class RequestCache:
     request_id: object
     slot: int
     length: int = 0                                   # committed tokens
+    reused: int = 0                                   # of these, taken over from a kept prefix at admission
     tables: list = field(default_factory=list)        # per group: page id per block, -1 once released
     first_live_block: list = field(default_factory=list)   # per group
     arrays: list = field(default_factory=list)        # per group: the table as int32 (released blocks read 0),
@@ -117,7 +145,7 @@ class RequestCache:
 
 
 class CacheManager:
-    def __init__(self, groups, page_size: int, pages_per_group, max_requests: int):
+    def __init__(self, groups, page_size: int, pages_per_group, max_requests: int, keep_prefixes: bool = False):
         if page_size < 16 or page_size & (page_size - 1):
             raise CacheError(f"page_size must be a power of two >= 16, got {page_size}")
         self.groups = tuple(groups)
@@ -130,9 +158,22 @@ class CacheManager:
         self.max_requests = max_requests
         self._free_slots = list(range(max_requests - 1, -1, -1))
         self.requests: dict = {}
+        if keep_prefixes and any(g.kind != "full" for g in self.groups):
+            raise CacheError("prefixes can be kept only where every cache group keeps every token")
+        self.keep_prefixes = bool(keep_prefixes) and bool(self.groups)
+        # digest of the tokens up to a page's end -> (the page in every group, the page's own tokens);
+        # the oldest entry first
+        self._kept: OrderedDict = OrderedDict()
+        self.prefix_hits = 0          # tokens taken over from kept prefixes so far
+        for pool in self.pools:
+            pool.reclaimable = lambda: len(self._kept)
+            pool.reclaim = self._drop_oldest_kept
 
     # ------------------------------------------------------------ requests
-    def admit(self, request_id) -> RequestCache:
+    def admit(self, request_id, tokens=None) -> RequestCache:
+        """A new request.  With `tokens` (its prompt) and kept prefixes, it takes over the kept
+        pages that hold the beginning of the prompt, whole pages only and never the whole
+        prompt: its `length` (= `reused`) says how many tokens need not be run."""
         if request_id in self.requests:
             raise CacheError(f"request {request_id!r} is already live")
         if not self._free_slots:
@@ -141,6 +182,19 @@ class CacheManager:
                           tables=[[] for _ in self.groups], first_live_block=[0] * len(self.groups),
                           arrays=[np.zeros(16, dtype=np.int32) for _ in self.groups])
         self.requests[request_id] = rc
+        if self.keep_prefixes and tokens is not None and self._kept:
+            ps = self.page_size
+            for b, digest in enumerate(self._digests(tokens, (len(tokens) - 1) // ps)):
+                entry = self._kept.get(digest)
+                if entry is None or entry[1] != tuple(tokens[b * ps:(b + 1) * ps]):
+                    break
+                del self._kept[digest]
+                for g, page in enumerate(entry[0]):
+                    self.pools[g].hand_over(page, KEPT, request_id)
+                    rc._append(g, page)
+                rc.length += ps
+            rc.reused = rc.length
+            self.prefix_hits += rc.reused
         return rc
 
     def get(self, request_id) -> RequestCache:
@@ -149,14 +203,56 @@ class CacheManager:
         except KeyError:
             raise CacheError(f"request {request_id!r} is not live") from None
 
-    def release(self, request_id) -> None:
+    def release(self, request_id, tokens=None) -> None:
+        """The request is over: its pages and its slot come back.  With `tokens` (what the
+        positions of its cache hold, from the first on; it may know fewer or more than
+        `length`) and kept prefixes, the full pages that these tokens cover stay behind for a
+        request that begins alike."""
         rc = self.get(request_id)
+        keep = 0
+        if self.keep_prefixes and tokens is not None:
+            keep = min(len(tokens), rc.length) // self.page_size
+            digests = self._digests(tokens, keep)
+            for b in range(keep - 1, -1, -1):           # the deepest page first: it is the first to go
+                if digests[b] in self._kept:            # the same prefix is kept already: this copy is not needed
+                    for g in range(len(self.groups)):
+                        self.pools[g].give_back(rc.tables[g][b], request_id)
+                    continue
+                pages = tuple(rc.tables[g][b] for g in range(len(self.groups)))
+                for g, page in enumerate(pages):
+                    self.pools[g].hand_over(page, request_id, KEPT)
+                self._kept[digests[b]] = (pages, tuple(tokens[b * self.page_size:(b + 1) * self.page_size]))
         for g, table in enumerate(rc.tables):
-            for page in table:
+            for page in table[keep:]:
                 if page >= 0:
                     self.pools[g].give_back(page, request_id)
         del self.requests[request_id]
         self._free_slots.append(rc.slot)
+
+    # ------------------------------------------------------- kept prefixes
+    def _digests(self, tokens, n_pages: int) -> list:
+        """For each of the first n_pages pages, a digest of all tokens up to its end."""
+        out, h, ps = [], hashlib.blake2b(digest_size=16), self.page_size
+        for b in range(n_pages):
+            h.update(np.asarray(tokens[b * ps:(b + 1) * ps], dtype=np.int64).tobytes())
+            out.append(h.copy().digest())
+        return out
+
+    def _drop_oldest_kept(self) -> None:
+        if not self._kept:
+            return
+        _, (pages, _) = self._kept.popitem(last=False)
+        for g, page in enumerate(pages):
+            self.pools[g].give_back(page, KEPT)
+
+    def drop_kept(self) -> None:
+        """Gives every kept page back (nothing is reused after this until requests end again)."""
+        while self._kept:
+            self._drop_oldest_kept()
+
+    @property
+    def num_kept_pages(self) -> int:
+        return len(self._kept)
 
     @property
     def num_free_slots(self) -> int:
@@ -182,6 +278,7 @@ class CacheManager:
         return all(need <= pool.num_free for need, pool in zip(self.pages_needed(request_id, n_new), self.pools))
 
     def free_pages(self) -> list:
+        """Pages per group that can be taken now (kept prefixes give theirs up when asked)."""
         return [p.num_free for p in self.pools]
 
     def reserve(self, request_id, n_new: int) -> None:
@@ -256,6 +353,10 @@ class CacheManager:
                             raise CacheError(f"group {g}: page {page} in the table of {rid!r} is owned by "
                                              f"{pool.owner_of(page)!r}")
                         held.append(page)
+            for pages, tokens in self._kept.values():
+                if pool.owner_of(pages[g]) != KEPT or len(tokens) != self.page_size:
+                    raise CacheError(f"group {g}: kept page {pages[g]} is owned by {pool.owner_of(pages[g])!r}")
+                held.append(pages[g])
             if len(held) != len(set(held)):
                 raise CacheError(f"group {g}: a page is held twice")
             free = list(pool._free)

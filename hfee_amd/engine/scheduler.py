@@ -59,7 +59,8 @@ from .step import StepEntry
 @dataclass
 class Stats:
     """/root/reference/internal/llm/runner.go:15-21"""
-    prompt_tokens: int = 0
+    prompt_tokens: int = 0          # tokens of the prompt that were run (runner.go:222: what is fed)
+    reused_tokens: int = 0          # tokens of the prompt found in the cache from an earlier request
     prompt_duration: float = 0.0
     eval_tokens: int = 0
     eval_duration: float = 0.0
@@ -148,7 +149,7 @@ class Scheduler:
         return max(room or 0, 0)
 
     def _preempt(self, victim: Request) -> None:
-        self.engine.release(victim.request_id)
+        self.engine.release(victim.request_id, victim.history)
         self.running.remove(victim)
         victim.feed = list(victim.prompt) + list(victim.generated)
         victim.decoding = False
@@ -161,7 +162,9 @@ class Scheduler:
         if request.eval_started:
             request.stats.eval_duration = now - request.eval_started
         if self.engine.is_live(request.request_id):
-            self.engine.release(request.request_id)
+            # (position p of its cache holds history[p]; a last token that was drawn but never
+            # run, or run ahead and dropped, is beyond what the two have in common)
+            self.engine.release(request.request_id, request.history)
         if request in self.running:
             self.running.remove(request)
         finished.append(Finished(request, reason, error))
@@ -286,7 +289,14 @@ class Scheduler:
                 self._finish(r, "length", finished, "the cache has no free page for this request")
                 continue
             self.waiting.popleft()
-            self.engine.admit(r.request_id)
+            # the beginning of the prompt may lie in the cache from an earlier request
+            # (runner.go:198-223): whole pages, and never the whole prompt
+            reused = self.engine.admit(r.request_id, r.feed).length
+            if reused:
+                r.feed = r.feed[reused:]
+                if not r.stats.preemptions:
+                    r.stats.reused_tokens = reused
+                    r.stats.prompt_tokens = len(r.prompt) - reused
             r.admitted_order = self._order
             self._order += 1
             if not r.started:

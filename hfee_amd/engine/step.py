@@ -53,7 +53,7 @@ class Engine:
 
     def __init__(self, model: Model, *, num_pages=None, cache_tokens=None, page_size: int = 16,
                  max_requests: int = 64, max_batch_tokens: int = 2048, num_positions: int | None = None,
-                 device="cuda:0", use_graphs: bool = True):
+                 device="cuda:0", use_graphs: bool = True, keep_prefixes: bool = False):
         if not model.bound:
             raise ValueError("the model has no weights bound")
         if not torch.cuda.is_available():
@@ -70,7 +70,10 @@ class Engine:
                 cache_tokens = self.num_positions * max_requests
             num_pages = (cache_tokens + page_size - 1) // page_size
         self.num_pages = num_pages
-        self.cache = CacheManager(self.groups, page_size, num_pages, max_requests)
+        # (a finished request's full pages wait for a request that begins alike: only where every
+        # group keeps every token and no part has state that cannot be cut back)
+        keep_prefixes = bool(keep_prefixes) and all(g.kind == "full" for g in self.groups) and not model.state_specs()
+        self.cache = CacheManager(self.groups, page_size, num_pages, max_requests, keep_prefixes=keep_prefixes)
         self.storage = CacheStorage(self.groups, page_size, num_pages, max_requests, self.dtype, self.device)
         self.workspace = Workspace(max_batch_tokens, self.device)
         info = EngineInfo(self.num_positions, self.device, self.dtype, page_size, max_requests, self.storage)
@@ -90,14 +93,18 @@ class Engine:
         self.graph_replays = 0
 
     # ------------------------------------------------------------ requests
-    def admit(self, request_id):
-        rc = self.cache.admit(request_id)
+    def admit(self, request_id, tokens=None):
+        """tokens: the request's prompt; with kept prefixes the request starts with the pages
+        that hold its beginning (`.length` of what is returned: tokens that need not be run)."""
+        rc = self.cache.admit(request_id, tokens)
         self.storage.clear_slot(rc.slot)
         self._prepared = None
         return rc
 
-    def release(self, request_id):
-        self.cache.release(request_id)
+    def release(self, request_id, tokens=None):
+        """tokens: what the request's cache holds, position by position (prompt and generated
+        tokens); with kept prefixes its full pages stay behind for a request that begins alike."""
+        self.cache.release(request_id, tokens)
         self._prepared = None
 
     def is_live(self, request_id) -> bool:

@@ -118,3 +118,126 @@ def test_random_orders_keep_every_invariant(seed):
         m.release(rid)
     m.check()
     assert m.free_pages() == [40, 12] and m.num_free_slots == 5
+
+
+# ------------------------------------------------------- prefixes kept between requests
+def keeping(pages=16, requests=4, groups=1):
+    specs = [CacheGroupSpec("full", (2, 1, 16), (g,)) for g in range(groups)]
+    return CacheManager(specs, 16, pages, requests, keep_prefixes=True)
+
+
+def run_whole(m, rid, tokens):
+    rc = m.admit(rid, tokens)
+    m.reserve(rid, len(tokens) - rc.length)
+    m.commit(rid, len(tokens) - rc.length)
+    return rc
+
+
+def test_full_pages_of_a_released_request_wait_for_one_that_begins_alike():
+    m = keeping(pages=8, groups=2)
+    a = list(range(100, 140))                         # 40 tokens: two full pages and a half
+    rc = run_whole(m, "a", a)
+    pages = [list(t) for t in rc.tables]
+    m.release("a", a)
+    m.check()
+    assert m.num_kept_pages == 2 and m.free_pages() == [8, 8]          # kept pages count as free
+    # the same 32 tokens and then others: both pages come back, as this request's own, in every group
+    rc = m.admit("b", a[:32] + [7, 8, 9])
+    assert rc.length == rc.reused == 32 and [t[:2] for t in rc.tables] == [p[:2] for p in pages]
+    assert m.num_kept_pages == 0 and m.pages_needed("b", 3) == [1, 1]
+    m.check()
+    m.release("b", a[:32])
+    # exactly the kept tokens: one token must still be run (runner.go:219), so the second page stays
+    rc = m.admit("c", a[:32])
+    assert rc.length == 16 and m.num_kept_pages == 1
+    m.release("c", a[:16])
+    m.check()
+    # the first page differs in its last token: nothing is taken, although the second page's own tokens agree
+    rc = m.admit("d", a[:15] + [0] + a[16:40])
+    assert rc.length == 0 and m.num_kept_pages == 2
+    m.release("d")
+    # a page is known by everything before it as well: these 16 tokens behind another beginning are another page
+    rc = m.admit("e", [1] * 16 + a[16:40])
+    assert rc.length == 0
+    m.release("e")
+    m.check()
+
+
+def test_kept_pages_give_way_when_pages_are_needed_the_deepest_of_the_oldest_first():
+    m = keeping(pages=4)
+    a, b = list(range(200, 232)) + [1], list(range(300, 316)) + [1]
+    run_whole(m, "a", a)                      # pages 0, 1, 2
+    m.release("a", a)                         # two kept
+    run_whole(m, "b", b)                      # two more pages
+    m.release("b", b)                         # one kept
+    assert m.num_kept_pages == 3 and m.free_pages() == [4]
+    m.admit("c")
+    m.reserve("c", 32)                        # one page is free, the other comes from a's second page
+    assert m.num_kept_pages == 2
+    m.check()
+    assert m.admit("a2", a).length == 16      # a's first page is still there, its second is gone
+    assert m.admit("b2", b).length == 16
+    m.check()
+    m.release("a2"), m.release("b2")
+    with pytest.raises(OutOfPages):
+        m.reserve("c", 80)                    # five pages: nothing kept is left to give way
+    m.release("c", None)
+    m.drop_kept()
+    assert m.free_pages() == [4] and m.num_kept_pages == 0
+    m.check()
+
+
+def test_the_same_prefix_is_kept_once():
+    m = keeping(pages=8)
+    a = list(range(50, 83))
+    run_whole(m, "a", a)
+    m.admit("b")                              # the same tokens run again beside it (nothing was kept yet)
+    m.reserve("b", 33), m.commit("b", 33)
+    m.release("a", a), m.release("b", a)
+    assert m.num_kept_pages == 2 and len(m.pools[0]._free) == 6
+    m.check()
+
+
+def test_prefixes_are_not_kept_where_a_window_has_given_pages_back():
+    with pytest.raises(CacheError, match="every cache group keeps every token"):
+        CacheManager([CacheGroupSpec("window", (2, 1, 16), (0,), window=32)], 16, 8, 2, keep_prefixes=True)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_with_kept_prefixes(seed):
+    """Requests from a small family of prompts that begin alike come and go in random order on
+    few pages.  A model of the memory (what was written where) shows that every position of a
+    live request, taken over or written, holds that request's token, and check() that no page
+    is lost, held twice or both kept and owned."""
+    rng = random.Random(seed)
+    ps = 16
+    m = keeping(pages=12, requests=3)
+    stems = [[rng.randrange(1000) for _ in range(70)] for _ in range(2)]
+    content, live, n = {}, {}, 0          # (page, slot) -> token; rid -> its tokens
+    reused = 0
+    for _ in range(400):
+        if live and (len(live) == 3 or rng.random() < 0.4):
+            rid = rng.choice(sorted(live))
+            rc = m.get(rid)
+            assert [content[(rc.tables[0][p // ps], p % ps)] for p in range(rc.length)] == live[rid][:rc.length]
+            m.release(rid, live[rid] if rng.random() < 0.8 else None)
+            del live[rid]
+        else:
+            stem = rng.choice(stems)
+            tokens = stem[:rng.randrange(1, 70)] + [rng.randrange(1000) for _ in range(rng.randrange(0, 20))]
+            rid, n = n, n + 1
+            rc = m.admit(rid, tokens)
+            assert rc.length % ps == 0 and rc.length < len(tokens)
+            reused += rc.length
+            try:
+                m.reserve(rid, len(tokens) - rc.length)
+            except OutOfPages:
+                m.release(rid, tokens)            # only what it took over can stay behind
+                m.check()
+                continue
+            for p in range(rc.length, len(tokens)):
+                content[(rc.tables[0][p // ps], p % ps)] = tokens[p]
+            m.commit(rid, len(tokens) - rc.length)
+            live[rid] = tokens
+        m.check()
+    assert reused > 0

@@ -42,7 +42,9 @@ def test_seeded_sampling_does_not_depend_on_the_batch(model_folders, dtype):
         order = [2, 0, 1]
         again = llm.generate([prompts[i] for i in order], [params[i] for i in order])
         assert [o.token_ids for o in again] == [together[i].token_ids for i in order]
-    wide = LLM(folder, dtype=dtype, num_ctx=256, num_parallel=3, max_batch_tokens=256)
+    # (nothing kept between the calls: a prompt of which whole pages are found in the cache runs
+    # its rest as a smaller step, through other kernels, and bfloat16 rounds differently there)
+    wide = LLM(folder, dtype=dtype, num_ctx=256, num_parallel=3, max_batch_tokens=256, keep_prefixes=False)
     a = wide.generate(prompts, params)
     b = wide.generate(list(reversed(prompts)), list(reversed(params)))
     assert all(len(o.token_ids) == 24 for o in a) and len({tuple(o.token_ids) for o in a}) == 3
@@ -173,6 +175,37 @@ def test_a_prompt_given_as_text(model_folders, tmp_path):
     o = llm.generate([prompt], SamplingParams.greedy(num_predict=24, stop=(stop,)))[0]
     assert o.text == text[:text.index(stop)] and o.done_reason == "stop"
     assert len(o.token_ids) < len(want) and o.token_ids == want[:len(o.token_ids)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_conversation_that_goes_on_runs_only_what_is_new(model_folders, dtype):
+    """Through the entry point: the second call's prompt is the first prompt, its answer and a
+    few more tokens.  Whole pages of it are found in the cache (the statistics say how many
+    tokens were run, as the reference counts them), and the tokens are those of the plain
+    model over the whole prompt.  With keep_prefixes=False everything is run."""
+    from plain_llama import PlainLlama
+    from hfee_amd import LLM, SamplingParams
+    folder = model_folders[("A", dtype)]
+    plain = PlainLlama(folder)
+    prompt = tu.make_requests(256, [40], seed=12)["r0"]
+    llm = LLM(folder, dtype=dtype, num_ctx=128, num_parallel=2)
+    first = llm.generate([prompt], SamplingParams.greedy(num_predict=12))[0]
+    assert first.stats.prompt_tokens == 40 and first.stats.reused_tokens == 0
+    follow = prompt + first.token_ids + [3, 1, 4]
+    out = llm.generate([follow], SamplingParams.greedy(num_predict=10))[0]
+    assert out.stats.reused_tokens == 48 and out.stats.prompt_tokens == len(follow) - 48      # 51 tokens lie in the cache
+    want = plain.greedy(follow, 10)
+    if dtype == "float32":
+        assert out.token_ids == want
+    else:
+        assert tu.agree_until_a_near_tie(out.token_ids, want, tu.greedy_margins(plain, follow, want), "after a kept prefix") >= 3
+    plain_llm = LLM(folder, dtype=dtype, num_ctx=128, num_parallel=2, keep_prefixes=False)
+    plain_llm.generate([prompt], SamplingParams.greedy(num_predict=12))
+    again = plain_llm.generate([follow], SamplingParams.greedy(num_predict=10))[0]
+    assert again.stats.reused_tokens == 0 and again.stats.prompt_tokens == len(follow)
+    if dtype == "float32":
+        assert again.token_ids == out.token_ids
+    llm.engine.cache.check()
 
 
 def test_an_interrupted_call_leaves_nothing_behind(model_folders):

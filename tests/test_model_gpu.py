@@ -65,3 +65,59 @@ def test_a_step_planned_ahead_is_the_same_step(model_folders, dtype):
     plain, right, wrong = run(None), run("right"), run("wrong")
     for a, b, c in zip(plain, right, wrong):
         assert torch.equal(a, b) and torch.equal(a, c)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prefix_kept_from_an_earlier_request(model_folders, dtype):
+    """A request whose prompt begins with 50 tokens of an earlier one takes over the three full
+    pages that hold 48 of them and runs the rest: the logits are those of the plain model over
+    the whole prompt, in 32-bit bit for bit those of an engine that keeps nothing; the pages
+    are the same ones; and when other requests have needed the memory in between, the prefix
+    is gone and everything is run again, with the same result."""
+    from plain_llama import PlainLlama
+    from hfee_amd.engine import Engine, StepEntry, load_model
+    folder = model_folders[("B", dtype)]
+    plain = PlainLlama(folder)
+    model, cfg = load_model(folder, dtype)
+    g = torch.Generator().manual_seed(9)
+    stem = torch.randint(0, cfg.vocab_size, (50,), generator=g).tolist()
+    first = stem + torch.randint(0, cfg.vocab_size, (9,), generator=g).tolist()
+    second = stem + torch.randint(0, cfg.vocab_size, (21,), generator=g).tolist()
+    other = torch.randint(0, cfg.vocab_size, (100,), generator=g).tolist()
+
+    def run(eng, rid, tokens):
+        rc = eng.admit(rid, tokens)
+        have, pages = rc.length, list(rc.tables[0])
+        rest = tokens[have:]
+        logits = eng.step([StepEntry(rid, rest, list(range(len(rest))))]).clone()
+        return have, pages, logits
+
+    keeping = Engine(model, num_pages=8, page_size=16, max_requests=2, max_batch_tokens=128, keep_prefixes=True)
+    fresh = Engine(model, num_pages=8, page_size=16, max_requests=2, max_batch_tokens=128)
+    have, pages_first, _ = run(keeping, "first", first)
+    assert have == 0
+    pages_first = list(keeping.cache.get("first").tables[0])
+    keeping.release("first", first)
+    have, pages, got = run(keeping, "second", second)
+    assert have == 48 and pages == pages_first[:3]
+    _, _, want = run(fresh, "second", second)
+    ref = plain.forward(second)[48:]
+    assert rel_err(got, ref) < TOL[dtype]
+    if dtype == "float32":
+        assert torch.equal(got, want[48:])
+    else:
+        assert rel_err(got, want[48:]) < 2e-2
+    keeping.release("second", second)
+    keeping.cache.check()
+    # 100 tokens of something else take seven of the eight pages: what was kept has to go
+    keeping.admit("other", other)
+    keeping.step([StepEntry("other", other, [])])
+    keeping.release("other")
+    have, _, again = run(keeping, "third", second)
+    assert have < 48
+    assert rel_err(again[48 - have:], ref) < TOL[dtype]
+    if dtype == "float32":
+        assert torch.equal(again[48 - have:], got)
+    keeping.release("third")
+    keeping.cache.check()
+    assert keeping.cache.free_pages() == [8]

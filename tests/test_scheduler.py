@@ -14,20 +14,27 @@ EOS = 49
 
 
 class FakeEngine:
-    def __init__(self, num_pages, max_requests, page_size=16):
-        self.cache = CacheManager([CacheGroupSpec("full", (2, 1, 16), (0,))], page_size, num_pages, max_requests)
-        self.fed = {}          # request -> tokens in its cache
+    """Pages and their contents without a GPU: a step writes its tokens into the places that
+    the block table names, and the "logits" of a row are the tokens read back through the
+    table, so that a page that holds something else than its request's history shows."""
+
+    def __init__(self, num_pages, max_requests, page_size=16, keep_prefixes=False):
+        self.cache = CacheManager([CacheGroupSpec("full", (2, 1, 16), (0,))], page_size, num_pages, max_requests,
+                                  keep_prefixes=keep_prefixes)
+        self.content = {}      # (page, slot) -> token
         self.batches = []      # per step: [(request, n tokens, wants logits)]
         self.prepared = None   # the shape that the scheduler announced for the next step
         self.guesses = []      # per announced shape: did the next step have it?
 
-    def admit(self, rid):
-        self.fed[rid] = []
-        return self.cache.admit(rid)
+    def admit(self, rid, tokens=None):
+        return self.cache.admit(rid, tokens)
 
-    def release(self, rid):
-        self.cache.release(rid)
-        del self.fed[rid]
+    def release(self, rid, tokens=None):
+        self.cache.release(rid, tokens)
+
+    def held(self, rid):
+        rc, ps = self.cache.get(rid), self.cache.page_size
+        return [self.content[(rc.tables[0][p // ps], p % ps)] for p in range(rc.length)]
 
     def is_live(self, rid):
         return rid in self.cache.requests
@@ -50,14 +57,17 @@ class FakeEngine:
         if self.prepared is not None:
             self.guesses.append(self.prepared == [(e.request_id, len(e.tokens), list(e.want)) for e in entries])
             self.prepared = None
+        ps = self.cache.page_size
         for e in entries:
-            assert len(self.fed[e.request_id]) == self.cache.get(e.request_id).length
+            rc = self.cache.get(e.request_id)
+            start = rc.length
             self.cache.reserve(e.request_id, len(e.tokens))
-            self.fed[e.request_id] += list(e.tokens)
+            for i, t in enumerate(e.tokens):
+                self.content[(rc.tables[0][(start + i) // ps], (start + i) % ps)] = t
             self.cache.commit(e.request_id, len(e.tokens))
             assert e.want in ([], [len(e.tokens) - 1])
             if e.want:
-                rows.append(tuple(self.fed[e.request_id]))
+                rows.append(tuple(self.held(e.request_id)))
         self.batches.append([(e.request_id, len(e.tokens), bool(e.want)) for e in entries])
         self.cache.check()
         return rows
@@ -80,8 +90,8 @@ class FakeSampler:
         return out
 
 
-def make(num_pages=64, seqs=4, budget=32, ctx=256, eos=()):
-    eng = FakeEngine(num_pages, seqs)
+def make(num_pages=64, seqs=4, budget=32, ctx=256, eos=(), keep_prefixes=False):
+    eng = FakeEngine(num_pages, seqs, keep_prefixes=keep_prefixes)
     return eng, Scheduler(eng, FakeSampler(), max_num_seqs=seqs, max_batch_tokens=budget, num_ctx=ctx,
                           eos_token_ids=eos, clock=lambda: 0.0)
 
@@ -205,6 +215,71 @@ def test_random_arrivals_under_scarce_pages_never_preempt_an_older_request_for_a
                 assert done[i].request.generated == solo(p, i, n), (trial, i)
         eng.cache.check()
         assert eng.cache.free_pages() == [pages]
+
+
+def test_a_prompt_that_begins_like_an_earlier_request_runs_only_its_rest():
+    """/root/reference/internal/llm/runner.go:198-223: the longest common prefix of a free
+    slot's tokens is kept, at least one token is run, and the prompt count is what was run.
+    Here whole pages of 16 tokens: a shared beginning of 50 tokens saves 48."""
+    eng, s = make(keep_prefixes=True, budget=64)
+    stem = [(5 * j + 3) % (VOCAB - 1) for j in range(50)]
+    first, second = stem + [1, 2, 3], stem + [9, 8, 7, 6]
+    s.add(Request(0, first, SamplingParams.greedy(num_predict=20), seed=0))
+    done = run_all(s)
+    assert done[0].request.stats.prompt_tokens == 53 and done[0].request.stats.reused_tokens == 0
+    assert eng.cache.num_kept_pages == (53 + 20 - 1) // 16          # the last token was drawn, never run
+    answer = done[0].request.generated
+    steps_before = len(eng.batches)
+    s.add(Request(1, second, SamplingParams.greedy(num_predict=6), seed=1))
+    done = run_all(s)
+    st = done[1].request.stats
+    assert st.reused_tokens == 48 and st.prompt_tokens == 54 - 48
+    assert eng.batches[steps_before] == [(1, 6, True)]                # one step of six tokens, not of 54
+    assert done[1].request.generated == solo(second, 1, 6)            # (the sampler saw the whole history in the cache)
+    # the same prompt again: everything but the last page's worth is there; one token at least is run
+    s.add(Request(2, second, SamplingParams.greedy(num_predict=6), seed=1))
+    done = run_all(s)
+    assert done[2].request.stats.reused_tokens == 48 and done[2].request.generated == solo(second, 1, 6)
+    # a continuation of the first conversation finds prompt and answer
+    follow = first + answer + [4, 4]
+    s.add(Request(3, follow, SamplingParams.greedy(num_predict=3), seed=3))
+    done3 = run_all(s)[3]
+    assert done3.request.stats.reused_tokens == 64 and done3.request.generated == solo(follow, 3, 3)
+    eng.cache.check()
+    assert eng.cache.free_pages() == [64]
+
+
+def test_random_arrivals_with_kept_prefixes_under_scarce_pages_give_the_same_tokens():
+    """Prompts from a family with common beginnings, few pages, preemption: kept pages give
+    way, are taken over, come back: the tokens are those of each request alone without any
+    reuse (and the sampler checks at every draw that the cache holds the request's history)."""
+    import random
+    rng = random.Random(5)
+    reused = preempted = 0
+    for trial in range(30):
+        pages = rng.randint(4, 10)
+        eng, s = make(num_pages=pages, seqs=rng.randint(2, 4), budget=rng.choice([8, 24, 64]), keep_prefixes=True)
+        stem = [rng.randrange(VOCAB - 1) for _ in range(40)]
+        want, done = {}, {}
+        for i in range(rng.randint(3, 7)):
+            p = stem[:rng.randint(1, 40)] + [rng.randrange(VOCAB - 1) for _ in range(rng.randint(0, 6))]
+            n = rng.randint(1, 20)
+            want[i] = (p, n)
+            s.add(Request(i, p, SamplingParams.greedy(num_predict=n), seed=i))
+            for _ in range(rng.randint(0, 12)):           # the next one arrives a few steps later
+                if s.has_work():
+                    for f in s.step():
+                        done[f.request.request_id] = f
+                eng.cache.check()
+        done.update(run_all(s))
+        for i, (p, n) in want.items():
+            if done[i].error is None:
+                assert done[i].request.generated == solo(p, i, n), (trial, i)
+            reused += done[i].request.stats.reused_tokens
+            preempted += done[i].request.stats.preemptions
+        eng.cache.check()
+        assert eng.cache.free_pages() == [pages] and not eng.cache.requests
+    assert reused > 200 and preempted > 0
 
 
 def test_a_request_too_large_for_the_cache_ends_with_length():
