@@ -66,6 +66,10 @@ struct TileOps {
   Op v[2][NDT];
 };
 
+// The operand of s_waitcnt that waits until at most n vector memory operations are outstanding
+// and for nothing else (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
+constexpr int vmcnt_only(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+
 // 64 consecutive entries of a sequence's block table, one per lane, so that a tile's
 // page numbers come from a register shuffle instead of a load that the tile's own loads
 // would have to wait for.
@@ -139,9 +143,16 @@ __device__ __forceinline__ void load_tile(TileOps& ops, const bf16_t* __restrict
 // as NC operands.  pos: this slot's position (keys lo..pos are visible; -1 for an unused
 // slot).  key_op(c) and value_op(u, t) hand over the tile's operands: from registers, or
 // from a tile in LDS that several waves share.
-template <class KeyOp, class ValueOp>
+struct Nothing {
+  __device__ __forceinline__ void operator()() const {}
+};
+
+// under_scores(): what the caller wants issued behind the score products, while the matrix pipe
+// works on them (a request for a tile to come).
+template <class KeyOp, class ValueOp, class Under = Nothing>
 __device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyOp key_op, ValueOp value_op, int k0,
-                                                  int pos, int lo, float scale_log2, bool all_visible) {
+                                                  int pos, int lo, float scale_log2, bool all_visible,
+                                                  Under under_scores = Nothing()) {
   const int lane = threadIdx.x & 63, G = lane >> 5;
 
   // ---- S^T = K Q^T ------------------------------------------------------------
@@ -163,6 +174,9 @@ __device__ __forceinline__ void compute_tile_with(Tile& st, const Op* q_op, KeyO
   __builtin_amdgcn_sched_barrier(0);          // (the reads stay in front of the products)
 #pragma unroll
   for (int c = 0; c < NC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_ops[c], q_op[c].v, s, 0, 0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  under_scores();
+  __builtin_amdgcn_sched_barrier(0);
 
   // ---- mask, running maximum and sum ------------------------------------------
   // all_visible (the same for the whole wave): every key of the tile is visible to every
@@ -452,7 +466,36 @@ __device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds,
   typedef __attribute__((address_space(3))) void* lds_ptr;
   typedef const __attribute__((address_space(1))) void* global_ptr;
   const int block_a = k0 >> lay.page_shift, block_b = (k0 + 16) >> lay.page_shift;
-  if (pages.base < 0 || block_a < pages.base || block_b >= pages.base + 64) pages.fill(bt, bt_stride, block_a);
+  if (pages.base < 0 || block_a < pages.base || block_b >= pages.base + 64) {
+    pages.fill(bt, bt_stride, block_a);
+    // (every 64 pages.  The window is waited for here, where it is loaded: a load that may or may
+    // not be on its way when the loop comes round makes the compiler wait for every load in flight,
+    // the tiles to come among them, in front of each use of the window, in every step)
+    if constexpr (BUFFER) __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+  }
+  if constexpr (BUFFER && NC % WAVES == 0) {
+    // A wave issues an instruction every four to five cycles, and what is computed per request
+    // stands in every step's chain.  With the key chunks a whole number of rounds of the waves, a
+    // wave's first NC / WAVES blocks are keys and the rest values, whichever wave it is: a key
+    // block's lanes choose between the two pages once for all key blocks, and everything that is
+    // the same for all lanes goes into the load's scalar offset; a value block lies in one page,
+    // so its lanes' offsets never change at all.  (The layer is smaller than 4 GB here.)
+    // (No look at kv_first..kv_last: a block table holds page 0 where a sequence has no page, or
+    // no longer has one, and whatever a page holds is finite; keys out of range are masked.)
+    const uint32_t page_bytes = (uint32_t)lay.page_stride * 2u;
+    const uint32_t a32 = (uint32_t)__builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_a - pages.base)) * page_bytes;
+    const uint32_t b32 = (uint32_t)__builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_b - pages.base)) * page_bytes;
+    const uint32_t in_a = (uint32_t)(k0 & (lay.page_size - 1)), in_b = (uint32_t)((k0 + 16) & (lay.page_size - 1));
+    const uint32_t s_key = in_a * (uint32_t)lay.head_dim * 2u, s_va = a32 + in_a * 2u, s_vb = b32 + in_b * 2u;
+    const uint32_t lane_page = w.second[0] ? b32 : a32;            // (block 0 of a wave is a key block)
+#pragma unroll
+    for (int j = 0; j < WaveBlocks<WAVES>::J; ++j) {
+      lds_ptr dst = (lds_ptr)(tile_lds + (wave + WAVES * j) * 1024);
+      if (j < NC / WAVES) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, dst, 16, lane_page + w.lane_off[j], s_key, 0, 0);
+      else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, dst, 16, w.lane_off[j], w.kind[j] == 2 ? s_vb : s_va, 0, 0);
+    }
+    return;
+  }
   // pages outside kv_first..kv_last may have been given back: page 0 is read instead
   const bool ok_a = k0 <= kv_last && k0 + 15 >= kv_first, ok_b = k0 + 16 <= kv_last && k0 + 31 >= kv_first;
   const int page_a = ok_a ? __builtin_amdgcn_readlane(pages.page, __builtin_amdgcn_readfirstlane(block_a - pages.base)) : 0;
@@ -481,10 +524,6 @@ __device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds,
     }
   }
 }
-
-// The operand of s_waitcnt that waits until at most n vector memory operations are outstanding
-// and for nothing else (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
-constexpr int vmcnt_only(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 
 // work: per row tile 4 ints (first row, rows <= 32, first position, block-table row).
 // WAVES: the waves of a workgroup if they are SHARED_WAVES, 0 for any other number.
@@ -542,12 +581,12 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
   const WaveBlocks<WAVES == 0 ? 1 : WAVES> mine = wave_blocks<WAVES == 0 ? 1 : WAVES>(lay, kvh, wave);
   // (a raw buffer of 32-bit data over the layer; only the ring's loads go through it)
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cache, 0, (int)layer_bytes, 0x00020000);
-  auto compute = [&](int t, const char* tile_at) {
+  auto compute = [&](int t, const char* tile_at, auto under_scores) {
     const char* cur = tile_at + lane * 16;
     compute_tile_with(
         st, q_op, [&](int c) { return *reinterpret_cast<const bf16x8*>(cur + c * 1024); },
         [&](int u, int tt) { return *reinterpret_cast<const bf16x8*>(cur + (NC + u * NDT + tt) * 1024); }, t * 32, pos, lo,
-        scale_log2, t * 32 >= all_first && t * 32 + 31 <= pos0);
+        scale_log2, t * 32 >= all_first && t * 32 + 31 <= pos0, under_scores);
   };
   if constexpr (RING) {
     // Every wave brings the same number of blocks of a tile, so a wave can wait for its loads by
@@ -583,8 +622,12 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
       asm volatile("" ::: "memory");
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
-      if (t + SHARED_TILES - 1 < t_end) request(t + SHARED_TILES - 1);
-      compute(t, kv_lds + ((t - t_first) % SHARED_TILES) * TILE_BYTES);
+      // (the request behind the tile's score products: asked for right after the barrier, the
+      // sixteen loads of a workgroup's four waves meet at the CU's one path into LDS, and a wave
+      // stands four hundred cycles at its four loads before it reads its first operand)
+      compute(t, kv_lds + ((t - t_first) % SHARED_TILES) * TILE_BYTES, [&]() {
+        if (t + SHARED_TILES - 1 < t_end) request(t + SHARED_TILES - 1);
+      });
     }
   } else {
     auto request = [&](int t) {
@@ -598,7 +641,7 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
     __syncthreads();               // waits for the loads too
     for (int t = t_first; t < t_end; ++t) {
       if (t + 1 < t_end) request(t + 1);
-      compute(t, kv_lds + ((t - t_first) & 1) * TILE_BYTES);
+      compute(t, kv_lds + ((t - t_first) & 1) * TILE_BYTES, Nothing());
       __syncthreads();             // the next tile has landed; nobody reads this one any more
     }
   }
