@@ -219,6 +219,58 @@ __device__ __forceinline__ void row_scales(const Args& a, float* out) {
   }
 }
 
+// The same in three parts, for kernels that end in an exchange through LDS anyway: the loads are
+// asked for at the start and nothing waits for them there (row_scales' barrier, standing in
+// front of the loop, kept every wave from asking for its next weights until the shares, which
+// the product before has only just written, had come from memory: 1.4 us a product inside the
+// decode step); the sums go into LDS together with the kernel's own partial sums, in front of the
+// barrier that those need, and a finishing thread adds the waves' parts up for its row.  One
+// round of loads: scale_blocks <= Shares<TILES>::BLOCKS (else row_scales).
+template <int TILES>
+struct Shares {
+  static constexpr int ROUND = TILES == 1 ? 16 : 8;
+  static constexpr int BLOCKS = ROUND * WAVES * 4;
+  float v[ROUND][TILES];
+};
+
+template <int TILES>
+__device__ __forceinline__ void ask_shares(const Args& a, Shares<TILES>& sh) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, j = lane >> 4;
+#pragma unroll
+  for (int r = 0; r < Shares<TILES>::ROUND; ++r) {
+    const int b = min(wave * 4 + j + r * WAVES * 4, a.scale_blocks - 1);       // past the end: a repeat that is not added
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+      sh.v[r][t] = 0.f;
+      if (r * WAVES * 4 < a.scale_blocks)        // (the same for everybody: whole rounds beyond the end are not asked for)
+        sh.v[r][t] = a.scale_ss[(int64_t)b * SS_STRIDE + min(t * 16 + m16, a.M - 1)];
+    }
+  }
+}
+
+// part: [WAVES][SS_STRIDE] floats of LDS; the caller's barrier follows.
+template <int TILES>
+__device__ __forceinline__ void put_shares(const Args& a, const Shares<TILES>& sh, float (*part)[SS_STRIDE]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, j = lane >> 4;
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) {
+    float v = 0.f;
+#pragma unroll
+    for (int r = 0; r < Shares<TILES>::ROUND; ++r) v += wave * 4 + j + r * WAVES * 4 < a.scale_blocks ? sh.v[r][t] : 0.f;
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    if (j == 0) part[wave][t * 16 + m16] = v;
+  }
+}
+
+// after the barrier: 1/sqrt(mean of squares + eps) of batch row m
+__device__ __forceinline__ float scale_of(const Args& a, const float (*part)[SS_STRIDE], int m) {
+  float v = 0.f;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) v += part[w][m];
+  return 1.0f / sqrtf(v / (float)a.K + a.scale_eps);
+}
+
 // What happens to four finished sums: weight rows n .. n+3 of batch row m.
 template <int EPI>
 __device__ __forceinline__ void epilogue(const Args& a, int m, int n, float* v) {
@@ -318,10 +370,13 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   __shared__ float partial[WAVES][MT][64][4];
   __shared__ float ss_part[WAVES][MT][16];
   __shared__ float row_scale[SS_STRIDE];
+  __shared__ float share_part[WAVES][SS_STRIDE];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * ROWS;
+  const bool scaled = !NORM && a.scale_ss != nullptr, late = scaled && a.scale_blocks <= Shares<MT>::BLOCKS;
+  Shares<MT> shares;
   // rows beyond N lie in the last row of tiles (zeros), rows beyond M read a valid row; what
   // they produce is never stored
   const bf16_t* w_row = WeightTiles::lane_place(a.W, a.w_stride, n0 + r16, g);
@@ -361,7 +416,8 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
     int kb = threadIdx.x >> 6;
     if (kb < nfull) load_block<MT, NORM, U>(cur, xcur, w_row, x_rows, a, kb * KBLOCK);
     // (behind the first loads of W, so that it costs no latency of its own)
-    if (!NORM && a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
+    if (late) ask_shares<MT>(a, shares);
+    else if (scaled) row_scales<MT>(a, row_scale);
     while (kb < nfull) {
       const int kn = kb + WAVES;
       if (kn < nfull) load_block<MT, NORM, U>(nxt, xnxt, w_row, x_rows, a, kn * KBLOCK);
@@ -417,6 +473,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
       if (g == 0) ss_part[wave][t][r16] = s;
     }
   }
+  if (late) put_shares<MT>(a, shares, share_part);
   __syncthreads();
 
   // D layout of the 16x16 tile: register i of lane l is weight row 4*(l/16) + i, batch row l%16
@@ -442,7 +499,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= scale;
     } else if (a.scale_ss != nullptr) {
-      const float scale = row_scale[min(m, SS_STRIDE - 1)];
+      const float scale = late ? scale_of(a, share_part, min(m, SS_STRIDE - 1)) : row_scale[min(m, SS_STRIDE - 1)];
 #pragma unroll
       for (int i = 0; i < 4; ++i) v[i] *= scale;
     }
@@ -897,7 +954,13 @@ __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups
   Chunk ring[RING];
 #pragma unroll
   for (int s = 0; s < RING; ++s) ring[s].u = load_streamed(reinterpret_cast<const u32x4*>(w_cur + koff(s) * WeightTiles::PER_COLUMN));
-  if (!NORM && a.scale_ss != nullptr) {      // (behind the first loads of W: it costs no latency of its own)
+  __shared__ float share_part[WAVES][SS_STRIDE];
+  const bool scaled = !NORM && a.scale_ss != nullptr;
+  bool late = scaled && a.scale_blocks <= Shares<1>::BLOCKS;      // the shares meet at the first row group's barrier
+  Shares<1> shares;
+  if (late) {
+    ask_shares<1>(a, shares);
+  } else if (scaled) {
     __shared__ float row_scale[SS_STRIDE];
     row_scales<1>(a, row_scale);
     __syncthreads();
@@ -918,7 +981,12 @@ __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) partial[wave][lane][i] = acc[i];
+    if (late) put_shares<1>(a, shares, share_part);
     __syncthreads();
+    if (late) {
+      scale = scale_of(a, share_part, min(r16, a.M - 1));
+      late = false;
+    }
     if (wave == 0) {
       // register i of lane l: weight row 4*(l/16) + i, batch row l%16
       const int m = r16, n = rg * ROWS + 4 * g;
