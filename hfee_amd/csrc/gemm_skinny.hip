@@ -792,7 +792,12 @@ __global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_gr
 #pragma unroll
   for (int st = 0; st < RING; ++st) ring[st].u = load_streamed(reinterpret_cast<const u32x4*>(w_cur + st * WeightTiles::TILE));
   put(fill, 0);
-  if (a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
+  // (the rows' shares meet at the first slice's barrier: see ask_shares; with one slice there is none)
+  __shared__ float share_part[WAVES][SS_STRIDE];
+  bool late = a.scale_ss != nullptr && slices > 1 && a.scale_blocks <= Shares<MT>::BLOCKS;
+  Shares<MT> shares;
+  if (late) ask_shares<MT>(a, shares);
+  else if (a.scale_ss != nullptr) row_scales<MT>(a, row_scale);
   __syncthreads();
 
   int buf = 0;
@@ -826,7 +831,12 @@ __global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_gr
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       }
       put(fill, buf ^ 1);          // read last in the slice before this one: everybody has passed that barrier
+      if (late && s == 0) put_shares<MT>(a, shares, share_part);
       __syncthreads();
+      if (late && s == 0) {        // (read after the next slice's barrier at the earliest)
+        if (threadIdx.x < MT * 16) row_scale[threadIdx.x] = scale_of(a, share_part, threadIdx.x);
+        late = false;
+      }
       buf ^= 1;
     }
     if (rg < row_groups) {
