@@ -177,7 +177,8 @@ def run(args):
     steps_total = args.steps + args.warmup
 
     page_size = 16
-    tokens_cached = max_batch * (PROMPT + steps_total + page_size) + PREFILL + page_size
+    # (while the later prompts are read, the earlier requests already decode: a token a step)
+    tokens_cached = max_batch * (PROMPT + steps_total + page_size + max_batch * PROMPT // PREFILL) + PREFILL + page_size
     if args.serving:
         context = min(context, 4096)
         tokens_cached = args.serving * (2048 + 128 + page_size)
