@@ -22,8 +22,20 @@ def _dt(t: torch.Tensor) -> int:
         raise KernelError(f"unsupported dtype {t.dtype}") from None
 
 
+_DEVICE = None
+
+
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """The current stream's handle (asked for at every launch: under graph capture it is another one).
+    torch's own accessor for the raw handle: `torch.cuda.current_stream()` builds a Python object
+    and took 9 us a launch, a quarter of the host's time in a step that is not replayed from a graph."""
+    global _DEVICE
+    if _DEVICE is None:
+        _DEVICE = torch.cuda.current_device()
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is None:
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return ctypes.c_void_p(raw(_DEVICE))
 
 
 def _ptr(t):
