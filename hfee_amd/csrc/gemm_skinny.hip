@@ -1040,10 +1040,11 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
   }
   const int row_groups = (a.N + ROWS - 1) / ROWS;
   if (a.M > 16 || a.K % (128 * WAVES) != 0 || a.K > 16 * 32 * WAVES) return false;
-  // converting the batch rows once per workgroup pays when a workgroup walks several
-  // row groups; with the norm folded in it pays from two on
+  // from two row groups a workgroup on: the workgroups then share the weight rows evenly, where
+  // one row group each leaves a second round that fills a part of the chip only (q/k/v of the 8B
+  // shape, 384 row groups: 1.5 us a layer inside the decode step)
   const int per = (row_groups + num_cus - 1) / num_cus;       // row groups per workgroup, all but equal
-  if (per < (norm ? 2 : 4)) return false;
+  if (per < 2) return false;
   const int grid = (row_groups + per - 1) / per;
 #define GO(NORM_, E) return launch_wide_steps<NORM_, E>(a, row_groups, grid, stream)
   if (norm) {
