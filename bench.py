@@ -173,7 +173,7 @@ def run(args):
     layer_params = d * (H + 2 * K) * hd + H * hd * d + 3 * d * F
     weight_bytes = 2 * (L * layer_params + V * d)              # every matrix a decode step reads, once
     kv_bytes_per_token = L * 2 * K * hd * 2
-    max_batch = max(64, args.batch, args.serving)
+    max_batch = max(64 if args.no_points else 128, args.batch, args.serving)
     steps_total = args.steps + args.warmup
 
     page_size = 16
@@ -353,7 +353,7 @@ def run(args):
         line["prefill"] = {"value": round(PREFILL / pt, 1), "tokens": PREFILL, "ms": round(pt * 1e3, 3),
                            "frac": round(flops / pt / BF16_PEAK, 4)}
         points = {}
-        for b in (() if getattr(args, "only_prefill_point", False) else (1, 64)):
+        for b in (() if getattr(args, "only_prefill_point", False) else (1, 64, 128)):
             steps = max(8, min(args.steps, 64))
             dtb, _ = decode_run(b, steps, min(args.warmup, 4))
             points[f"decode_b{b}"] = round(b * steps / dtb, 2)
