@@ -476,6 +476,34 @@ def test_steps_launched_ahead_give_the_same_tokens_and_reasons(pages):
     engine.cache.check()
 
 
+@pytest.mark.parametrize("pages", [40, 12])
+def test_steps_launched_ahead_with_kept_prefixes(pages):
+    """Both together: requests that begin alike arrive one after the other, end on an
+    end-of-sequence id or at their limit while a step made ahead for them is under way, leave
+    their full pages behind and the next one takes them over, with pages to spare and with few.
+    The tokens are those of a scheduler that waits for every step and keeps nothing; the
+    sampler checks at every draw that the cache holds the request's history."""
+    stem = [(11 * j + 5) % (VOCAB - 1) for j in range(70)]
+    limits = [30, 12, 25, 18, 40, 9]
+    def arrivals():
+        reqs = [Request(i, stem[:20 + 9 * i] + [i, i + 1], SamplingParams.greedy(num_predict=limits[i]), seed=i) for i in range(6)]
+        return {0: reqs[:2], 14: reqs[2:3], 50: reqs[3:5], 90: reqs[5:]}
+    _, plain = run_staggered(FakeEngine(64, 3), FakeSampler(), arrivals(), seqs=3)
+    tokens = [t for f in plain.values() for t in f.request.generated[2:-2]]
+    eos = max(set(tokens), key=tokens.count)
+    _, plain = run_staggered(FakeEngine(64, 3), FakeSampler(), arrivals(), eos=[eos], seqs=3)
+    assert any(f.reason == "stop" for f in plain.values()) and any(f.reason == "length" for f in plain.values())
+    engine = DeviceTokenEngine(pages, 3, keep_prefixes=True)
+    sched, ahead = run_staggered(engine, DeviceIdsSampler(), arrivals(), eos=[eos], seqs=3)
+    assert sched.steps_ahead > 10
+    for rid in plain:
+        assert ahead[rid].error is None and ahead[rid].request.generated == plain[rid].request.generated, rid
+        assert ahead[rid].reason == plain[rid].reason
+    assert sum(f.request.stats.reused_tokens for f in ahead.values()) >= 48
+    engine.cache.check()
+    assert engine.cache.free_pages() == [pages] and not engine.cache.requests
+
+
 def test_a_penalty_on_earlier_tokens_is_launched_ahead_too_and_a_cancellation_ends_it():
     ps = prompts()
     engine = DeviceTokenEngine(64, 4)
