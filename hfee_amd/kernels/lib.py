@@ -27,7 +27,7 @@ _CORE_SIGNATURES = {
     "hfee_rmsnorm": [P, I, P, P, I, P, F, I, I, P],
     "hfee_swiglu": [P, L, P, P, L, I, I, I, I, P],
     "hfee_residual_add": [P, P, I, L, P],
-    "hfee_rope_cache_write": [P, L, P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, P, I, I, I, I, I, P],
+    "hfee_rope_cache_write": [P, L, P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, P, I, I, I, I, I, I, P],
     "hfee_gemm_f32": [P, L, P, L, P, L, I, I, I, I, P],
     "hfee_attention_ref": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "hfee_gemm_bf16": [P, I, L, P, L, P, L, I, I, I, I, P, L, P],

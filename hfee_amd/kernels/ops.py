@@ -196,8 +196,10 @@ def tiled_plan(m: int, n: int, k: int) -> tuple:
 
 def rope_cache_write(q, k, v, positions, token_segment, block_tables, cos, sin, pairing: int,
                      cache_layer, num_heads: int, kv_heads: int, head_dim: int, page_size: int,
-                     max_position: int):
+                     max_position: int, portions: bool = True):
     """Rotates q in place, writes rotated k and v into the pages of `cache_layer`.
+    portions: the tokens hold runs of consecutive positions (portions of prompts); False for
+    single tokens of many sequences, whose values are then written by each token's own workgroup.
     q, k, v: 2-D views [n, heads * head_dim] (any leading dimension), or None.
     cos/sin: [positions, half] float32 or None (no rotation).  cache_layer:
     [pages, 2, kv_heads, page_size * head_dim] or None (no write)."""
@@ -233,7 +235,7 @@ def rope_cache_write(q, k, v, positions, token_segment, block_tables, cos, sin, 
                     block_tables.stride(0) if k is not None else 0,
                     _ptr(cos), _ptr(sin), half, pairing, table_positions, max_position,
                     _ptr(cache_layer if k is not None else None), num_heads, kv_heads, head_dim, page_size,
-                    n, _stream())
+                    n, int(portions), _stream())
 
 
 def attention_plain(out, q, cache_layer, positions, token_segment, block_tables, num_heads: int,

@@ -171,8 +171,10 @@ class Attention(Mixer):
             else:   # this run of the layer reads keys and values that another run wrote
                 ops.linear(q, hn, self.w_qkv[:self.q_width])
                 k = v = None
+            portions = self.dtype != torch.bfloat16 or ctx.extra["attention.tiles"].shape[0] > 0
             ops.rope_cache_write(q, k, v, ctx.positions, ctx.token_segment, tables, cos, sin, self.pairing,
-                                 cache if writes_cache else None, H, K, hd, ctx.page_size, ctx.max_position)
+                                 cache if writes_cache else None, H, K, hd, ctx.page_size, ctx.max_position,
+                                 portions=portions)
         att = ctx.rows("attention.out", self.q_width)
         if self.dtype == torch.float32:
             ops.attention_plain(att, q, cache, ctx.positions, ctx.token_segment, tables, H, K, hd,

@@ -671,6 +671,12 @@ def test_rope_cache_write_of_long_portions(ps):
                              torch.zeros(1, dtype=torch.int32, device=DEV), tables[int(seg[t]):int(seg[t]) + 1].to(DEV),
                              *args, one_by_one, H, K, hd, ps, int(pos.max()))
     assert torch.equal(layer, one_by_one)
+    # and told that the tokens are no portions (single tokens of many sequences): every token's own
+    # workgroup writes its values; the same cache
+    alone = torch.zeros_like(layer)
+    ops.rope_cache_write(q.clone().to(DEV), k.to(DEV), v.to(DEV), pos.to(DEV), seg.to(DEV), tables.to(DEV), *args,
+                         alone, H, K, hd, ps, int(pos.max()), portions=False)
+    assert torch.equal(layer, alone)
     lay = layer.cpu()
     for t in range(T):
         p = int(pos[t])
