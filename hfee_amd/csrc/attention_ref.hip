@@ -40,8 +40,10 @@ __global__ __launch_bounds__(64) void attention_ref_kernel(
     const int j = base + lane;
     if (j >= lo && j <= pos) {
       const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
+      const int kc = lay.key_chunk();
+      const int64_t chunk_stride = lay.key_chunk_stride();
       float s = 0.f;
-      for (int d = 0; d < hd; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
+      for (int d = 0; d < hd; ++d) s = fmaf(qs[d], to_float<T>(kr[(d / kc) * chunk_stride + d % kc]), s);
       m = fmaxf(m, s * scale);
     }
   }
@@ -55,8 +57,10 @@ __global__ __launch_bounds__(64) void attention_ref_kernel(
     float e = 0.f;
     if (j >= lo && j <= pos) {
       const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
+      const int kc = lay.key_chunk();
+      const int64_t chunk_stride = lay.key_chunk_stride();
       float s = 0.f;
-      for (int d = 0; d < hd; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
+      for (int d = 0; d < hd; ++d) s = fmaf(qs[d], to_float<T>(kr[(d / kc) * chunk_stride + d % kc]), s);
       e = expf(s * scale - m);
       lsum += e;
     }

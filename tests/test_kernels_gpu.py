@@ -15,6 +15,15 @@ def vslot(s):
     return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1)
 
 
+def kslot(keys, ps, hd, s):
+    """Where the cache keeps the key of slot s of one (page, head): `keys` is that head's
+    ps * hd elements; chunks of 16 dims lie together ([hd / 16][slot][16]) where hd is a
+    multiple of 16, else a key's dims in a row.  A view of shape [hd / chunk, chunk]: assign
+    `k.view(-1, chunk)` to it, or read it with `.reshape(hd)`."""
+    kc = 16 if hd % 16 == 0 else hd
+    return keys.view(hd // kc, ps, kc)[:, s, :]
+
+
 def close(a, b, tol):
     """|a - b| <= tol * (1 + |b|), the reference's form (/root/reference/internal/ggml/q8_test.go:24-26)."""
     a, b = a.double().cpu(), b.double().cpu()
@@ -442,7 +451,7 @@ def _check_fused_qkv(H, K, hd, half, M, norm, d, **kw):
         p = int(pos[m])
         page, slot = int(tables[m, p // ps]), p % ps
         for kh in range(K):
-            close(lay[page, 0, kh].view(ps, hd)[slot], k_ref[m, kh], 2e-2)
+            close(kslot(lay[page, 0, kh], ps, hd, slot).reshape(hd), k_ref[m, kh], 2e-2)
             close(lay[page, 1, kh].view(hd, ps)[:, vslot(slot)], v_ref[m, kh], 2e-2)
     assert int((lay != 0).sum()) <= M * 2 * K * hd, "nothing but the tokens' own slots is written"
 
@@ -490,7 +499,7 @@ def _paged(kv, page_size, pages_order):
         for s in range(min(page_size, T - b * page_size)):
             t = b * page_size + s
             for h in range(K):
-                layer[p, 0, h].view(page_size, hd)[s] = kv[0][t, h]
+                kslot(layer[p, 0, h], page_size, hd, s)[:] = kv[0][t, h].view(-1, 16 if hd % 16 == 0 else hd)
                 layer[p, 1, h].view(hd, page_size)[:, vslot(s)] = kv[1][t, h]
     return layer, torch.tensor([pages_order[:nblocks]], dtype=torch.int32)
 
@@ -634,7 +643,7 @@ def test_rope_cache_write(pairing, dtype):
         p = int(pos[t])
         page, slot = [2, 0, 3, 1][p // ps], p % ps
         for h in range(K):
-            close(lay[page, 0, h].view(ps, hd)[slot], k_ref[t, h], tol)
+            close(kslot(lay[page, 0, h], ps, hd, slot).reshape(hd), k_ref[t, h], tol)
             assert torch.equal(lay[page, 1, h].view(hd, ps)[:, vslot(slot)], v[t].view(K, hd)[h])
 
 
@@ -751,7 +760,7 @@ def test_attention_over_long_contexts(H, K, hd, ps, ctx):
         for kh in range(K):
             rows = q[:T] if b == 0 else q[T + b:T + b + 1]
             mean = rows.float().view(-1, H, hd)[:, kh * (H // K)].mean(0)
-            cache[page, 0, kh].view(ps, hd)[slot] = (mean / mean.norm() * 30).to(torch.bfloat16)
+            kslot(cache[page, 0, kh], ps, hd, slot)[:] = (mean / mean.norm() * 30).to(torch.bfloat16).view(-1, 16)
     positions = torch.cat([torch.arange(ctx - T, ctx), torch.tensor([ctx - 1, ctx - 8])]).to(torch.int32).to(DEV)
     seg = torch.tensor([0] * T + [0, 1], dtype=torch.int32, device=DEV)
     ref = torch.zeros(T + B, H * hd, dtype=torch.bfloat16, device=DEV)

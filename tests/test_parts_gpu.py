@@ -16,6 +16,15 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+def kslot(keys, ps, hd, s):
+    """Where the cache keeps the key of slot s of one (page, head): `keys` is that head's
+    ps * hd elements; chunks of 16 dims lie together ([hd / 16][slot][16]) where hd is a
+    multiple of 16, else a key's dims in a row.  A view of shape [hd / chunk, chunk]: assign
+    `k.view(-1, chunk)` to it, or read it with `.reshape(hd)`."""
+    kc = 16 if hd % 16 == 0 else hd
+    return keys.view(hd // kc, ps, kc)[:, s, :]
+
+
 def vslot(s):
     """Where the cache keeps slot s of a value column: bits 2 and 3 exchanged."""
     return (s & ~12) | ((s & 4) << 1) | ((s & 8) >> 1)
@@ -609,7 +618,8 @@ def test_attention_finds_a_far_key_among_hundreds():
             layer = torch.zeros(nblocks + 3, 2, K, ps * hd)
             for t in range(T):
                 p, s = order[t // ps], t % ps
-                layer[p, 0].view(K, ps, hd)[:, s] = k[t]
+                for kh in range(K):
+                    kslot(layer[p, 0, kh], ps, hd, s)[:] = k[t].view(K, -1, 16 if hd % 16 == 0 else hd)[kh]
                 layer[p, 1].view(K, hd, ps)[:, :, vslot(s)] = v[t]
             layer = layer.to(dtype).to(DEV)
             table = torch.tensor([order], dtype=torch.int32, device=DEV)
@@ -665,7 +675,8 @@ def test_attention_window_edge():
                 layer = torch.full((nblocks + 2, 2, K, ps * hd), 9.0)
                 for t in range(T):
                     p, sl = order[t // ps], t % ps
-                    layer[p, 0].view(K, ps, hd)[:, sl] = k[t]
+                    for kh in range(K):
+                        kslot(layer[p, 0, kh], ps, hd, sl)[:] = k[t].view(K, -1, 16 if hd % 16 == 0 else hd)[kh]
                     layer[p, 1].view(K, hd, ps)[:, :, vslot(sl)] = v[t]
                 layer = layer.to(dtype).to(DEV)
                 table = torch.tensor([order], dtype=torch.int32, device=DEV)
