@@ -9,12 +9,11 @@
 //   SiLU gate   internal/ggml/ops.go:159-165  (g / (1 + exp(-g)) * up)
 //   residual    internal/ggml/ops.go:152-157
 #include "common.h"
+#include "gemm_entry.h"
 
 using namespace hfee;
 
 HFEE_DEFINE_LAST_ERROR
-
-enum { DT_F32 = 0, DT_BF16 = 1 };
 
 // ------------------------------------------------------------------ embedding
 template <typename T>

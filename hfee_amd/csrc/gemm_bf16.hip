@@ -582,6 +582,88 @@ __global__ __launch_bounds__(256) void gemm_split_finish_kernel(void* __restrict
   }
 }
 
+// What comes after a product that adds into the residual stream: the norm of the new rows.
+// normed null: no norm.
+struct NormAfter {
+  bf16_t* normed = nullptr;     // [M, N] bfloat16, rows ldn apart
+  int64_t ldn = 0;
+  const void* weight = nullptr; // [N]
+  bool weight_is_f32 = false;
+  float eps = 0.f;
+};
+
+// The second kernel of a cut product that adds into the residual stream, together with the
+// norm that reads the new rows next: one workgroup a row, which stays in registers between
+// the sum of its squares and the scaling.  The same sums in the same order as
+// gemm_split_finish_kernel followed by the norm's own kernel.  N a multiple of 4 and at
+// most 16 * blockDim.x; rows of C, of the partial products and of normed aligned for
+// 16-byte (normed: 8-byte) accesses.
+template <typename TW, int NV>
+__global__ void gemm_split_finish_norm_kernel(float* __restrict__ C, int64_t ldc, const float* __restrict__ partial,
+                                              int splits, int M, int N, bf16_t* __restrict__ normed, int64_t ldn,
+                                              const TW* __restrict__ w, float eps) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  constexpr int MOST = 8;
+  f32x4 v[NV];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int n = 4 * (threadIdx.x + i * blockDim.x);
+    v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (n < N) {
+      f32x4 part[MOST];
+#pragma unroll
+      for (int z = 0; z < MOST; ++z)      // all asked for together; past the last one: a repeat that is not added
+        part[z] = *reinterpret_cast<const f32x4*>(partial + ((int64_t)min(z, splits - 1) * M + m) * N + n);
+      f32x4* c = reinterpret_cast<f32x4*>(C + (int64_t)m * ldc + n);
+      const f32x4 old = *c;
+      f32x4 sum = part[0];
+#pragma unroll
+      for (int z = 1; z < MOST; ++z)
+        if (z < splits) sum += part[z];
+      sum += old;
+      *c = sum;
+      v[i] = sum;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss = fmaf(v[i][e], v[i][e], ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)N + eps);
+  bf16_t* o = normed + (int64_t)m * ldn;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int n = 4 * (threadIdx.x + i * blockDim.x);
+    if (n < N) {
+      u32x2 y;
+      y[0] = (uint32_t)float_to_bf16(v[i][0] * scale * to_float<TW>(w[n])) |
+             ((uint32_t)float_to_bf16(v[i][1] * scale * to_float<TW>(w[n + 1])) << 16);
+      y[1] = (uint32_t)float_to_bf16(v[i][2] * scale * to_float<TW>(w[n + 2])) |
+             ((uint32_t)float_to_bf16(v[i][3] * scale * to_float<TW>(w[n + 3])) << 16);
+      *reinterpret_cast<u32x2*>(o + n) = y;
+    }
+  }
+}
+
+// Launches it; false if the sizes do not fit it (nothing has been launched then).
+inline bool launch_finish_norm(float* C, int64_t ldc, const float* partial, int splits, int M, int N,
+                               const NormAfter& norm, hipStream_t stream) {
+  const int threads = N >= 2048 ? 512 : 256;
+  if (N % 4 != 0 || N > 16 * threads || norm.ldn % 4 != 0 || (uintptr_t)norm.normed % 8 != 0) return false;
+  const int nv = (N + 4 * threads - 1) / (4 * threads);          // 1 .. 4
+#define GO(TW)                                                                                                   \
+  do {                                                                                                           \
+    if (nv <= 1) gemm_split_finish_norm_kernel<TW, 1><<<M, threads, 0, stream>>>(C, ldc, partial, splits, M, N, norm.normed, norm.ldn, (const TW*)norm.weight, norm.eps);      \
+    else if (nv == 2) gemm_split_finish_norm_kernel<TW, 2><<<M, threads, 0, stream>>>(C, ldc, partial, splits, M, N, norm.normed, norm.ldn, (const TW*)norm.weight, norm.eps); \
+    else gemm_split_finish_norm_kernel<TW, 4><<<M, threads, 0, stream>>>(C, ldc, partial, splits, M, N, norm.normed, norm.ldn, (const TW*)norm.weight, norm.eps);              \
+  } while (0)
+  if (norm.weight_is_f32) GO(float);
+  else GO(bf16_t);
+#undef GO
+  return true;
+}
+
 template <int MODE>
 int raise_pipelined_lds(size_t lds) {
   static bool raised = false;
@@ -615,9 +697,11 @@ inline int pipelined_splits(int M, int N, int K) {
 template <int MODE>
 int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
                      int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, const RowScale& rs = RowScale{},
-                     const Partial& partial = Partial{}) {
+                     const Partial& partial = Partial{}, const NormAfter& norm = NormAfter{}, bool* normed = nullptr) {
   // 128 x 128 tiles, two workgroups per CU.  (128 x 256 tiles halve the LDS reads per
-  // matrix instruction but leave one wave per SIMD, and measured 20 % slower.)
+  // matrix instruction but leave one wave per SIMD, and measured 20 % slower; 128 x 64
+  // tiles, which put two workgroups on a CU where 128 x 128 leave one, 15 % slower at 65
+  // to 256 rows.)
   constexpr int TM = 2, TN = 2, STAGES = 3;
   const size_t lds = (size_t)2 * (64 * TM + 64 * TN) * PPITCH * sizeof(bf16_t);
   if (raise_pipelined_lds<MODE>(lds)) return 1;
@@ -634,6 +718,12 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
       grid.y = splits;
       gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
           partial.at, N, A, lda, W, ldw, M, N, K, qkv, rs, k_split, (int64_t)M * N);
+      if constexpr (MODE == OUT_ADD_F32) {
+        if (norm.normed != nullptr && launch_finish_norm((float*)C, ldc, partial.at, splits, M, N, norm, stream)) {
+          *normed = true;
+          return 0;
+        }
+      }
       const int64_t threads = (int64_t)M * (N / 4);
       gemm_split_finish_kernel<MODE><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(C, ldc, partial.at, splits, M, N);
       return 0;
@@ -1307,6 +1397,45 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
   if (rc) return rc;
   HFEE_CHECK_LAUNCH("gemm_bf16");
   return 0;
+}
+
+// C (float32, the residual stream) += A W^T, and normed (bfloat16) = C_new / sqrt(mean(C_new^2) + eps)
+// * norm_weight, the norm that reads the new rows next.  Where K is cut over workgroups (see
+// hfee_gemm_bf16_scratch) the kernel that adds the partial products up also does the norm;
+// otherwise the product and the norm are two launches, as if the caller had made them.
+// C and normed: rows of N elements without gaps.  scratch as for hfee_gemm_bf16.
+HFEE_API int hfee_gemm_bf16_add_norm(float* C, const void* A, int64_t lda, const void* W, int64_t ldw, int M, int N,
+                                     int K, float* scratch, int64_t scratch_floats, void* normed,
+                                     const void* norm_weight, int norm_weight_is_f32, float eps, hipStream_t stream) {
+  HFEE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16_add_norm: bad sizes M=%d N=%d K=%d", M, N, K);
+  HFEE_REQUIRE(C != nullptr && normed != nullptr && norm_weight != nullptr && eps >= 0.f,
+               "gemm_bf16_add_norm: C, normed and the norm's weight are needed, and eps must not be negative");
+  HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16_add_norm: a leading dimension is shorter than its row");
+  if (M == 0) return 0;
+  const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+  bool done = false;
+  if (vec && !skinny_pays(M, N)) {
+    const TiledPlan plan = plan_tiled(M, N, K, large_fits(lda, ldw, M, N, K), true);
+    if (plan.first == 2 && plan.second == 0) {
+      Partial partial;
+      partial.at = scratch;
+      partial.floats = scratch != nullptr ? scratch_floats : 0;
+      NormAfter norm;
+      norm.normed = (bf16_t*)normed;
+      norm.ldn = N;
+      norm.weight = norm_weight;
+      norm.weight_is_f32 = norm_weight_is_f32 != 0;
+      norm.eps = eps;
+      if (launch_pipelined<OUT_ADD_F32>(C, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, stream,
+                                        RowScale{}, partial, norm, &done))
+        return 1;
+      HFEE_CHECK_LAUNCH("gemm_bf16_add_norm");
+      if (done) return 0;
+      return hfee_rmsnorm(normed, DT_BF16, C, norm_weight, norm_weight_is_f32 ? DT_F32 : DT_BF16, nullptr, eps, M, N, stream);
+    }
+  }
+  if (int rc = hfee_gemm_bf16(C, OUT_ADD_F32, N, A, lda, W, ldw, M, N, K, 0, scratch, scratch_floats, stream)) return rc;
+  return hfee_rmsnorm(normed, DT_BF16, C, norm_weight, norm_weight_is_f32 ? DT_F32 : DT_BF16, nullptr, eps, M, N, stream);
 }
 
 // The q/k/v product of more than 64 rows: C = q part of A W^T rotated, k and v rotated

@@ -31,6 +31,7 @@ _CORE_SIGNATURES = {
     "hfee_gemm_f32": [P, L, P, L, P, L, I, I, I, I, P],
     "hfee_attention_ref": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "hfee_gemm_bf16": [P, I, L, P, L, P, L, I, I, I, I, P, L, P],
+    "hfee_gemm_bf16_add_norm": [P, P, L, P, L, I, I, I, P, L, P, P, I, F, P],
     "hfee_gemm_bf16_scratch": [I, I, I],
     "hfee_gemm_bf16_plan": [I, I, I, P, P, P],
     "hfee_gemm_skinny": [P, L, P, I, L, P, L, I, I, I, I, P, I, F, P, P, P, P, I, P, P, I, I, P, I, I, I, I,

@@ -138,6 +138,29 @@ def linear_scratch(m: int, n: int, k: int) -> int:
     return int(lib.core().raw("hfee_gemm_bf16_scratch")(int(m), int(n), int(k)))
 
 
+def linear_add_norm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, normed: torch.Tensor,
+                    norm_weight: torch.Tensor, eps: float, scratch=None):
+    """out (float32, the residual stream) += x @ weight.T, and normed (bfloat16) = the RMS norm of the
+    new rows of out times norm_weight.  bfloat16 x and weight.  Where the product's K is cut over
+    workgroups (`linear_scratch` > 0 and scratch given) the kernel that adds the partial products
+    up does the norm as well; otherwise it is the product and the norm, one after the other."""
+    _gpu(out, x, weight, normed, norm_weight)
+    M, K, lda = _rows2d(x, "linear_add_norm x")
+    N, Kw, ldw = _rows2d(weight, "linear_add_norm weight")
+    _check(x.dtype == weight.dtype == torch.bfloat16 and out.dtype == torch.float32 and normed.dtype == torch.bfloat16,
+           "linear_add_norm: bfloat16 x, weight and normed, float32 out")
+    _check(Kw == K and tuple(out.shape) == (M, N) == tuple(normed.shape) and out.is_contiguous() and normed.is_contiguous(),
+           f"linear_add_norm: shapes x{list(x.shape)} w{list(weight.shape)} out{list(out.shape)} normed{list(normed.shape)}")
+    _check(norm_weight.numel() == N and norm_weight.is_contiguous() and norm_weight.dtype in (torch.float32, torch.bfloat16),
+           "linear_add_norm: the norm's weight must have the width of out, float32 or bfloat16")
+    if scratch is not None:
+        _gpu(scratch)
+        _check(scratch.dtype == torch.float32 and scratch.is_contiguous(), "linear_add_norm: float32 scratch expected")
+    lib.core().call("hfee_gemm_bf16_add_norm", _ptr(out), _ptr(x), lda, _ptr(weight), ldw, M, N, K, _ptr(scratch),
+                    0 if scratch is None else scratch.numel(), _ptr(normed), _ptr(norm_weight),
+                    1 if norm_weight.dtype == torch.float32 else 0, float(eps), _stream())
+
+
 def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate: bool = False, kernel: int = 0,
            gate: bool = False, scratch=None):
     """out (+)= x @ weight.T, weight stored [out_features, in_features].

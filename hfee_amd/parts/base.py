@@ -177,6 +177,20 @@ class LazyNorm:
         self.pending = dict(out=out, shares=shares, blocks=blocks, eps=eps)
         return dict(weight=weight, out=out, shares=shares)
 
+    def offer_whole(self):
+        """For the part that adds into x last with bfloat16 operands: dict(out, weight, eps) if
+        its adding product may also write the whole norm of the new rows into `out`
+        (`ops.linear_add_norm`); the part that takes the offer has to fill `out`.  None if this
+        norm is not of that form (then nothing changes for anybody)."""
+        form = self.fusable()
+        if form is None or self.x.dtype != torch.float32 or self._tensor is not None or self.pending is not None:
+            return None
+        out = self.ctx.rows("block.normed", self.x.shape[1])
+        if out.dtype != torch.bfloat16:
+            return None
+        self._tensor = out
+        return dict(out=out, weight=form[0], eps=form[1])
+
     def row_scale(self):
         """For the consuming part: (emitted tensor, `row_scale` arguments) if a producer has
         done the first half, else None."""

@@ -74,4 +74,10 @@ class GatedMLP(FeedForward):
             gate_up = ctx.rows("mlp.gate_up", 2 * F)
             ops.linear(gate_up, hn, self.w_gate_up)
             ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
-        ops.linear(x, act, self.w_down, accumulate=True, **ctx.workspace.split_scratch(n, self.w_down))
+        # the down projection adds into x and, if asked, goes on with the norm that follows
+        after = then.offer_whole() if then is not None and aligned else None
+        if after:
+            ops.linear_add_norm(x, act, self.w_down, after["out"], after["weight"], after["eps"],
+                                **ctx.workspace.split_scratch(n, self.w_down))
+        else:
+            ops.linear(x, act, self.w_down, accumulate=True, **ctx.workspace.split_scratch(n, self.w_down))

@@ -147,6 +147,38 @@ def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
     assert ops.linear_scratch(64, N, K) == 0 and ops.linear_scratch(2048, 4096, K) == 0
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 4096, 2112),
+                                   (100, 2052, 2048), (100, 512, 1024), (70, 1001, 2048), (2048, 512, 1024), (40, 512, 2048),
+                                   (90, 260, 2050)])
+@pytest.mark.parametrize("weight_dtype", [torch.float32, torch.bfloat16])
+def test_product_that_adds_into_the_stream_and_goes_on_with_the_norm(M, N, K, weight_dtype):
+    """The product that adds into the residual stream together with the norm of the new rows:
+    where K is cut over workgroups one kernel adds the partial products and norms the row; in
+    every other case (too few or too many rows, a short K, a width that the kernel does not
+    take, unaligned operands, no scratch) it is the two launches.  Bit-equal to the product
+    followed by the norm either way, and right against float64."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(M + 3 * N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    c0 = torch.randn(M, N, generator=g).to(DEV)
+    nw = (1.0 + 0.2 * torch.randn(N, generator=g)).to(weight_dtype).to(DEV)
+    eps = 1e-5
+    words = ops.linear_scratch(M, N, K)
+    for with_scratch in (True, False):
+        kw = dict(scratch=torch.full((words,), float("nan"), dtype=torch.float32, device=DEV)) if words and with_scratch else {}
+        two, normed_two = c0.clone(), torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.linear(two, x, w, accumulate=True, **kw)
+        ops.rmsnorm(normed_two, two, nw, eps)
+        one, normed_one = c0.clone(), torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.linear_add_norm(one, x, w, normed_one, nw, eps, **kw)
+        assert torch.equal(one, two)
+        assert torch.equal(normed_one, normed_two)
+    ref = c0.double().cpu() + x.double().cpu() @ w.double().cpu().t()
+    ref_normed = ref / torch.sqrt((ref * ref).mean(dim=1, keepdim=True) + eps) * nw.double().cpu()
+    assert (normed_one.double().cpu() - ref_normed).abs().max() <= 1e-2 * (1 + ref_normed.abs().max())
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 128, 32), (300, 200, 520), (2048, 512, 1024), (129, 258, 72), (65, 130, 200),
                                    (257, 384, 64), (1000, 96, 4096), (600, 520, 192), (256, 512, 64),
                                    (513, 258, 320)])
