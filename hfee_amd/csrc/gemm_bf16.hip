@@ -686,7 +686,10 @@ inline int pipelined_splits(int M, int N, int K) {
   if (M <= 64 || tiles >= (long_k ? 384 : 256) || K < 2048 || N % 4 != 0) return 1;
   // (two workgroups of this kernel fit a CU; measured, a prompt of 128 tokens is faster with one a CU
   // and fewer partial products, one of 512 tokens with two; two cuts only pay where K is long)
-  int splits = tiles < 128 ? (int)(256 / tiles) : tiles < 256 ? (int)(512 / tiles) : 2;
+  // (measured at 128 to 512 rows on the three narrow products of the 8B shape, µs for the pair of
+  // kernels: 48 tiles in 5 cuts 24, in 8 cuts 31; 64 tiles in 4 cuts 25, in 6 cuts 30; 96 tiles whole
+  // 46, in 3 cuts 38 to 41, in 5 cuts 32 to 36; 144 tiles in 2 cuts 50, in 3 cuts 42, in 4 cuts 51)
+  int splits = tiles < 86 ? (int)(256 / tiles) : tiles < 256 ? (int)(512 / tiles) : 2;
   if (splits > 8) splits = 8;
   if (splits > K / 512) splits = K / 512;
   if (splits < 2 || (splits == 2 && !long_k)) return 1;
