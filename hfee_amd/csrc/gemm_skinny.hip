@@ -361,12 +361,16 @@ __device__ __forceinline__ void finish_rows_ahead(const Args& a, const Ahead<EPI
   }
 }
 
-template <int MT, bool NORM, int EPI>
-__global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
+// TWO_A_CU (at most 16 batch rows): blocks of half the size, so that the registers allow two
+// workgroups a CU.  For launches of more workgroups than CUs and at most twice as many (5,120
+// weight rows: 320): all of them are on the chip from the start and share the memory's
+// bandwidth, where one a CU leaves a second round that fills a part of the chip only.
+template <int MT, bool NORM, int EPI, bool TWO_A_CU = false>
+__global__ __launch_bounds__(WAVES * 64, TWO_A_CU ? 4 : 2) void skinny_kernel(Args a) {
   // (two kilobytes of weights a wave and step of the loop for up to 16 batch rows, one beyond:
   // with 8 waves a CU and a block in flight that is 64 KB a CU on its way, what the memory's
   // latency takes at the CU's share of the bandwidth)
-  constexpr int U = MT == 1 ? 8 : 4, KBLOCK = 32 * U;
+  constexpr int U = MT == 1 && !TWO_A_CU ? 8 : 4, KBLOCK = 32 * U;
   __shared__ float partial[WAVES][MT][64][4];
   __shared__ float ss_part[WAVES][MT][16];
   __shared__ float row_scale[SS_STRIDE];
@@ -508,12 +512,39 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(Args a) {
   }
 }
 
+// The CUs of the current device (256 if it cannot be asked).
+inline int cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+           prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+  }
+  return cus;
+}
+
 template <int MT, bool NORM>
 void launch_epi(const Args& a, int epi, hipStream_t stream) {
   // (a workgroup takes a whole row of tiles: with 8 or 12 rows a workgroup, which spread 6,144
   // rows more evenly over 256 CUs, a wave's load is no longer a whole kilobyte, and that costs
   // more than the uneven rounds: q/k/v of the 8B shape 16.6 us against 12.7)
   dim3 grid((a.N + ROWS - 1) / ROWS);
+  if constexpr (MT == 1 && !NORM) {
+    const int cus = cu_count();
+    if ((int)grid.x > cus && (int)grid.x <= 2 * cus) {
+#define GO2(E) skinny_kernel<MT, NORM, E, true><<<grid, WAVES * 64, 0, stream>>>(a)
+      switch (epi) {
+        case EPI_BF16: GO2(EPI_BF16); break;
+        case EPI_F32: GO2(EPI_F32); break;
+        case EPI_ADD: GO2(EPI_ADD); break;
+        case EPI_SWIGLU: GO2(EPI_SWIGLU); break;
+        default: GO2(EPI_QKV); break;
+      }
+#undef GO2
+      return;
+    }
+  }
 #define GO(E) skinny_kernel<MT, NORM, E><<<grid, WAVES * 64, 0, stream>>>(a)
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
@@ -899,7 +930,7 @@ template <int STEPS, bool NORM, int EPI>
 __global__ __launch_bounds__(WAVES * 64) void wide_kernel(Args a, int row_groups) {
   // (loads in flight a wave; it must divide STEPS.  Measured inside the decode step, gate/up of the
   // 8B shape: 44.7 µs with 16, 43.0 with 8, 43.8 with 4)
-  constexpr int RING = STEPS % 8 == 0 ? 8 : STEPS % 6 == 0 ? 6 : 4;
+  constexpr int RING = STEPS % 8 == 0 ? 8 : STEPS % 10 == 0 ? 10 : STEPS % 6 == 0 ? 6 : 4;
   static_assert(STEPS % RING == 0, "a ring slot must mean the same step in every row group");
   __shared__ float partial[WAVES][64][4];
   __shared__ float ss_part[WAVES][16];
@@ -1025,7 +1056,12 @@ bool launch_wide_steps(const Args& a, int row_groups, int grid, hipStream_t stre
   else if (steps == 8) wide_kernel<8, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
   else if (steps == 12) wide_kernel<12, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
   else if (steps == 16) wide_kernel<16, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
-  else return false;      // other widths: the streaming kernel takes them
+  else if (steps == 20) {
+    // (with the norm folded in, the float32 rows on their way to operands need more registers
+    // than a wave of eight a CU has: those products stay with the streaming kernel)
+    if constexpr (NORM) return false;
+    else wide_kernel<20, false, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
+  } else return false;      // other widths: the streaming kernel takes them
   return true;
 }
 
@@ -1039,10 +1075,11 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
     num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
   const int row_groups = (a.N + ROWS - 1) / ROWS;
-  if (a.M > 16 || a.K % (128 * WAVES) != 0 || a.K > 16 * 32 * WAVES) return false;
+  if (a.M > 16 || a.K % (128 * WAVES) != 0 || a.K > 20 * 32 * WAVES) return false;
   // from two row groups a workgroup on: the workgroups then share the weight rows evenly, where
   // one row group each leaves a second round that fills a part of the chip only (q/k/v of the 8B
-  // shape, 384 row groups: 1.5 us a layer inside the decode step)
+  // shape, 384 row groups: 1.5 us a layer inside the decode step; and better than the streaming
+  // kernel with two workgroups a CU: 3.465 ms a step against 3.52)
   const int per = (row_groups + num_cus - 1) / num_cus;       // row groups per workgroup, all but equal
   if (per < 2) return false;
   const int grid = (row_groups + per - 1) / per;

@@ -262,7 +262,9 @@ def test_weights_in_tiles():
 
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (8, 344, 96), (16, 100, 256), (3, 16400, 1024), (16, 16500, 2048),
                                    (5, 17000, 4096), (2, 16390, 3072), (33, 200, 128), (64, 52, 1024),
-                                   (7, 50, 40), (12, 107, 200), (4, 20, 8), (9, 6144, 512)])
+                                   (7, 50, 40), (12, 107, 200), (4, 20, 8), (9, 6144, 512),
+                                   (16, 5130, 1280), (3, 8000, 200),      # more workgroups than CUs, at most twice as many
+                                   (5, 8300, 5120)])                       # the persistent kernel at K = 5,120
 @pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu"])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_decode_products(M, N, K, epilogue, norm):
@@ -376,7 +378,8 @@ def _products_of_17_to_64_rows(M, N, K, epilogue, kernel):
 
 
 @pytest.mark.parametrize("M,N,K,N2", [(1, 64, 96, 48), (8, 200, 256, 344), (16, 4096, 1024, 16400), (33, 104, 64, 72),
-                                       (64, 520, 128, 100), (40, 200, 64, 16400), (64, 2048, 128, 17000), (17, 96, 64, 16384)])
+                                       (64, 520, 128, 100), (40, 200, 64, 16400), (64, 2048, 128, 17000), (17, 96, 64, 16384),
+                                       (9, 5120, 320, 6000)])     # both products: more workgroups than CUs, at most twice as many
 @pytest.mark.parametrize("epilogue2", ["bf16", "swiglu", "add"])
 def test_norm_in_two_halves(M, N, K, N2, epilogue2):
     """A norm between two products, without a launch of its own: the product that adds
@@ -424,7 +427,8 @@ def test_norm_in_two_halves(M, N, K, N2, epilogue2):
 
 
 @pytest.mark.parametrize("H,K,hd,half,M", [(4, 2, 16, 8, 5), (3, 1, 32, 16, 16), (6, 3, 48, 8, 1), (2, 2, 128, 64, 9),
-                                           (4, 2, 16, 8, 100), (6, 3, 48, 8, 130), (2, 2, 128, 64, 300), (5, 1, 64, 32, 65)])
+                                           (4, 2, 16, 8, 100), (6, 3, 48, 8, 130), (2, 2, 128, 64, 300), (5, 1, 64, 32, 65),
+                                           (40, 8, 128, 64, 9)])      # 7,168 weight rows: more workgroups than CUs
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rotation_and_cache_write(H, K, hd, half, M, norm):
     """Projection + rotation (pairs 2i, 2i+1) + cache write in one launch against the
