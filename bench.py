@@ -38,8 +38,17 @@ SHAPES = {
     "llama-2-13b": dict(BASE_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40,
                         num_key_value_heads=40, intermediate_size=13824, vocab_size=32000,
                         max_position_embeddings=4096, rope_theta=10000.0, rope_scaling=None),
+    "llama-3.2-3b": dict(BASE_8B, num_hidden_layers=28, hidden_size=3072, num_attention_heads=24,
+                         intermediate_size=8192, tie_word_embeddings=True,
+                         rope_scaling=dict(BASE_8B["rope_scaling"], factor=32.0)),
+    "llama-2-7b": dict(BASE_8B, num_hidden_layers=32, num_key_value_heads=32, intermediate_size=11008,
+                       vocab_size=32000, max_position_embeddings=4096, rope_theta=10000.0, rope_scaling=None),
+    # (80 layers of it do not fit beside their second copy in tiles: run it with --layers)
+    "llama-3.1-70b": dict(BASE_8B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                          intermediate_size=28672),
 }
-SHAPE_NAMES = {"llama-3.1-8b": "Llama-3.1-8B", "llama-3.2-1b": "Llama-3.2-1B", "llama-2-13b": "Llama-2-13B"}
+SHAPE_NAMES = {"llama-3.1-8b": "Llama-3.1-8B", "llama-3.2-1b": "Llama-3.2-1B", "llama-2-13b": "Llama-2-13B",
+               "llama-3.2-3b": "Llama-3.2-3B", "llama-2-7b": "Llama-2-7B", "llama-3.1-70b": "Llama-3.1-70B"}
 CONTEXT = 8192
 PROMPT = 1024
 PREFILL = 2048
