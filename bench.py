@@ -43,7 +43,7 @@ SHAPES = {
                          rope_scaling=dict(BASE_8B["rope_scaling"], factor=32.0)),
     "llama-2-7b": dict(BASE_8B, num_hidden_layers=32, num_key_value_heads=32, intermediate_size=11008,
                        vocab_size=32000, max_position_embeddings=4096, rope_theta=10000.0, rope_scaling=None),
-    # (80 layers of it do not fit beside their second copy in tiles: run it with --layers)
+    # (141 GB of weights: the layers bound last do without their second copy in tiles)
     "llama-3.1-70b": dict(BASE_8B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
                           intermediate_size=28672),
 }

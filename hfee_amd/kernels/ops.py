@@ -444,6 +444,25 @@ def tile_weight(weight: torch.Tensor) -> TiledWeight:
     return TiledWeight(tiles, n, k)
 
 
+# The part of the device's memory that the second copies of the weights leave free (for the cache,
+# the workspace, and whatever else the process holds).
+TILES_LEAVE_FREE = 0.2
+
+
+def tile_weights_if_room(*weights: torch.Tensor):
+    """The weights' second copies in tiles (`tile_weight`), all of them or none: None where they
+    would leave less than TILES_LEAVE_FREE of the device's memory free.  A model too large to lie
+    in memory twice then has the layers that were bound last without tiles; their steps of at
+    most 64 rows go through the kernels that read the rows as they lie."""
+    device = weights[0].device
+    if device.type == "cuda":
+        need = sum(w.numel() * w.element_size() for w in weights)
+        free, total = torch.cuda.mem_get_info(device)
+        if free - need < TILES_LEAVE_FREE * total:
+            return None
+    return tuple(tile_weight(w) for w in weights)
+
+
 SS_STRIDE = 64     # rows of a table of sum-of-squares shares (one row of the table per 16 weight rows)
 
 

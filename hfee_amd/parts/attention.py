@@ -91,8 +91,11 @@ class Attention(Mixer):
         # a second copy in tiles for steps of up to 64 rows, whose products stream the weights
         # (as rows they serve the tiled products of longer portions)
         self.streams = self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.q_width % 8 == 0
-        self.w_qkv_tiles = ops.tile_weight(self.w_qkv) if self.streams else None
-        self.w_o_tiles = ops.tile_weight(self.w_o) if self.streams else None
+        tiles = ops.tile_weights_if_room(self.w_qkv, self.w_o) if self.streams else None
+        self.streams = tiles is not None
+        self.w_qkv_tiles, self.w_o_tiles = tiles if tiles else (None, None)
+        if not self.streams:      # (nobody finishes a norm here that the part before has begun)
+            self.second_half_rows = 0
 
     def key_layout(self):
         """What two layers must share to read one cache layer."""

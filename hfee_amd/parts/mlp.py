@@ -41,16 +41,19 @@ class GatedMLP(FeedForward):
                                      dim=1).reshape(2 * self.intermediate, self.hidden).contiguous()
         self.w_down = tensors.pop(p + "down_proj.weight").contiguous()
         # a second copy in tiles for steps of up to 64 rows, whose products stream the weights
-        self.streams = self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.intermediate % 8 == 0
-        self.w_gate_up_tiles = ops.tile_weight(self.w_gate_up) if self.streams else None
-        self.w_down_tiles = ops.tile_weight(self.w_down) if self.streams else None
+        self.aligned = self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.intermediate % 8 == 0
+        tiles = ops.tile_weights_if_room(self.w_gate_up, self.w_down) if self.aligned else None
+        self.streams = tiles is not None
+        self.w_gate_up_tiles, self.w_down_tiles = tiles if tiles else (None, None)
+        if not self.streams:      # (nobody finishes a norm here that the part before has begun)
+            self.second_half_rows = 0
 
     def forward_add(self, ctx, x, h, then=None):
         F, n = self.intermediate, ctx.n
         act = ctx.rows("mlp.act", F)
-        aligned = self.streams
+        aligned = self.aligned
         lazy = isinstance(h, LazyNorm)
-        if aligned and n <= ops.SKINNY_MAX_ROWS:        # both products stream the weights' tiles
+        if self.streams and n <= ops.SKINNY_MAX_ROWS:        # both products stream the weights' tiles
             w = self.w_gate_up_tiles
             halves = h.row_scale() if lazy else None     # (offered for few rows only)
             norm = None

@@ -121,3 +121,41 @@ def test_a_prefix_kept_from_an_earlier_request(model_folders, dtype):
     keeping.release("third")
     keeping.cache.check()
     assert keeping.cache.free_pages() == [8]
+
+
+@pytest.mark.parametrize("tiled_calls", [0, 2])
+def test_a_model_too_large_for_second_copies_of_its_weights(model_folders, monkeypatch, tiled_calls):
+    """Where the weights' second copies in tiles would not leave room, the parts bound last do
+    without them (none of them, or all but the first layer's attention and feed-forward): steps
+    of few rows then go through the kernels that read the weights' rows as they lie, beside
+    layers that have their tiles, and give the plain model's logits, whole and decoding."""
+    from plain_llama import PlainLlama
+    from hfee_amd.engine import Engine, StepEntry, load_model
+    from hfee_amd.kernels import ops
+    made = ops.tile_weights_if_room
+    calls = {"n": 0}
+
+    def no_room(*weights):
+        calls["n"] += 1
+        return made(*weights) if calls["n"] <= tiled_calls else None
+
+    monkeypatch.setattr(ops, "tile_weights_if_room", no_room)
+    folder = model_folders[("B", "bfloat16")]
+    plain = PlainLlama(folder)
+    model, cfg = load_model(folder, "bfloat16")
+    with_tiles = [b.mixer.streams for b in model.blocks] + [b.feed_forward.streams for b in model.blocks]
+    assert sum(with_tiles) == tiled_calls and calls["n"] == len(with_tiles)
+    eng = Engine(model, num_pages=64, page_size=16, max_requests=4, max_batch_tokens=256)
+    g = torch.Generator().manual_seed(2)
+    toks = torch.randint(0, cfg.vocab_size, (90,), generator=g).tolist()
+    ref = plain.forward(toks)
+    eng.admit("r")
+    got = [eng.step([StepEntry("r", toks[:70], list(range(70)))]).clone()]
+    for t in toks[70:]:
+        got.append(eng.step([StepEntry("r", [t], [0])]).clone())
+    assert rel_err(torch.cat(got), ref) < TOL["bfloat16"]
+    # another request beside it: 17 to 64 rows in a step, then both decoding
+    other = torch.randint(0, cfg.vocab_size, (40,), generator=g).tolist()
+    eng.admit("s")
+    both = eng.step([StepEntry("r", [toks[0]], []), StepEntry("s", other, list(range(40)))])
+    assert rel_err(both, plain.forward(other)) < TOL["bfloat16"]
