@@ -560,7 +560,8 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 // ------------------------------------------------------------ 17 to 64 rows ---
 // With more than 16 batch rows the streaming kernel reads the batch again for every 16
 // weight rows, and that traffic (from L2) outgrows the weights.  Here K is cut into
-// slices of 1,024 columns (the last one may be half a slice), each with workgroups of its own.  A workgroup keeps its slice
+// slices of 1,024 columns (the last one may be shorter: a multiple of 512 columns, of 256 from 33
+// batch rows on), each with workgroups of its own.  A workgroup keeps its slice
 // of the batch, all rows, in LDS; each of its waves walks over groups of 16 weight rows
 // on its own: the weights come straight from global memory through a ring of 4 or 16 loads
 // that runs across group boundaries, the batch operands from LDS; no barrier stands in
@@ -568,11 +569,16 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 // scratch buffer and goes on; a second, short kernel (one wave for 16 batch rows of a row
 // group, so that the whole chip takes part) adds the shares in the order of the slices and
 // runs the epilogue.  Nobody waits for anybody, and nothing is counted.
-constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32, MID_HALF = MID_STEPS / 2;
+constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32;
 // loads a wave keeps in flight.  Measured inside the decode step at 64 rows (q/k/v, output, down
 // of the 8B shape): 20.3 / 14.2 / 27.2 µs with 8, 15.0 / 13.8 / 27.1 with 4, 19.7 / 15.2 / 30.4 with 2;
 // at 24 and 32 rows 4 and 16 measured alike.
 constexpr int mid_ring(int mt) { return mt >= 3 ? 4 : 16; }
+// steps that the loop is unrolled over (whole turns of the ring): the last slice of K is a whole
+// number of these, so K is a multiple of 256 columns from 33 batch rows on, of 512 below.  (The
+// same loop over 16 steps with a last turn of 8, written as one body for both, measured 3 %
+// slower over the whole step at 64 rows: 5.91 ms against 5.73.)
+constexpr int mid_unroll(int mt) { return mt >= 3 ? 8 : 16; }
 constexpr int MID_PITCH = MID_KS + 8;        // LDS row pitch of the batch slice in elements: rows 16 bytes askew
 
 constexpr size_t mid_lds_bytes(int mt) { return (size_t)mt * 16 * MID_PITCH * sizeof(bf16_t); }
@@ -616,7 +622,8 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   const int per_slice = gridDim.x / slices;
   int rg = blockIdx.x / slices + per_slice * wave;
   const bf16_t* w_cur = row_ptr(min(rg, row_groups - 1));
-  constexpr int MID_RING = mid_ring(MT);
+  constexpr int MID_RING = mid_ring(MT), MID_HALF = mid_unroll(MT);
+  static_assert(MID_HALF % MID_RING == 0 && MID_STEPS % MID_HALF == 0, "a ring slot means the same step in every turn of the loop");
   Chunk ring[MID_RING];
 #pragma unroll
   for (int st = 0; st < MID_RING; ++st) ring[st].u = load_streamed(reinterpret_cast<const u32x4*>(w_cur + st * WeightTiles::TILE));
@@ -639,7 +646,7 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   __syncthreads();
 
   const bf16_t* x_lane = xs + r16 * MID_PITCH + g * 8;
-  const int steps = min(MID_STEPS, (a.K - k0) / 32);      // of this slice: 32, or 16 in a last half slice
+  const int steps = min(MID_STEPS, (a.K - k0) / 32);      // of this slice: 32, or fewer in a last, shorter one
   while (rg < row_groups) {
     const int rg_next = rg + stride;
     const bf16_t* w_next = row_ptr(rg_next < row_groups ? rg_next : rg);    // past the end: a repeat that nobody uses
@@ -1207,7 +1214,7 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
       return 0;
     }
   }
-  if (!norm && mt > 1 && K % (MID_KS / 2) == 0 && (mid_pays || force_mid == 1)) {
+  if (!norm && mt > 1 && K % (32 * mid_unroll(mt)) == 0 && (mid_pays || force_mid == 1)) {
     const bool took = mt == 2 ? launch_mid_rows<2>(a, epi, scratch, scratch_floats, num_cus, stream)
                     : mt == 3 ? launch_mid_rows<3>(a, epi, scratch, scratch_floats, num_cus, stream)
                               : launch_mid_rows<4>(a, epi, scratch, scratch_floats, num_cus, stream);
