@@ -266,10 +266,24 @@ __global__ void rope_cache_kernel(T* __restrict__ q, int64_t ldq, const T* __res
   }
 }
 
+// Where q, k and v come from when the product that makes them was cut along K over
+// workgroups and its partial products have not been added up: `count` matrices of float32
+// [rows, ld], `stride` floats apart, whose columns are q, then k (from k_col), then v (from
+// v_col).  at null: q, k and v are read as bfloat16 rows.
+struct QkvCuts {
+  const float* at;
+  int count;
+  int64_t stride, ld;
+  int k_col, v_col;
+};
+
 // The same for bfloat16 with adjacent pairs (2i, 2i + 1), eight elements (16 bytes, four
 // pairs) per thread and step: head_dim and 2 * half multiples of 8, rows 16-byte aligned.
+// With `cuts`, the partial products are added up here, in their order, and rounded to
+// bfloat16 as the kernel that would have added them does: q is only written, k and v only
+// say that the cache is written.
 __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, const bf16_t* __restrict__ k, int64_t ldk,
-                                        const bf16_t* __restrict__ v, int64_t ldv,
+                                        const bf16_t* __restrict__ v, int64_t ldv, QkvCuts cuts,
                                         const int* __restrict__ positions, const int* __restrict__ token_segment,
                                         const int* __restrict__ block_tables, int bt_stride,
                                         const float* __restrict__ cos_table, const float* __restrict__ sin_table,
@@ -280,6 +294,36 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
   union Eight {
     u32x4 u;
     bf16_t e[8];
+  };
+  // elements col .. col + 7 of row t: from the bfloat16 row, or the sum of the cuts
+  auto eight = [&](const bf16_t* row, int t, int col) {
+    Eight x;
+    if (cuts.at == nullptr) {
+      x.u = *reinterpret_cast<const u32x4*>(row);
+      return x;
+    }
+    constexpr int MOST = 8;
+    const float* p = cuts.at + (int64_t)t * cuts.ld + col;
+    f32x4 lo[MOST], hi[MOST];
+#pragma unroll
+    for (int z = 0; z < MOST; ++z) {      // all asked for together; past the last one: a repeat that is not added
+      const float* pz = p + (int64_t)min(z, cuts.count - 1) * cuts.stride;
+      lo[z] = *reinterpret_cast<const f32x4*>(pz);
+      hi[z] = *reinterpret_cast<const f32x4*>(pz + 4);
+    }
+    f32x4 a = lo[0], b = hi[0];
+#pragma unroll
+    for (int z = 1; z < MOST; ++z)
+      if (z < cuts.count) {
+        a += lo[z];
+        b += hi[z];
+      }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x.e[i] = float_to_bf16(a[i]);
+      x.e[4 + i] = float_to_bf16(b[i]);
+    }
+    return x;
   };
   // Some workgroups take the values of 16 consecutive tokens each.  The cache keeps values
   // transposed (a column of a head holds the page's slots side by side), so a token alone
@@ -298,7 +342,7 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int idx = min(first + u * (int)blockDim.x, pieces - 1), j = idx / chunks, c = idx - j * chunks;
-        piece[u] = *reinterpret_cast<const u32x4*>(v + (int64_t)(t0 + j) * ldv + 8 * c);
+        piece[u] = eight(v + (int64_t)(t0 + j) * ldv + 8 * c, t0 + j, cuts.v_col + 8 * c).u;
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -347,26 +391,30 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
       x.e[2 * p + 1] = float_to_bf16(x0 * s[p] + x1 * c[p]);
     }
   };
-  if (q != nullptr && cs != nullptr) {
-    bf16_t* qt = q + (int64_t)t * ldq;
-    for (int w = threadIdx.x; w < num_heads * per_head; w += blockDim.x) {
-      const int d = (w % per_head) * 8;
-      Eight x;
-      x.u = *reinterpret_cast<const u32x4*>(qt + w * 8);
-      rotate(x, d);
-      *reinterpret_cast<u32x4*>(qt + w * 8) = x.u;
-    }
-  }
-  if (k == nullptr || cache == nullptr) return;
-  const int page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
+  // One walk over the token's pieces of eight elements, q's first and then k's (with v's): what
+  // a thread needs of the tables is asked for before the first piece, so that the workgroups of
+  // few tokens (a decode step) wait once for memory and not once for q and once again for k.
+  const bool with_q = q != nullptr && (cs != nullptr || cuts.at != nullptr);
+  const bool with_kv = k != nullptr && cache != nullptr;
+  const int q_pieces = with_q ? num_heads * per_head : 0, kv_pieces = with_kv ? lay.kv_heads * per_head : 0;
+  int page = 0;
+  if (with_kv) page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
   const int slot = pos & (lay.page_size - 1);
+  bf16_t* qt = q + (int64_t)t * ldq;
   const bf16_t* kt = k + (int64_t)t * ldk;
   const bf16_t* vt = v + (int64_t)t * ldv;
-  for (int w = threadIdx.x; w < lay.kv_heads * per_head; w += blockDim.x) {
+  for (int u = threadIdx.x; u < q_pieces + kv_pieces; u += blockDim.x) {
+    if (u < q_pieces) {
+      const int d = (u % per_head) * 8;
+      Eight x = eight(qt + u * 8, t, u * 8);
+      rotate(x, d);
+      *reinterpret_cast<u32x4*>(qt + u * 8) = x.u;
+      continue;
+    }
+    const int w = u - q_pieces;
     const int h = w / per_head, d = (w - h * per_head) * 8;
-    Eight x, y;
-    x.u = *reinterpret_cast<const u32x4*>(kt + w * 8);
-    if (!values_by_groups) y.u = *reinterpret_cast<const u32x4*>(vt + w * 8);
+    Eight x = eight(kt + w * 8, t, cuts.k_col + w * 8), y;
+    if (!values_by_groups) y = eight(vt + w * 8, t, cuts.v_col + w * 8);
     rotate(x, d);
 #pragma unroll
     for (int c = 0; c < 4; ++c) x.u[c] = finite_bf16x2(x.u[c]);       // only finite values go into the cache
@@ -416,8 +464,8 @@ HFEE_API int hfee_rope_cache_write(void* q, int64_t ldq, const void* k, int64_t 
     // against 5 at 128 rows)
     const int by_groups = portions != 0 && k != nullptr && cache != nullptr && n >= 32 && group_bytes <= 48 * 1024;
     rope_cache_pairs_kernel<<<n + (by_groups ? (n + 15) / 16 : 0), 256, by_groups ? group_bytes : 0, stream>>>(
-        (bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv, positions, token_segment, block_tables, bt_stride,
-        cos_table, sin_table, half, (bf16_t*)cache, lay, num_heads, n, by_groups);
+        (bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv, QkvCuts{nullptr, 0, 0, 0, 0, 0}, positions,
+        token_segment, block_tables, bt_stride, cos_table, sin_table, half, (bf16_t*)cache, lay, num_heads, n, by_groups);
   }
   else if (dtype == DT_BF16)
     rope_cache_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv,
@@ -426,5 +474,51 @@ HFEE_API int hfee_rope_cache_write(void* q, int64_t ldq, const void* k, int64_t 
   else
     return fail("rope_cache_write: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("rope_cache_write");
+  return 0;
+}
+
+// The same for q, k and v that lie as the partial products of a q/k/v product cut along K
+// (hfee_gemm_bf16_cuts): `cuts` matrices of float32 [n, width], width = (num_heads + 2 *
+// kv_heads) * head_dim, one after the other.  The partial products are added up in their
+// order and rounded to bfloat16, then rotated (adjacent pairs); q goes to `q` (bfloat16, rows
+// ldq apart), k and v into the cache: the numbers of the adding kernel followed by
+// hfee_rope_cache_write, in one launch.  bfloat16 cache, adjacent pairs, head_dim and the
+// rotary width multiples of 8.
+HFEE_API int hfee_rope_cache_write_cuts(void* q, int64_t ldq, const float* partial, int cuts,
+                                        const int* positions, const int* token_segment, const int* block_tables,
+                                        int bt_stride, const float* cos_table, const float* sin_table, int half,
+                                        int table_positions, int max_position, void* cache, int num_heads,
+                                        int kv_heads, int head_dim, int page_size, int n, int portions,
+                                        hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0, "rope_cache_write_cuts: bad token count");
+  if (n == 0) return 0;
+  HFEE_REQUIRE(q != nullptr && partial != nullptr && cache != nullptr && positions != nullptr &&
+                   token_segment != nullptr && block_tables != nullptr,
+               "rope_cache_write_cuts: q, the partial products, the cache and its tables are needed");
+  HFEE_REQUIRE(cuts >= 1 && cuts <= 8, "rope_cache_write_cuts: 1 to 8 cuts, got %d", cuts);
+  HFEE_REQUIRE(half >= 0 && 2 * half <= head_dim, "rope_cache_write_cuts: rotary width %d exceeds head_dim %d",
+               2 * half, head_dim);
+  HFEE_REQUIRE(cos_table == nullptr || max_position < table_positions,
+               "rope_cache_write_cuts: position %d is beyond the rotation table (%d positions)", max_position,
+               table_positions);
+  CacheLayout lay;
+  if (make_cache_layout(&lay, kv_heads, head_dim, page_size)) return 1;
+  const int64_t width = (int64_t)(num_heads + 2 * kv_heads) * head_dim;
+  HFEE_REQUIRE(head_dim % 8 == 0 && half % 4 == 0 && ldq % 8 == 0 && ldq >= (int64_t)num_heads * head_dim &&
+                   (uintptr_t)q % 16 == 0 && (uintptr_t)partial % 16 == 0 && (uintptr_t)cos_table % 16 == 0 &&
+                   (uintptr_t)sin_table % 16 == 0 && (uintptr_t)cache % 16 == 0,
+               "rope_cache_write_cuts: head_dim and the rotary width must be multiples of 8 and the operands 16-byte aligned");
+  const QkvCuts c{partial, cuts, (int64_t)n * width, width, num_heads * head_dim, (num_heads + kv_heads) * head_dim};
+  const size_t group_bytes = (size_t)32 * kv_heads * head_dim;
+  const int by_groups = portions != 0 && n >= 32 && group_bytes <= 48 * 1024;
+  // (k and v: any pointers that are not null; with cuts they are never read.  More threads than
+  // the plain kernel has, a piece each where that is at most 768: a thread's eight elements
+  // are up to sixteen loads, and few tokens leave CUs without a workgroup)
+  const int pieces = (num_heads + kv_heads) * (head_dim / 8);
+  const int threads = pieces >= 768 ? 768 : pieces > 512 ? (pieces + 63) / 64 * 64 : 512;
+  rope_cache_pairs_kernel<<<n + (by_groups ? (n + 15) / 16 : 0), threads, by_groups ? group_bytes : 0, stream>>>(
+      (bf16_t*)q, ldq, (const bf16_t*)q, 0, (const bf16_t*)q, 0, c, positions, token_segment, block_tables, bt_stride,
+      cos_table, sin_table, half, (bf16_t*)cache, lay, num_heads, n, by_groups);
+  HFEE_CHECK_LAUNCH("rope_cache_write_cuts");
   return 0;
 }

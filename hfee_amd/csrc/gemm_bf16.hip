@@ -1442,6 +1442,34 @@ HFEE_API int hfee_gemm_bf16_add_norm(float* C, const void* A, int64_t lda, const
   return hfee_rmsnorm(normed, DT_BF16, C, norm_weight, norm_weight_is_f32 ? DT_F32 : DT_BF16, nullptr, eps, M, N, stream);
 }
 
+// A W^T cut along K over workgroups, the partial products left as they are: *cuts matrices of
+// float32 [M, N], one after the other in scratch, for a caller whose next kernel adds them up
+// on its way (hfee_rope_cache_write_cuts).  *cuts = 0 and nothing launched where the product
+// would not be cut (see hfee_gemm_bf16_scratch) or the scratch is too small: the caller then
+// takes the plain product.
+HFEE_API int hfee_gemm_bf16_cuts(const void* A, int64_t lda, const void* W, int64_t ldw, int M, int N, int K,
+                                 float* scratch, int64_t scratch_floats, int* cuts, hipStream_t stream) {
+  HFEE_REQUIRE(M > 0 && N > 0 && K > 0 && cuts != nullptr, "gemm_bf16_cuts: bad arguments");
+  HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16_cuts: a leading dimension is shorter than its row");
+  *cuts = 0;
+  const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+  if (!vec || skinny_pays(M, N) || scratch == nullptr || (uintptr_t)scratch % 16 != 0 || N % 4 != 0) return 0;
+  const TiledPlan plan = plan_tiled(M, N, K, large_fits(lda, ldw, M, N, K), true);
+  const int splits = pipelined_splits(M, N, K);
+  if (plan.first != 2 || plan.second != 0 || splits < 2 || scratch_floats < (int64_t)splits * M * N) return 0;
+  constexpr int TM = 2, TN = 2, STAGES = 3;
+  const size_t lds = (size_t)2 * (64 * TM + 64 * TN) * PPITCH * sizeof(bf16_t);
+  if (raise_pipelined_lds<OUT_F32>(lds)) return 1;
+  const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
+  dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS), splits);
+  const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+  gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
+      scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, RowScale{}, k_split, (int64_t)M * N);
+  HFEE_CHECK_LAUNCH("gemm_bf16_cuts");
+  *cuts = splits;
+  return 0;
+}
+
 // The q/k/v product of more than 64 rows: C = q part of A W^T rotated, k and v rotated
 // and written into the paged cache by the product's epilogue (see qkv_epilogue.h).
 // Operands must be aligned as the tiled kernels need them.  For the callers of

@@ -32,6 +32,8 @@ _CORE_SIGNATURES = {
     "hfee_attention_ref": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
     "hfee_gemm_bf16": [P, I, L, P, L, P, L, I, I, I, I, P, L, P],
     "hfee_gemm_bf16_add_norm": [P, P, L, P, L, I, I, I, P, L, P, P, I, F, P],
+    "hfee_gemm_bf16_cuts": [P, L, P, L, I, I, I, P, L, P, P],
+    "hfee_rope_cache_write_cuts": [P, L, P, I, P, P, P, I, P, P, I, I, I, P, I, I, I, I, I, I, P],
     "hfee_gemm_bf16_scratch": [I, I, I],
     "hfee_gemm_bf16_plan": [I, I, I, P, P, P],
     "hfee_gemm_skinny": [P, L, P, I, L, P, L, I, I, I, I, P, I, F, P, P, P, P, I, P, P, I, I, P, I, I, I, I,

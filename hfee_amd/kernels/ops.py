@@ -138,6 +138,53 @@ def linear_scratch(m: int, n: int, k: int) -> int:
     return int(lib.core().raw("hfee_gemm_bf16_scratch")(int(m), int(n), int(k)))
 
 
+def linear_cuts(x: torch.Tensor, weight: torch.Tensor, scratch) -> int:
+    """x @ weight.T (bfloat16) cut along K over workgroups, the partial products left in scratch
+    as that many float32 matrices [M, N] one after the other, for a kernel that adds them up on
+    its way (`rope_cache_write_cuts`).  Returns the number of cuts; 0 (and nothing launched)
+    where the product is not one that is cut (`linear_scratch`) or scratch is missing."""
+    if scratch is None:
+        return 0
+    _gpu(x, weight, scratch)
+    M, K, lda = _rows2d(x, "linear_cuts x")
+    N, Kw, ldw = _rows2d(weight, "linear_cuts weight")
+    _check(x.dtype == weight.dtype == torch.bfloat16 and Kw == K, "linear_cuts: bfloat16 x and weight of one width")
+    _check(scratch.dtype == torch.float32 and scratch.is_contiguous(), "linear_cuts: float32 scratch expected")
+    cuts = ctypes.c_int(0)
+    lib.core().call("hfee_gemm_bf16_cuts", _ptr(x), lda, _ptr(weight), ldw, M, N, K, _ptr(scratch), scratch.numel(),
+                    ctypes.byref(cuts), _stream())
+    return cuts.value
+
+
+def rope_cache_write_cuts(q, partial, cuts: int, positions, token_segment, block_tables, cos, sin, cache_layer,
+                          num_heads: int, kv_heads: int, head_dim: int, page_size: int, max_position: int,
+                          portions: bool = True):
+    """`rope_cache_write` for q, k and v that lie as the `cuts` partial products of `linear_cuts`
+    ([n, (num_heads + 2 kv_heads) * head_dim] float32 each): they are added up in their order and
+    rounded to bfloat16, rotated (adjacent pairs), q written to `q` (bfloat16 [n, num_heads *
+    head_dim], any leading dimension), k and v into the pages of `cache_layer` (bfloat16)."""
+    _gpu(q, partial, positions, cos, sin, cache_layer)
+    n, wq, ldq = _rows2d(q, "rope q")
+    _check(wq == num_heads * head_dim and q.dtype == torch.bfloat16 and cache_layer.dtype == torch.bfloat16,
+           "rope_cache_write_cuts: bfloat16 q of num_heads * head_dim columns and a bfloat16 cache")
+    _check(partial.dtype == torch.float32 and partial.is_contiguous() and
+           partial.numel() >= cuts * n * (num_heads + 2 * kv_heads) * head_dim, "rope_cache_write_cuts: partial products too short")
+    _check(cache_layer.is_contiguous() and cache_layer.dim() == 4 and
+           tuple(cache_layer.shape[1:]) == (2, kv_heads, page_size * head_dim), "rope: cache layer shape")
+    _i32(token_segment, "rope token_segment", n)
+    _i32(positions, "rope positions", n)
+    _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1, "rope: block tables")
+    half = table_positions = 0
+    if cos is not None:
+        _check(cos.shape == sin.shape and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous()
+               and cos.dtype == sin.dtype == torch.float32, "rope: cos/sin tables")
+        table_positions, half = cos.shape
+    lib.core().call("hfee_rope_cache_write_cuts", _ptr(q), ldq, _ptr(partial), int(cuts), _ptr(positions),
+                    _ptr(token_segment), _ptr(block_tables), block_tables.stride(0), _ptr(cos), _ptr(sin), half,
+                    table_positions, max_position, _ptr(cache_layer), num_heads, kv_heads, head_dim, page_size, n,
+                    1 if portions else 0, _stream())
+
+
 def linear_add_norm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, normed: torch.Tensor,
                     norm_weight: torch.Tensor, eps: float, scratch=None):
     """out (float32, the residual stream) += x @ weight.T, and normed (bfloat16) = the RMS norm of the

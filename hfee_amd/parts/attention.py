@@ -96,6 +96,10 @@ class Attention(Mixer):
         self.w_qkv_tiles, self.w_o_tiles = tiles if tiles else (None, None)
         if not self.streams:      # (nobody finishes a norm here that the part before has begun)
             self.second_half_rows = 0
+        # where the q/k/v product of a portion is cut along K, the rotation kernel can add the cuts up
+        half = self.position.rotary_dim // 2 if self.position is not None else 0
+        self.cuts_into_rotation = (self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.head_dim % 8 == 0
+                                   and half % 4 == 0)
 
     def key_layout(self):
         """What two layers must share to read one cache layer."""
@@ -167,17 +171,26 @@ class Attention(Mixer):
                              **ctx.workspace.product_scratch(n, self.w_qkv_tiles))
         else:
             hn = h.tensor() if isinstance(h, LazyNorm) else h
-            if writes_cache:
-                ops.linear(qkv, hn, self.w_qkv, **ctx.workspace.split_scratch(n, self.w_qkv))
-                k = qkv[:, self.q_width:self.q_width + self.kv_width]
-                v = qkv[:, self.q_width + self.kv_width:]
-            else:   # this run of the layer reads keys and values that another run wrote
-                ops.linear(q, hn, self.w_qkv[:self.q_width])
-                k = v = None
             portions = self.dtype != torch.bfloat16 or ctx.extra["attention.tiles"].shape[0] > 0
-            ops.rope_cache_write(q, k, v, ctx.positions, ctx.token_segment, tables, cos, sin, self.pairing,
-                                 cache if writes_cache else None, H, K, hd, ctx.page_size, ctx.max_position,
-                                 portions=portions)
+            cuts = 0
+            if writes_cache and self.cuts_into_rotation:
+                # a product of few tiles, cut along K: the rotation adds the cuts up on its way
+                scratch = ctx.workspace.split_scratch(n, self.w_qkv).get("scratch")
+                cuts = ops.linear_cuts(hn, self.w_qkv, scratch)
+                if cuts:
+                    ops.rope_cache_write_cuts(q, scratch, cuts, ctx.positions, ctx.token_segment, tables, cos, sin,
+                                              cache, H, K, hd, ctx.page_size, ctx.max_position, portions=portions)
+            if not cuts:
+                if writes_cache:
+                    ops.linear(qkv, hn, self.w_qkv, **ctx.workspace.split_scratch(n, self.w_qkv))
+                    k = qkv[:, self.q_width:self.q_width + self.kv_width]
+                    v = qkv[:, self.q_width + self.kv_width:]
+                else:   # this run of the layer reads keys and values that another run wrote
+                    ops.linear(q, hn, self.w_qkv[:self.q_width])
+                    k = v = None
+                ops.rope_cache_write(q, k, v, ctx.positions, ctx.token_segment, tables, cos, sin, self.pairing,
+                                     cache if writes_cache else None, H, K, hd, ctx.page_size, ctx.max_position,
+                                     portions=portions)
         att = ctx.rows("attention.out", self.q_width)
         if self.dtype == torch.float32:
             ops.attention_plain(att, q, cache, ctx.positions, ctx.token_segment, tables, H, K, hd,

@@ -684,6 +684,60 @@ def test_rope_cache_write(pairing, dtype):
             assert torch.equal(lay[page, 1, h].view(hd, ps)[:, vslot(slot)], v[t].view(K, hd)[h])
 
 
+@pytest.mark.parametrize("H,K,hd,rotary,d,n,portions", [(8, 2, 64, 64, 2048, 100, True), (4, 4, 128, 128, 4096, 65, False),
+                                                        (6, 2, 48, 32, 2304, 130, True), (8, 2, 64, 0, 2048, 70, True),
+                                                        (8, 2, 64, 64, 1024, 100, True), (8, 2, 64, 64, 2048, 40, True)])
+def test_rotation_that_adds_up_a_cut_product(H, K, hd, rotary, d, n, portions):
+    """The q/k/v product of a portion cut along K, its partial products added up by the
+    rotation kernel on its way to q and to the cache: bit-equal to the product (with the kernel
+    that adds the cuts) followed by the rotation.  Part of the head rotated, nothing rotated;
+    portions of prompts (values through groups of 16 tokens) and single tokens of many
+    sequences; and the cases that are not cut (a short K, few rows): no cuts, nothing launched."""
+    from hfee_amd.kernels import ops
+    from hfee_amd.parts.rotary import Rotary
+    from hfee_amd.config.specs import PositionSpec, params
+    ps = 16
+    g = torch.Generator().manual_seed(n + d + hd)
+    width = (H + 2 * K) * hd
+    x = torch.randn(n, d, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(width, d, generator=g) / math.sqrt(d)).to(torch.bfloat16).to(DEV)
+    cos = sin = None
+    if rotary:
+        rot = Rotary(PositionSpec("rope", params(head_dim=hd, rotary_dim=rotary, theta=10000.0, scaling=None, pairing="interleaved")))
+        rot.prepare(512, DEV)
+        cos, sin = rot.cos, rot.sin
+    if portions:      # two requests, portions of consecutive positions
+        first = n // 2
+        pos = torch.cat([torch.arange(32, 32 + first), torch.arange(5, 5 + n - first)]).to(torch.int32)
+        seg = torch.cat([torch.zeros(first), torch.ones(n - first)]).to(torch.int32)
+        tables = torch.stack([torch.randperm(24, generator=g)[:16], 24 + torch.randperm(24, generator=g)[:16]]).to(torch.int32)
+    else:             # one token each of n sequences
+        pos = torch.randint(0, 200, (n,), generator=g).to(torch.int32)
+        seg = torch.arange(n, dtype=torch.int32)
+        tables = torch.stack([i * 13 + torch.randperm(13, generator=g) for i in range(n)]).to(torch.int32)
+    pages = int(tables.max()) + 1
+    pos, seg, tables = pos.to(DEV), seg.to(DEV), tables.to(DEV)
+    words = ops.linear_scratch(n, width, d)
+    scratch = torch.full((max(words, 1),), float("nan"), dtype=torch.float32, device=DEV)
+    cuts = ops.linear_cuts(x, w, scratch if words else None)
+    assert (cuts > 1) == (words > 0) and (cuts == 0 or words == cuts * n * width)
+    if d <= 1024 or n <= 64:
+        assert cuts == 0
+        return
+    got_q = torch.full((n, width), float("nan"), dtype=torch.bfloat16, device=DEV)[:, :H * hd]
+    got_cache = torch.zeros(pages, 2, K, ps * hd, dtype=torch.bfloat16, device=DEV)
+    ops.rope_cache_write_cuts(got_q, scratch, cuts, pos, seg, tables, cos, sin, got_cache, H, K, hd, ps, int(pos.max()),
+                              portions=portions)
+    qkv = torch.zeros(n, width, dtype=torch.bfloat16, device=DEV)
+    ops.linear(qkv, x, w, scratch=scratch)
+    want_cache = torch.zeros_like(got_cache)
+    ops.rope_cache_write(qkv[:, :H * hd], qkv[:, H * hd:(H + K) * hd], qkv[:, (H + K) * hd:], pos, seg, tables, cos, sin, 1,
+                         want_cache, H, K, hd, ps, int(pos.max()), portions=portions)
+    assert torch.equal(got_q, qkv[:, :H * hd])
+    assert torch.equal(got_cache, want_cache)
+    assert got_cache.abs().sum() > 0
+
+
 @pytest.mark.parametrize("ps", [16, 32])
 def test_rope_cache_write_of_long_portions(ps):
     """From 32 tokens on the values of 16 consecutive tokens are written together: whole
