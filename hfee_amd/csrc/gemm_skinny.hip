@@ -1118,7 +1118,7 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 // product's shares of the rows' sums of squares to emit_ss (ceil(N / 16) x 64 floats).
 // scale_ss: shares left by such a product (scale_blocks x 64 floats) over rows of width K:
 // the finished sums are scaled by 1 / sqrt(sum / K + scale_eps).
-// scratch: for 17 to 64 rows and K a multiple of 512, a faster pair of kernels that needs
+// scratch: for 17 to 64 rows and K a multiple of 512 (of 256 from 33 rows on), a faster pair of kernels that needs
 // ceil(N / 16) * ceil(K / 1024) * ceil(M / 16) * 256 + 64 floats of scratch (none for K <= 1,024);
 // without it, or for other sizes, or where it would not pay, the streaming kernel takes
 // the product (force_mid: 1 takes the pair of kernels with slices of K wherever it applies,
