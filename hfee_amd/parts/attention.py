@@ -224,9 +224,9 @@ class Attention(Mixer):
             emit = then.offer() if then is not None else None
             ops.linear_fused(x, att, self.w_o_tiles, "add", emit=emit, **ctx.workspace.product_scratch(n, self.w_o_tiles))
         else:
-            after = then.offer_whole() if then is not None and self.dtype == torch.bfloat16 else None
-            if after:      # ... goes on with the whole norm that follows
-                ops.linear_add_norm(x, att, self.w_o, after["out"], after["weight"], after["eps"],
-                                    **ctx.workspace.split_scratch(n, self.w_o))
+            cut = ctx.workspace.split_scratch(n, self.w_o)
+            after = then.offer_whole() if then is not None and self.dtype == torch.bfloat16 and cut else None
+            if after:      # ... goes on with the whole norm that follows, where its K is cut over workgroups
+                ops.linear_add_norm(x, att, self.w_o, after["out"], after["weight"], after["eps"], **cut)
             else:
-                ops.linear(x, att, self.w_o, accumulate=True, **ctx.workspace.split_scratch(n, self.w_o))
+                ops.linear(x, att, self.w_o, accumulate=True, **cut)

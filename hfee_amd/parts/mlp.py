@@ -78,9 +78,10 @@ class GatedMLP(FeedForward):
             ops.linear(gate_up, hn, self.w_gate_up)
             ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
         # the down projection adds into x and, if asked, goes on with the norm that follows
-        after = then.offer_whole() if then is not None and aligned else None
+        # (where its K is cut over workgroups: the kernel that adds the cuts up has the row at hand)
+        cut = ctx.workspace.split_scratch(n, self.w_down)
+        after = then.offer_whole() if then is not None and aligned and cut else None
         if after:
-            ops.linear_add_norm(x, act, self.w_down, after["out"], after["weight"], after["eps"],
-                                **ctx.workspace.split_scratch(n, self.w_down))
+            ops.linear_add_norm(x, act, self.w_down, after["out"], after["weight"], after["eps"], **cut)
         else:
-            ops.linear(x, act, self.w_down, accumulate=True, **ctx.workspace.split_scratch(n, self.w_down))
+            ops.linear(x, act, self.w_down, accumulate=True, **cut)
