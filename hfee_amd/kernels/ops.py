@@ -503,11 +503,15 @@ def tile_weights_if_room(*weights: torch.Tensor):
     most 64 rows go through the kernels that read the rows as they lie."""
     device = weights[0].device
     if device.type == "cuda":
-        need = sum(w.numel() * w.element_size() for w in weights)
         free, total = torch.cuda.mem_get_info(device)
-        if free - need < TILES_LEAVE_FREE * total:
+        if not room_for_tiles(sum(w.numel() * w.element_size() for w in weights), free, total):
             return None
     return tuple(tile_weight(w) for w in weights)
+
+
+def room_for_tiles(need: int, free: int, total: int) -> bool:
+    """Whether copies of `need` bytes leave TILES_LEAVE_FREE of the `total` bytes free, `free` being free now."""
+    return free - need >= TILES_LEAVE_FREE * total
 
 
 SS_STRIDE = 64     # rows of a table of sum-of-squares shares (one row of the table per 16 weight rows)

@@ -179,3 +179,25 @@ def test_the_benchmark_refuses_more_than_one_gpu():
     assert done.returncode == 2
     lines = [l for l in (done.stdout + done.stderr).splitlines() if l.strip()]
     assert len(lines) == 1 and "one GPU" in lines[0]
+
+
+def test_second_copies_of_the_weights_only_while_they_leave_room():
+    """The weights' second copies in tiles are made while a fifth of the device's memory stays
+    free; on tensors that are not on a GPU nothing is asked and the tiles are made (all of a
+    part's weights or none), in the layout the kernels read: 16 rows x 32 columns a kilobyte."""
+    import torch
+    from hfee_amd.kernels import ops
+    gib = 1 << 30
+    assert ops.room_for_tiles(2 * gib, free=100 * gib, total=288 * gib)
+    assert ops.room_for_tiles(42 * gib, free=100 * gib, total=288 * gib)
+    assert not ops.room_for_tiles(43 * gib, free=100 * gib, total=288 * gib)
+    assert not ops.room_for_tiles(1, free=57 * gib, total=288 * gib)
+    w = torch.arange(40 * 72, dtype=torch.float32).reshape(40, 72).to(torch.bfloat16)
+    tiles = ops.tile_weights_if_room(w, w[:16])
+    assert len(tiles) == 2 and (tiles[0].n, tiles[0].k) == (40, 72)
+    t = tiles[0].tiles
+    assert t.shape == (3, 3, 512)                        # rows and columns padded to whole tiles
+    # element (row r, column c) lies in tile (r // 16, c // 32) at ((c % 32) // 8) * 128 + (r % 16) * 8 + c % 8
+    for r, c in ((0, 0), (5, 9), (17, 40), (39, 71)):
+        assert t[r // 16, c // 32, ((c % 32) // 8) * 128 + (r % 16) * 8 + c % 8] == w[r, c]
+    assert t[2, 2, 511] == 0                             # padding
