@@ -542,28 +542,43 @@ template <int WAVES, bool RING>
 __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, uint32_t layer_bytes, CacheLayout lay, const int* __restrict__ work, int num_tiles,
+    const int* __restrict__ runs, int num_runs,
     const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2, int window) {
   extern __shared__ __attribute__((aligned(1024))) char kv_lds[];     // two tiles of KV_BLOCKS KB
   const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), waves = blockDim.x >> 6;
   const int group = num_heads / lay.kv_heads, chunks = (group + waves - 1) / waves;
+  // What the waves of a workgroup share a key tile for: the heads of a KV head over one row
+  // tile, or (runs: heads that share no keys with another) up to four row tiles of one head
+  // that follow one another in a sequence, run (first tile, count): the keys of the last of
+  // them are the keys of all, and a wave leaves out the tiles beyond its own rows.
+  const bool by_rows = runs != nullptr;
   // Workgroups go to the eight XCDs in turn; every XCD gets a contiguous run of the work,
   // ordered by KV head first (its keys then live in one L2), later row tiles first.
-  int tile, kvh, chunk;
+  int tile, last_tile, kvh, chunk;
   {
-    const int per_kv = num_tiles * chunks, total = per_kv * lay.kv_heads, per_xcd = (total + 7) / 8;
+    const int per_kv = by_rows ? num_runs : num_tiles * chunks, total = per_kv * lay.kv_heads, per_xcd = (total + 7) / 8;
     const int u = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (u >= total) return;
     kvh = u / per_kv;
     const int rest = u - kvh * per_kv;
-    tile = num_tiles - 1 - rest / chunks;
-    chunk = rest % chunks;
+    if (by_rows) {
+      const int* run = runs + 2 * (num_runs - 1 - rest);
+      tile = run[0];
+      last_tile = tile + run[1] - 1;
+      chunk = 0;
+    } else {
+      tile = last_tile = num_tiles - 1 - rest / chunks;
+      chunk = rest % chunks;
+    }
   }
-  const int* wk = work + 4 * tile;
+  // the keys that the workgroup walks: from the first tile's first key to the last tile's last
+  const int wg_pos0 = work[4 * tile + 2], wg_last = work[4 * last_tile + 2] + work[4 * last_tile + 1] - 1;
+  const bool head_ok = by_rows ? tile + wave <= last_tile : chunk * waves + wave < group;      // a wave without work still loads its share
+  const int* wk = work + 4 * (by_rows && head_ok ? tile + wave : tile);
   const int row0 = wk[0], rows = wk[1], pos0 = wk[2], seg = wk[3];
   const int* bt = block_tables + (int64_t)seg * bt_stride;
-  const bool head_ok = chunk * waves + wave < group;      // a wave without a head still loads its share
-  const int h = kvh * group + (head_ok ? chunk * waves + wave : 0);
+  const int h = by_rows ? kvh : kvh * group + (head_ok ? chunk * waves + wave : 0);
 
   const bool slot_ok = r32 < rows && head_ok;
   const int pos = slot_ok ? pos0 + r32 : -1;
@@ -573,10 +588,11 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
 
   Tile st;
   init_tile(st);
-  const int kv_last = pos0 + rows - 1;
-  const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int kv_last = wg_last;
+  const int kv_first = window > 0 ? max(0, wg_pos0 - window + 1) : 0;
   const int t_first = kv_first >> 5, t_end = (kv_last >> 5) + 1;
-  const int all_first = window > 0 ? max(0, kv_last - window + 1) : 0;   // every row in use sees all_first .. pos0
+  const int my_last = pos0 + rows - 1;                                    // this wave's last key
+  const int all_first = window > 0 ? max(0, my_last - window + 1) : 0;   // every row in use sees all_first .. pos0
   PageWindow pages;
   pages.base = -1;
   constexpr int TILE_BYTES = KV_BLOCKS * 1024;
@@ -585,6 +601,10 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
   // (a raw buffer of 32-bit data over the layer; only the ring's loads go through it)
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cache, 0, (int)layer_bytes, 0x00020000);
   auto compute = [&](int t, const char* tile_at, auto under_scores) {
+    if (!head_ok || t * 32 > my_last) {      // (a wave without work, or of earlier rows: nothing here is visible to it)
+      under_scores();
+      return;
+    }
     const char* cur = tile_at + lane * 16;
     compute_tile_with(
         st, q_op, [&](int c) { return *reinterpret_cast<const bf16x8*>(cur + c * 1024); },
@@ -891,6 +911,7 @@ static int check_common(const char* name, int64_t ld_out, int64_t ldq, int num_h
 // of a KV head (for tests of each kernel alone).
 HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* q, int64_t ldq,
                                          const void* cache, int cache_pages, const int* work, int num_tiles,
+                                         const int* runs, int num_runs,
                                          const int* block_tables, int bt_stride, int num_heads, int kv_heads,
                                          int page_size, float scale, int window, int variant, hipStream_t stream) {
   HFEE_REQUIRE(num_tiles >= 0, "attention_bf16_prefill: bad tile count");
@@ -902,15 +923,20 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
     return 1;
   HFEE_REQUIRE((int64_t)num_tiles * num_heads < (1ll << 30), "attention_bf16_prefill: too much work for one launch");
   const int group = num_heads / kv_heads;
-  if (variant == 1 || (variant == 0 && group == 1)) {      // nothing to share: one wave per (tile, head)
+  HFEE_REQUIRE(runs == nullptr || num_runs > 0, "attention_bf16_prefill: runs of row tiles without their number");
+  const int64_t layer_bytes = (int64_t)cache_pages * lay.page_stride * 2;
+  // heads that share no keys with another: the row tiles of a head that follow one another
+  // share them instead, four at a time, where the caller has listed such runs
+  const bool by_rows = group == 1 && runs != nullptr && variant != 1 && KV_BLOCKS % SHARED_WAVES == 0 &&
+                       layer_bytes < (1ll << 32);
+  if (!by_rows && (variant == 1 || (variant == 0 && group == 1))) {      // nothing to share: one wave per (tile, head)
     dim3 grid((unsigned)(((int64_t)num_tiles * num_heads + 7) / 8 * 8));
     prefill_kernel<<<grid, 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
                                             work, num_tiles, block_tables, bt_stride, num_heads, scale * LOG2E, window);
   } else {
-    const int waves = group < SHARED_WAVES ? group : SHARED_WAVES, chunks = (group + waves - 1) / waves;
+    const int waves = by_rows ? SHARED_WAVES : group < SHARED_WAVES ? group : SHARED_WAVES, chunks = (group + waves - 1) / waves;
     // the ring of tiles with loads waited for by count: four waves that bring equal shares of a
     // tile, and a layer that 32 bits address
-    const int64_t layer_bytes = (int64_t)cache_pages * lay.page_stride * 2;
     const bool ring = waves == SHARED_WAVES && KV_BLOCKS % SHARED_WAVES == 0 && layer_bytes < (1ll << 32);
     const size_t lds = (size_t)(ring ? SHARED_TILES : 2) * KV_BLOCKS * 1024;
     static bool raised = false;
@@ -927,12 +953,13 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
       HFEE_REQUIRE(e == hipSuccess, "attention_bf16_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
       raised = true;
     }
-    dim3 grid((unsigned)(((int64_t)num_tiles * kv_heads * chunks + 7) / 8 * 8));
+    dim3 grid((unsigned)(((int64_t)(by_rows ? num_runs : num_tiles * chunks) * kv_heads + 7) / 8 * 8));
+    const int* runs_or_none = by_rows ? runs : nullptr;
 #define GO(W, R)                                                                                                    \
   prefill_shared_kernel<W, R><<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,         \
                                                                 (const bf16_t*)cache, (uint32_t)(ring ? layer_bytes : 0),  \
-                                                                lay, work, num_tiles, block_tables, bt_stride, num_heads, \
-                                                                scale * LOG2E, window)
+                                                                lay, work, num_tiles, runs_or_none, num_runs, block_tables, \
+                                                                bt_stride, num_heads, scale * LOG2E, window)
     if (ring) GO(SHARED_WAVES, (KV_BLOCKS % SHARED_WAVES == 0));
     else if (waves == SHARED_WAVES) GO(SHARED_WAVES, false);
     else GO(0, false);

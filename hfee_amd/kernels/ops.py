@@ -388,17 +388,25 @@ def _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, he
 
 
 def attention_bf16_prefill(out, q, cache_layer, tiles, block_tables, num_heads: int, kv_heads: int,
-                           head_dim: int, page_size: int, scale: float, window: int = 0, kernel: int = 0):
+                           head_dim: int, page_size: int, scale: float, window: int = 0, kernel: int = 0, runs=None):
     """tiles: [num_tiles, 4] int32 (first row, rows <= 32, first position, block-table row).
     kernel: 0 automatic, 1 one wave per (tile, head), 2 the heads of a KV head share its
-    key tiles through LDS."""
+    key tiles through LDS.
+    runs: [num_runs, 2] int32 (first tile, count <= 4) or None: every tile in exactly one run of
+    tiles that follow one another in `tiles` and in one sequence, rows and positions going on
+    where the tile before ended.  For heads that share no keys with another head (kv_heads ==
+    num_heads) the row tiles of a run then share the head's key tiles through LDS."""
     n, ldq, ldo = _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size)
     _check(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
            "attention: tiles must be [num_tiles, 4] int32")
+    if runs is not None:
+        _gpu(runs)
+        _check(runs.dtype == torch.int32 and runs.dim() == 2 and runs.shape[1] == 2 and runs.is_contiguous() and runs.shape[0] > 0,
+               "attention: runs must be [num_runs, 2] int32")
     lib.attention_bf16(head_dim).call(
         "hfee_attention_bf16_prefill", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), cache_layer.shape[0], _ptr(tiles),
-        tiles.shape[0], _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, page_size,
-        float(scale), int(window), int(kernel), _stream())
+        tiles.shape[0], _ptr(runs), 0 if runs is None else runs.shape[0], _ptr(block_tables), block_tables.stride(0),
+        num_heads, kv_heads, page_size, float(scale), int(window), int(kernel), _stream())
 
 
 def attention_bf16_decode(out, q, cache_layer, seg_rows, seg_positions, seg_tables, block_tables,

@@ -544,7 +544,8 @@ def _paged(kv, page_size, pages_order):
 @pytest.mark.parametrize("H,K,hd,T,window", [(4, 2, 16, 37, 0), (3, 1, 32, 100, 0), (6, 3, 48, 70, 0),
                                              (2, 2, 64, 33, 0), (4, 1, 128, 130, 0), (4, 2, 16, 90, 20),
                                              (5, 5, 80, 40, 0), (1, 1, 256, 35, 0), (12, 2, 64, 200, 0),
-                                             (8, 1, 256, 70, 33)])
+                                             (8, 1, 256, 70, 33),
+                                             (3, 3, 128, 300, 0), (5, 5, 64, 200, 70), (2, 2, 48, 129, 0)])     # no two heads share keys
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_kernels(H, K, hd, T, window, dtype):
     """Plain kernel (both dtypes) and the matrix-core kernels (bfloat16) against
@@ -585,6 +586,12 @@ def _check_attention(H, K, hd, T, window, dtype, ps):
             out2 = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
             ops.attention_bf16_prefill(out2, qd, layer, tiles, table, H, K, hd, ps, scale, window, kernel=kernel)
             close(out2, ref, tol)
+        # runs of up to four row tiles of a head that share its key tiles (taken where no two heads share keys)
+        n_tiles = tiles.shape[0]
+        runs = torch.tensor([(t, min(4, n_tiles - t)) for t in range(0, n_tiles, 4)], dtype=torch.int32, device=DEV)
+        out2 = torch.full((T, H * hd), float("nan"), dtype=dtype, device=DEV)
+        ops.attention_bf16_prefill(out2, qd, layer, tiles, table, H, K, hd, ps, scale, window, runs=runs)
+        close(out2, ref, tol)
         # decode kernel: the last rows as single queries, with and without split keys
         # (joined by a second launch, and by the workgroup that finishes last: twice, the
         # second time on the counters that the first call left)
