@@ -934,7 +934,12 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
     prefill_kernel<<<grid, 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
                                             work, num_tiles, block_tables, bt_stride, num_heads, scale * LOG2E, window);
   } else {
-    const int waves = by_rows ? SHARED_WAVES : group < SHARED_WAVES ? group : SHARED_WAVES, chunks = (group + waves - 1) / waves;
+    const bool can_ring = KV_BLOCKS % SHARED_WAVES == 0 && layer_bytes < (1ll << 32);
+    // (two or three heads to a KV head: four waves all the same, of which the others only bring
+    // their shares of the tiles, so that the ring applies: 16 heads over 8 KV heads 92 -> 69 µs
+    // at 2,048 tokens, 24 heads 96 -> 76)
+    const int waves = by_rows || (can_ring && group >= 2) ? SHARED_WAVES : group < SHARED_WAVES ? group : SHARED_WAVES;
+    const int chunks = (group + waves - 1) / waves;
     // the ring of tiles with loads waited for by count: four waves that bring equal shares of a
     // tile, and a layer that 32 bits address
     const bool ring = waves == SHARED_WAVES && KV_BLOCKS % SHARED_WAVES == 0 && layer_bytes < (1ll << 32);
