@@ -1063,11 +1063,12 @@ bool launch_wide_steps(const Args& a, int row_groups, int grid, hipStream_t stre
   else if (steps == 8) wide_kernel<8, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
   else if (steps == 12) wide_kernel<12, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
   else if (steps == 16) wide_kernel<16, NORM, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
-  else if (steps == 20) {
+  else if (steps == 20 || steps == 32) {
     // (with the norm folded in, the float32 rows on their way to operands need more registers
     // than a wave of eight a CU has: those products stay with the streaming kernel)
     if constexpr (NORM) return false;
-    else wide_kernel<20, false, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
+    else if (steps == 20) wide_kernel<20, false, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
+    else wide_kernel<32, false, EPI><<<grid, WAVES * 64, 0, stream>>>(a, row_groups);
   } else return false;      // other widths: the streaming kernel takes them
   return true;
 }
@@ -1082,7 +1083,7 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
     num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
   const int row_groups = (a.N + ROWS - 1) / ROWS;
-  if (a.M > 16 || a.K % (128 * WAVES) != 0 || a.K > 20 * 32 * WAVES) return false;
+  if (a.M > 16 || a.K % (128 * WAVES) != 0 || a.K > 32 * 32 * WAVES) return false;
   // from two row groups a workgroup on: the workgroups then share the weight rows evenly, where
   // one row group each leaves a second round that fills a part of the chip only (q/k/v of the 8B
   // shape, 384 row groups: 1.5 us a layer inside the decode step; and better than the streaming

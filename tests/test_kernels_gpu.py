@@ -264,7 +264,7 @@ def test_weights_in_tiles():
                                    (5, 17000, 4096), (2, 16390, 3072), (33, 200, 128), (64, 52, 1024),
                                    (7, 50, 40), (12, 107, 200), (4, 20, 8), (9, 6144, 512),
                                    (16, 5130, 1280), (3, 8000, 200),      # more workgroups than CUs, at most twice as many
-                                   (5, 8300, 5120)])                       # the persistent kernel at K = 5,120
+                                   (5, 8300, 5120), (7, 8200, 8192)])      # the persistent kernel at K = 5,120 and 8,192
 @pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu"])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_decode_products(M, N, K, epilogue, norm):
