@@ -560,8 +560,8 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 // ------------------------------------------------------------ 17 to 64 rows ---
 // With more than 16 batch rows the streaming kernel reads the batch again for every 16
 // weight rows, and that traffic (from L2) outgrows the weights.  Here K is cut into
-// slices of 1,024 columns (the last one may be shorter: a multiple of 512 columns, of 256 from 33
-// batch rows on), each with workgroups of its own.  A workgroup keeps its slice
+// slices of 1,024 columns (the last one may be shorter: a multiple of 256 columns), each with
+// workgroups of its own.  A workgroup keeps its slice
 // of the batch, all rows, in LDS; each of its waves walks over groups of 16 weight rows
 // on its own: the weights come straight from global memory through a ring of 4 or 16 loads
 // that runs across group boundaries, the batch operands from LDS; no barrier stands in
@@ -570,15 +570,16 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 // group, so that the whole chip takes part) adds the shares in the order of the slices and
 // runs the epilogue.  Nobody waits for anybody, and nothing is counted.
 constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32;
-// loads a wave keeps in flight.  Measured inside the decode step at 64 rows (q/k/v, output, down
-// of the 8B shape): 20.3 / 14.2 / 27.2 µs with 8, 15.0 / 13.8 / 27.1 with 4, 19.7 / 15.2 / 30.4 with 2;
-// at 24 and 32 rows 4 and 16 measured alike.
+// Loads a wave keeps in flight: four.  Measured inside the decode step at 64 rows (q/k/v, output,
+// down of the 8B shape): 20.3 / 14.2 / 27.2 µs with 8, 15.0 / 13.8 / 27.1 with 4, 19.7 / 15.2 / 30.4
+// with 2; at 24 and 32 rows 4 against 16: 4.41 against 4.46 ms a step, 4.70 against 4.73.
+// The loop is unrolled over eight steps (whole turns of the ring), and the last slice of K is
+// a whole number of these: K is a multiple of 256 columns.  (The same loop over 16 steps with
+// a last turn of 8, written as one body for both, measured 3 % slower over the whole step at
+// 64 rows: 5.91 ms against 5.73.)
+constexpr int MID_RING = 4, MID_HALF = 8;
+// (the kernel for many weight rows, below, keeps its own count)
 constexpr int mid_ring(int mt) { return mt >= 3 ? 4 : 16; }
-// steps that the loop is unrolled over (whole turns of the ring): the last slice of K is a whole
-// number of these, so K is a multiple of 256 columns from 33 batch rows on, of 512 below.  (The
-// same loop over 16 steps with a last turn of 8, written as one body for both, measured 3 %
-// slower over the whole step at 64 rows: 5.91 ms against 5.73.)
-constexpr int mid_unroll(int mt) { return mt >= 3 ? 8 : 16; }
 constexpr int MID_PITCH = MID_KS + 8;        // LDS row pitch of the batch slice in elements: rows 16 bytes askew
 
 constexpr size_t mid_lds_bytes(int mt) { return (size_t)mt * 16 * MID_PITCH * sizeof(bf16_t); }
@@ -622,7 +623,6 @@ __global__ __launch_bounds__(WAVES * 64) void mid_kernel(Args a, int row_groups,
   const int per_slice = gridDim.x / slices;
   int rg = blockIdx.x / slices + per_slice * wave;
   const bf16_t* w_cur = row_ptr(min(rg, row_groups - 1));
-  constexpr int MID_RING = mid_ring(MT), MID_HALF = mid_unroll(MT);
   static_assert(MID_HALF % MID_RING == 0 && MID_STEPS % MID_HALF == 0, "a ring slot means the same step in every turn of the loop");
   Chunk ring[MID_RING];
 #pragma unroll
@@ -1119,7 +1119,7 @@ bool launch_wide(const Args& a, bool norm, int epi, hipStream_t stream) {
 // product's shares of the rows' sums of squares to emit_ss (ceil(N / 16) x 64 floats).
 // scale_ss: shares left by such a product (scale_blocks x 64 floats) over rows of width K:
 // the finished sums are scaled by 1 / sqrt(sum / K + scale_eps).
-// scratch: for 17 to 64 rows and K a multiple of 512 (of 256 from 33 rows on), a faster pair of kernels that needs
+// scratch: for 17 to 64 rows and K a multiple of 256, a faster pair of kernels that needs
 // ceil(N / 16) * ceil(K / 1024) * ceil(M / 16) * 256 + 64 floats of scratch (none for K <= 1,024);
 // without it, or for other sizes, or where it would not pay, the streaming kernel takes
 // the product (force_mid: 1 takes the pair of kernels with slices of K wherever it applies,
@@ -1215,7 +1215,7 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
       return 0;
     }
   }
-  if (!norm && mt > 1 && K % (32 * mid_unroll(mt)) == 0 && (mid_pays || force_mid == 1)) {
+  if (!norm && mt > 1 && K % 256 == 0 && (mid_pays || force_mid == 1)) {
     const bool took = mt == 2 ? launch_mid_rows<2>(a, epi, scratch, scratch_floats, num_cus, stream)
                     : mt == 3 ? launch_mid_rows<3>(a, epi, scratch, scratch_floats, num_cus, stream)
                               : launch_mid_rows<4>(a, epi, scratch, scratch_floats, num_cus, stream);

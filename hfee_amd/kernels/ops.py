@@ -528,7 +528,7 @@ SS_STRIDE = 64     # rows of a table of sum-of-squares shares (one row of the ta
 def mid_rows_scratch(n_rows: int, n_weight_rows: int, k: int) -> int:
     """float32 words of scratch that a product of 17 to 64 rows wants for its faster kernel
     (0: it has no use for scratch)."""
-    if n_rows <= 16 or n_rows > SKINNY_MAX_ROWS or k % (256 if n_rows > 32 else 512) or k <= 1024:
+    if n_rows <= 16 or n_rows > SKINNY_MAX_ROWS or k % 256 or k <= 1024:
         return 0
     return ((n_weight_rows + 15) // 16) * ((k + 1023) // 1024) * ((n_rows + 15) // 16) * 256 + SS_STRIDE
 
@@ -545,7 +545,7 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
     ceil(N / 16) * 64).  row_scale: dict(shares, blocks, eps): the other half: x is such an
     emitted tensor, and the finished sums are scaled by 1 / sqrt(sum of shares / K + eps).
     scratch (float32, `mid_rows_scratch` words): lets products of 17 to 64 rows over
-    K % 512 == 0 (K % 256 == 0 from 33 rows on) take a kernel that keeps the batch in LDS and cuts K over workgroups, and a
+    K % 256 == 0 take a kernel that keeps the batch in LDS and cuts K over workgroups, and a
     second one that adds the slices up, where that pays.  Products with weight rows enough to
     fill the chip take a kernel that cuts nothing and needs no scratch.  (force_mid_rows, for
     tests: 1 takes the first wherever it applies, 2 the second.)

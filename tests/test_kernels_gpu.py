@@ -309,11 +309,11 @@ def test_fused_decode_products(M, N, K, epilogue, norm):
 
 @pytest.mark.parametrize("M,N,K", [(17, 48, 1024), (33, 200, 2048), (64, 344, 3072), (40, 6150, 4096), (64, 100, 1024),
                                    (48, 30, 2048), (64, 200, 512), (33, 520, 1536), (50, 344, 3584),
-                                   (64, 136, 2304), (40, 72, 1280), (33, 200, 11008)])     # last slices of 256 and of 768 columns
+                                   (64, 136, 2304), (40, 72, 1280), (33, 200, 11008), (20, 136, 2304), (32, 72, 11008)])     # last slices of 256 and of 768 columns
 @pytest.mark.parametrize("epilogue", ["bf16", "f32", "add", "swiglu", "emit", "scaled"])
 def test_products_of_17_to_64_rows(M, N, K, epilogue):
     """The kernel that keeps the batch in LDS and cuts K over workgroups (17 to 64 rows,
-    K a multiple of 512, of 256 from 33 rows on: slices of 1,024 and a last, shorter one) and the kernel that adds its
+    K a multiple of 256: slices of 1,024 and a last, shorter one) and the kernel that adds its
     slices up, with every epilogue, twice in a row on the same scratch, against the unfused formulas."""
     _products_of_17_to_64_rows(M, N, K, epilogue, 1)
 
