@@ -579,8 +579,9 @@ constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32;
 // 64 rows: 5.91 ms against 5.73.)
 constexpr int MID_RING = 4, MID_HALF = 8;
 // (the kernel for many weight rows, below, keeps its own count: at 24 and 32 rows 4.36 and 4.68 ms
-// a step with 8, 4.41 and 4.70 with 16, 4.40 and 4.74 with 4)
-constexpr int mid_ring(int mt) { return mt >= 3 ? 4 : 8; }
+// a step with 8, 4.41 and 4.70 with 16, 4.40 and 4.74 with 4; at 48 rows 5.28 with 8 and 5.33 with
+// 4; at 64 rows 5.94 with 8 and 5.75 with 4)
+constexpr int mid_ring(int mt) { return mt >= 4 ? 4 : 8; }
 constexpr int MID_PITCH = MID_KS + 8;        // LDS row pitch of the batch slice in elements: rows 16 bytes askew
 
 constexpr size_t mid_lds_bytes(int mt) { return (size_t)mt * 16 * MID_PITCH * sizeof(bf16_t); }
