@@ -572,7 +572,8 @@ void launch_epi(const Args& a, int epi, hipStream_t stream) {
 constexpr int MID_KS = 1024, MID_STEPS = MID_KS / 32;
 // Loads a wave keeps in flight: four.  Measured inside the decode step at 64 rows (q/k/v, output,
 // down of the 8B shape): 20.3 / 14.2 / 27.2 µs with 8, 15.0 / 13.8 / 27.1 with 4, 19.7 / 15.2 / 30.4
-// with 2; at 24 and 32 rows 4 against 16: 4.41 against 4.46 ms a step, 4.70 against 4.73.
+// with 2; at 24 and 32 rows 4 against 16: 4.41 against 4.46 ms a step, 4.70 against 4.73; at 24
+// and 48 rows 4 against 8: 4.35 against 4.44, 5.29 against 5.36.
 // The loop is unrolled over eight steps (whole turns of the ring), and the last slice of K is
 // a whole number of these: K is a multiple of 256 columns.  (The same loop over 16 steps with
 // a last turn of 8, written as one body for both, measured 3 % slower over the whole step at
