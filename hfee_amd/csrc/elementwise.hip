@@ -47,6 +47,72 @@ __global__ __launch_bounds__(256) void embed_bf16_wide_kernel(float* __restrict_
   *reinterpret_cast<f32x4*>(o + 4) = hi;
 }
 
+// The same for at most 64 rows, with the first half of the norm that follows: also
+// bfloat16(x * weight) into emit_out and, for the row's columns that this workgroup takes,
+// their sum of squares into emit_ss[blockIdx.y * 64 + row] (the form in which the products
+// of at most 64 rows take a norm in two halves: hfee_gemm_skinny's scale_ss).
+template <typename TW>
+__global__ __launch_bounds__(256) void embed_bf16_emit_kernel(float* __restrict__ out, const bf16_t* __restrict__ table,
+                                                              const int* __restrict__ ids, int d,
+                                                              const TW* __restrict__ weight, bf16_t* __restrict__ emit_out,
+                                                              int64_t ld_emit, float* __restrict__ emit_ss) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  __shared__ float parts[4];
+  const int row = blockIdx.x, j = 8 * (blockIdx.y * 256 + threadIdx.x);
+  float ss = 0.f;
+  if (j < d) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(table + (int64_t)ids[row] * d + j);
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = __uint_as_float(v[i] << 16);
+      x[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+    }
+    float* o = out + (int64_t)row * d + j;
+    *reinterpret_cast<f32x4*>(o) = f32x4{x[0], x[1], x[2], x[3]};
+    *reinterpret_cast<f32x4*>(o + 4) = f32x4{x[4], x[5], x[6], x[7]};
+    u32x4 e;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ss = fmaf(x[2 * i], x[2 * i], ss);
+      ss = fmaf(x[2 * i + 1], x[2 * i + 1], ss);
+      e[i] = (uint32_t)float_to_bf16(x[2 * i] * to_float<TW>(weight[j + 2 * i])) |
+             (uint32_t)float_to_bf16(x[2 * i + 1] * to_float<TW>(weight[j + 2 * i + 1])) << 16;
+    }
+    *reinterpret_cast<u32x4*>(emit_out + (int64_t)row * ld_emit + j) = e;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  if ((threadIdx.x & 63) == 0) parts[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  if (threadIdx.x == 0) emit_ss[blockIdx.y * 64 + row] = (parts[0] + parts[1]) + (parts[2] + parts[3]);
+}
+
+// hfee_embed of a bfloat16 table for at most 64 rows, which also writes bfloat16(out * emit_weight)
+// to emit_out [n, d] (rows ld_emit apart, 16-byte aligned) and the rows' sums of squares to
+// emit_ss, in ceil(d / 2,048) shares of 64 floats (a workgroup takes 2,048 columns of a row).
+HFEE_API int hfee_embed_emit(float* out, const void* table, const int* ids, int n, int d, const void* emit_weight,
+                             int emit_weight_dtype, void* emit_out, int64_t ld_emit, float* emit_ss,
+                             int64_t emit_ss_floats, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && n <= 64 && d > 0 && d % 8 == 0, "embed_emit: at most 64 rows of a width that is a multiple of 8 (n=%d d=%d)", n, d);
+  HFEE_REQUIRE((uintptr_t)table % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)emit_out % 16 == 0 && ld_emit % 8 == 0 &&
+               ld_emit >= d && emit_weight && emit_ss, "embed_emit: 16-byte aligned rows expected");
+  const dim3 grid(n > 0 ? n : 1, (d + 2047) / 2048);
+  HFEE_REQUIRE(emit_ss_floats >= (int64_t)grid.y * 64, "embed_emit: %d shares of 64 floats expected", (int)grid.y);
+  if (n == 0) return 0;
+  if (emit_weight_dtype == DT_F32)
+    embed_bf16_emit_kernel<float><<<grid, 256, 0, stream>>>(out, (const bf16_t*)table, ids, d, (const float*)emit_weight,
+                                                            (bf16_t*)emit_out, ld_emit, emit_ss);
+  else if (emit_weight_dtype == DT_BF16)
+    embed_bf16_emit_kernel<bf16_t><<<grid, 256, 0, stream>>>(out, (const bf16_t*)table, ids, d, (const bf16_t*)emit_weight,
+                                                             (bf16_t*)emit_out, ld_emit, emit_ss);
+  else
+    return fail("embed_emit: unknown dtype %d", emit_weight_dtype);
+  HFEE_CHECK_LAUNCH("embed_emit");
+  return 0;
+}
+
 HFEE_API int hfee_embed(float* out, const void* table, int table_dtype, const int* ids,
                         int n, int d, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && d > 0, "embed: bad sizes n=%d d=%d", n, d);

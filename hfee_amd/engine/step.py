@@ -355,9 +355,14 @@ class Engine:
 
     def _forward(self, ctx, n: int, w: int, dev: dict):
         x = self.workspace.rows("residual", n, self.model.spec.hidden, torch.float32)
-        self.model.embedding.forward(ctx, x)
         schedule, blocks = self.model.schedule, self.model.blocks
-        carried = None          # the next block's normed input, if the block before has begun it
+        carried = None          # the next block's normed input, if what ran before has begun it
+        first = blocks[schedule[0].layer] if schedule else None
+        if getattr(self.model.embedding, "emits_norm", False) and getattr(first, "chains_norms", False):
+            carried = first.begin(ctx, x)
+            self.model.embedding.forward(ctx, x, then=carried)
+        else:
+            self.model.embedding.forward(ctx, x)
         for i, entry in enumerate(schedule):
             block = blocks[entry.layer]
             if getattr(block, "chains_norms", False):

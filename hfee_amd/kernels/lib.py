@@ -24,6 +24,7 @@ P, I, L, F, U64 = c_void_p, c_int, c_int64, c_float, c_uint64
 
 _CORE_SIGNATURES = {
     "hfee_embed": [P, P, I, P, I, I, P],
+    "hfee_embed_emit": [P, P, P, I, I, P, I, P, L, P, L, P],
     "hfee_rmsnorm": [P, I, P, P, I, P, F, I, I, P],
     "hfee_swiglu": [P, L, P, P, L, I, I, I, I, P],
     "hfee_residual_add": [P, P, I, L, P],

@@ -67,14 +67,44 @@ def _i32(t, what, n=None):
 
 # ------------------------------------------------------------------ simple ops
 
-def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor):
-    """out[i, :] = table[ids[i], :] as float32."""
+def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, emit: dict | None = None):
+    """out[i, :] = table[ids[i], :] as float32.
+
+    emit: dict(weight, out, shares) as for `linear_fused`: the first half of the norm that
+    follows, bfloat16(out * weight) into emit["out"] and the rows' sums of squares in
+    `embed_emit_blocks(width)` shares of 64 floats into emit["shares"] (`can_embed_emit` says
+    for which tables and rows)."""
     _gpu(out, table, ids)
     n, d, _ = _rows2d(out, "embed out")
     _check(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous float32")
     _check(table.dim() == 2 and table.is_contiguous() and table.shape[1] == d, "embed: table shape")
     _i32(ids, "embed ids", n)
-    lib.core().call("hfee_embed", _ptr(out), _ptr(table), _dt(table), _ptr(ids), n, d, _stream())
+    if emit is None:
+        lib.core().call("hfee_embed", _ptr(out), _ptr(table), _dt(table), _ptr(ids), n, d, _stream())
+        return
+    eo, es, ew = emit["out"], emit["shares"], emit["weight"]
+    _gpu(eo, es, ew)
+    _check(can_embed_emit(table, n), "embed: the norm's first half only with a bfloat16 table of a width that is a "
+           "multiple of 8, for at most 64 rows")
+    Me, Ne, lde = _rows2d(eo, "embed emit out")
+    _check(eo.dtype == torch.bfloat16 and Me >= n and Ne == d, "embed: emit out must be bfloat16 [n, width]")
+    _check(ew.numel() == d and ew.is_contiguous(), "embed: emit weight")
+    _check(es.dtype == torch.float32 and es.is_contiguous() and es.numel() >= embed_emit_blocks(d) * SS_STRIDE,
+           "embed: the shares need embed_emit_blocks(width) * 64 float32")
+    lib.core().call("hfee_embed_emit", _ptr(out), _ptr(table), _ptr(ids), n, d, _ptr(ew), _dt(ew), _ptr(eo), lde,
+                    _ptr(es), es.numel(), _stream())
+
+
+EMBED_COLUMNS_A_WORKGROUP = 2048     # of a row, in the embedding kernels for bfloat16 tables
+
+
+def can_embed_emit(table: torch.Tensor, n: int) -> bool:
+    return table.dtype == torch.bfloat16 and table.shape[1] % 8 == 0 and n <= SS_STRIDE
+
+
+def embed_emit_blocks(width: int) -> int:
+    """Shares of a row's sum of squares that `embed(..., emit=...)` leaves."""
+    return (width + EMBED_COLUMNS_A_WORKGROUP - 1) // EMBED_COLUMNS_A_WORKGROUP
 
 
 def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None):

@@ -6,6 +6,7 @@ model it is in.  Seven kinds, each with a registry from the spec's `kind` string
 a class:
 
   embedding       forward(ctx, x): the residual stream's first value from the token ids
+                  (with `emits_norm = True`: forward(ctx, x, then=None), see LazyNorm)
   norm            forward(ctx, out, x, rows=None)
   position        prepare(num_positions, device); applied by the mixer that owns it
   mixer           forward_add(ctx, x, h, cache_layer, writes_cache): x += mix(h)
@@ -151,7 +152,8 @@ class LazyNorm:
     the LazyNorm of what follows it as `then`; if `then.offer()` returns arguments, its
     adding product also writes bfloat16(x_new * weight) and the rows' sums of squares
     (`ops.linear_fused(..., emit=...)`).  The part that consumes the norm then finds
-    `pending` set and gives it to its first product as `row_scale`."""
+    `pending` set and gives it to its first product as `row_scale`.  An embedding with
+    `emits_norm = True` is handed the first block's LazyNorm in the same way."""
 
     def __init__(self, ctx, norm, x, second_half_rows: int = 0):
         self.ctx, self.norm, self.x = ctx, norm, x
@@ -163,17 +165,21 @@ class LazyNorm:
         """(weight, eps) if the norm is y = x / sqrt(mean(x^2) + eps) * weight, else None."""
         return getattr(self.norm, "fused_form", lambda: None)()
 
-    def offer(self):
-        """For the part that adds into x last: the `emit` arguments of its adding product,
-        or None if this norm cannot be split (then nothing changes for anybody)."""
+    def offer(self, blocks: int | None = None):
+        """For the part that writes x last: the `emit` arguments of its adding product, or None
+        if this norm cannot be split (then nothing changes for anybody).  blocks: in how many
+        shares the producer leaves a row's sum of squares (one for every 16 columns unless it
+        says otherwise)."""
         form = self.fusable()
         if form is None or self.x.dtype != torch.float32 or self.ctx.n > self.second_half_rows:
             return None
         weight, eps = form
         width = self.x.shape[1]
-        blocks = (width + 15) // 16
+        most = (width + 15) // 16
+        blocks = blocks or most
         out = self.ctx.rows("block.emitted", width, torch.bfloat16)
-        shares = self.ctx.workspace.flat("block.emitted_shares", blocks * 64, torch.float32)
+        # (one size for every producer: the buffer is made once)
+        shares = self.ctx.workspace.flat("block.emitted_shares", max(blocks, most) * 64, torch.float32)[:blocks * 64]
         self.pending = dict(out=out, shares=shares, blocks=blocks, eps=eps)
         return dict(weight=weight, out=out, shares=shares)
 

@@ -32,8 +32,15 @@ class Embedding(Part):
     def bind(self, tensors):
         self.table = tensors[self.name].contiguous()
 
-    def forward(self, ctx, x):
-        ops.embed(x, self.table, ctx.token_ids)
+    # forward takes the normed input of the first block as `then` (a LazyNorm), and may do
+    # the first half of that norm on its way
+    emits_norm = True
+
+    def forward(self, ctx, x, then=None):
+        emit = None
+        if then is not None and ops.can_embed_emit(self.table, ctx.n):
+            emit = then.offer(blocks=ops.embed_emit_blocks(self.hidden))
+        ops.embed(x, self.table, ctx.token_ids, emit=emit)
 
 
 @register_head("norm_linear")

@@ -524,6 +524,34 @@ def test_embed(dtype, d):
     assert torch.equal(out.cpu(), table[ids.long()].float())
 
 
+@pytest.mark.parametrize("d,n,wdtype", [(4096, 8, torch.bfloat16), (2048, 1, torch.float32), (5128, 64, torch.bfloat16),
+                                        (40, 3, torch.float32)])
+def test_embed_with_the_first_half_of_the_norm_that_follows(d, n, wdtype):
+    """The rows as float32, bfloat16(row * weight), and the rows' sums of squares in shares
+    that a product with `row_scale` turns into the norm: the two halves together against the
+    norm in one piece (the shares against a float64 sum)."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(d + n)
+    table = torch.randn(97, d, generator=g).to(torch.bfloat16)
+    weight = (1 + 0.2 * torch.randn(d, generator=g)).to(wdtype)
+    ids = torch.randint(0, 97, (n,), generator=g, dtype=torch.int32)
+    blocks = ops.embed_emit_blocks(d)
+    out = torch.empty(n, d, dtype=torch.float32, device=DEV)
+    emitted = torch.full((n, d), 7.0, dtype=torch.bfloat16, device=DEV)
+    shares = torch.full((blocks * 64,), 7.0, dtype=torch.float32, device=DEV)
+    assert ops.can_embed_emit(table, n) and not ops.can_embed_emit(table, 65) and not ops.can_embed_emit(table.float(), n)
+    ops.embed(out, table.to(DEV), ids.to(DEV), emit=dict(weight=weight.to(DEV), out=emitted, shares=shares))
+    rows = table[ids.long()].float()
+    assert torch.equal(out.cpu(), rows)
+    assert torch.equal(emitted.cpu(), (rows * weight.float()).to(torch.bfloat16))
+    sums = shares.cpu().view(blocks, 64)[:, :n].double().sum(0)
+    assert torch.allclose(sums, rows.double().pow(2).sum(1), rtol=1e-5)
+    with pytest.raises(Exception, match="64 rows"):
+        ops.embed(torch.empty(65, d, dtype=torch.float32, device=DEV), table.to(DEV),
+                  torch.zeros(65, dtype=torch.int32, device=DEV),
+                  emit=dict(weight=weight.to(DEV), out=torch.empty(65, d, dtype=torch.bfloat16, device=DEV), shares=shares))
+
+
 def _paged(kv, page_size, pages_order):
     """kv: [T, K, hd] -> cache layer tensor with the pages in the given order, and the table."""
     T, K, hd = kv[0].shape
