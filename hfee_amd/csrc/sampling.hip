@@ -15,6 +15,10 @@
 // probability mass for top_p.  All sums run in a fixed order (thread-owned contiguous
 // chunks, then a fixed tree), so a row's result is the same in every batch.
 //
+// A row of a large vocabulary goes through sample_slices_kernel first, 32 workgroups a row
+// (penalty, maximum, and each slice's own top_k for a small top_k); sample_kernel then
+// works on what the slices left.  Smaller vocabularies: sample_kernel alone.
+//
 // The random number is counter based: splitmix64 of (seed, draw index), one stream
 // per request, independent of what else is sampled in the same call.
 #include "common.h"
@@ -86,6 +90,38 @@ __device__ __forceinline__ MaxIdx better(MaxIdx a, MaxIdx b) {   // greater valu
   if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
   return a;
 }
+
+// The sum of a wave's 64 values, the same in every lane's return value: four steps inside
+// the rows of 16 lanes and two across them, all in the data path of the vector unit (a
+// shuffle goes through the LDS crossbar and takes ten times as long; the bisection for
+// top_p waits for 32 such sums in turn).  A fixed tree: the same sum for the same values.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_total(float v) {
+  v = dpp_add<0xB1, 0xf>(v);          // quad_perm [1, 0, 3, 2]
+  v = dpp_add<0x4E, 0xf>(v);          // quad_perm [2, 3, 0, 1]
+  v = dpp_add<0x141, 0xf>(v);         // row_half_mirror
+  v = dpp_add<0x140, 0xf>(v);         // row_mirror: every lane has its row's sum
+  v = dpp_add<0x142, 0xa>(v);         // row_bcast 15: rows 1 and 3 add the row before
+  v = dpp_add<0x143, 0xc>(v);         // row_bcast 31: rows 2 and 3 add rows 0 + 1
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_add(int v) {
+  return v + __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ int wave_total(int v) {
+  v = dpp_add<0xB1, 0xf>(v);
+  v = dpp_add<0x4E, 0xf>(v);
+  v = dpp_add<0x141, 0xf>(v);
+  v = dpp_add<0x140, 0xf>(v);
+  v = dpp_add<0x142, 0xa>(v);
+  v = dpp_add<0x143, 0xc>(v);
+  return __builtin_amdgcn_readlane(v, 63);
+}
+
 
 // One pass of the block over lg[0 .. V-1]: see(j, lg[j]) for every j, ascending within a
 // thread.  Rows that are 16-byte aligned are read four logits a load, four loads in flight;
@@ -224,6 +260,18 @@ __device__ __forceinline__ T team_exclusive_scan(T v, T* wave_totals, T* total) 
   }
 }
 
+// The team's sum alone (no prefix).
+template <bool WAVE>
+__device__ __forceinline__ float team_total(float v, float* scratch) {
+  if constexpr (WAVE) {
+    return wave_total(v);
+  } else {
+    float total;
+    block_exclusive_scan<float>(v, scratch, &total);
+    return total;
+  }
+}
+
 template <bool WAVE>
 __device__ __forceinline__ float team_max(float v, float* scratch) {
   if constexpr (WAVE) return wave_max(v);
@@ -258,8 +306,7 @@ __device__ __forceinline__ void draw_from_kept(const SampleParams& p, const MaxI
     my_mass += e;
   }
   if (!WAVE) __threadfence_block();
-  float Z;
-  team_exclusive_scan<float, WAVE>(my_mass, fscratch, &Z);
+  const float Z = team_total<WAVE>(my_mass, fscratch);
 
   // ---- top_p: threshold key and how many of its ties belong (sampler.go:98-108)
   uint32_t t_p = 0u;
@@ -271,9 +318,7 @@ __device__ __forceinline__ void draw_from_kept(const SampleParams& p, const MaxI
       const uint32_t cand = t | (1u << bit);
       float mass = 0.f;
       for (int j = j0; j < j1; ++j) mass += order_key(lgp[j]) >= cand ? qp[j] : 0.f;
-      float total;
-      team_exclusive_scan<float, WAVE>(mass, fscratch, &total);
-      if (total >= target) t = cand;
+      if (team_total<WAVE>(mass, fscratch) >= target) t = cand;
     }
     t_p = t;
     float above = 0.f, tie_p = 0.f;
@@ -282,8 +327,7 @@ __device__ __forceinline__ void draw_from_kept(const SampleParams& p, const MaxI
       if (key > t_p) above += qp[j];
       else if (key == t_p && qp[j] > 0.f) tie_p = qp[j];
     }
-    float mass_above;
-    team_exclusive_scan<float, WAVE>(above, fscratch, &mass_above);
+    const float mass_above = team_total<WAVE>(above, fscratch);
     tie_p = team_max<WAVE>(tie_p, fscratch);
     r_p = tie_p > 0.f ? max(1, (int)ceilf((target - mass_above) / tie_p)) : 1;
   }
@@ -358,6 +402,168 @@ __device__ __forceinline__ void draw_from_kept(const SampleParams& p, const MaxI
   }
 }
 
+// ---- a row spread over workgroups ------------------------------------------------------
+// With a top_k of at most SLICE_K (the default is 40) a row of a large vocabulary is cut into
+// SLICES slices, a workgroup each: the slice comes into LDS once, gets its share of the
+// repeat penalty, and leaves its maximum and its own top_k (value desc, id asc: the order in
+// which the whole row's top_k is taken, so the row's top_k lies within the slices' top_ks)
+// in the row's scratch.  The row's workgroup (sample_kernel) then selects among at most
+// SLICES x top_k candidates instead of reading the vocabulary seven times.  Rows that are
+// greedy, or whose top_k is off or larger, get the penalty and the maxima here and the rest
+// in sample_kernel as before.
+constexpr int SLICES = 32, SLICE_K = 64, SLICE_THREADS = 256, SPAN_MAX = 8192;
+constexpr int SLICE_HEAD = 128;                                   // words: SLICES maxima (value, id), SLICES counts
+constexpr int SLICE_WORDS = SLICE_HEAD + SLICES * 2 * SLICE_K;    // of a row's scratch
+constexpr int SLICED_MIN_V = 8192;
+
+__device__ __forceinline__ MaxIdx* slice_tops(float* q) { return reinterpret_cast<MaxIdx*>(q); }
+__device__ __forceinline__ int* slice_counts(float* q) { return reinterpret_cast<int*>(q) + 2 * SLICES; }
+__device__ __forceinline__ float* slice_vals(float* q, int s) { return q + SLICE_HEAD + s * 2 * SLICE_K; }
+__device__ __forceinline__ int* slice_ids(float* q, int s) {
+  return reinterpret_cast<int*>(q) + SLICE_HEAD + s * 2 * SLICE_K + SLICE_K;
+}
+__device__ __forceinline__ bool sliced_top_k(const SampleParams& p) {
+  return p.temperature > 0.f && p.top_k > 0 && p.top_k <= SLICE_K;
+}
+
+template <int KPT>       // keys a thread: the slice has at most KPT * SLICE_THREADS ids
+__global__ __launch_bounds__(SLICE_THREADS) void sample_slices_kernel(float* __restrict__ logits, int64_t ld, int V,
+                                                                      int span, const SampleParams* __restrict__ params,
+                                                                      const int* __restrict__ history, const int* latest,
+                                                                      float* __restrict__ scratch, int64_t ld_scratch) {
+  constexpr int WAVES_HERE = SLICE_THREADS / 64;
+  __shared__ __align__(16) float vals[SPAN_MAX];
+  __shared__ uint32_t seen[SPAN_MAX / 32];
+  __shared__ MaxIdx mscratch[WAVES_HERE];
+  __shared__ int counts[2][WAVES_HERE];
+  __shared__ int wave_above[WAVES_HERE], wave_ties[WAVES_HERE];
+  const int s = blockIdx.x, row = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const SampleParams p = params[row];
+  float* lg = logits + (int64_t)p.logits_row * ld;
+  float* q = scratch + (int64_t)row * ld_scratch;
+  const int lo = min(V, s * span), n = min(V, lo + span) - lo;
+
+  if ((((uintptr_t)(lg + lo)) & 15) == 0) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const f32x4* src = reinterpret_cast<const f32x4*>(lg + lo);
+    for (int i = tid; i < (n >> 2); i += SLICE_THREADS) *reinterpret_cast<f32x4*>(&vals[4 * i]) = src[i];
+    for (int j = (n & ~3) + tid; j < n; j += SLICE_THREADS) vals[j] = lg[lo + j];
+  } else {
+    for (int j = tid; j < n; j += SLICE_THREADS) vals[j] = lg[lo + j];
+  }
+  for (int w = tid; w < (n + 31) / 32; w += SLICE_THREADS) seen[w] = 0u;
+  __syncthreads();
+
+  // ---- repeat penalty on the ids of this slice (see sample_kernel)
+  if (p.repeat_penalty != 1.0f && (p.history_length > 0 || latest != nullptr)) {
+    const int count = p.history_length + (latest != nullptr ? 1 : 0);
+    for (int i = tid; i < count; i += SLICE_THREADS) {
+      const int id = i < p.history_length ? history[p.history_offset + i] : latest[row];
+      if (id >= lo && id < lo + n) {
+        const int k = id - lo;
+        const uint32_t bit = 1u << (k & 31);
+        if (!(atomicOr(&seen[k >> 5], bit) & bit)) {
+          const float v = vals[k];
+          const float w = v > 0.f ? v / p.repeat_penalty : v * p.repeat_penalty;
+          vals[k] = w;
+          lg[id] = w;
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- the slice's first maximum
+  MaxIdx best{-INFINITY, 0x7fffffff};
+  for (int j = tid; j < n; j += SLICE_THREADS) {
+    const float v = vals[j];
+    if (v > best.v) best = MaxIdx{v, lo + j};
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    MaxIdx o{__shfl_xor(best.v, off, 64), __shfl_xor(best.i, off, 64)};
+    best = better(best, o);
+  }
+  if (lane == 0) mscratch[wave] = best;
+  __syncthreads();
+  if (tid == 0) {
+    MaxIdx r = mscratch[0];
+    for (int w = 1; w < WAVES_HERE; ++w) r = better(r, mscratch[w]);
+    slice_tops(q)[s] = r;
+  }
+  if (!sliced_top_k(p)) return;
+
+  // ---- the key of the slice's kk-th largest logit, bit by bit: the largest t with
+  // at least kk keys >= t
+  const int kk = min(p.top_k, n);
+  if (kk == 0) {
+    if (tid == 0) slice_counts(q)[s] = 0;
+    return;
+  }
+  // (a thread's keys in registers: a count is a few dozen instructions and one barrier, where
+  // a loop over LDS waited for every read in turn: 55 us a slice instead of 10)
+  uint32_t key[KPT];
+#pragma unroll
+  for (int i = 0; i < KPT; ++i) {
+    const int j = tid + i * SLICE_THREADS;
+    key[i] = j < n ? order_key(vals[j]) : 0u;              // (no count asks for keys >= 0)
+  }
+  int turn = 0;
+  auto count_from = [&](uint32_t t) {                      // keys >= t in the slice, t > 0
+    int c = 0;                                             // (by ballots: the wave's count is a scalar; a count
+#pragma unroll                                             //  a lane and one sum over the wave measured 2 us slower)
+    for (int i = 0; i < KPT; ++i) c += __popcll(__ballot(key[i] >= t));
+    if (lane == 0) counts[turn][wave] = c;
+    __syncthreads();                                       // (two sets in turn: one barrier a count)
+    int all = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES_HERE; ++w) all += counts[turn][w];
+    turn ^= 1;
+    return all;
+  };
+  uint32_t t_k = 0u;
+  for (int bit = 31; bit >= 0; --bit) {
+    const uint32_t cand = t_k | (1u << bit);
+    if (count_from(cand) >= kk) t_k = cand;
+  }
+  const int r_k = kk - (t_k == 0xffffffffu ? 0 : count_from(t_k + 1u));      // ties at t_k that belong
+
+  // ---- {key > t_k} and the first r_k ties, ids ascending: wave w takes the w-th quarter
+  // of the slice, 64 consecutive ids at a time; it counts, then places
+  const int wspan = ((n + WAVES_HERE - 1) / WAVES_HERE + 63) / 64 * 64;
+  const int first = min(n, wave * wspan), last = min(n, first + wspan);
+  int above = 0, ties = 0;
+  for (int j = first + lane; j - lane < last; j += 64) {
+    const uint32_t key = j < last ? order_key(vals[j]) : 0u;
+    above += __popcll(__ballot(j < last && key > t_k));
+    ties += __popcll(__ballot(j < last && key == t_k));
+  }
+  if (lane == 0) { wave_above[wave] = above; wave_ties[wave] = ties; }
+  __syncthreads();
+  int above_before = 0, ties_before = 0;
+  for (int w = 0; w < wave; ++w) { above_before += wave_above[w]; ties_before += wave_ties[w]; }
+  int at = above_before + min(ties_before, r_k);
+  int ties_seen = ties_before;
+  const uint64_t below = (1ull << lane) - 1ull;
+  float* out_v = slice_vals(q, s);
+  int* out_i = slice_ids(q, s);
+  for (int j = first + lane; j - lane < last; j += 64) {
+    const float v = j < last ? vals[j] : 0.f;
+    const uint32_t key = order_key(v);
+    const bool tie = j < last && key == t_k;
+    const uint64_t tie_mask = __ballot(tie);
+    const bool in = j < last && (key > t_k || (tie && ties_seen + __popcll(tie_mask & below) < r_k));
+    const uint64_t in_mask = __ballot(in);
+    if (in) {
+      const int slot = at + __popcll(in_mask & below);
+      if (slot < SLICE_K) { out_v[slot] = v; out_i[slot] = lo + j; }
+    }
+    at += __popcll(in_mask);
+    ties_seen += __popcll(tie_mask);
+  }
+  if (tid == 0) slice_counts(q)[s] = kk;
+}
+
 // The largest top_k whose kept set is gathered into LDS (ids ascending): every rule after
 // top_k then runs over at most this many entries instead of the whole vocabulary.
 constexpr int GATHER_MAX = 1024;
@@ -367,7 +573,8 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
                                                          int64_t ld, int V, const SampleParams* __restrict__ params,
                                                          const int* __restrict__ history,
                                                          const int* latest,
-                                                         float* __restrict__ scratch, int64_t ld_scratch) {
+                                                         float* __restrict__ scratch, int64_t ld_scratch,
+                                                         bool sliced) {
   extern __shared__ uint32_t bits[];            // (V + 31) / 32 words, used by the repeat penalty
   __shared__ MaxIdx mscratch[16];
   __shared__ float fscratch[16];
@@ -393,7 +600,9 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
   // step before, which lies on the device and which the host has not seen yet when this
   // sampling is launched.  It may be the very place that `out` names: it is read here,
   // before anything is written there.)
-  if (p.repeat_penalty != 1.0f && (p.history_length > 0 || latest != nullptr)) {
+  // (sliced: sample_slices_kernel has run over this row; the penalty is done, and the
+  // slices' maxima lie at the head of the row's scratch)
+  if (!sliced && p.repeat_penalty != 1.0f && (p.history_length > 0 || latest != nullptr)) {
     const int words = (V + 31) / 32;
     for (int w = tid; w < words; w += THREADS) bits[w] = 0u;
     __syncthreads();
@@ -413,9 +622,115 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
   }
 
   // ---- greedy (sampler.go:76-84)
-  const MaxIdx top = block_argmax(lg, V, mscratch);
+  MaxIdx top;
+  if (sliced) {
+    if (wave == 0) {
+      MaxIdx best = lane < SLICES ? slice_tops(q)[lane] : MaxIdx{-INFINITY, 0x7fffffff};
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        MaxIdx o{__shfl_xor(best.v, off, 64), __shfl_xor(best.i, off, 64)};
+        best = better(best, o);
+      }
+      if (lane == 0) mscratch[0] = best;
+    }
+    __syncthreads();
+    top = mscratch[0];
+    if (top.i == 0x7fffffff) top.i = 0;
+  } else {
+    top = block_argmax(lg, V, mscratch);
+  }
   if (p.temperature <= 0.f) {
     if (tid == 0) out[row] = top.i;
+    return;
+  }
+  __shared__ int sh_choice;
+
+  // ---- a small top_k over a row in slices: the slices' candidates (ids ascending: slice by
+  // slice, and ascending within each) come into LDS in their order; the key of the top_k-th
+  // largest among them bit by bit, then {key > t_k} and the first ties as below
+  if (sliced && sliced_top_k(p)) {
+    __shared__ int cand_before[SLICES + 1];
+    float* cand_val = reinterpret_cast<float*>(hist);              // (the radix counters are not used on this path)
+    constexpr int CAND_WORDS = SLICES * SLICE_K + SLICES * SLICE_K / 32;
+    int* cand_id = hist + CAND_WORDS;
+    static_assert(2 * CAND_WORDS <= HIST_COPIES * HIST_PITCH && SLICES * SLICE_K % 64 == 0 && SLICES * SLICE_K / 64 <= 64 &&
+                  SLICES <= 64 && SLICE_K <= GATHER_MAX, "the candidates of a row: within the counters' LDS, 32 a lane");
+    if (wave == 0) {
+      const int c = lane < SLICES ? slice_counts(q)[lane] : 0;
+      int incl = c;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += up;
+      }
+      if (lane < SLICES) cand_before[lane] = incl - c;
+      if (lane == SLICES - 1) cand_before[SLICES] = incl;
+    }
+    __syncthreads();
+    for (int e = tid; e < SLICES * SLICE_K; e += THREADS) {
+      const int sl = e / SLICE_K, k = e % SLICE_K;
+      if (k < cand_before[sl + 1] - cand_before[sl]) {
+        const int at = cand_before[sl] + k;
+        cand_val[at + at / 32] = slice_vals(q, sl)[k];             // (a word of padding every 32: lane l reads 33 l + i)
+        cand_id[at + at / 32] = slice_ids(q, sl)[k];
+      }
+    }
+    __syncthreads();
+    // wave 0 alone from here: lane l holds candidates 32 l .. 32 l + 31 as keys in registers,
+    // counts meet by shuffles, no barrier
+    if (wave != 0) return;
+    constexpr int PER = SLICES * SLICE_K / 64;
+    const int N = cand_before[SLICES], kk = min(p.top_k, N);
+    uint32_t key[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = lane * PER + i;
+      key[i] = e < N ? order_key(cand_val[e + e / 32]) : 0u;       // (no count asks for keys >= 0)
+    }
+    auto wave_before = [&](int c) {                  // of the lanes before this one
+      int incl = c;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += up;
+      }
+      return incl - c;
+    };
+    uint32_t t = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t cand = t | (1u << bit);
+      int c[4] = {0, 0, 0, 0};                       // (a lane's own count in four chains, then one sum over the
+#pragma unroll                                       //  wave: 1,024 ballots in a row took 17 us)
+      for (int i = 0; i < PER; ++i) c[i & 3] += key[i] >= cand;
+      if (wave_total((c[0] + c[1]) + (c[2] + c[3])) >= kk) t = cand;
+    }
+    int above = 0, ties = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      above += key[i] > t;
+      ties += lane * PER + i < N && key[i] == t;
+    }
+    const int r = kk - wave_total(above);
+    int tie_rank = wave_before(ties);
+    uint64_t in = 0ull;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const bool have = lane * PER + i < N;
+      bool take = have && key[i] > t;
+      if (have && key[i] == t) take = tie_rank++ < r;
+      in |= (uint64_t)take << i;
+    }
+    int slot = wave_before(__popcll(in));
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if ((in >> i) & 1ull) {
+        const int e = lane * PER + i;
+        kept_logit[slot] = cand_val[e + e / 32];
+        kept_id[slot] = cand_id[e + e / 32];
+        ++slot;
+      }
+    draw_from_kept<true>(p, top, kk, kept_logit, kept_q, kept_id, 0u, 0x7fffffff, out + row, fscratch, iscratch,
+                         &sh_choice);
     return;
   }
 
@@ -524,7 +839,6 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(int* __restrict__ out, 
     t_k = 0u;                                   // top_k is done: every gathered entry belongs
     r_k = 0x7fffffff;
   }
-  __shared__ int sh_choice;
   if (gathered) {
     if (wave == 0)
       draw_from_kept<true>(p, top, Vn, lgp, qp, kept_id, t_k, r_k, out + row, fscratch, iscratch, &sh_choice);
@@ -618,7 +932,22 @@ HFEE_API int hfee_sample(int* out, float* logits, int64_t ld, int rows, int V, c
                          hipStream_t stream) {
   HFEE_REQUIRE(rows >= 0 && V > 0 && ld >= V && ld_scratch >= V, "sample: bad sizes rows=%d V=%d", rows, V);
   if (rows == 0) return 0;
-  const size_t lds = (size_t)((V + 31) / 32) * 4;
+  // a large vocabulary goes through the slices first (the penalty's bit set is then theirs)
+  const bool sliced = V >= SLICED_MIN_V && V <= SLICES * SPAN_MAX && ld_scratch >= SLICE_WORDS && rows <= 65535;
+  if (sliced) {
+    const int span = ((V + SLICES - 1) / SLICES + 3) & ~3;
+    const dim3 grid(SLICES, rows);
+    const SampleParams* sp = (const SampleParams*)params;
+    if (span <= 8 * SLICE_THREADS)
+      sample_slices_kernel<8><<<grid, SLICE_THREADS, 0, stream>>>(logits, ld, V, span, sp, history, latest, scratch, ld_scratch);
+    else if (span <= 16 * SLICE_THREADS)
+      sample_slices_kernel<16><<<grid, SLICE_THREADS, 0, stream>>>(logits, ld, V, span, sp, history, latest, scratch, ld_scratch);
+    else
+      sample_slices_kernel<SPAN_MAX / SLICE_THREADS><<<grid, SLICE_THREADS, 0, stream>>>(logits, ld, V, span, sp, history, latest,
+                                                                                       scratch, ld_scratch);
+    HFEE_CHECK_LAUNCH("sample slices");
+  }
+  const size_t lds = sliced ? 0 : (size_t)((V + 31) / 32) * 4;
   HFEE_REQUIRE(lds <= 96 * 1024, "sample: a vocabulary of %d ids does not fit the penalty's bit set", V);
   static bool raised = false;
   if (lds > 32 * 1024 && !raised) {
@@ -628,7 +957,7 @@ HFEE_API int hfee_sample(int* out, float* logits, int64_t ld, int rows, int V, c
     raised = true;
   }
   sample_kernel<<<rows, THREADS, lds, stream>>>(out, logits, ld, V, (const SampleParams*)params, history, latest,
-                                                scratch, ld_scratch);
+                                                scratch, ld_scratch, sliced);
   HFEE_CHECK_LAUNCH("sample");
   return 0;
 }

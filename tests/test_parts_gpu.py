@@ -424,7 +424,7 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path):
 
 # -------------------------------------------------------------- the sampler ---
 
-@pytest.mark.parametrize("V", [1000, 1001])
+@pytest.mark.parametrize("V", [1000, 1001, 8201])      # (from 8,192 ids on a row is cut into slices first)
 def test_sampler_kernel_follows_the_plain_rules(V):
     from plain_llama import plain_repeat_penalty, plain_sampling_distribution
     from hfee_amd.sampling import SampleRow, Sampler, SamplingParams, uniform
@@ -457,8 +457,9 @@ def test_sampler_kernel_follows_the_plain_rules(V):
                 exact += int(i == int((cum >= uniform(99, c * 64 + r)).nonzero()[0]))
         assert set(counts.nonzero().flatten().tolist()) <= support, f"{p}: sampled outside the kept set"
         assert exact >= 0.99 * draws, f"{p}: only {exact} of {draws} draws match the inverse CDF"
-        tv = 0.5 * float((counts / draws - dist.float()).abs().sum())
-        assert tv < 0.12, f"{p}: total variation {tv}"
+        if V <= 1001:      # (over thousands of ids 1,920 draws say too little about the shape; the check above is the exact one)
+            tv = 0.5 * float((counts / draws - dist.float()).abs().sum())
+            assert tv < 0.12, f"{p}: total variation {tv}"
     # greedy with and without penalty; one stream per request, whatever shares the call
     greedy = SamplingParams(temperature=0.0, repeat_penalty=1.0)
     logits = base.repeat(3, 1).to(DEV)
@@ -472,14 +473,14 @@ def test_sampler_kernel_follows_the_plain_rules(V):
     assert mixed[2] == alone[0] and mixed[1] == 17
 
 
-@pytest.mark.parametrize("top_k", [40, 700, 1500])
-def test_sampler_takes_the_first_ties_at_the_top_k_threshold(top_k):
+@pytest.mark.parametrize("top_k,V", [(40, 9001), (700, 9001), (1500, 9001), (40, 7001), (64, 9004), (65, 9004), (12, 200000)])
+def test_sampler_takes_the_first_ties_at_the_top_k_threshold(top_k, V):
     """Thousands of equal logits at the top_k threshold, spread over the whole vocabulary (so
-    over all the waves that gather the kept set): the ones with the smallest ids belong, as
+    over all the waves that gather the kept set, and over all the slices of a large
+    vocabulary with a small top_k): the ones with the smallest ids belong, as
     many as top_k leaves room for after the larger logits (sampler.go:132-151)."""
     from plain_llama import plain_sampling_distribution
     from hfee_amd.sampling import SampleRow, Sampler, SamplingParams
-    V = 9001
     g = torch.Generator().manual_seed(top_k)
     base = torch.full((V,), -2.0)
     tied = torch.randperm(V, generator=g)[:4000]
@@ -551,7 +552,7 @@ def test_sampler_at_the_vocabulary_of_the_real_models(top_k):
     assert exact >= 0.99 * draws, f"top_k {top_k}: only {exact} of {draws} draws match the inverse CDF ({kept} ids kept)"
 
 
-@pytest.mark.parametrize("V", [700, 1003, 4099])
+@pytest.mark.parametrize("V", [700, 1003, 4099, 8209, 8212])
 def test_sampler_takes_the_newest_id_of_a_history_from_the_device(V):
     """The newest id of each row's history may lie on the device only (`latest`: the ids of
     the sampling before, not yet collected), even in the tensor that takes this sampling's
