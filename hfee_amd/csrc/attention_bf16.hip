@@ -528,6 +528,19 @@ __device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds,
   }
 }
 
+// The same as a static member of a class template: nothing is deduced at the call.  (The host
+// pass of the compiler takes the call of the function template in the first specialization of
+// the kernel below that makes it and reports no match in the second.)
+template <int WAVES, bool BUFFER>
+struct RequestBlocks {
+  static __device__ __forceinline__ void go(char* __restrict__ tile_lds, const bf16_t* __restrict__ cache,
+                                            __amdgpu_buffer_rsrc_t rsrc, const CacheLayout& lay, const WaveBlocks<WAVES>& w,
+                                            const int* __restrict__ bt, int bt_stride, PageWindow& pages, int k0, int kv_first,
+                                            int kv_last, int wave) {
+    request_wave_blocks<WAVES, BUFFER>(tile_lds, cache, rsrc, lay, w, bt, bt_stride, pages, k0, kv_first, kv_last, wave);
+  }
+};
+
 // work: per row tile 4 ints (first row, rows <= 32, first position, block-table row).
 // WAVES: the waves of a workgroup if they are SHARED_WAVES, 0 for any other number.
 // RING: key tiles come through buffer loads (layer_bytes < 4 GB) into a ring of SHARED_TILES
@@ -538,7 +551,12 @@ __device__ __forceinline__ void request_wave_blocks(char* __restrict__ tile_lds,
 // a step.  History of this kernel at the 8B shape, 2,048 tokens, us a layer: 85 with one tile
 // ahead behind a fence; 81.5 with the ring; 71.5 within 256 registers; 67.6 with a tile's
 // sixteen operand reads in front of its products; 65.0 with four tiles.)
-template <int WAVES, bool RING>
+// IDLERS: some waves of a workgroup may have nothing to multiply at a key tile (a wave without a
+// head, or a row tile of earlier rows) and skip it.  Where the heads of a KV head fill the waves
+// the kernel holds no trace of that: the check in every step's chain, and what the compiler made
+// of the loop around it, cost 16 to 20 % at four heads to a KV head (69 -> 81 us a layer at
+// 2,048 tokens, 275 -> 330 at 8,192, 1,093 -> 1,267 at 32,768).
+template <int WAVES, bool RING, bool IDLERS = true>
 __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, uint32_t layer_bytes, CacheLayout lay, const int* __restrict__ work, int num_tiles,
@@ -601,9 +619,11 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
   // (a raw buffer of 32-bit data over the layer; only the ring's loads go through it)
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cache, 0, (int)layer_bytes, 0x00020000);
   auto compute = [&](int t, const char* tile_at, auto under_scores) {
-    if (!head_ok || t * 32 > my_last) {      // (a wave without work, or of earlier rows: nothing here is visible to it)
-      under_scores();
-      return;
+    if constexpr (IDLERS) {
+      if (!head_ok || t * 32 > my_last) {    // (a wave without work, or of earlier rows: nothing here is visible to it)
+        under_scores();
+        return;
+      }
     }
     const char* cur = tile_at + lane * 16;
     compute_tile_with(
@@ -620,7 +640,7 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
     static_assert(WAVES != 0 && KV_BLOCKS % (WAVES == 0 ? 1 : WAVES) == 0, "a wave's loads of a tile must be a fixed number");
     constexpr int W = WAVES == 0 ? 1 : WAVES, MINE = KV_BLOCKS / W;     // loads a wave issues for a tile
     auto request = [&](int t) {
-      request_wave_blocks<W, true>(kv_lds + ((t - t_first) % SHARED_TILES) * TILE_BYTES, cache, rsrc, lay, mine, bt, bt_stride,
+      RequestBlocks<W, true>::go(kv_lds + ((t - t_first) % SHARED_TILES) * TILE_BYTES, cache, rsrc, lay, mine, bt, bt_stride,
                                    pages, t * 32, kv_first, kv_last, wave);
     };
     // Nothing is on its way when the loop begins but what the loop itself asks for: the compiler
@@ -955,17 +975,23 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
       if (e == hipSuccess && KV_BLOCKS % SHARED_WAVES == 0)
         e = hipFuncSetAttribute((const void*)prefill_shared_kernel<SHARED_WAVES, KV_BLOCKS % SHARED_WAVES == 0>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, most);
+      if (e == hipSuccess && KV_BLOCKS % SHARED_WAVES == 0)
+        e = hipFuncSetAttribute((const void*)prefill_shared_kernel<SHARED_WAVES, KV_BLOCKS % SHARED_WAVES == 0, false>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, most);
       HFEE_REQUIRE(e == hipSuccess, "attention_bf16_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
       raised = true;
     }
     dim3 grid((unsigned)(((int64_t)(by_rows ? num_runs : num_tiles * chunks) * kv_heads + 7) / 8 * 8));
     const int* runs_or_none = by_rows ? runs : nullptr;
-#define GO(W, R)                                                                                                    \
-  prefill_shared_kernel<W, R><<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,         \
+    // (every wave has a head at every key tile: the heads of a KV head are whole rounds of the waves)
+    const bool all_busy = !by_rows && group % waves == 0;
+#define GO(W, R, ...)                                                                                               \
+  prefill_shared_kernel<W, R, ##__VA_ARGS__><<<grid, waves * 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, \
                                                                 (const bf16_t*)cache, (uint32_t)(ring ? layer_bytes : 0),  \
                                                                 lay, work, num_tiles, runs_or_none, num_runs, block_tables, \
                                                                 bt_stride, num_heads, scale * LOG2E, window)
-    if (ring) GO(SHARED_WAVES, (KV_BLOCKS % SHARED_WAVES == 0));
+    if (ring && all_busy) GO(SHARED_WAVES, (KV_BLOCKS % SHARED_WAVES == 0), false);
+    else if (ring) GO(SHARED_WAVES, (KV_BLOCKS % SHARED_WAVES == 0));
     else if (waves == SHARED_WAVES) GO(SHARED_WAVES, false);
     else GO(0, false);
 #undef GO
