@@ -79,6 +79,9 @@ def parse(argv=None):
     ap.add_argument("--yardsticks", action="store_true",
                     help="only measure what the simplest kernels get from this GPU: a read-only stream over 4 GiB "
                          "and a loop of nothing but bfloat16 matrix instructions; prints its own line")
+    ap.add_argument("--attention-alone", action="store_true",
+                    help="only time the prefill attention kernel by itself: the last 2,048 rows of one sequence of "
+                         "2,048, 8,192 and 32,768 tokens (heads and head size of --shape); prints its own line")
     ap.add_argument("--no-extra-points", action="store_true",
                     help="skip the other shapes and the longer context that the default run adds under `points`")
     return ap.parse_args(argv)
@@ -113,6 +116,43 @@ def yardsticks():
     return (4 << 30) / read_s / 1e9, flops / mfma_s / 1e12
 
 
+def attention_alone(shape: dict) -> dict:
+    """The prefill attention kernel by itself, as a yardstick for changes to it: one sequence of T
+    tokens in the cache, its last 2,048 rows attending: {T: (microseconds, TFLOP/s)}."""
+    import torch
+    from hfee_amd.kernels import ops
+    dev, page_size, rows = "cuda:0", 16, 2048
+    heads, kv_heads = shape["num_attention_heads"], shape["num_key_value_heads"]
+    head_dim = shape.get("head_dim") or shape["hidden_size"] // heads
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    out = {}
+    for tokens in (2048, 8192, 32768):
+        pages = (tokens + page_size - 1) // page_size
+        cache = (torch.randn(pages, 2, kv_heads, page_size * head_dim, device=dev) * 0.5).to(torch.bfloat16)
+        q = (torch.randn(rows, heads * head_dim, device=dev) * 0.5).to(torch.bfloat16)
+        o = torch.zeros_like(q)
+        tables = torch.arange(pages, dtype=torch.int32, device=dev).view(1, -1)
+        tiles = torch.tensor([(r, 32, tokens - rows + r, 0) for r in range(0, rows, 32)], dtype=torch.int32, device=dev)
+        runs = None
+        if heads == kv_heads:      # heads that share no keys: row tiles that follow one another share them, four at a time
+            runs = torch.tensor([(i, min(4, rows // 32 - i)) for i in range(0, rows // 32, 4)], dtype=torch.int32, device=dev)
+        call = lambda: ops.attention_bf16_prefill(o, q, cache, tiles, tables, heads, kv_heads, head_dim, page_size,
+                                                  head_dim ** -0.5, runs=runs)
+        call()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(20):
+            start.record()
+            call()
+            stop.record()
+            torch.cuda.synchronize()
+            best = min(best, start.elapsed_time(stop) * 1e3)
+        visible = sum(tokens - rows + r + 1 for r in range(rows))          # keys that the rows see, causal
+        out[tokens] = (round(best, 1), round(4.0 * visible * head_dim * heads / best / 1e6, 1))
+        del cache
+    return out
+
+
 def main(argv=None) -> int:
     args = parse(argv)
     if args.gpus != 1:
@@ -124,6 +164,13 @@ def main(argv=None) -> int:
         print(json.dumps({"read_stream_gb_per_s": round(gbs, 1), "hbm_published_gb_per_s": HBM_PEAK / 1e9,
                           "mfma_loop_tflop_per_s": round(tflops, 1), "bf16_published_tflop_per_s": BF16_PEAK / 1e12}),
               flush=True)
+        return 0
+    if args.attention_alone:
+        import hfee_amd  # noqa: F401
+        timed = attention_alone(SHAPES[args.shape])
+        print(json.dumps({"kernel": "prefill attention alone, the last 2,048 rows of a sequence", "shape": args.shape,
+                          "microseconds": {str(t): v[0] for t, v in timed.items()},
+                          "tflop_per_s": {str(t): v[1] for t, v in timed.items()}}), flush=True)
         return 0
     line = run(args)
     if isinstance(line, int):
