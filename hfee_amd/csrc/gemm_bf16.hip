@@ -697,6 +697,23 @@ inline int pipelined_splits(int M, int N, int K) {
   return (K + k_split - 1) / k_split;
 }
 
+template <int MODE, int TM, int TN, int NBUF>
+int launch_direct64(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
+                    int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, int k_split = 0, int splits = 1,
+                    int64_t split_stride = 0);
+inline bool large_fits(int64_t lda, int64_t ldw, int M, int N, int K);
+
+// Whether the cuts of a product are better made by the kernel of 256 x 128 tiles: its loop runs
+// at 1.2 PFLOP/s where the 128 x 128 kernel's, two workgroups a CU, reaches 0.7 (the down
+// product of the 1B shape at 2,048 rows, N 2,048, K 8,192 in two cuts: 95 us against 70).  Its
+// tiles are half as many: with the cuts they must still fill most of the chip, and the rows
+// must be whole tiles of 256, or nearly.
+inline bool cuts_by_large_tiles(int M, int N, int K, int splits, int k_split) {
+  const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 255) / 256);
+  return (int64_t)((M + 255) / 256) * 256 * 10 <= (int64_t)((M + 127) / 128) * 128 * 11 && tiles * splits >= 192 &&
+         tiles * splits <= 256 && k_split >= 1024 && k_split % 64 == 0 && K % 64 == 0;
+}
+
 template <int MODE>
 int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
                      int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, const RowScale& rs = RowScale{},
@@ -719,9 +736,15 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
         partial.floats >= (int64_t)splits * M * N) {
       if (raise_pipelined_lds<OUT_F32>(lds)) return 1;
       const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
-      grid.y = splits;
-      gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
-          partial.at, N, A, lda, W, ldw, M, N, K, qkv, rs, k_split, (int64_t)M * N);
+      if (cuts_by_large_tiles(M, N, K, splits, k_split) && large_fits(lda, ldw, M, N, K)) {
+        if (launch_direct64<OUT_F32, 4, 2, 3>(partial.at, N, A, lda, W, ldw, M, N, K, qkv, stream, k_split, splits,
+                                              (int64_t)M * N))
+          return 1;
+      } else {
+        grid.y = splits;
+        gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
+            partial.at, N, A, lda, W, ldw, M, N, K, qkv, rs, k_split, (int64_t)M * N);
+      }
       if constexpr (MODE == OUT_ADD_F32) {
         if (norm.normed != nullptr && launch_finish_norm((float*)C, ldc, partial.at, splits, M, N, norm, stream)) {
           *normed = true;
@@ -958,14 +981,25 @@ constexpr int EROW = 128;                    // bytes of a tile row in a buffer
 // depends on the low five bits of the row only: a lane's operand rows are 32 apart
 __device__ __forceinline__ uint32_t swizzle8(uint32_t row) { return (row ^ ((row >> 3) & 3u)) & 7u; }
 
-template <int MODE, int TM, int TN, int NBUF>
+// (CUT is a compile-time choice: the kernel of whole products holds no trace of it)
+template <int MODE, int TM, int TN, int NBUF, bool CUT = false>
 __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restrict__ C, int64_t ldc,
                                                                  const bf16_t* __restrict__ A, int64_t lda,
                                                                  const bf16_t* __restrict__ W, int64_t ldw,
-                                                                 int M, int N, int K, QkvArgs qkv) {
+                                                                 int M, int N, int K, QkvArgs qkv, int k_split,
+                                                                 int64_t split_stride) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int BM = 64 * TM, BN = 64 * TN, CA = BM / 32, CW = BN / 32;
   constexpr int BUF = (BM + BN) * EROW;
+  if constexpr (CUT) {
+    // K cut over workgroups: blockIdx.y takes columns blockIdx.y * k_split .. of A and W (a multiple
+    // of 64) and leaves its partial product, float32, split_stride words after the one before
+    const int k_first = (int)blockIdx.y * k_split;
+    A += k_first;
+    W += k_first;
+    K = min(K - k_first, k_split);
+    C = (void*)((float*)C + (int64_t)blockIdx.y * split_stride);
+  }
   extern __shared__ __attribute__((aligned(1024))) char lds_bytes[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1103,20 +1137,31 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
 #endif
 }
 
+// (k_split > 0: K in `splits` cuts of k_split columns, MODE a float32 store, the partial products
+// split_stride words apart from C on)
 template <int MODE, int TM, int TN, int NBUF>
 int launch_direct64(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                    int M, int N, int K, const QkvArgs& qkv, hipStream_t stream) {
+                    int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, int k_split, int splits,
+                    int64_t split_stride) {
   const size_t lds = (size_t)NBUF * (64 * TM + 64 * TN) * EROW;
   static bool raised = false;
   if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF, false>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF, true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return fail("gemm_bf16: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = true;
   }
   const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
-  dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS));
-  gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv);
+  dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS), k_split > 0 ? splits : 1);
+  if (k_split > 0)
+    gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF, true><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv,
+                                                                                   k_split, split_stride);
+  else
+    gemm_bf16_direct64_kernel<MODE, TM, TN, NBUF, false><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv,
+                                                                                    0, 0);
   return 0;
 }
 

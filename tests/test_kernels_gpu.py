@@ -110,13 +110,14 @@ def test_gemm_bf16(M, N, K, kernel, mode):
 
 
 @pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 640, 2112),
-                                   (100, 2048, 2048)])
+                                   (100, 2048, 2048), (512, 4096, 8192), (1000, 2048, 8256), (2048, 2048, 8192)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "add"])
 def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
     """Products with too few 128 x 128 tiles for the chip: given scratch, K is cut over up to
     eight times as many workgroups and a second kernel adds the partial products (K that is
-    no multiple of the cut, M and N that are no multiples of a tile); the same numbers as
-    without scratch up to the order of the sums."""
+    no multiple of the cut, M and N that are no multiples of a tile; the last three sizes: the
+    cuts made by the kernel of 256 x 128 tiles, whole tiles of rows and not, a last cut that is
+    shorter); the same numbers as without scratch up to the order of the sums."""
     from hfee_amd.kernels import ops
     g = torch.Generator().manual_seed(M + 3 * N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -149,7 +150,7 @@ def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
 
 @pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 4096, 2112),
                                    (100, 2052, 2048), (100, 512, 1024), (70, 1001, 2048), (2048, 512, 1024), (40, 512, 2048),
-                                   (90, 260, 2050)])
+                                   (90, 260, 2050), (512, 4096, 8192), (1000, 2048, 8256)])
 @pytest.mark.parametrize("weight_dtype", [torch.float32, torch.bfloat16])
 def test_product_that_adds_into_the_stream_and_goes_on_with_the_norm(M, N, K, weight_dtype):
     """The product that adds into the residual stream together with the norm of the new rows:
