@@ -348,6 +348,19 @@ struct QkvCuts {
 // With `cuts`, the partial products are added up here, in their order, and rounded to
 // bfloat16 as the kernel that would have added them does: q is only written, k and v only
 // say that the cache is written.
+// Into how many workgroups the KV heads of 16 tokens' values are dealt (0: a head alone does not
+// fit), and the LDS of each: at most 48 KB, 32 bytes a column.
+struct GroupShares {
+  int parts;
+  size_t bytes;
+};
+inline GroupShares group_shares(int kv_heads, int head_dim) {
+  const int most = (int)(48 * 1024 / ((size_t)32 * head_dim));       // heads a workgroup
+  if (most < 1) return GroupShares{0, 0};
+  const int parts = (kv_heads + most - 1) / most, heads_a_part = (kv_heads + parts - 1) / parts;
+  return GroupShares{parts, (size_t)32 * heads_a_part * head_dim};
+}
+
 // (CUTS is a compile-time choice: as a check at run time in front of every load it cost the
 // plain kernel 3.6 us of 14 at 2,048 tokens)
 template <bool CUTS>
@@ -399,19 +412,23 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
   // writes two bytes here and two bytes there; 16 tokens that fill 16 slots in a row of one
   // page (a prompt's portion that starts on a page's edge) write 32 bytes a column at once.
   // (the groups' workgroups, which run longer than a token's, come first: none is left over at the end)
-  const int groups = values_by_groups ? (n + 15) / 16 : 0;
+  // (values_by_groups: into how many workgroups the KV heads of such a group are dealt, so that a
+  // workgroup's share of the 16 tokens' values fits its LDS: 40 heads of 128 are four of ten)
+  const int groups = values_by_groups ? ((n + 15) / 16) * values_by_groups : 0;
   if ((int)blockIdx.x < groups) {
-    extern __shared__ __attribute__((aligned(16))) bf16_t group_values[];      // [16][kv_heads * head_dim]
+    extern __shared__ __attribute__((aligned(16))) bf16_t group_values[];      // [16][heads of this workgroup * head_dim]
     __shared__ int g_pos[16], g_page[16];
-    const int t0 = 16 * (int)blockIdx.x, count = min(16, n - t0);
-    const int width = lay.kv_heads * lay.head_dim, chunks = width / 8;
+    const int part = (int)blockIdx.x % values_by_groups, heads_a_part = (lay.kv_heads + values_by_groups - 1) / values_by_groups;
+    const int h_first = part * heads_a_part, c_first = h_first * lay.head_dim;
+    const int t0 = 16 * ((int)blockIdx.x / values_by_groups), count = min(16, n - t0);
+    const int width = max(0, min(lay.kv_heads - h_first, heads_a_part)) * lay.head_dim, chunks = width / 8;
     const int pieces = count * chunks;
     for (int first = threadIdx.x; first < pieces; first += 8 * blockDim.x) {      // eight loads in flight
       u32x4 piece[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int idx = min(first + u * (int)blockDim.x, pieces - 1), j = idx / chunks, c = idx - j * chunks;
-        piece[u] = eight(v + (int64_t)(t0 + j) * ldv + 8 * c, t0 + j, cuts.v_col + 8 * c).u;
+        piece[u] = eight(v + (int64_t)(t0 + j) * ldv + c_first + 8 * c, t0 + j, cuts.v_col + c_first + 8 * c).u;
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -428,7 +445,7 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
     bool in_a_row = count == 16 && (g_pos[0] & 15) == 0;
     for (int j = 1; j < count; ++j) in_a_row = in_a_row && g_pos[j] == g_pos[0] + j && g_page[j] == g_page[0];
     for (int col = threadIdx.x; col < width; col += blockDim.x) {
-      const int h = col / lay.head_dim, d = col - h * lay.head_dim;
+      const int h = h_first + col / lay.head_dim, d = col % lay.head_dim;
       if (in_a_row) {
         union { u32x4 u[2]; bf16_t e[16]; } row;
 #pragma unroll
@@ -526,13 +543,13 @@ HFEE_API int hfee_rope_cache_write(void* q, int64_t ldq, const void* k, int64_t 
            (uintptr_t)cos_table % 16 == 0 && (uintptr_t)sin_table % 16 == 0 && (uintptr_t)cache % 16 == 0)
   {
     // (the values of 16 tokens through LDS, if a workgroup's share of it fits and there is more than one group)
-    const size_t group_bytes = (size_t)32 * kv_heads * head_dim;
+    const GroupShares shares = group_shares(kv_heads, head_dim);
     // (`portions`: the tokens hold runs of consecutive positions of a sequence.  Without them, single
     // tokens of many sequences, a group's workgroup would write 16 tokens' values two bytes at a time
     // on its own, eight workgroups for 128 tokens where every token's own workgroup can do it: 13 us
     // against 5 at 128 rows)
-    const int by_groups = portions != 0 && k != nullptr && cache != nullptr && n >= 32 && group_bytes <= 48 * 1024;
-    rope_cache_pairs_kernel<false><<<n + (by_groups ? (n + 15) / 16 : 0), 256, by_groups ? group_bytes : 0, stream>>>(
+    const int by_groups = portions != 0 && k != nullptr && cache != nullptr && n >= 32 ? shares.parts : 0;
+    rope_cache_pairs_kernel<false><<<n + by_groups * ((n + 15) / 16), 256, by_groups ? shares.bytes : 0, stream>>>(
         (bf16_t*)q, ldq, (const bf16_t*)k, ldk, (const bf16_t*)v, ldv, QkvCuts{nullptr, 0, 0, 0, 0, 0}, positions,
         token_segment, block_tables, bt_stride, cos_table, sin_table, half, (bf16_t*)cache, lay, num_heads, n, by_groups);
   }
@@ -578,14 +595,14 @@ HFEE_API int hfee_rope_cache_write_cuts(void* q, int64_t ldq, const float* parti
                    (uintptr_t)sin_table % 16 == 0 && (uintptr_t)cache % 16 == 0,
                "rope_cache_write_cuts: head_dim and the rotary width must be multiples of 8 and the operands 16-byte aligned");
   const QkvCuts c{partial, cuts, (int64_t)n * width, width, num_heads * head_dim, (num_heads + kv_heads) * head_dim};
-  const size_t group_bytes = (size_t)32 * kv_heads * head_dim;
-  const int by_groups = portions != 0 && n >= 32 && group_bytes <= 48 * 1024;
+  const GroupShares shares = group_shares(kv_heads, head_dim);
+  const int by_groups = portions != 0 && n >= 32 ? shares.parts : 0;
   // (k and v: any pointers that are not null; with cuts they are never read.  More threads than
   // the plain kernel has, a piece each where that is at most 768: a thread's eight elements
   // are up to sixteen loads, and few tokens leave CUs without a workgroup)
   const int pieces = (num_heads + kv_heads) * (head_dim / 8);
   const int threads = pieces >= 768 ? 768 : pieces > 512 ? (pieces + 63) / 64 * 64 : 512;
-  rope_cache_pairs_kernel<true><<<n + (by_groups ? (n + 15) / 16 : 0), threads, by_groups ? group_bytes : 0, stream>>>(
+  rope_cache_pairs_kernel<true><<<n + by_groups * ((n + 15) / 16), threads, by_groups ? shares.bytes : 0, stream>>>(
       (bf16_t*)q, ldq, (const bf16_t*)q, 0, (const bf16_t*)q, 0, c, positions, token_segment, block_tables, bt_stride,
       cos_table, sin_table, half, (bf16_t*)cache, lay, num_heads, n, by_groups);
   HFEE_CHECK_LAUNCH("rope_cache_write_cuts");

@@ -774,17 +774,18 @@ def test_rotation_that_adds_up_a_cut_product(H, K, hd, rotary, d, n, portions):
     assert got_cache.abs().sum() > 0
 
 
-@pytest.mark.parametrize("ps", [16, 32])
-def test_rope_cache_write_of_long_portions(ps):
+@pytest.mark.parametrize("ps,H,K,hd", [(16, 3, 2, 32), (32, 3, 2, 32), (16, 13, 13, 128), (16, 5, 5, 256), (32, 20, 20, 80)])
+def test_rope_cache_write_of_long_portions(ps, H, K, hd):
     """From 32 tokens on the values of 16 consecutive tokens are written together: whole
     32-byte runs of the transposed value layout where the 16 tokens fill 16 slots in a row of
     one page, element by element where they do not (a portion that starts inside a page, a
     group that spans two requests, the last, partial group).  Two requests with their own
-    block tables; every key and value is found where the layout says."""
+    block tables; every key and value is found where the layout says.  With many KV heads
+    (13 of 128, 5 of 256, 20 of 80) a group's heads are dealt over two or three workgroups,
+    the last of them with fewer heads."""
     from hfee_amd.kernels import ops
     from hfee_amd.parts.rotary import Rotary
     from hfee_amd.config.specs import PositionSpec, params
-    H, K, hd = 3, 2, 32
     rot = Rotary(PositionSpec("rope", params(head_dim=hd, rotary_dim=hd, theta=10000.0, scaling=None, pairing="interleaved")))
     rot.prepare(256, DEV)
     # request 0: positions 32 .. 84 (starts on a page's edge); request 1: positions 5 .. 58 (does not)
