@@ -151,6 +151,56 @@ class PlainLlama:
             for name in f.keys():
                 self.w[name] = f.get_tensor(name).to(F64)
 
+    def embed(self, tokens) -> torch.Tensor:
+        """/root/reference/internal/llm/forward.go:75-77: the token's row of the table,
+        as it is stored (no scaling by sqrt(width) or anything else)."""
+        return self.w["model.embed_tokens.weight"][torch.as_tensor(tokens, dtype=torch.long)]
+
+    def attention_sublayer(self, x, l, pos, kv=None, window=0):
+        """/root/reference/internal/llm/forward.go:82-107: what the attention half of
+        layer l adds to the stream x [T, d] at positions pos: norm first, then q/k/v,
+        rotation of q and k, attention, output projection.  Returns (delta, (k, v));
+        with kv given, those keys and values are read instead of made."""
+        w, T = self.w, x.shape[0]
+        p = f"model.layers.{l}."
+        xb = plain_rmsnorm(x, w[p + "input_layernorm.weight"], self.eps)               # forward.go:82
+        q = plain_matmul(xb, w[p + "self_attn.q_proj.weight"]).reshape(T, self.H, self.hd)
+        q = plain_rope(q, pos, self.inv_freq)                                          # forward.go:96-97
+        if kv is None:
+            k = plain_matmul(xb, w[p + "self_attn.k_proj.weight"]).reshape(T, self.K, self.hd)
+            v = plain_matmul(xb, w[p + "self_attn.v_proj.weight"]).reshape(T, self.K, self.hd)
+            kv = (plain_rope(k, pos, self.inv_freq), v)                                # forward.go:99-101
+        att = plain_attention(q, kv[0], kv[1], window=window).reshape(T, self.H * self.hd)          # forward.go:104
+        return plain_matmul(att, w[p + "self_attn.o_proj.weight"]), kv                 # forward.go:106
+
+    def feed_forward_sublayer(self, x, l):
+        """/root/reference/internal/llm/forward.go:109-113: what the feed-forward half
+        of layer l adds to the stream: norm first, then down(silu(gate) * up)."""
+        w = self.w
+        p = f"model.layers.{l}."
+        xb = plain_rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps)      # forward.go:109
+        h = plain_swiglu(plain_matmul(xb, w[p + "mlp.gate_proj.weight"]),
+                         plain_matmul(xb, w[p + "mlp.up_proj.weight"]))                # forward.go:110-112
+        return plain_matmul(h, w[p + "mlp.down_proj.weight"])                          # forward.go:113
+
+    def block(self, x, l, pos, kv=None, window=0):
+        """/root/reference/internal/llm/forward.go:80-115: x <- x + attention(norm(x));
+        x <- x + feed_forward(norm(x)): each half reads the normed stream and adds to
+        the stream itself.  Returns (x, (k, v))."""
+        delta, kv = self.attention_sublayer(x, l, pos, kv, window)
+        x = x + delta                                                                  # forward.go:107
+        x = x + self.feed_forward_sublayer(x, l)                                       # forward.go:114
+        return x, kv
+
+    def head(self, x) -> torch.Tensor:
+        """/root/reference/internal/llm/forward.go:124-141: the final norm, then the
+        product with the output matrix (the embedding table itself when tied,
+        model.go:118-121); nothing scales the logits."""
+        w = self.w
+        x = plain_rmsnorm(x, w["model.norm.weight"], self.eps)                         # forward.go:124-128
+        head = w["model.embed_tokens.weight"] if self.tied else w["lm_head.weight"]    # model.go:118-121
+        return plain_matmul(x, head)                                                   # forward.go:132-141
+
     def forward(self, tokens, schedule=None, windows=None, rows=None) -> torch.Tensor:
         """/root/reference/internal/llm/forward.go:51-142 for one sequence from
         position 0, logits at every position (or at the positions `rows` only: the
@@ -158,35 +208,20 @@ class PlainLlama:
         running order (default: every layer once, its own cache); an entry that does
         not write reads the keys and values that the entry which wrote `cache` made.
         windows: {layer: keys kept} for layers with a window."""
-        w = self.w
         T = len(tokens)
         pos = list(range(T))
-        x = w["model.embed_tokens.weight"][torch.as_tensor(tokens, dtype=torch.long)]   # forward.go:75-77
+        x = self.embed(tokens)
         if schedule is None:
             schedule = [(l, l, True) for l in range(self.L)]
         windows = windows or {}
         caches = {}
         for l, cache, writes in schedule:
-            p = f"model.layers.{l}."
-            xb = plain_rmsnorm(x, w[p + "input_layernorm.weight"], self.eps)           # forward.go:82
-            q = plain_matmul(xb, w[p + "self_attn.q_proj.weight"]).reshape(T, self.H, self.hd)
-            q = plain_rope(q, pos, self.inv_freq)                                      # forward.go:96-97
+            x, kv = self.block(x, l, pos, None if writes else caches[cache], windows.get(l, 0))
             if writes:
-                k = plain_matmul(xb, w[p + "self_attn.k_proj.weight"]).reshape(T, self.K, self.hd)
-                v = plain_matmul(xb, w[p + "self_attn.v_proj.weight"]).reshape(T, self.K, self.hd)
-                caches[cache] = (plain_rope(k, pos, self.inv_freq), v)                 # forward.go:99-101
-            k, v = caches[cache]
-            att = plain_attention(q, k, v, window=windows.get(l, 0)).reshape(T, self.H * self.hd)   # forward.go:104
-            x = x + plain_matmul(att, w[p + "self_attn.o_proj.weight"])                # forward.go:106-107
-            xb = plain_rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps)  # forward.go:109
-            h = plain_swiglu(plain_matmul(xb, w[p + "mlp.gate_proj.weight"]),
-                             plain_matmul(xb, w[p + "mlp.up_proj.weight"]))            # forward.go:110-112
-            x = x + plain_matmul(h, w[p + "mlp.down_proj.weight"])                     # forward.go:113-114
+                caches[cache] = kv
         if rows is not None:
             x = x[torch.as_tensor(list(rows), dtype=torch.long)]
-        x = plain_rmsnorm(x, w["model.norm.weight"], self.eps)                         # forward.go:124-128
-        head = w["model.embed_tokens.weight"] if self.tied else w["lm_head.weight"]    # model.go:118-121
-        return plain_matmul(x, head)                                                   # forward.go:132-141
+        return self.head(x)
 
     def greedy(self, prompt, n_new: int) -> list:
         """Greedy continuation: first maximum wins (/root/reference/internal/llm/sampler.go:76-84)."""
