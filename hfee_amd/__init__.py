@@ -9,13 +9,16 @@ from .config import ConfigError, LlamaConfig, register_architecture
 from .weights import WeightsError, write_model_folder
 
 __all__ = ["LLM", "SamplingParams", "ConfigError", "WeightsError", "LlamaConfig",
-           "register_architecture", "write_model_folder"]
+           "register_architecture", "write_model_folder", "replay"]
 
 
 def __getattr__(name):
     if name in ("LLM", "Output"):
         from . import api
         return getattr(api, name)
+    if name == "replay":
+        from .trace_replay import replay
+        return replay
     if name == "SamplingParams":
         from .sampling import SamplingParams
         return SamplingParams

@@ -204,7 +204,7 @@ def main(argv=None) -> int:
     if cmd == "run":
         return run(rest)
     if cmd == "replay":
-        from .replay import main as replay_main
+        from .trace_replay import main as replay_main
         return replay_main(rest)
     if cmd == "bench":
         return bench(rest)

@@ -1,7 +1,6 @@
 // An entry point that allocates nothing.
 //
-// It has no counterpart in the reference (which picks its greedy token on the host,
-// /root/reference/internal/llm/sampler.go:76-84).  It is for callers that cannot
+// It has no counterpart in the reference.  It is for callers that cannot
 // allocate device memory: code under HIP graph capture, tight serving loops, harnesses
 // that forbid hipMalloc.  hfee_argmax spreads a row over several workgroups only when
 // its caller brings a buffer for their partial results and counters that are zero;

@@ -31,7 +31,7 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fvisibility=h
          "-Wno-unused-command-line-argument"]
 
 CORE_SOURCES = ["elementwise.hip", "gemm_f32.hip", "attention_ref.hip", "gemm_bf16.hip", "gemm_skinny.hip",
-                "sampling.hip", "yardstick.hip"]
+                "sampling.hip", "random_fill.hip", "yardstick.hip"]
 ATTENTION_SOURCE = "attention_bf16.hip"
 HEAD_DIMS = tuple(range(16, 257, 16))
 

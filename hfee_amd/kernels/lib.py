@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import threading
-from ctypes import c_void_p, c_int, c_int64, c_float, c_uint64, c_char_p
+from ctypes import c_void_p, c_int, c_int64, c_float, c_double, c_uint64, c_char_p
 
 from . import build
 
@@ -20,7 +20,7 @@ class KernelError(RuntimeError):
     """An entry point refused its arguments or its launch failed."""
 
 
-P, I, L, F, U64 = c_void_p, c_int, c_int64, c_float, c_uint64
+P, I, L, F, D, U64 = c_void_p, c_int, c_int64, c_float, c_double, c_uint64
 
 _CORE_SIGNATURES = {
     "hfee_embed": [P, P, I, P, I, I, P],
@@ -43,6 +43,7 @@ _CORE_SIGNATURES = {
     "hfee_argmax": [P, P, L, I, I, P, L, P, I, P],
     "hfee_sample": [P, P, L, I, I, P, P, P, P, L, P],
     "hfee_argmax_static": [P, P, L, I, I, P],
+    "hfee_random_fill": [P, I, L, U64, I, D, L, P],
     "hfee_read_stream": [P, L, P, I, I, P],
     "hfee_mfma_loop": [P, I, I, P],
 }

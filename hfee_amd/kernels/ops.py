@@ -134,6 +134,21 @@ def swiglu(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
     lib.core().call("hfee_swiglu", _ptr(out), ldo, _ptr(gate), _ptr(up), ld, gate.stride(1), _dt(out), n, w, _stream())
 
 
+def random_fill(out: torch.Tensor, key: int, kind: str, std: float = 1.0, bound: int = 0):
+    """Fills `out` with element i = f(key, i): kind "normal" (N(0, std)), "one_plus_normal"
+    (1 + N(0, std)) into a float32 or bfloat16 tensor, "integers" (in [0, bound)) into an int32
+    tensor.  The host twin is weights/random_stream.py: the same bits."""
+    _gpu(out)
+    _check(out.is_contiguous(), "random_fill: the tensor must be contiguous")
+    if kind == "integers":
+        _check(out.dtype == torch.int32, "random_fill: integers go into an int32 tensor")
+        lib.core().call("hfee_random_fill", _ptr(out), 0, out.numel(), key, 2, 0.0, int(bound), _stream())
+        return
+    _check(kind in ("normal", "one_plus_normal"), f"random_fill: unknown kind {kind!r}")
+    lib.core().call("hfee_random_fill", _ptr(out), _dt(out), out.numel(), key, 1 if kind == "one_plus_normal" else 0,
+                    float(std), 0, _stream())
+
+
 def residual_add(x: torch.Tensor, y: torch.Tensor):
     """x (float32) += y."""
     _gpu(x, y)

@@ -55,14 +55,14 @@ TINY_C = {
 TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 
 
-def make_model_folder(path, config_json, seed, dtype="float32", std=0.02, norm_init=None):
+def make_model_folder(path, config_json, seed, dtype="float32", std=0.02, norm_init=None, device="cpu"):
     import torch
     import hfee_amd  # noqa: F401  (registers the architecture)
     from hfee_amd.config import config_from_dict
     from hfee_amd.weights import write_model_folder
     cfg = config_from_dict(config_json)
     dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype]
-    return write_model_folder(str(path), cfg, seed=seed, std=std, dtype=dt, norm_init=norm_init)
+    return write_model_folder(str(path), cfg, seed=seed, std=std, dtype=dt, norm_init=norm_init, device=device)
 
 
 @pytest.fixture(scope="session")

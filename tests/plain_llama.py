@@ -18,6 +18,15 @@ import torch
 F64 = torch.float64
 
 
+def to_bfloat16(x: torch.Tensor) -> torch.Tensor:
+    """x rounded to the nearest bfloat16 number (ties to even), as float64 again."""
+    return x.to(torch.float32).to(torch.bfloat16).to(F64)
+
+
+def same(x: torch.Tensor) -> torch.Tensor:
+    return x
+
+
 # ---------------------------------------------------------------- parts -----
 
 def plain_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
@@ -70,14 +79,14 @@ def plain_rope(x: torch.Tensor, positions, inv_freq: torch.Tensor, pairing: str 
     x = x.to(F64).clone()
     T, _, hd = x.shape
     half = inv_freq.numel()
-    pos = torch.as_tensor(positions, dtype=F64).reshape(T, 1)
-    ang = pos * inv_freq.reshape(1, half)          # [T, half]
+    pos = torch.as_tensor(positions, dtype=F64, device=x.device).reshape(T, 1)
+    ang = pos * inv_freq.to(x.device).reshape(1, half)          # [T, half]
     cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
     if pairing == "half":
-        a = torch.arange(half)
+        a = torch.arange(half, device=x.device)
         b = a + half
     elif pairing == "interleaved":
-        a = 2 * torch.arange(half)
+        a = 2 * torch.arange(half, device=x.device)
         b = a + 1
     else:
         raise ValueError(pairing)
@@ -89,33 +98,40 @@ def plain_rope(x: torch.Tensor, positions, inv_freq: torch.Tensor, pairing: str 
 
 def plain_softmax(s: torch.Tensor) -> torch.Tensor:
     """/root/reference/internal/ggml/ops.go:136-150: subtract the maximum,
-    exponentiate, divide by the sum."""
+    exponentiate, divide by the sum (along the last dimension)."""
     s = s.to(F64)
-    e = torch.exp(s - s.max())
-    return e / e.sum()
+    e = torch.exp(s - s.max(dim=-1, keepdim=True).values)
+    return e / e.sum(dim=-1, keepdim=True)
 
 
 def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None = None,
-                    window: int = 0, positions=None) -> torch.Tensor:
+                    window: int = 0, positions=None, round_terms=None) -> torch.Tensor:
     """/root/reference/internal/llm/forward.go:144-178.  q: [T, H, hd], k, v:
     [T, K, hd] (k already rotated).  Head h reads KV head h // (H/K); token i
     scores keys 0..i (no mask values: the range is the mask), score = dot * scale,
     softmax, weighted sum of v.  `window` > 0 narrows the range to the last
-    `window` keys (the reference has no window; 0 is its behaviour)."""
+    `window` keys (the reference has no window; 0 is its behaviour).  round_terms
+    (not in the reference): a function that the terms exp(score - max) go through
+    on their way into the weighted sum, while their sum is taken unrounded, as an
+    engine does that multiplies in a narrow format and divides by a float32 sum."""
     T, H, hd = q.shape
     K = k.shape[1]
     group = H // K
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
     q, k, v = q.to(F64), k.to(F64), v.to(F64)
-    out = torch.zeros(T, H, hd, dtype=F64)
+    out = torch.zeros(T, H, hd, dtype=F64, device=q.device)
     for i in range(T):
         lo = 0 if window <= 0 else max(0, i - window + 1)
-        for h in range(H):
-            kvh = h // group
-            scores = (k[lo:i + 1, kvh, :] @ q[i, h, :]) * scale
+        # the heads of a group side by side: qi[kvh, g] is head kvh * group + g, which reads KV head kvh
+        qi = q[i].reshape(K, group, hd)
+        scores = torch.einsum("nkd,kgd->kgn", k[lo:i + 1], qi) * scale
+        if round_terms is None:
             p = plain_softmax(scores)
-            out[i, h, :] = p @ v[lo:i + 1, kvh, :]
+            out[i] = torch.einsum("kgn,nkd->kgd", p, v[lo:i + 1]).reshape(H, hd)
+        else:
+            e = torch.exp(scores - scores.max(dim=-1, keepdim=True).values)
+            out[i] = (torch.einsum("kgn,nkd->kgd", round_terms(e), v[lo:i + 1]) / e.sum(dim=-1, keepdim=True)).reshape(H, hd)
     return out
 
 
@@ -130,8 +146,16 @@ def plain_swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 class PlainLlama:
     """Reads a model folder; forward(tokens) -> logits [T, vocab] (float64)."""
 
-    def __init__(self, model_dir: str):
+    def __init__(self, model_dir: str, round_like_engine: bool = False, device: str = "cpu", weights=None):
+        """weights: the tensors of another PlainLlama of the same folder, to share (read only).  device: where torch keeps the tensors and does the arithmetic (the same
+        float64 library routines either way).  round_like_engine (not in the reference): what a bfloat16 engine keeps in
+        bfloat16 between its kernels is rounded to bfloat16 here too (the normed
+        stream, q and k after the rotation, v, the terms of the softmax on their way
+        into the weighted sum, the attention's output, the gated product); sums
+        stay float64 and the stream itself is not rounded.  The distance of an
+        engine to this twin is what its kernels add beyond the format."""
         from safetensors import safe_open
+        self.r = to_bfloat16 if round_like_engine else same
         with open(os.path.join(model_dir, "config.json"), "r", encoding="utf-8") as f:
             c = json.load(f)
         self.c = c
@@ -146,15 +170,19 @@ class PlainLlama:
         if scaling is not None and scaling.get("rope_type", scaling.get("type")) != "llama3":
             scaling = None
         self.inv_freq = plain_rope_frequencies(self.hd, c.get("rope_theta", 10000.0), scaling)
+        self.device = device
+        if weights is not None:
+            self.w = weights
+            return
         self.w = {}
         with safe_open(os.path.join(model_dir, "model.safetensors"), framework="pt") as f:
             for name in f.keys():
-                self.w[name] = f.get_tensor(name).to(F64)
+                self.w[name] = f.get_tensor(name).to(device=device).to(F64)
 
     def embed(self, tokens) -> torch.Tensor:
         """/root/reference/internal/llm/forward.go:75-77: the token's row of the table,
         as it is stored (no scaling by sqrt(width) or anything else)."""
-        return self.w["model.embed_tokens.weight"][torch.as_tensor(tokens, dtype=torch.long)]
+        return self.w["model.embed_tokens.weight"][torch.as_tensor(tokens, dtype=torch.long, device=self.device)]
 
     def attention_sublayer(self, x, l, pos, kv=None, window=0):
         """/root/reference/internal/llm/forward.go:82-107: what the attention half of
@@ -163,25 +191,27 @@ class PlainLlama:
         with kv given, those keys and values are read instead of made."""
         w, T = self.w, x.shape[0]
         p = f"model.layers.{l}."
-        xb = plain_rmsnorm(x, w[p + "input_layernorm.weight"], self.eps)               # forward.go:82
+        r = self.r
+        xb = r(plain_rmsnorm(x, w[p + "input_layernorm.weight"], self.eps))            # forward.go:82
         q = plain_matmul(xb, w[p + "self_attn.q_proj.weight"]).reshape(T, self.H, self.hd)
-        q = plain_rope(q, pos, self.inv_freq)                                          # forward.go:96-97
+        q = r(plain_rope(q, pos, self.inv_freq))                                       # forward.go:96-97
         if kv is None:
             k = plain_matmul(xb, w[p + "self_attn.k_proj.weight"]).reshape(T, self.K, self.hd)
             v = plain_matmul(xb, w[p + "self_attn.v_proj.weight"]).reshape(T, self.K, self.hd)
-            kv = (plain_rope(k, pos, self.inv_freq), v)                                # forward.go:99-101
-        att = plain_attention(q, kv[0], kv[1], window=window).reshape(T, self.H * self.hd)          # forward.go:104
-        return plain_matmul(att, w[p + "self_attn.o_proj.weight"]), kv                 # forward.go:106
+            kv = (r(plain_rope(k, pos, self.inv_freq)), r(v))                          # forward.go:99-101
+        att = plain_attention(q, kv[0], kv[1], window=window,
+                              round_terms=None if r is same else r).reshape(T, self.H * self.hd)    # forward.go:104
+        return plain_matmul(r(att), w[p + "self_attn.o_proj.weight"]), kv              # forward.go:106
 
     def feed_forward_sublayer(self, x, l):
         """/root/reference/internal/llm/forward.go:109-113: what the feed-forward half
         of layer l adds to the stream: norm first, then down(silu(gate) * up)."""
         w = self.w
         p = f"model.layers.{l}."
-        xb = plain_rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps)      # forward.go:109
+        xb = self.r(plain_rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps))    # forward.go:109
         h = plain_swiglu(plain_matmul(xb, w[p + "mlp.gate_proj.weight"]),
                          plain_matmul(xb, w[p + "mlp.up_proj.weight"]))                # forward.go:110-112
-        return plain_matmul(h, w[p + "mlp.down_proj.weight"])                          # forward.go:113
+        return plain_matmul(self.r(h), w[p + "mlp.down_proj.weight"])                  # forward.go:113
 
     def block(self, x, l, pos, kv=None, window=0):
         """/root/reference/internal/llm/forward.go:80-115: x <- x + attention(norm(x));
@@ -197,7 +227,7 @@ class PlainLlama:
         product with the output matrix (the embedding table itself when tied,
         model.go:118-121); nothing scales the logits."""
         w = self.w
-        x = plain_rmsnorm(x, w["model.norm.weight"], self.eps)                         # forward.go:124-128
+        x = self.r(plain_rmsnorm(x, w["model.norm.weight"], self.eps))                 # forward.go:124-128
         head = w["model.embed_tokens.weight"] if self.tied else w["lm_head.weight"]    # model.go:118-121
         return plain_matmul(x, head)                                                   # forward.go:132-141
 
@@ -220,8 +250,8 @@ class PlainLlama:
             if writes:
                 caches[cache] = kv
         if rows is not None:
-            x = x[torch.as_tensor(list(rows), dtype=torch.long)]
-        return self.head(x)
+            x = x[torch.as_tensor(list(rows), dtype=torch.long, device=self.device)]
+        return self.head(x).cpu()
 
     def greedy(self, prompt, n_new: int) -> list:
         """Greedy continuation: first maximum wins (/root/reference/internal/llm/sampler.go:76-84)."""

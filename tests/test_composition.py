@@ -225,7 +225,7 @@ def test_the_engine_satisfies_every_identity(tmp_path, cut):
     """The same four vectors through the engine's own block, embedding and head, in 32-bit, whole
     and token by token; then the scaling of the stream (the embedding table times 3 with a
     negligible eps changes the logits exactly as the identity says: 3x + a, not 3(x + a))."""
-    from hfee_amd.replay import Replayer
+    from hfee_amd.trace_replay import Replayer
 
     def engine_logits(folder):
         rep = Replayer(folder, "float32", max_tokens=64)

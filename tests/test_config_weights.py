@@ -149,6 +149,37 @@ def test_safetensors_reader_refuses_broken_files(tmp_path):
     assert sorted(ck.names()) == ["a", "b"] and torch.equal(ck.tensor("b"), torch.ones(3))
 
 
+def test_a_checkpoint_in_two_shards_loads_like_the_single_file(tmp_path):
+    """A folder whose tensors lie in two safetensors files behind model.safetensors.index.json
+    is read end to end: the same tensors, in both engine types, come out of `load_tensors` as
+    from the single file."""
+    from safetensors.torch import load_file
+    folder = make_model_folder(tmp_path / "one", TINY_B, seed=3, dtype="bfloat16", std=0.1)
+    tensors = load_file(os.path.join(folder, "model.safetensors"))
+    names = sorted(tensors)
+    first = {n: tensors[n] for n in names[::2]}
+    second = {n: tensors[n] for n in names[1::2]}
+    two = tmp_path / "two"
+    os.makedirs(two)
+    write_safetensors(str(two / "model-00001-of-00002.safetensors"), first)
+    write_safetensors(str(two / "model-00002-of-00002.safetensors"), second)
+    weight_map = {n: "model-00001-of-00002.safetensors" for n in first}
+    weight_map.update({n: "model-00002-of-00002.safetensors" for n in second})
+    json.dump({"metadata": {"total_size": 0}, "weight_map": weight_map}, open(two / "model.safetensors.index.json", "w"))
+    json.dump(json.load(open(os.path.join(folder, "config.json"))), open(two / "config.json", "w"))
+    cfg = config_from_folder(str(two))
+    specs = declared_tensors(cfg)
+    for dtype in (torch.bfloat16, torch.float32):
+        a = load_tensors(folder, specs, dtype, "cpu")
+        b = load_tensors(str(two), specs, dtype, "cpu")
+        assert set(a) == set(b) == set(names)
+        assert all(torch.equal(a[n], b[n]) and a[n].dtype == b[n].dtype for n in names)
+    # a tensor missing from one shard is reported by name, with everything else that is wrong
+    write_safetensors(str(two / "model-00002-of-00002.safetensors"), {n: t for n, t in second.items() if n != "model.norm.weight"})
+    with pytest.raises(Exception, match="model.norm.weight"):
+        load_tensors(str(two), specs, torch.bfloat16, "cpu")
+
+
 def test_schedule_and_cache_groups_are_data():
     """A layer may run twice, or read another layer's cache; layers with different
     needs land in different cache groups."""
