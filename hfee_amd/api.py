@@ -40,7 +40,9 @@ class LLM:
         budget of a step (256 in the reference, /root/reference/internal/llm/runner.go:11).
         keep_prefixes: a finished request's full pages stay in the cache, and a prompt that
         begins with the same tokens does not run them again (the reference reuses the longest
-        common prefix of a free slot's tokens, runner.go:198-229)."""
+        common prefix of a free slot's tokens, runner.go:198-229).  num_pages: the cache pool in
+        pages of page_size tokens; by default every request slot can hold its whole context, as
+        far as the device's free memory allows after the weights."""
         from .config import config_from_folder
         if model is not None and not random_weights:
             self.model, self.config = load_model(model, dtype, device)
@@ -50,8 +52,8 @@ class LLM:
         spec = self.model.spec
         self.num_ctx = max(1, min(num_ctx, spec.max_positions))
         max_batch_tokens = max(1, min(max_batch_tokens, 65536))
-        if num_pages is None:
-            num_pages = num_parallel * ((self.num_ctx + page_size - 1) // page_size)
+        # (num_pages None: what num_parallel requests of num_ctx tokens take, or what the free memory
+        # holds if that is less; a number that does not fit is refused before anything is allocated)
         self.engine = Engine(self.model, num_pages=num_pages, page_size=page_size, max_requests=num_parallel,
                              keep_prefixes=keep_prefixes,
                              max_batch_tokens=max_batch_tokens, num_positions=self.num_ctx, device=device)

@@ -1,2 +1,3 @@
 from .manager import CacheManager, CacheGroupSpec, PagePool, RequestCache, OutOfPages, CacheError
 from .storage import CacheStorage, bytes_per_token
+from . import capacity

@@ -72,6 +72,8 @@ struct TileOps {
 // The operand of s_waitcnt that waits until at most n vector memory operations are outstanding
 // and for nothing else (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
 constexpr int vmcnt_only(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+// The same, and until every LDS read of this wave has returned (lgkmcnt 0).
+constexpr int vmcnt_and_lds_reads(int n) { return (n & 15) | (7 << 4) | (0 << 8) | ((n >> 4) << 14); }
 
 // 64 consecutive entries of a sequence's block table, one per lane, so that a tile's
 // page numbers come from a register shuffle instead of a load that the tile's own loads
@@ -666,9 +668,12 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
       // (the wait is the compiler's own builtin, not text it cannot read: it then knows that
       // the loads of before the loop, the queries, have arrived, and does not wait for them,
       // and with them for every load behind them, in front of every product)
-      if (behind >= 2) __builtin_amdgcn_s_waitcnt(vmcnt_only(2 * MINE));
-      else if (behind == 1) __builtin_amdgcn_s_waitcnt(vmcnt_only(MINE));
-      else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+      // (and this wave's own LDS reads of tile t - 1 have returned: the products that consume them
+      // stand before this point, but nothing else would make a read that is still on its way
+      // come back before another wave's load lands in the place it reads)
+      if (behind >= 2) __builtin_amdgcn_s_waitcnt(vmcnt_and_lds_reads(2 * MINE));
+      else if (behind == 1) __builtin_amdgcn_s_waitcnt(vmcnt_and_lds_reads(MINE));
+      else __builtin_amdgcn_s_waitcnt(vmcnt_and_lds_reads(0));
       // ... and after the barrier everybody's have, and nobody reads tile t - 1 any more, whose
       // place the next request takes.  (No fence: it would wait for every load in flight.)
       asm volatile("" ::: "memory");
@@ -930,6 +935,9 @@ __global__ __launch_bounds__(64) void combine_kernel(bf16_t* __restrict__ out, i
 }  // namespace
 
 HFEE_API int hfee_attention_bf16_head_dim() { return HD; }
+
+// The most row tiles in a run of `runs` (hfee_attention_bf16_prefill): one wave a row tile.
+HFEE_API int hfee_attention_bf16_run_tiles() { return SHARED_WAVES; }
 
 static int check_common(const char* name, int64_t ld_out, int64_t ldq, int num_heads, int kv_heads,
                         int page_size, int window, float scale, const void* out, const void* q, CacheLayout* lay) {

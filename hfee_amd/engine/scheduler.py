@@ -20,9 +20,12 @@ there.  Here they can, and this is what happens:
 
   1. requests that run come before requests that wait: decoding requests first, then the
      prompts that are still being read, oldest first, and only then is a waiting request
-     admitted, if a state slot is free and the free pages cover its first portion (so the
-     pages that a preemption frees go to those who needed them, not back to the request
-     that gave them up);
+     admitted, if a state slot is free and a page is free for the beginning of its first
+     portion (so the pages that a preemption frees go to those who needed them, not back to
+     the request that gave them up); a request that was preempted comes back, while others
+     run, not in the step that preempted it and only when the free pages hold all it has to
+     run again, its next token, and a page for every running request's next page edge (let
+     in on less it would run its tokens again only to give way again);
   2. a prompt portion is shortened to what the free pages hold (or waits a step);
   3. if a decoding request cannot get the page its next token needs, requests younger than
      it are preempted, youngest first: their pages go back, and they return to the front
@@ -109,6 +112,7 @@ class Scheduler:
         self.eos = set(eos_token_ids)
         self.clock = clock
         self.waiting: deque = deque()
+        self._preempted_now: set = set()      # requests preempted by the step being put together
         self.running: list = []          # in admission order
         self._order = 0
         self.last_batch: list = []       # (request_id, tokens in the step) of the latest step, for tests
@@ -148,9 +152,18 @@ class Scheduler:
             room = r if room is None else min(room, r)
         return max(room or 0, 0)
 
+    def _comes_back_with(self, request: Request) -> int:
+        """Free tokens that a preempted request waits for while others run: room for all it has
+        to run again and its next token, and a page for every running request's next page edge.
+        Let in on a single free page it would run its prompt and its tokens again only to be
+        preempted at the next edge of an older request, step after step."""
+        ps = self.cache.page_size
+        return (len(request.feed) + 1 + ps - 1) // ps * ps + len(self.running) * ps
+
     def _preempt(self, victim: Request) -> None:
         self.engine.release(victim.request_id, victim.history)
         self.running.remove(victim)
+        self._preempted_now.add(victim.request_id)
         victim.feed = list(victim.prompt) + list(victim.generated)
         victim.decoding = False
         victim.stats.preemptions += 1
@@ -239,6 +252,7 @@ class Scheduler:
 
         budget = self.max_batch_tokens
         batch: list = []     # (request, tokens, wants_logits)
+        self._preempted_now.clear()
 
         # decoding requests first, oldest first; preempt from the young end if pages run out
         ps = self.cache.page_size
@@ -284,6 +298,10 @@ class Scheduler:
             free_tokens = min(p.num_free for p in self.cache.pools) * self.cache.page_size if self.cache.pools else first
             if free_tokens < min(first, self.cache.page_size) and self.running:
                 break                      # wait until pages come back
+            if r.request_id in self._preempted_now:
+                break                      # it has just given its pages up: not back in the same step
+            if r.stats.preemptions and self.running and free_tokens < self._comes_back_with(r):
+                break                      # it would run its tokens again only to give way again
             if free_tokens < 1:
                 self.waiting.popleft()
                 self._finish(r, "length", finished, "the cache has no free page for this request")

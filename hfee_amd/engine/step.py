@@ -15,7 +15,7 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
-from ..cache import CacheManager, CacheStorage, OutOfPages
+from ..cache import CacheManager, CacheStorage, OutOfPages, bytes_per_token, capacity
 from ..parts.base import Segment, StepContext, Workspace
 from .model import EngineInfo, Model
 
@@ -65,10 +65,24 @@ class Engine:
         self.num_positions = min(num_positions or model.spec.max_positions, model.spec.max_positions)
         self.vocab = model.spec.vocab
         self.groups = model.cache_groups()
-        if num_pages is None:
-            if cache_tokens is None:
-                cache_tokens = self.num_positions * max_requests
-            num_pages = (cache_tokens + page_size - 1) // page_size
+        # The pool: as many pages as were asked for (by number or by tokens), or what every slot at
+        # its full context takes; never more than the device's free memory holds beside the
+        # workspace of the largest step and a reserve (the weights are there already).
+        wanted = None
+        if num_pages is not None:
+            wanted = num_pages
+        elif cache_tokens is not None:
+            wanted = (cache_tokens + page_size - 1) // page_size
+        at_most = max_requests * ((self.num_positions + page_size - 1) // page_size)
+        if isinstance(wanted, (list, tuple)):          # a number for every group
+            need = sum(n * page_size * bytes_per_token([g], self.dtype) for n, g in zip(wanted, self.groups))
+            capacity.require_room(need + self._state_bytes(), f"the cache of {list(wanted)} pages in its groups",
+                                  *self._memory(), self._workspace_estimate())
+            num_pages = list(wanted)
+        else:
+            num_pages = capacity.choose_pages(wanted, at_most, *self._memory(), self._workspace_estimate(),
+                                              page_size * bytes_per_token(self.groups, self.dtype),
+                                              self._state_bytes())
         self.num_pages = num_pages
         # (a finished request's full pages wait for a request that begins alike: only where every
         # group keeps every token and no part has state that cannot be cut back)
@@ -91,6 +105,27 @@ class Engine:
         self.use_graphs = use_graphs and model.graph_safe
         self._graphs: dict = {}
         self.graph_replays = 0
+
+    # ------------------------------------------------------------ memory
+    def _memory(self):
+        """(free, total) bytes of the device; what torch holds in its pool without using it counts as free."""
+        free, total = torch.cuda.mem_get_info(self.device)
+        idle = torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
+        return free + max(0, idle), total
+
+    def _workspace_estimate(self) -> int:
+        widest = max([s.shape[0] for s in self.model.tensor_specs() if len(s.shape) == 2 and s.shape[0] != self.vocab]
+                     or [self.model.spec.hidden])
+        return capacity.workspace_bytes(self.max_batch_tokens, self.vocab, max(widest, self.model.spec.hidden))
+
+    def _state_bytes(self) -> int:
+        total = 0
+        for _, shape, dt in self.model.state_specs():
+            n = self.max_requests
+            for d in shape:
+                n *= d
+            total += n * torch.empty((), dtype=dt).element_size()
+        return total
 
     # ------------------------------------------------------------ requests
     def admit(self, request_id, tokens=None):

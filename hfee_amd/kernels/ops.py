@@ -432,14 +432,38 @@ def _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, he
     return n, ldq, ldo
 
 
+def attention_run_tiles(head_dim: int) -> int:
+    """The most row tiles that a run of `attention_bf16_prefill`'s `runs` may hold."""
+    return int(lib.attention_bf16(head_dim).raw("hfee_attention_bf16_run_tiles")())
+
+
+def attention_runs(tiles, head_dim: int) -> list:
+    """The runs of a step's row tiles, on the host: tiles is the list of (first row, rows, first
+    position, block-table row) that `attention_bf16_prefill` takes; a run is (first tile, count) of
+    tiles of one sequence whose rows and positions go on where the tile before ended, at most
+    `attention_run_tiles` of them, every tile in exactly one run."""
+    most = attention_run_tiles(head_dim)
+    runs = []
+    for t, (row, rows, pos, table) in enumerate(tiles):
+        if runs and runs[-1][1] < most:
+            first, count = runs[-1]
+            prow, prows, ppos, ptable = tiles[first + count - 1]
+            if ptable == table and prow + prows == row and ppos + prows == pos:
+                runs[-1] = (first, count + 1)
+                continue
+        runs.append((t, 1))
+    return runs
+
+
 def attention_bf16_prefill(out, q, cache_layer, tiles, block_tables, num_heads: int, kv_heads: int,
                            head_dim: int, page_size: int, scale: float, window: int = 0, kernel: int = 0, runs=None):
     """tiles: [num_tiles, 4] int32 (first row, rows <= 32, first position, block-table row).
     kernel: 0 automatic, 1 one wave per (tile, head), 2 the heads of a KV head share its
     key tiles through LDS.
-    runs: [num_runs, 2] int32 (first tile, count <= 4) or None: every tile in exactly one run of
-    tiles that follow one another in `tiles` and in one sequence, rows and positions going on
-    where the tile before ended.  For heads that share no keys with another head (kv_heads ==
+    runs: [num_runs, 2] int32 (first tile, count <= attention_run_tiles) or None: every tile in
+    exactly one run of tiles that follow one another in `tiles` and in one sequence, rows and
+    positions going on where the tile before ended (`attention_runs` makes them; a longer run
+    would leave row tiles without output).  For heads that share no keys with another head (kv_heads ==
     num_heads) the row tiles of a run then share the head's key tiles through LDS."""
     n, ldq, ldo = _attention_common(out, q, cache_layer, block_tables, num_heads, kv_heads, head_dim, page_size)
     _check(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),

@@ -29,7 +29,6 @@ from ..weights.spec import TensorSpec
 from .base import LazyNorm, Mixer, lookup, register_mixer
 
 _TILE = 32            # query rows per workgroup of the prefill kernel, keys per tile
-_RUN = 4              # row tiles of one head that share its key tiles where no other head does
 _DECODE_WAVES = 4     # waves of a decode workgroup; each takes every 4th key tile
 _TILES_PER_WAVE = 16  # beyond this many tiles per wave the keys are always split over workgroups
 _DECODE_WORKGROUPS = 256   # with fewer (segment, KV head) pairs than this the keys are split to fill the chip
@@ -131,11 +130,10 @@ class Attention(Mixer):
                 d_pos.append(seg.start)
                 d_tab.append(s)
             else:
-                first = len(tiles)
                 for off in range(0, seg.length, _TILE):
                     tiles.append((seg.row0 + off, min(_TILE, seg.length - off), seg.start + off, s))
-                # (runs of up to four row tiles of the portion: for heads that share no keys with another)
-                runs += [(t, min(_RUN, len(tiles) - t)) for t in range(first, len(tiles), _RUN)]
+        # (runs of row tiles of a portion that follow one another: for heads that share no keys with another)
+        runs = ops.attention_runs(tiles, self.head_dim)
         plan.add("attention.tiles", np.asarray(tiles, dtype=np.int32).reshape(-1, 4))
         plan.add("attention.runs", np.asarray(runs, dtype=np.int32).reshape(-1, 2))
         plan.add("attention.decode_rows", np.asarray(d_rows, dtype=np.int32))

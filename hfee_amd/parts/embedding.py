@@ -66,9 +66,14 @@ class Head(Part):
     def bind(self, tensors):
         self.norm.bind(tensors)
         self.weight = tensors[self.name].contiguous() if self.name is not None else self.embedding.table
-        # a second copy in tiles for up to 64 wanted rows, whose product streams the weights
-        self.streams = self.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.hidden % 8 == 0
-        self.weight_tiles = ops.tile_weight(self.weight) if self.streams else None
+        # a second copy in tiles for up to 64 wanted rows, whose product streams the weights (of a
+        # table shared with the embedding too: the lookup reads rows as they lie); like every second
+        # copy only while it leaves room, else the wanted rows go through the kernels for rows
+        self.weight_tiles = None
+        if self.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.hidden % 8 == 0:
+            tiles = ops.tile_weights_if_room(self.weight)
+            self.weight_tiles = tiles[0] if tiles else None
+        self.streams = self.weight_tiles is not None
 
     def forward(self, ctx, logits, x, rows):
         """logits[i] = head(norm(x[rows[i]])); logits float32 [len(rows), vocab]."""

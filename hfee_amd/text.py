@@ -211,7 +211,10 @@ class FolderTokenizer:
     """A model folder's tokenizer.json: text -> ids, id -> bytes.  Byte-level vocabularies
     (words cut by the llama3 or the gpt2 rule, bytes written as printable characters) and
     vocabularies of the sentencepiece kind (spaces written as U+2581, bytes without a piece
-    as <0xNN>) are read; the merges' order is their rank."""
+    as <0xNN>) are read; the merges' order is their rank.  (The reference joins the pieces of a
+    sentencepiece vocabulary by the scores in its model file, tokenizer.go:185-212; a
+    tokenizer.json has none, and its merges are taken to be in descending score, as the
+    converters write them.  A piece without an id and without byte pieces is dropped, as there.)"""
 
     def __init__(self, path: str):
         import json

@@ -241,3 +241,36 @@ def test_random_orders_with_kept_prefixes(seed):
             live[rid] = tokens
         m.check()
     assert reused > 0
+
+
+def test_the_pool_is_sized_from_the_free_memory():
+    """The arithmetic of `capacity`: by default the pool is what every slot at its full context
+    takes, or what fits if that is less; a number that was asked for and does not fit is refused
+    with the bytes it needs and the bytes there are; a pool of no page is refused."""
+    from hfee_amd.cache import capacity
+    from hfee_amd.cache.manager import CacheError
+    gib = 1 << 30
+    total = 288 * gib
+    page = 2 << 20                                     # the 8B shape: 128 KiB a token, 16 tokens
+    work = capacity.workspace_bytes(2048, 128256, 28672)
+    assert work == 2048 * (4 * 128256 + 16 * 28672)
+    reserve = int(capacity.RESERVE_FRACTION * total)
+    # plenty of room: the slots' full contexts decide
+    assert capacity.choose_pages(None, 8 * 512, 200 * gib, total, work, page) == 8 * 512
+    # little room: what fits, to the page
+    free = 30 * gib
+    fit = (free - work - reserve) // page
+    assert capacity.pages_that_fit(free, total, work, page) == fit and 0 < fit < 64 * 8192 // 16
+    assert capacity.choose_pages(None, 64 * 8192 // 16, free, total, work, page) == fit
+    assert capacity.choose_pages(fit, 1, free, total, work, page) == fit          # asked for: taken as it is
+    with pytest.raises(CacheError) as e:
+        capacity.choose_pages(fit + 1, 1, free, total, work, page)
+    msg = str(e.value)
+    assert f"needs {(fit + 1) * page:,} bytes" in msg and f"{free:,}" in msg and f"{fit} pages would fit" in msg
+    # the states' bytes come off first
+    spare = (free - work - reserve) % page
+    assert capacity.pages_that_fit(free, total, work, page, state_bytes=3 * page + spare) == fit - 3
+    assert capacity.pages_that_fit(free, total, work, page, state_bytes=3 * page + spare + 1) == fit - 4
+    with pytest.raises(CacheError, match="no page of the cache fits"):
+        capacity.choose_pages(None, 100, work + reserve + page - 1, total, work, page)
+    assert capacity.choose_pages(None, 100, work + reserve + page, total, work, page) == 1

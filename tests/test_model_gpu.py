@@ -126,7 +126,7 @@ def test_a_prefix_kept_from_an_earlier_request(model_folders, dtype):
 @pytest.mark.parametrize("tiled_calls", [0, 2])
 def test_a_model_too_large_for_second_copies_of_its_weights(model_folders, monkeypatch, tiled_calls):
     """Where the weights' second copies in tiles would not leave room, the parts bound last do
-    without them (none of them, or all but the first layer's attention and feed-forward): steps
+    without them (none of them, or all but the first layer's attention and feed-forward; the head, bound last, in neither case): steps
     of few rows then go through the kernels that read the weights' rows as they lie, beside
     layers that have their tiles, and give the plain model's logits, whole and decoding."""
     from plain_llama import PlainLlama
@@ -143,8 +143,9 @@ def test_a_model_too_large_for_second_copies_of_its_weights(model_folders, monke
     folder = model_folders[("B", "bfloat16")]
     plain = PlainLlama(folder)
     model, cfg = load_model(folder, "bfloat16")
-    with_tiles = [b.mixer.streams for b in model.blocks] + [b.feed_forward.streams for b in model.blocks]
+    with_tiles = [b.mixer.streams for b in model.blocks] + [b.feed_forward.streams for b in model.blocks] + [model.head.streams]
     assert sum(with_tiles) == tiled_calls and calls["n"] == len(with_tiles)
+    assert not model.head.streams            # the head is bound last: it is the first to do without
     eng = Engine(model, num_pages=64, page_size=16, max_requests=4, max_batch_tokens=256)
     g = torch.Generator().manual_seed(2)
     toks = torch.randint(0, cfg.vocab_size, (90,), generator=g).tolist()
@@ -159,3 +160,21 @@ def test_a_model_too_large_for_second_copies_of_its_weights(model_folders, monke
     eng.admit("s")
     both = eng.step([StepEntry("r", [toks[0]], []), StepEntry("s", other, list(range(40)))])
     assert rel_err(both, plain.forward(other)) < TOL["bfloat16"]
+
+
+def test_the_cache_pool_follows_the_free_memory(model_folders):
+    """Without a number the pool is what every slot at its full context takes (there is room for
+    that here); a number that the free memory does not hold is refused with the bytes it needs
+    and the bytes there are, and nothing has been allocated by then."""
+    from hfee_amd.cache import CacheError, bytes_per_token
+    from hfee_amd.engine import Engine, load_model
+    model, cfg = load_model(model_folders[("A", "bfloat16")], "bfloat16")
+    eng = Engine(model, page_size=16, max_requests=4, max_batch_tokens=64)
+    assert eng.num_pages == 4 * (cfg.max_position_embeddings // 16) == eng.cache.pools[0].num_pages
+    assert Engine(model, page_size=16, max_requests=4, max_batch_tokens=64, cache_tokens=100).num_pages == 7
+    free, total = torch.cuda.mem_get_info()
+    page = 16 * bytes_per_token(eng.groups, torch.bfloat16)
+    before = torch.cuda.memory_allocated()
+    with pytest.raises(CacheError, match="pages would fit") as e:
+        Engine(model, num_pages=free // page + 10, page_size=16, max_requests=4, max_batch_tokens=64)
+    assert f"{total:,}" in str(e.value) and torch.cuda.memory_allocated() == before

@@ -177,4 +177,5 @@ def test_a_whole_trace_that_names_its_model_by_configuration_and_seed(tmp_path):
     last = np.fromfile(tmp_path / "out" / "3.f32", dtype="<f4")
     assert np.array_equal(last, r_whole[("b", 49)])
     with pytest.raises(Exception, match="pages"):          # the pool is what the trace says: five pages' worth is refused
-        hfee_amd.replay(dict(whole, steps=[{"segments": [{"req": "a", "tokens": a + b[:20], "want": "last"}]}]))
+        hfee_amd.replay(dict(whole, steps=[{"segments": [{"req": "a", "tokens": a, "want": "last"},
+                                                         {"req": "b", "tokens": b[:30], "want": "last"}]}]))

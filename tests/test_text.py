@@ -163,6 +163,27 @@ def test_a_vocabulary_of_the_sentencepiece_kind(tmp_path):
     assert tok.piece(vocab["<0xE2>"]) == b"\xe2" and tok.piece(1) == b"" and tok.piece(10 ** 6) == b""
 
 
+def test_the_order_of_the_merges_is_their_rank_in_a_sentencepiece_vocabulary_too(tmp_path):
+    """The reference reads scores from its model file and joins the neighbours whose concatenation
+    has the highest score (/root/reference/internal/tokenizer/tokenizer.go:185-212); a tokenizer.json
+    has no scores, only `merges`, which the converters write in descending score, so the place in
+    that list is taken as the rank.  Two lists over one vocabulary show that the list decides, not
+    the vocabulary: with (b, c) first "abc" becomes a + bc, with (a, b) first ab + c.  (Parity with
+    the reference is unpinned for a folder whose merges are not in the order of its scores: no
+    fixture of the reference covers one.)"""
+    path, vocab = sentencepiece_folder(tmp_path)
+    spec = json.loads(open(path, encoding="utf-8").read())
+    pieces = list(spec["model"]["vocab"]) + ["a", "b", "c", "ab", "bc", "▁a", "▁ab"]
+    spec["model"]["vocab"] = vocab = {p: i for i, p in enumerate(pieces)}
+    for merges, want in (([("b", "c"), ("a", "b"), ("▁", "a")], ["▁a", "bc"]),
+                         ([("a", "b"), ("b", "c"), ("▁", "ab"), ("▁", "a")], ["▁ab", "c"]),
+                         ([("▁", "a"), ("a", "b"), ("b", "c")], ["▁a", "bc"])):
+        spec["model"]["merges"] = [f"{l} {r}" for l, r in merges]
+        other = tmp_path / "other.json"
+        other.write_text(json.dumps(spec), encoding="utf-8")
+        assert FolderTokenizer(str(other)).encode("abc") == [vocab[p] for p in want], merges
+
+
 def test_other_kinds_of_tokenizer_are_refused(tmp_path):
     path = tmp_path / "tokenizer.json"
     path.write_text(json.dumps({"model": {"type": "Unigram", "vocab": [["a", 0.0]]}}))
