@@ -136,8 +136,9 @@ def attention_alone(shape: dict) -> dict:
         runs = None
         if heads == kv_heads:      # heads that share no keys: row tiles that follow one another share them, four at a time
             runs = torch.tensor([(i, min(4, rows // 32 - i)) for i in range(0, rows // 32, 4)], dtype=torch.int32, device=dev)
+        kernel = ops.prefill_attention_kernel(tiles.tolist(), 0, kv_heads, heads // kv_heads, head_dim)     # (as the engine chooses)
         call = lambda: ops.attention_bf16_prefill(o, q, cache, tiles, tables, heads, kv_heads, head_dim, page_size,
-                                                  head_dim ** -0.5, runs=runs)
+                                                  head_dim ** -0.5, runs=runs, kernel=kernel)
         call()
         torch.cuda.synchronize()
         best = float("inf")
@@ -183,13 +184,23 @@ def main(argv=None) -> int:
         for shape in ("llama-3.2-1b", "llama-2-13b"):
             other = copy.copy(args)
             other.shape, other.no_points, other.steps, other.warmup = shape, False, min(args.steps, 32), min(args.warmup, 4)
-            other.only_prefill_point = True
+            other.point_batches = (1, 64)
             got = run(other)
             torch.cuda.empty_cache()
             line["points"][f"decode_b8_{shape}"] = got["value"]
             line["points"][f"decode_b8_hbm_frac_{shape}"] = got["roofline"]["frac"]
+            for key, value in got["points"].items():
+                line["points"][f"{key}_{shape}"] = value
             line["points"][f"prefill_2048_{shape}"] = got["prefill"]["value"]
             line["points"][f"prefill_2048_frac_{shape}"] = got["prefill"]["frac"]
+        # continuous batching at the small shape: 128 requests at once, prompts of 64 to 2,048
+        # tokens, 128 new tokens each
+        serving = copy.copy(args)
+        serving.shape, serving.serving = "llama-3.2-1b", 128
+        got = run(serving)
+        torch.cuda.empty_cache()
+        line["points"]["serving_128_generated_tok_s_llama-3.2-1b"] = got["value"]
+        line["points"]["serving_128_all_tok_s_llama-3.2-1b"] = got["all_tokens_per_s"]
         longer = copy.copy(args)
         longer.context, longer.steps, longer.warmup = 8192, min(args.steps, 16), 2
         got = run(longer)
@@ -409,10 +420,11 @@ def run(args):
         line["prefill"] = {"value": round(PREFILL / pt, 1), "tokens": PREFILL, "ms": round(pt * 1e3, 3),
                            "frac": round(flops / pt / BF16_PEAK, 4)}
         points = {}
-        for b in (() if getattr(args, "only_prefill_point", False) else (1, 64, 128)):
+        for b in getattr(args, "point_batches", (1, 64, 128)):
             steps = max(8, min(args.steps, 64))
-            dtb, _ = decode_run(b, steps, min(args.warmup, 4))
+            dtb, ctx_b = decode_run(b, steps, min(args.warmup, 4))
             points[f"decode_b{b}"] = round(b * steps / dtb, 2)
+            points[f"decode_b{b}_hbm_frac"] = round((weight_bytes + b * ctx_b * kv_bytes_per_token) / (dtb / steps) / HBM_PEAK, 4)
         line["points"] = points
     return line
 

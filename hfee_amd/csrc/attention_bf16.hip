@@ -731,6 +731,153 @@ __global__ __launch_bounds__(SHARED_WAVES * 64, 2) void prefill_shared_kernel(
   }
 }
 
+// ------------------------------ prefill, a row tile's keys in two halves ---
+// At a few thousand tokens the launch above is as long as its longest workgroup: the last
+// row tile of a 2,048-token prompt walks 64 key tiles one after the other while most of the
+// chip has long finished (half of the time of the kernel is the tail).  Here a workgroup
+// has eight waves: four heads of a KV head over the first half of the row tile's key tiles,
+// and the same four heads over the second half, each half with its own ring of tiles in
+// LDS, both walking in step (one barrier a step for all eight).  At the end the second
+// half's state goes through the LDS to the first half's waves, which join the two (the
+// reference of the exponentials is per half; the quotient does not depend on it) and store.
+// One workgroup a CU, two waves a SIMD as before; the longest chain is half as long.
+// For four heads (or a multiple) to a KV head, head sizes up to 128 (two rings of four
+// tiles fit the LDS), a layer that 32 bits address.
+constexpr bool HALVES_FIT = KV_BLOCKS % SHARED_WAVES == 0 && 2 * 4 * KV_BLOCKS <= 160;
+constexpr int HALVES_TILES = 4;
+constexpr int JOIN_FLOATS = NDT * 16 + 2;          // a lane's share of a wave's state: O, reference, sum
+
+__global__ __launch_bounds__(2 * SHARED_WAVES * 64, 1) void prefill_halves_kernel(
+    bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
+    const bf16_t* __restrict__ cache, uint32_t layer_bytes, CacheLayout lay, const int* __restrict__ work, int num_tiles,
+    const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2, int window) {
+  extern __shared__ __attribute__((aligned(1024))) char kv_lds[];     // two rings of HALVES_TILES tiles
+  if constexpr (HALVES_FIT) {
+    constexpr int W = SHARED_WAVES, MINE = KV_BLOCKS / W, TILE_BYTES = KV_BLOCKS * 1024, RING_BYTES = HALVES_TILES * TILE_BYTES;
+    const int lane = threadIdx.x & 63, r32 = lane & 31, G = lane >> 5;
+    const int wave8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = wave8 & (W - 1), half = wave8 >> 2;
+    const int group = num_heads / lay.kv_heads, chunks = group / W;
+    int tile, kvh, chunk;
+    {
+      const int per_kv = num_tiles * chunks, total = per_kv * lay.kv_heads, per_xcd = (total + 7) / 8;
+      const int u = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+      if (u >= total) return;
+      kvh = u / per_kv;
+      const int rest = u - kvh * per_kv;
+      tile = num_tiles - 1 - rest / chunks;
+      chunk = rest % chunks;
+    }
+    const int* wk = work + 4 * tile;
+    const int row0 = wk[0], rows = wk[1], pos0 = wk[2], seg = wk[3];
+    const int* bt = block_tables + (int64_t)seg * bt_stride;
+    const int h = kvh * group + chunk * W + wave;
+    const bool slot_ok = r32 < rows;
+    const int pos = slot_ok ? pos0 + r32 : -1;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    Op q_op[NC];
+    load_query(q_op, q + (int64_t)(row0 + (slot_ok ? r32 : 0)) * ldq + h * HD, slot_ok);
+
+    Tile st;
+    init_tile(st);
+    const int kv_last = pos0 + rows - 1;
+    const int kv_first = window > 0 ? max(0, pos0 - window + 1) : 0;
+    const int t_first = kv_first >> 5, t_end = (kv_last >> 5) + 1;
+    // the first half takes the odd tile: it is the one that joins and stores at the end
+    const int t_mid = t_first + (t_end - t_first + 1) / 2;
+    const int my_first = half == 0 ? t_first : t_mid, my_end = half == 0 ? t_mid : t_end;
+    const int common = t_end - t_mid;                       // steps that both halves take
+    const int all_first = window > 0 ? max(0, kv_last - window + 1) : 0;
+    PageWindow pages;
+    pages.base = -1;
+    const WaveBlocks<W> mine = wave_blocks<W>(lay, kvh, wave);
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)cache, 0, (int)layer_bytes, 0x00020000);
+    char* ring = kv_lds + half * RING_BYTES;
+    auto request = [&](int t) {
+      RequestBlocks<W, true>::go(ring + ((t - my_first) % HALVES_TILES) * TILE_BYTES, cache, rsrc, lay, mine, bt, bt_stride,
+                                   pages, t * 32, kv_first, kv_last, wave);
+    };
+    // (as in the kernel above: nothing but the ring's own loads is on its way inside the loop)
+    if (my_first < my_end) request(my_first);
+    if (my_first + 1 < my_end) request(my_first + 1);
+    if (my_first + 2 < my_end) request(my_first + 2);
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    auto arrive = [&](int t) {
+      const int behind = min(HALVES_TILES - 2, my_end - 1 - t);
+      if (behind >= 2) __builtin_amdgcn_s_waitcnt(vmcnt_and_lds_reads(2 * MINE));
+      else if (behind == 1) __builtin_amdgcn_s_waitcnt(vmcnt_and_lds_reads(MINE));
+      else __builtin_amdgcn_s_waitcnt(vmcnt_and_lds_reads(0));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    };
+    auto step = [&](int t) {
+      arrive(t);
+      const char* cur = ring + ((t - my_first) % HALVES_TILES) * TILE_BYTES + lane * 16;
+      compute_tile_with(
+          st, q_op, [&](int c) { return *reinterpret_cast<const bf16x8*>(cur + c * 1024); },
+          [&](int u, int tt) { return *reinterpret_cast<const bf16x8*>(cur + (NC + u * NDT + tt) * 1024); }, t * 32, pos, lo,
+          scale_log2, t * 32 >= all_first && t * 32 + 31 <= pos0, [&]() {
+            if (t + HALVES_TILES - 1 < my_end) request(t + HALVES_TILES - 1);
+          });
+    };
+    for (int i = 0; i < common; ++i) step(my_first + i);
+    if (t_mid - t_first > common) {                         // (the same for the whole workgroup)
+      if (half == 0) {
+        step(my_first + common);
+      } else {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+      }
+    }
+
+    // ---- the second half's state to the first half's waves, through the LDS (every ring is done with)
+    __syncthreads();
+    float* mine_at = reinterpret_cast<float*>(kv_lds) + (size_t)wave * JOIN_FLOATS * 64 + lane;
+    if (half == 1) {
+#pragma unroll
+      for (int t = 0; t < NDT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mine_at[(t * 16 + r) * 64] = st.o[t][r];
+      mine_at[(NDT * 16) * 64] = st.m;
+      mine_at[(NDT * 16 + 1) * 64] = st.l;
+    }
+    __syncthreads();
+    if (half == 1) return;
+    {
+      const float m1 = mine_at[(NDT * 16) * 64], l1 = mine_at[(NDT * 16 + 1) * 64];
+      const float m_new = fmaxf(st.m, m1);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      // (a half without keys has a reference of minus infinity, a sum and an output of zero: its factor is zero)
+      const float f0 = st.m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(st.m - m_use);
+      const float f1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - m_use);
+      st.l = st.l * f0 + l1 * f1;
+#pragma unroll
+      for (int t = 0; t < NDT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st.o[t][r] = st.o[t][r] * f0 + mine_at[(t * 16 + r) * 64] * f1;
+    }
+    const float l_slot = finish_sum(st);
+    if (slot_ok) {
+      const float inv = 1.0f / l_slot;
+      bf16_t* orow = out + (int64_t)(row0 + r32) * ld_out + h * HD;
+#pragma unroll
+      for (int t = 0; t < NDT; ++t)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int d = 32 * t + 8 * b + 4 * G;
+          if (d < HD) {
+            bf16_t v4[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v4[i] = float_to_bf16(st.o[t][4 * b + i] * inv);
+            *reinterpret_cast<u32x2*>(orow + d) = *reinterpret_cast<const u32x2*>(v4);
+          }
+        }
+    }
+  }
+}
+
 // Joins the splits of one (segment, head) in ascending split order: lane s holds the
 // weight of split s, every lane then walks the splits for its own dims.  One wave.
 // COHERENT: the partial results were written by other workgroups of this launch, so
@@ -936,6 +1083,9 @@ __global__ __launch_bounds__(64) void combine_kernel(bf16_t* __restrict__ out, i
 
 HFEE_API int hfee_attention_bf16_head_dim() { return HD; }
 
+// Whether this head size has the prefill kernel with a row tile's keys in two halves (variant 3).
+HFEE_API int hfee_attention_bf16_halves() { return HALVES_FIT ? 1 : 0; }
+
 // The most row tiles in a run of `runs` (hfee_attention_bf16_prefill): one wave a row tile.
 HFEE_API int hfee_attention_bf16_run_tiles() { return SHARED_WAVES; }
 
@@ -954,14 +1104,14 @@ static int check_common(const char* name, int64_t ld_out, int64_t ldq, int num_h
 
 // work: num_tiles x 4 int32 (first row, rows <= 32, first position, block-table row).
 // variant: 0 choose, 1 one wave per (tile, head), 2 key tiles shared in LDS by the heads
-// of a KV head (for tests of each kernel alone).
+// of a KV head, 3 the same with a row tile's keys in two halves (for tests of each kernel alone).
 HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* q, int64_t ldq,
                                          const void* cache, int cache_pages, const int* work, int num_tiles,
                                          const int* runs, int num_runs,
                                          const int* block_tables, int bt_stride, int num_heads, int kv_heads,
                                          int page_size, float scale, int window, int variant, hipStream_t stream) {
   HFEE_REQUIRE(num_tiles >= 0, "attention_bf16_prefill: bad tile count");
-  HFEE_REQUIRE(variant >= 0 && variant <= 2, "attention_bf16_prefill: unknown kernel choice %d", variant);
+  HFEE_REQUIRE(variant >= 0 && variant <= 3, "attention_bf16_prefill: unknown kernel choice %d", variant);
   HFEE_REQUIRE(cache_pages > 0, "attention_bf16_prefill: a cache layer of %d pages", cache_pages);
   if (num_tiles == 0) return 0;
   CacheLayout lay;
@@ -975,7 +1125,25 @@ HFEE_API int hfee_attention_bf16_prefill(void* out, int64_t ld_out, const void* 
   // share them instead, four at a time, where the caller has listed such runs
   const bool by_rows = group == 1 && runs != nullptr && variant != 1 && KV_BLOCKS % SHARED_WAVES == 0 &&
                        layer_bytes < (1ll << 32);
-  if (!by_rows && (variant == 1 || (variant == 0 && group == 1))) {      // nothing to share: one wave per (tile, head)
+  // a row tile's keys in two halves, eight waves a workgroup: four heads (or a multiple) to a KV
+  // head; the caller asks for it where the longest row tile of the step is much longer than the
+  // chip's share of the whole step (it knows the positions)
+  const bool halves_fit = HALVES_FIT && !by_rows && group % SHARED_WAVES == 0 && layer_bytes < (1ll << 32);
+  HFEE_REQUIRE(variant != 3 || halves_fit, "attention_bf16_prefill: the kernel with a row tile's keys in two halves takes "
+               "four heads or a multiple to a KV head, head sizes up to 128 and a layer below 4 GB");
+  if (variant == 3) {
+    constexpr size_t lds = (size_t)2 * HALVES_TILES * KV_BLOCKS * 1024;
+    static bool raised_halves = false;
+    if (!raised_halves) {
+      hipError_t e = hipFuncSetAttribute((const void*)prefill_halves_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      HFEE_REQUIRE(e == hipSuccess, "attention_bf16_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
+      raised_halves = true;
+    }
+    dim3 grid((unsigned)(((int64_t)num_tiles * (group / SHARED_WAVES) * kv_heads + 7) / 8 * 8));
+    prefill_halves_kernel<<<grid, 2 * SHARED_WAVES * 64, lds, stream>>>(
+        (bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, (uint32_t)layer_bytes, lay, work, num_tiles,
+        block_tables, bt_stride, num_heads, scale * LOG2E, window);
+  } else if (!by_rows && (variant == 1 || (variant == 0 && group == 1))) {      // nothing to share: one wave per (tile, head)
     dim3 grid((unsigned)(((int64_t)num_tiles * num_heads + 7) / 8 * 8));
     prefill_kernel<<<grid, 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay,
                                             work, num_tiles, block_tables, bt_stride, num_heads, scale * LOG2E, window);

@@ -51,6 +51,7 @@ _CORE_SIGNATURES = {
 _ATTENTION_SIGNATURES = {
     "hfee_attention_bf16_head_dim": [],
     "hfee_attention_bf16_run_tiles": [],
+    "hfee_attention_bf16_halves": [],
     "hfee_attention_bf16_prefill": [P, L, P, L, P, I, P, I, P, I, P, I, I, I, I, F, I, I, P],
     "hfee_attention_bf16_decode": [P, L, P, L, P, P, P, P, I, P, I, I, I, I, F, I, P, L, I, I, P, I, P],
 }

@@ -437,6 +437,29 @@ def attention_run_tiles(head_dim: int) -> int:
     return int(lib.attention_bf16(head_dim).raw("hfee_attention_bf16_run_tiles")())
 
 
+def attention_halves_fit(head_dim: int, heads_per_kv_head: int) -> bool:
+    """Whether `attention_bf16_prefill(kernel=3)` takes this shape: a row tile's keys in two halves."""
+    return heads_per_kv_head % 4 == 0 and bool(lib.attention_bf16(head_dim).raw("hfee_attention_bf16_halves")())
+
+
+def prefill_attention_kernel(tiles, window: int, kv_heads: int, heads_per_kv_head: int, head_dim: int) -> int:
+    """The `kernel` argument of `attention_bf16_prefill` for a step's row tiles (first row, rows,
+    first position, block-table row), on the host.  A workgroup walks the key tiles of its row tile
+    one after the other, and two workgroups share a CU: where the longest row tile has many more
+    key tiles than a workgroup slot's share of all of them (a prompt read from its start: the last
+    row tile of 2,048 tokens has 64, the share is 32), the kernel that walks a row tile's keys in
+    two halves side by side is as long as half the longest (3); where the row tiles are alike (a
+    portion deep in a long context) two independent workgroups a CU do better (0)."""
+    if not tiles or not attention_halves_fit(head_dim, heads_per_kv_head):
+        return 0
+    steps = []
+    for _, rows, pos, _ in tiles:
+        first = (max(0, pos - window + 1) >> 5) if window > 0 else 0
+        steps.append(((pos + rows - 1) >> 5) + 1 - first)
+    share = sum(steps) * kv_heads * (heads_per_kv_head // 4) / (2 * compute_units())
+    return 3 if max(steps) >= 4 and max(steps) > 1.4 * max(share, 1.0) else 0
+
+
 def attention_runs(tiles, head_dim: int) -> list:
     """The runs of a step's row tiles, on the host: tiles is the list of (first row, rows, first
     position, block-table row) that `attention_bf16_prefill` takes; a run is (first tile, count) of
@@ -459,7 +482,8 @@ def attention_bf16_prefill(out, q, cache_layer, tiles, block_tables, num_heads: 
                            head_dim: int, page_size: int, scale: float, window: int = 0, kernel: int = 0, runs=None):
     """tiles: [num_tiles, 4] int32 (first row, rows <= 32, first position, block-table row).
     kernel: 0 automatic, 1 one wave per (tile, head), 2 the heads of a KV head share its
-    key tiles through LDS.
+    key tiles through LDS, 3 the same with a row tile's keys in two halves that eight waves
+    walk side by side (four heads or a multiple to a KV head, head sizes up to 128).
     runs: [num_runs, 2] int32 (first tile, count <= attention_run_tiles) or None: every tile in
     exactly one run of tiles that follow one another in `tiles` and in one sequence, rows and
     positions going on where the tile before ended (`attention_runs` makes them; a longer run
@@ -523,14 +547,19 @@ FUSED_NORM_MAX_N = 8192
 _cus = None
 
 
+def compute_units() -> int:
+    """CUs of the device (256 on an MI355X)."""
+    global _cus
+    if _cus is None:
+        _cus = torch.cuda.get_device_properties(0).multi_processor_count
+    return _cus
+
+
 def norm_fusion_pays(n_rows: int, k: int) -> bool:
     """Whether folding the norm into a product with n_rows weight rows is cheaper than
     a norm kernel of its own: narrow products, and the wide ones that the persistent
     kernel takes (there the activations are converted once per workgroup)."""
-    global _cus
-    if _cus is None:
-        _cus = torch.cuda.get_device_properties(0).multi_processor_count
-    wide = n_rows > 16 * _cus and k % 1024 == 0 and k <= 4096
+    wide = n_rows > 16 * compute_units() and k % 1024 == 0 and k <= 4096
     return wide or n_rows <= FUSED_NORM_MAX_N
 _EPI = {"bf16": 0, "f32": 1, "add": 2, "swiglu": 3, "qkv": 4}
 

@@ -139,6 +139,8 @@ class Attention(Mixer):
         plan.add("attention.decode_rows", np.asarray(d_rows, dtype=np.int32))
         plan.add("attention.decode_positions", np.asarray(d_pos, dtype=np.int32))
         plan.add("attention.decode_tables", np.asarray(d_tab, dtype=np.int32))
+        plan.host["attention.prefill_kernel"] = ops.prefill_attention_kernel(tiles, self.window, self.kv_heads,
+                                                                             self.num_heads // self.kv_heads, self.head_dim)
         plan.host["attention.decode_max_position"] = max(d_pos) if d_pos else 0
         # (a step of decoding requests only: segment i is row i and has block table i)
         plan.host["attention.decode_in_order"] = d_rows == list(range(len(d_rows))) and d_tab == d_rows
@@ -202,7 +204,8 @@ class Attention(Mixer):
             tiles = ctx.extra["attention.tiles"]
             if tiles.shape[0]:
                 ops.attention_bf16_prefill(att, q, cache, tiles, tables, H, K, hd, ctx.page_size,
-                                           self.scale, self.window, runs=ctx.extra["attention.runs"] if H == K else None)
+                                           self.scale, self.window, runs=ctx.extra["attention.runs"] if H == K else None,
+                                           kernel=ctx.host.get("attention.prefill_kernel", 0))
             rows = ctx.extra["attention.decode_rows"]
             if rows.numel():
                 nseg = rows.numel()

@@ -611,7 +611,9 @@ def _check_attention(H, K, hd, T, window, dtype, ps):
     close(out, ref, tol)
     if dtype == torch.bfloat16:
         tiles = torch.tensor([(o, min(32, T - o), o, 0) for o in range(0, T, 32)], dtype=torch.int32, device=DEV)
-        for kernel in (0, 1, 2):       # the automatic choice, one wave per (tile, head), tiles shared in LDS
+        # the automatic choice, one wave per (tile, head), tiles shared in LDS, and (four heads or a
+        # multiple to a KV head, head sizes up to 128) a row tile's keys in two halves
+        for kernel in (0, 1, 2) + ((3,) if ops.attention_halves_fit(hd, H // K) else ()):
             out2 = torch.zeros(T, H * hd, dtype=dtype, device=DEV)
             ops.attention_bf16_prefill(out2, qd, layer, tiles, table, H, K, hd, ps, scale, window, kernel=kernel)
             close(out2, ref, tol)
@@ -633,6 +635,61 @@ def _check_attention(H, K, hd, T, window, dtype, ps):
                                       table, H, K, hd, ps, scale, window, partial, splits, counters=cnt)
             close(out3[[T - 1, T // 2, 0]], ref[[T - 1, T // 2, 0]], tol)
             assert int(counters.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("H,K,hd,window", [(8, 2, 128, 0), (4, 1, 64, 0), (16, 2, 32, 300), (8, 1, 96, 0)])
+def test_prefill_attention_with_a_row_tiles_keys_in_two_halves(H, K, hd, window):
+    """One launch over portions of several sequences: a prompt of 1,500 tokens from its start (row
+    tiles with 1 to 47 key tiles, odd and even counts, the odd tile with the first half), a
+    portion of 70 rows deep in a context of 900, portions of 33, 2 and 1 rows; against the plain
+    formula for every row, with one key far back scaled up in every sequence so that a half that
+    is skipped, joined with a wrong weight or read from the other ring would show.  The host's
+    choice for these row tiles is this kernel; for the row tiles of a portion deep in a long
+    context, which are all alike, it is the other."""
+    from plain_llama import plain_attention
+    from hfee_amd.kernels import ops
+    ps = 16
+    g = torch.Generator().manual_seed(hd + H)
+    lengths = [1500, 900, 33, 2, 1]            # keys of each sequence
+    portions = [(0, 1500), (830, 70), (0, 33), (0, 2), (0, 1)]      # (first position, rows) that this step runs
+    scale = 1 / math.sqrt(hd)
+    blocks = [(n + ps - 1) // ps for n in lengths]
+    order = torch.randperm(sum(blocks) + 3, generator=g).tolist()
+    layer = torch.full((sum(blocks) + 3, 2, K, ps * hd), 7.0, dtype=torch.bfloat16)
+    table = torch.zeros(len(lengths), max(blocks), dtype=torch.int32)
+    qs, refs, tiles, row = [], [], [], 0
+    for s, (n, (first, rows)) in enumerate(zip(lengths, portions)):
+        q = torch.randn(n, H, hd, generator=g).to(torch.bfloat16)
+        k = (torch.randn(n, K, hd, generator=g) * 0.7).to(torch.bfloat16)
+        v = torch.randn(n, K, hd, generator=g).to(torch.bfloat16)
+        far = n // 3
+        k[far] = (q[first:first + rows].float().mean(0).view(K, H // K, hd).mean(1) * 6).to(torch.bfloat16)
+        pages = order[:blocks[s]]
+        order = order[blocks[s]:]
+        one, _ = _paged((k, v), ps, pages)
+        for p in pages:
+            layer[p] = one[p]
+        table[s, :blocks[s]] = torch.tensor(pages, dtype=torch.int32)
+        refs.append(plain_attention(q, k, v, scale, window=window)[first:first + rows].reshape(rows, H * hd))
+        qs.append(q[first:first + rows].reshape(rows, H * hd))
+        for off in range(0, rows, 32):
+            tiles.append((row + off, min(32, rows - off), first + off, s))
+        row += rows
+    q_all, ref = torch.cat(qs).to(DEV), torch.cat(refs)
+    tiles = torch.tensor(tiles, dtype=torch.int32, device=DEV)
+    outs = {}
+    for kernel in (3, 0, 2):
+        out = torch.full((row, H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.attention_bf16_prefill(out, q_all, layer.to(DEV), tiles, table.to(DEV), H, K, hd, ps, scale, window, kernel=kernel)
+        close(out, ref, 2e-2)
+    assert ops.attention_halves_fit(hd, H // K)
+    assert ops.prefill_attention_kernel(tiles.tolist(), window, K, H // K, hd) == 3
+    deep = [(32 * i, 32, 30000 + 32 * i, 0) for i in range(64)]
+    assert ops.prefill_attention_kernel(deep, 0, 8, 4, hd) == 0
+    assert ops.prefill_attention_kernel([(0, 32, 0, 0)], 0, 8, 4, hd) == 0 and ops.prefill_attention_kernel([], 0, 8, 4, hd) == 0
+    with pytest.raises(Exception, match="two halves"):
+        ops.attention_bf16_prefill(out[:, :K * hd].contiguous(), q_all[:, :K * hd].contiguous(), layer.to(DEV), tiles, table.to(DEV), K, K, hd, ps,
+                                   scale, window, kernel=3)           # (no two heads share keys: not this kernel's case)
 
 
 @pytest.mark.parametrize("B,splits", [(40, 1), (70, 2), (12, 3)])
@@ -895,7 +952,7 @@ def test_attention_over_long_contexts(H, K, hd, ps, ctx):
     ops.attention_plain(ref, q, cache, positions, seg, table, H, K, hd, ps, scale, 0)
     out = torch.zeros_like(ref)
     tiles = torch.tensor([(0, 32, ctx - T, 0), (32, T - 32, ctx - T + 32, 0)], dtype=torch.int32, device=DEV)
-    for kernel in (1, 2):
+    for kernel in (1, 2) + ((3,) if ops.attention_halves_fit(hd, H // K) else ()):
         out.zero_()
         ops.attention_bf16_prefill(out, q, cache, tiles, table, H, K, hd, ps, scale, 0, kernel=kernel)
         assert (out[:T].float() - ref[:T].float()).abs().max() <= 2e-2 * (1 + ref[:T].float().abs().max())
