@@ -104,6 +104,7 @@ class Engine:
         # cost more than the kernels at small batches
         self.use_graphs = use_graphs and model.graph_safe
         self._graphs: dict = {}
+        self._graph_seen: dict = {}        # shape -> how often it has come without a recording
         self.graph_replays = 0
 
     # ------------------------------------------------------------ memory
@@ -202,6 +203,7 @@ class Engine:
             self._meta_capacity = cap
             self._meta_views.clear()
             self._graphs.clear()      # captured graphs point into the old buffer
+            self._graph_seen.clear()
         views = self._meta_views.get(layout)
         if views is None:             # where each array lies, and its view of the device buffer
             if len(self._meta_views) > 256:
@@ -374,10 +376,16 @@ class Engine:
             graph = self._graphs.get(key)
             if graph is None:
                 logits = self._forward(ctx, n, w, dev)          # this step, eagerly; buffers get made
-                captured = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(captured):
-                    self._forward(ctx, n, w, dev)                # recorded, not run
-                self._graphs[key] = captured
+                # A shape is recorded when it comes a second time: recording takes as long as several
+                # steps, and while requests end one after the other every step has a batch size of
+                # its own that never comes again (128 requests at the 1B shape: a third of the run
+                # went into recordings that were replayed once or never).
+                self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
+                if self._graph_seen[key] >= 2:
+                    captured = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(captured):
+                        self._forward(ctx, n, w, dev)            # recorded, not run
+                    self._graphs[key] = captured
             else:
                 graph.replay()
                 self.graph_replays += 1
