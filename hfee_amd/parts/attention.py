@@ -57,6 +57,13 @@ class Attention(Mixer):
             raise ValueError(f"head sizes above 256 are not built, got {self.head_dim}")
         self.prefix, self.dtype = prefix, dtype
         self.position = lookup("position", spec.position.kind)(spec.position) if spec.position else None
+        # an optional step between the projections and the rotation: (kind, params)
+        step = spec.get("after_projection")
+        self.after_projection = None
+        if step is not None:
+            self.after_projection = lookup("projection_step", step[0])(dict(step[1]), prefix, self.num_heads, self.kv_heads,
+                                                                       self.head_dim, dtype)
+            self.second_half_rows = 0      # (the product that would finish a norm's second half is the fused one)
         self.q_width = self.num_heads * self.head_dim
         self.kv_width = self.kv_heads * self.head_dim
         self.w_qkv = self.w_o = None
@@ -67,7 +74,11 @@ class Attention(Mixer):
         return [TensorSpec(p + "q_proj.weight", (self.q_width, self.hidden)),
                 TensorSpec(p + "k_proj.weight", (self.kv_width, self.hidden)),
                 TensorSpec(p + "v_proj.weight", (self.kv_width, self.hidden)),
-                TensorSpec(p + "o_proj.weight", (self.hidden, self.q_width))]
+                TensorSpec(p + "o_proj.weight", (self.hidden, self.q_width))] + \
+            (self.after_projection.tensor_specs() if self.after_projection else [])
+
+    def parts(self):
+        return [self] + (self.after_projection.parts() if self.after_projection else [])
 
     def _pair_order(self, device):
         """Row order inside a head that puts rotation pairs side by side."""
@@ -87,6 +98,8 @@ class Attention(Mixer):
         wk = wk.view(self.kv_heads, self.head_dim, self.hidden)[:, order].reshape(self.kv_width, self.hidden)
         self.w_qkv = torch.cat([wq, wk, tensors.pop(p + "v_proj.weight")], dim=0).contiguous()
         self.w_o = tensors.pop(p + "o_proj.weight").contiguous()
+        if self.after_projection is not None:
+            self.after_projection.bind(tensors, order)
         self.pairing = 1          # pairs are (2i, 2i + 1) from here on
         # a second copy in tiles for steps of up to 64 rows, whose products stream the weights
         # (as rows they serve the tiled products of longer portions)
@@ -158,7 +171,7 @@ class Attention(Mixer):
         # as a kernel of its own, spread over the whole chip, measured faster than as the
         # tail of 256 x 256 tiles with one wave a SIMD: 135 us against 156 us a layer at
         # 2,048 rows)
-        fused = self.streams and n <= ops.SKINNY_MAX_ROWS
+        fused = self.streams and n <= ops.SKINNY_MAX_ROWS and self.after_projection is None
         qkv = ctx.rows("attention.qkv", self.q_width + 2 * self.kv_width)
         q = qkv[:, :self.q_width]
         if fused:
@@ -178,7 +191,7 @@ class Attention(Mixer):
             hn = h.tensor() if isinstance(h, LazyNorm) else h
             portions = self.dtype != torch.bfloat16 or ctx.extra["attention.tiles"].shape[0] > 0
             cuts = 0
-            if writes_cache and self.cuts_into_rotation:
+            if writes_cache and self.cuts_into_rotation and self.after_projection is None:
                 # a product of few tiles, cut along K: the rotation adds the cuts up on its way
                 scratch = ctx.workspace.split_scratch(n, self.w_qkv).get("scratch")
                 cuts = ops.linear_cuts(hn, self.w_qkv, scratch)
@@ -193,6 +206,8 @@ class Attention(Mixer):
                 else:   # this run of the layer reads keys and values that another run wrote
                     ops.linear(q, hn, self.w_qkv[:self.q_width])
                     k = v = None
+                if self.after_projection is not None:
+                    self.after_projection.forward(ctx, q, k, v)
                 ops.rope_cache_write(q, k, v, ctx.positions, ctx.token_segment, tables, cos, sin, self.pairing,
                                      cache if writes_cache else None, H, K, hd, ctx.page_size, ctx.max_position,
                                      portions=portions)

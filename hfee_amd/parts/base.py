@@ -2,7 +2,7 @@
 and what a step hands it.
 
 A part gets all its sizes and constants through its spec; it never learns which
-model it is in.  Seven kinds, each with a registry from the spec's `kind` string to
+model it is in.  Eight kinds, each with a registry from the spec's `kind` string to
 a class:
 
   embedding       forward(ctx, x): the residual stream's first value from the token ids
@@ -10,6 +10,9 @@ a class:
   norm            forward(ctx, out, x, rows=None)
   position        prepare(num_positions, device); applied by the mixer that owns it
   mixer           forward_add(ctx, x, h, cache_layer, writes_cache): x += mix(h)
+  projection_step forward(ctx, q, k, v): what a mixer does to its projections before it applies
+                  the position (a bias, a norm over each head); named by the attention
+                  mixer's `after_projection` parameter, see ProjectionStep
   feed_forward    forward_add(ctx, x, h):                            x += ffn(h)
   block           forward(ctx, x, entry): one layer's arrangement of the above
   head            forward(ctx, logits, x, rows): logits of the wanted rows
@@ -32,7 +35,7 @@ import torch
 
 
 _REGISTRIES: dict[str, dict] = {"norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {},
-                                "embedding": {}, "head": {}}
+                                "embedding": {}, "head": {}, "projection_step": {}}
 
 
 def _register(family: str, kind: str, cls):
@@ -62,6 +65,10 @@ def register_block(kind: str, cls=None):
 
 def register_embedding(kind: str, cls=None):
     return _register("embedding", kind, cls) if cls else (lambda c: _register("embedding", kind, c))
+
+
+def register_projection_step(kind: str, cls=None):
+    return _register("projection_step", kind, cls) if cls else (lambda c: _register("projection_step", kind, c))
 
 
 def register_head(kind: str, cls=None):
@@ -128,6 +135,25 @@ class Mixer(Part):
     """Mixes information between the tokens of a sequence."""
 
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool) -> None:
+        raise NotImplementedError
+
+
+class ProjectionStep(Part):
+    """What stands between a mixer's projections and the position encoding: a bias on q, k
+    and v, a norm over each head of q and k, anything that works row by row.  The attention
+    mixer builds one from its `after_projection` parameter, a (kind, params) pair, with the
+    constructor (params, prefix, num_heads, kv_heads, head_dim, dtype); a mixer that has one
+    runs its projections, this step and the rotation as launches of their own (the fused
+    epilogues know nothing of it)."""
+
+    def bind(self, tensors: dict, order=None) -> None:
+        """order: the attention mixer keeps the rows of a q or k head in an order of its own
+        (rotation pairs side by side); element j of a head as this step sees it is element
+        order[j] of the head in the checkpoint.  Per-dimension tensors of q and k must follow."""
+
+    def forward(self, ctx, q, k, v) -> None:
+        """In place: q [n, num_heads * head_dim], k and v [n, kv_heads * head_dim] (None where
+        this run of the layer reads another run's cache), in the engine's dtype."""
         raise NotImplementedError
 
 

@@ -422,6 +422,118 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path):
     assert torch.allclose(got, want, atol=2e-4, rtol=2e-4), float((got - want).abs().max())
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_step_between_the_projections_and_the_rotation(tmp_path, dtype):
+    """A bias on q, k and v and a norm over each head of q and k with a weight per dimension,
+    between the projections and the rotation: defined and registered here as a
+    `projection_step`, named by the attention mixer's `after_projection` parameter in a toy
+    architecture, stepped in portions and token by token (the mixer then runs projections,
+    this step and the rotation as launches of their own) and compared with a plain computation.
+    The rows of a q or k head lie in the mixer's own order; the step's tensors follow it."""
+    import hfee_amd  # noqa: F401
+    from hfee_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
+                                 ScheduleEntry, params, register_architecture)
+    from hfee_amd.config.base import KeyReader
+    from hfee_amd.engine import Engine, StepEntry, load_model
+    from hfee_amd.parts import ProjectionStep, register_projection_step
+    from hfee_amd.weights import Checkpoint, TensorSpec, write_model_folder
+    from plain_llama import plain_attention, plain_rmsnorm, plain_rope, plain_rope_frequencies, plain_swiglu
+
+    @register_projection_step("toy_bias_and_head_norm")
+    class BiasAndHeadNorm(ProjectionStep):
+        def __init__(self, options, prefix, num_heads, kv_heads, head_dim, dtype):
+            self.prefix, self.H, self.K, self.hd, self.eps = prefix, num_heads, kv_heads, head_dim, options["eps"]
+
+        def tensor_specs(self):
+            p = self.prefix
+            return [TensorSpec(p + "q_proj.bias", (self.H * self.hd,), role="vector", init=("normal",)),
+                    TensorSpec(p + "k_proj.bias", (self.K * self.hd,), role="vector", init=("normal",)),
+                    TensorSpec(p + "v_proj.bias", (self.K * self.hd,), role="vector", init=("normal",)),
+                    TensorSpec(p + "q_norm.weight", (self.hd,), role="vector", init=("one_plus_normal",)),
+                    TensorSpec(p + "k_norm.weight", (self.hd,), role="vector", init=("one_plus_normal",))]
+
+        def bind(self, tensors, order=None):
+            p = self.prefix
+            self.bq = tensors.pop(p + "q_proj.bias").float().view(self.H, self.hd)[:, order].reshape(-1)
+            self.bk = tensors.pop(p + "k_proj.bias").float().view(self.K, self.hd)[:, order].reshape(-1)
+            self.bv = tensors.pop(p + "v_proj.bias").float()
+            self.wq = tensors.pop(p + "q_norm.weight").float()[order]
+            self.wk = tensors.pop(p + "k_norm.weight").float()[order]
+
+        def forward(self, ctx, q, k, v):
+            def head_norm(t, bias, w, heads):
+                y = (t.float() + bias).view(t.shape[0], heads, self.hd)
+                y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + self.eps) * w
+                t.copy_(y.view(t.shape[0], -1))
+            head_norm(q, self.bq, self.wq, self.H)
+            if k is not None:
+                head_norm(k, self.bk, self.wk, self.K)
+                v.copy_(v.float() + self.bv)
+
+    @dataclass(frozen=True)
+    class StepConfig:
+        architecture: str
+        hidden: int
+        vocab: int
+
+        @staticmethod
+        def from_dict(d, where="config.json"):
+            r = KeyReader(d, where)
+            c = StepConfig("ToyStepForCausalLM", r.int("s_hidden"), r.int("s_vocab"))
+            r.finish()
+            return c
+
+        def to_dict(self):
+            return {"architectures": ["ToyStepForCausalLM"], "s_hidden": self.hidden, "s_vocab": self.vocab}
+
+    H, KV, HD, F, EPS = 4, 2, 32, 56, 1e-5
+
+    def spec_of(c):
+        norm = NormSpec("rmsnorm", c.hidden, EPS)
+        ffn = FeedForwardSpec("gated_mlp", params(hidden=c.hidden, intermediate=F))
+        att = MixerSpec("attention", params(hidden=c.hidden, num_heads=H, num_kv_heads=KV, head_dim=HD, window=0,
+                                            after_projection=("toy_bias_and_head_norm", params(eps=1e-3))),
+                        position=PositionSpec("rope", params(head_dim=HD, theta=10000.0, rotary_dim=HD, pairing="half", scaling=None)))
+        layers = tuple(LayerSpec("prenorm", c.hidden, att, ffn, norm, norm, f"s.{i}.") for i in range(2))
+        return ModelSpec("ToyStepForCausalLM", c.hidden, c.vocab, layers, tuple(ScheduleEntry(i, i) for i in range(2)),
+                         norm, "s.embed.weight", "s.norm.weight", None, max_positions=128)
+
+    register_architecture("ToyStepForCausalLM", StepConfig, spec_of)
+    cfg = StepConfig("ToyStepForCausalLM", 48, 90)
+    folder = write_model_folder(str(tmp_path / "m"), cfg, seed=6, std=0.15,
+                                dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype])
+    model, _ = load_model(folder, dtype)
+    assert model.blocks[0].mixer.after_projection is not None and model.blocks[0].mixer.second_half_rows == 0
+    eng = Engine(model, num_pages=8, page_size=16, max_requests=2, max_batch_tokens=64)
+    toks = tu.make_requests(90, [50], seed=4)["r0"]
+    eng.admit("a")
+    got, i = [], 0
+    for n in [33, 1, 1, 9, 2, 1, 1, 1, 1]:
+        got.append(eng.step([StepEntry("a", toks[i:i + n], list(range(n)))]).double().cpu())
+        i += n
+    got = torch.cat(got)
+
+    ck = Checkpoint(folder)
+    t = {n: ck.tensor(n).double() for n in ck.names()}
+    x = t["s.embed.weight"][toks]
+    T, pos, inv = len(toks), list(range(len(toks))), plain_rope_frequencies(HD, 10000.0)
+    for l in range(2):
+        p = f"s.{l}."
+        h = plain_rmsnorm(x, t[p + "mixer_norm.weight"], EPS)
+        q = (h @ t[p + "mixer.q_proj.weight"].t() + t[p + "mixer.q_proj.bias"]).view(T, H, HD)
+        k = (h @ t[p + "mixer.k_proj.weight"].t() + t[p + "mixer.k_proj.bias"]).view(T, KV, HD)
+        v = (h @ t[p + "mixer.v_proj.weight"].t() + t[p + "mixer.v_proj.bias"]).view(T, KV, HD)
+        q = plain_rope(plain_rmsnorm(q, t[p + "mixer.q_norm.weight"], 1e-3), pos, inv)
+        k = plain_rope(plain_rmsnorm(k, t[p + "mixer.k_norm.weight"], 1e-3), pos, inv)
+        x = x + plain_attention(q, k, v).reshape(T, H * HD) @ t[p + "mixer.o_proj.weight"].t()
+        h = plain_rmsnorm(x, t[p + "feed_forward_norm.weight"], EPS)
+        x = x + plain_swiglu(h @ t[p + "feed_forward.gate_proj.weight"].t(), h @ t[p + "feed_forward.up_proj.weight"].t()) \
+            @ t[p + "feed_forward.down_proj.weight"].t()
+    want = plain_rmsnorm(x, t["s.norm.weight"], EPS) @ t["s.embed.weight"].t()
+    assert rel(got, want) < (3e-5 if dtype == "float32" else 5e-2), rel(got, want)
+    assert float(t["s.0.mixer.q_proj.bias"].abs().max()) > 0.1          # (the step has something to add)
+
+
 # -------------------------------------------------------------- the sampler ---
 
 @pytest.mark.parametrize("V", [1000, 1001, 8201])      # (from 8,192 ids on a row is cut into slices first)
