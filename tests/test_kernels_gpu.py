@@ -692,6 +692,67 @@ def test_prefill_attention_with_a_row_tiles_keys_in_two_halves(H, K, hd, window)
                                    scale, window, kernel=3)           # (no two heads share keys: not this kernel's case)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_prefill_attention_kernels_on_drawn_steps(seed):
+    """Steps drawn at random: head sizes, heads to a KV head, page sizes, windows, and a mix of
+    portions (some from a sequence's start, some deep in a context, some of a few rows) over
+    pages in scrambled order with stale contents elsewhere.  Every matrix-core prefill kernel
+    that takes the shape (the choice of the host among them) against the plain kernel, which is
+    checked against the formula at small sizes."""
+    import random
+    from hfee_amd.kernels import ops
+    rng = random.Random(900 + seed)
+    hd = rng.choice([16, 32, 64, 64, 96, 128, 128, 48, 160])
+    K = rng.choice([1, 2, 3])
+    group = rng.choice([4, 4, 8, 1, 2, 12])
+    H = K * group
+    ps = rng.choice([16, 16, 32, 64])
+    window = rng.choice([0, 0, 0, 40, 257])
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    portions = []          # (keys before the portion, rows)
+    for _ in range(rng.randint(1, 5)):
+        kind = rng.random()
+        before = 0 if kind < 0.4 else rng.randint(1, 3000)
+        rows = rng.choice([1, 2, 31, 32, 33, rng.randint(2, 700)])
+        portions.append((before, rows))
+    blocks = [(b + r + ps - 1) // ps for b, r in portions]
+    total_pages = sum(blocks) + 4
+    cache = (torch.randn(total_pages, 2, K, ps * hd, generator=g, device=DEV) * 0.6).to(torch.bfloat16)
+    order = torch.randperm(total_pages, generator=g, device=DEV).to(torch.int32)
+    table = torch.zeros(len(portions), max(blocks), dtype=torch.int32, device=DEV)
+    tiles, positions, seg, at = [], [], [], 0
+    row = 0
+    for s, ((before, rows), nb) in enumerate(zip(portions, blocks)):
+        table[s, :nb] = order[at:at + nb]
+        at += nb
+        for off in range(0, rows, 32):
+            tiles.append((row + off, min(32, rows - off), before + off, s))
+        positions += list(range(before, before + rows))
+        seg += [s] * rows
+        row += rows
+    q = (torch.randn(row, H * hd, generator=g, device=DEV) * 0.8).to(torch.bfloat16)
+    positions = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    seg = torch.tensor(seg, dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(hd)
+    ref = torch.zeros(row, H * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention_plain(ref, q, cache, positions, seg, table, H, K, hd, ps, scale, window)
+    dev_tiles = torch.tensor(tiles, dtype=torch.int32, device=DEV)
+    choice = ops.prefill_attention_kernel(tiles, window, K, group, hd)
+    kernels = [1, 2] + ([3] if ops.attention_halves_fit(hd, group) else [])
+    assert choice in (0, 3) and (choice == 0 or 3 in kernels)
+    what = dict(hd=hd, K=K, group=group, ps=ps, window=window, portions=portions)
+    for kernel in kernels:
+        out = torch.full((row, H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.attention_bf16_prefill(out, q, cache, dev_tiles, table, H, K, hd, ps, scale, window, kernel=kernel)
+        worst = float((out.float() - ref.float()).abs().max())
+        assert worst <= 2e-2 * (1 + float(ref.float().abs().max())), (kernel, worst, what)
+    if group == 1:
+        runs = torch.tensor(ops.attention_runs(tiles, hd), dtype=torch.int32, device=DEV)
+        out = torch.full((row, H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.attention_bf16_prefill(out, q, cache, dev_tiles, table, H, K, hd, ps, scale, window, runs=runs)
+        assert float((out.float() - ref.float()).abs().max()) <= 2e-2 * (1 + float(ref.float().abs().max())), what
+
+
 @pytest.mark.parametrize("B,splits", [(40, 1), (70, 2), (12, 3)])
 def test_decode_attention_with_more_workgroups_than_cus(B, splits):
     """With more (segment, KV head, split) workgroups than the chip has CUs the decode kernel
