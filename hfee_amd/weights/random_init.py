@@ -19,8 +19,6 @@ from . import random_stream
 from .safetensors_io import write_safetensors
 from .spec import TensorSpec
 
-_tensor_seed = random_stream.tensor_key
-
 
 def random_tensor(spec: TensorSpec, seed: int, std: float, dtype: torch.dtype,
                   device="cpu") -> torch.Tensor:
