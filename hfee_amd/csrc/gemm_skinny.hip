@@ -797,7 +797,7 @@ constexpr int WIDE_MIN_GROUPS_A_CU = 6;       // of eight: below, the kernels ab
 constexpr size_t mid_wide_lds_bytes(int mt) { return (size_t)2 * mt * 16 * WIDE_PITCH * sizeof(bf16_t); }
 
 template <int MT, int EPI>
-__global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_groups) {
+__global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_groups, int busy) {
   extern __shared__ __attribute__((aligned(16))) char wide_lds[];
   bf16_t* xs = (bf16_t*)wide_lds;                                    // [2][MT * 16][WIDE_PITCH]
   __shared__ float row_scale[SS_STRIDE];
@@ -828,13 +828,19 @@ __global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_gr
   // the batch first (from L2: it must not wait in line behind weights from memory), then the ring
   u32x4 fill[FILL];
   ask(fill, 0);
-  const int stride = gridDim.x * WAVES;
-  const bf16_t* w_cur = row_ptr(blockIdx.x * WAVES + wave);
+  // `busy` waves of a workgroup take a row group each in every round; the others only help to bring
+  // the batch (1,792 row groups over 256 CUs are seven a workgroup: with eight, 224 workgroups would
+  // leave 32 CUs without work)
+  const int stride = gridDim.x * busy;
+  const bool works = wave < busy;
+  const bf16_t* w_cur = row_ptr(blockIdx.x * busy + wave);
   constexpr int RING = mid_ring(MT);          // (8 or 16 loads a wave in flight at 64 rows: the step within 1 %)
   static_assert(WIDE_STEPS % RING == 0, "a ring slot must mean the same step in every slice");
   Chunk ring[RING];
+  if (works) {
 #pragma unroll
-  for (int st = 0; st < RING; ++st) ring[st].u = load_streamed(reinterpret_cast<const u32x4*>(w_cur + st * WeightTiles::TILE));
+    for (int st = 0; st < RING; ++st) ring[st].u = load_streamed(reinterpret_cast<const u32x4*>(w_cur + st * WeightTiles::TILE));
+  }
   put(fill, 0);
   // (the rows' shares meet at the first slice's barrier: see ask_shares; with one slice there is none)
   __shared__ float share_part[WAVES][SS_STRIDE];
@@ -845,8 +851,8 @@ __global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_gr
   __syncthreads();
 
   int buf = 0;
-  for (int first = blockIdx.x * WAVES; first < row_groups; first += stride) {      // (the same for all waves: barriers inside)
-    const int rg = first + wave;
+  for (int first = blockIdx.x * busy; first < row_groups; first += stride) {      // (the same for all waves: barriers inside)
+    const int rg = works ? first + wave : row_groups;
     const bf16_t* w_next = row_ptr(rg + stride);                     // past the end: a repeat that nobody uses
     f32x4 acc[MT];
 #pragma unroll
@@ -854,25 +860,27 @@ __global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_gr
     for (int s = 0; s < slices; ++s) {
       ask(fill, s + 1 < slices ? s + 1 : 0);
       const bf16_t* x_lane = xs + (buf * MT * 16 + r16) * WIDE_PITCH + g * 8;
+      if (works) {                 // (the same for the whole wave)
 #pragma unroll
-      for (int st = 0; st < WIDE_STEPS; ++st) {
+        for (int st = 0; st < WIDE_STEPS; ++st) {
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          const bf16x8 b = *reinterpret_cast<const bf16x8*>(x_lane + t * 16 * WIDE_PITCH + st * 32);
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st % RING].v, b, acc[t], 0, 0, 0);
+          for (int t = 0; t < MT; ++t) {
+            const bf16x8 b = *reinterpret_cast<const bf16x8*>(x_lane + t * 16 * WIDE_PITCH + st * 32);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[st % RING].v, b, acc[t], 0, 0, 0);
+          }
+          const int ahead = s * WIDE_STEPS + st + RING;
+          const bf16_t* src = ahead < tiles ? w_cur + (int64_t)ahead * WeightTiles::TILE : w_next + (int64_t)(ahead - tiles) * WeightTiles::TILE;
+          ring[st % RING].u = load_streamed(reinterpret_cast<const u32x4*>(src));
         }
-        const int ahead = s * WIDE_STEPS + st + RING;
-        const bf16_t* src = ahead < tiles ? w_cur + (int64_t)ahead * WeightTiles::TILE : w_next + (int64_t)(ahead - tiles) * WeightTiles::TILE;
-        ring[st % RING].u = load_streamed(reinterpret_cast<const u32x4*>(src));
-      }
-      // (the order of issue as in the kernel above: LDS reads of a step under the products of the
-      // step before, a ring slot refilled as soon as its step has been multiplied)
-      __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+        // (the order of issue as in the kernel above: LDS reads of a step under the products of the
+        // step before, a ring slot refilled as soon as its step has been multiplied)
+        __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
 #pragma unroll
-      for (int st = 0; st < WIDE_STEPS; ++st) {
-        if (st + 1 < WIDE_STEPS) __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        for (int st = 0; st < WIDE_STEPS; ++st) {
+          if (st + 1 < WIDE_STEPS) __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, MT, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
       }
       put(fill, buf ^ 1);          // read last in the slice before this one: everybody has passed that barrier
       if (late && s == 0) put_shares<MT>(a, shares, share_part);
@@ -905,9 +913,13 @@ __global__ __launch_bounds__(WAVES * 64) void mid_wide_kernel(Args a, int row_gr
 // Returns true if the kernel for 17 to 64 rows and many weight rows took the product.
 template <int MT>
 bool launch_mid_wide(const Args& a, int epi, int num_cus, hipStream_t stream) {
-  const int row_groups = (a.N + ROWS - 1) / ROWS, groups = (row_groups + WAVES - 1) / WAVES;
-  const int per = (groups + num_cus - 1) / num_cus;                  // rounds of a workgroup, all but equal
-  const int grid = (groups + per - 1) / per;
+  const int row_groups = (a.N + ROWS - 1) / ROWS;
+  const int per = (row_groups + num_cus * WAVES - 1) / (num_cus * WAVES);      // rounds of a workgroup, all but equal
+  // (gate/up of the 8B shape: seven waves on 256 CUs instead of eight on 224: a decode step at batch 64
+  // 5.73 -> 5.61 ms, at 32 4.68 -> 4.60, at 24 4.38 -> 4.30, the two libraries in turn on one box)
+  int busy = (row_groups + num_cus * per - 1) / (num_cus * per);                // waves of a workgroup with a row group a round
+  if (busy > WAVES) busy = WAVES;
+  const int grid = (row_groups + busy * per - 1) / (busy * per);
   const size_t lds = mid_wide_lds_bytes(MT);
 #define GO(E)                                                                                                  \
   do {                                                                                                         \
@@ -918,7 +930,7 @@ bool launch_mid_wide(const Args& a, int epi, int num_cus, hipStream_t stream) {
         return false;                                                                                          \
       raised = true;                                                                                           \
     }                                                                                                          \
-    mid_wide_kernel<MT, E><<<grid, WAVES * 64, lds, stream>>>(a, row_groups);                                  \
+    mid_wide_kernel<MT, E><<<grid, WAVES * 64, lds, stream>>>(a, row_groups, busy);                            \
   } while (0)
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
