@@ -792,7 +792,11 @@ bool launch_mid_rows(const Args& a, int epi, float* scratch, int64_t scratch_flo
 // above, through a ring of loads that runs on across slices and row groups.
 constexpr int WIDE_KS = 512, WIDE_STEPS = WIDE_KS / 32, WIDE_PITCH = WIDE_KS + 8;
 
-constexpr int WIDE_MIN_GROUPS_A_CU = 6;       // of eight: below, the kernels above with their slices of K spread better
+constexpr int WIDE_MIN_GROUPS_A_CU = 6;
+// (up to 48 rows from four on: gate/up of the 1B shape, 1,024 row groups on 256 workgroups of four busy
+// waves, a decode step at batch 20 / 24 / 32 / 40 / 48 1.181 / 1.210 / 1.288 / 1.329 / 1.405 -> 1.139 / 1.166 /
+// 1.240 / 1.326 / 1.399 ms; at 64 rows the pair of kernels stays, 1.591 against 1.616)
+constexpr int WIDE_MIN_GROUPS_A_CU_FEW_ROWS = 4;       // of eight: below, the kernels above with their slices of K spread better
 
 constexpr size_t mid_wide_lds_bytes(int mt) { return (size_t)2 * mt * 16 * WIDE_PITCH * sizeof(bf16_t); }
 
@@ -1223,7 +1227,8 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
                prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
   }
   // weight rows enough for most of the CUs to have eight row groups each: nothing is cut along K
-  const bool wide_rows = (N + ROWS - 1) / ROWS >= WIDE_MIN_GROUPS_A_CU * num_cus;
+  const bool wide_rows = (N + ROWS - 1) / ROWS >= WIDE_MIN_GROUPS_A_CU * num_cus ||
+                         ((N + ROWS - 1) / ROWS >= WIDE_MIN_GROUPS_A_CU_FEW_ROWS * num_cus && mt <= 3);
   if (!norm && mt > 1 && K % WIDE_KS == 0 && (force_mid == 2 || (force_mid == 0 && wide_rows))) {
     const bool took = mt == 2 ? launch_mid_wide<2>(a, epi, num_cus, stream)
                     : mt == 3 ? launch_mid_wide<3>(a, epi, num_cus, stream)
