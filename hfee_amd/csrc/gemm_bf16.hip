@@ -17,7 +17,6 @@
 #include "qkv_epilogue.h"
 #include "gemm_entry.h"
 
-#include <type_traits>
 
 using namespace hfee;
 
@@ -760,22 +759,6 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
   return 0;
 }
 
-// Tells the scheduler to issue N matrix instructions with R instructions of another
-// group (0x100 LDS read, 0x200 LDS write, 0x020 global load) spread evenly between them.
-template <int OTHER, int N, int R, int G = 0>
-struct Interleave {
-  static __device__ __forceinline__ void emit() {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    constexpr int c = (R * (G + 1)) / N - (R * G) / N;
-    if constexpr (c > 0) __builtin_amdgcn_sched_group_barrier(OTHER, c, 0);
-    Interleave<OTHER, N, R, G + 1>::emit();
-  }
-};
-template <int OTHER, int N, int R>
-struct Interleave<OTHER, N, R, N> {
-  static __device__ __forceinline__ void emit() {}
-};
-
 // ------------------------------------ tiled, one wave a SIMD, loads into the LDS ---
 // Products with enough tiles of 256 rows to fill the chip.  A 128 x 128 tile at the
 // full matrix rate asks the L1 for 64 bytes a clock, which is all a CU has, and the LDS
@@ -796,8 +779,16 @@ struct Interleave<OTHER, N, R, N> {
 //  * The one barrier of a step stands where the wave has nothing outstanding in the LDS,
 //    and carries no fence (a fence would wait for every load in flight); what must have
 //    landed is waited for by count.
-//  * The order of issue is spelled out with scheduling groups: what does not stand
-//    between two matrix instructions is not overlapped with them.
+//  * The order of issue is written out and pinned, every matrix instruction and what follows
+//    it between two scheduling barriers: what does not stand between two matrix
+//    instructions is not overlapped with them, and a burst of requests from four waves in
+//    step queues at the CU's one address unit while the matrix pipes run dry.
+//  * The kernel is bound by power, not by its schedule: by the cycle counter and the
+//    constant-rate counter read around the loop (K = 8,192, all CUs busy), a loop of the
+//    matrix instructions alone takes 32.7 cycles an instruction at 1.82 GHz; with the LDS
+//    reads and the barrier 36.7 at 1.68; with the requests too, all to one address, 37.3 at
+//    1.47; the whole loop 36.0 at 1.39 (38.9 at 1.42 while the requests of a step stood
+//    together under a quarter of its matrix instructions).
 //  * The products are formed transposed (weights as the row operand): a lane then holds
 //    four consecutive columns of one row of C and stores them with one instruction.
 // K must be a multiple of 32 and every row's byte offset must fit 31 bits.
@@ -857,16 +848,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
       __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)(((int64_t)(M - 1) * lda + K) * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t w_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)(((int64_t)(N - 1) * ldw + K) * 2), 0x00020000);
-  auto load_step = [&](int kt) {
-    const int buf = kt & 3;
+  auto load_one = [&](int kt, int p) {            // request p of K step kt: CA of A, then CW of W
     const int koff = min(kt, ktiles - 1) * DROW;          // past the end: a repeat that nobody uses
-    char* dst = lds_bytes + buf * BUF + wave * 1024;
+    char* dst = lds_bytes + (kt & 3) * BUF + wave * 1024;
+    if (p < CA) __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(dst + p * 4096), 16, a_off[p], koff, 0, 0);
+    else __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)(dst + BM * DROW + (p - CA) * 4096), 16, w_off[p - CA], koff, 0, 0);
+  };
+  auto load_step = [&](int kt) {
 #pragma unroll
-    for (int p = 0; p < CA; ++p)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(dst + p * 4096), 16, a_off[p], koff, 0, 0);
-#pragma unroll
-    for (int p = 0; p < CW; ++p)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)(dst + BM * DROW + p * 4096), 16, w_off[p], koff, 0, 0);
+    for (int p = 0; p < CA + CW; ++p) load_one(kt, p);
   };
 
   f32x16 acc[TM][TN];
@@ -891,16 +881,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
 #pragma unroll
     for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * DROW);
   };
-  auto multiply = [&](const bf16x8* af, const bf16x8* bf, int from, int to) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        if (i * TN + j >= from && i * TN + j < to)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);   // transposed
-  };
 
-  constexpr int RD = TM + TN, MF = TM * TN, LD = CA + CW, HALF = MF / 2;
+  constexpr int RD = TM + TN, MF = TM * TN, LD = CA + CW;
   load_step(0);
   load_step(1);
   load_step(2);
@@ -908,26 +890,45 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
   barrier_no_fence();
   read_operands(0, 0, a[0], b[0]);
 
-  // One step: columns 0..15 with the reads of columns 16..31 under them; the first half
-  // of columns 16..31 with the requests for K step kt + 3 (its buffer was last read in
-  // step kt - 1, before that step's barrier); then the barrier, and the second half with
-  // the first reads of the next step.  At the barrier this wave's part of K step kt + 1
-  // (asked for two steps ago) has landed: at most the loads of two steps are outstanding.
-  // After the barrier everybody's has, and nobody reads this step's buffer any more.
-  // No fence: it would wait for every load in flight.
+  // One step in two stretches of MF matrix instructions with the barrier between them: columns
+  // 0..15 with the reads of columns 16..31 under the first matrix instructions of the stretch, so
+  // that the last read is READ_SPAN matrix instructions old when its value is needed; then the
+  // barrier; then columns 16..31 with the first reads of the next step.  The requests for K step
+  // kt + 3 (its buffer was last read in step kt - 1, before that step's barrier) are spread over
+  // the whole step, one for every 32 / LD matrix instructions: a request of a kilobyte keeps the
+  // CU's one address unit busy for 16 cycles, and the four waves ask at the same time.  At the
+  // barrier this wave's part of K step kt + 1 (asked for two steps ago) has landed when at most
+  // the loads of step kt + 2 and the first CA of this step are outstanding; after it everybody's
+  // has, and nobody reads this step's buffer any more.  No fence: it would wait for every load.
+  constexpr int READ_SPAN = MF / 2;
+  // (the order is written out and pinned: every matrix instruction with what follows it stands
+  // between two scheduling barriers)
+  auto read_one = [&](int buf, int ks, bf16x8* af, bf16x8* bf, int r) {      // in the order in which the products need them
+    const char* tile = lds_bytes + buf * BUF + rd[ks];
+    const int j = r - 1, i = r - TN;
+    if (r == 0) af[0] = *reinterpret_cast<const bf16x8*>(tile + a_rd);
+    else if (r <= TN) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * DROW);
+    else af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 32 * DROW);
+  };
+  auto stretch = [&](const bf16x8* af, const bf16x8* bf, int rbuf, int rks, bf16x8* raf, bf16x8* rbf, int kt_load, int l0, int l1) {
+#pragma unroll
+    for (int g = 0; g < MF; ++g) {
+      const int i = g / TN, j = g % TN;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);   // transposed
+      if (g < READ_SPAN) {
+#pragma unroll
+        for (int r = (RD * g) / READ_SPAN; r < (RD * (g + 1)) / READ_SPAN; ++r) read_one(rbuf, rks, raf, rbf, r);
+      }
+#pragma unroll
+      for (int l = l0 + ((l1 - l0) * g) / MF; l < l0 + ((l1 - l0) * (g + 1)) / MF; ++l) load_one(kt_load, l);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
   for (int kt = 0; kt < ktiles; ++kt) {
-    const int buf = kt & 3;
-    read_operands(buf, 1, a[1], b[1]);
-    multiply(a[0], b[0], 0, MF);
-    Interleave<0x100, MF, RD>::emit();
-    multiply(a[1], b[1], 0, HALF);
-    load_step(kt + 3);
-    Interleave<0x020, HALF, LD>::emit();
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * LD) : "memory");
+    stretch(a[0], b[0], kt & 3, 1, a[1], b[1], kt + 3, 0, CA);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LD + CA) : "memory");
     barrier_no_fence();
-    read_operands((kt + 1) & 3, 0, a[0], b[0]);
-    multiply(a[1], b[1], HALF, MF);
-    Interleave<0x100, MF - HALF, RD>::emit();
+    stretch(a[1], b[1], (kt + 1) & 3, 0, a[0], b[0], kt + 3, CA, LD);
   }
   // the repeats asked for past the end still write into this workgroup's LDS: let them
   // land before the wave can end and the LDS go to another workgroup
@@ -1033,15 +1034,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
       __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)(((int64_t)(M - 1) * lda + K) * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t w_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)(((int64_t)(N - 1) * ldw + K) * 2), 0x00020000);
-  auto load_step = [&](int kt, int buf) {
-    const int koff = min(kt, ktiles - 1) * EROW;
+  auto load_one = [&](int kt, int buf, int p) {     // request p of K step kt: CA of A, then CW of W
+    const int koff = min(kt, ktiles - 1) * EROW;         // past the end: a repeat that nobody uses
     char* dst = lds_bytes + buf * BUF + wave * 1024;
+    if (p < CA) __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(dst + p * 4096), 16, a_off[p], koff, 0, 0);
+    else __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)(dst + BM * EROW + (p - CA) * 4096), 16, w_off[p - CA], koff, 0, 0);
+  };
+  auto load_step = [&](int kt, int buf) {
 #pragma unroll
-    for (int p = 0; p < CA; ++p)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(dst + p * 4096), 16, a_off[p], koff, 0, 0);
-#pragma unroll
-    for (int p = 0; p < CW; ++p)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)(dst + BM * EROW + p * 4096), 16, w_off[p], koff, 0, 0);
+    for (int p = 0; p < CA + CW; ++p) load_one(kt, buf, p);
   };
 
   f32x16 acc[TM][TN];
@@ -1065,51 +1066,55 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
 #pragma unroll
     for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * EROW);
   };
-  auto multiply = [&](const bf16x8* af, const bf16x8* bf, int from, int to) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        if (i * TN + j >= from && i * TN + j < to)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);   // transposed
-  };
 
-  constexpr int RD = TM + TN, MF = TM * TN, LD = CA + CW, HALF = MF / 2;
+  constexpr int RD = TM + TN, MF = TM * TN, LD = CA + CW;
 #pragma unroll
   for (int s = 0; s < NBUF - 1; ++s) load_step(s, s);
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 2) * LD) : "memory");     // K step 0 has landed
   barrier_no_fence();
   read_operands(0, 0, a[0], b[0]);
 
-  // One step of 64 columns in four quarters.  The requests for K step kt + NBUF - 1 go out
-  // under the first quarter (its buffer was last read in step kt - 1, before that step's
-  // barrier).  The barrier stands in the middle of the last quarter: this wave's part of
-  // K step kt + 1 has landed when at most the loads of NBUF - 2 steps are outstanding;
-  // after it everybody's has, and nobody reads this step's buffer any more.
+  // One step of 64 columns in four quarters of MF matrix instructions; the order is written out
+  // and pinned (every matrix instruction with what follows it stands between two scheduling
+  // barriers).  Under a quarter's first matrix instructions go the reads of the next quarter's
+  // operands.  The requests for K step kt + NBUF - 1 (its buffer was last read in step kt - 1,
+  // before that step's barrier) are spread over the first three quarters, one for every second
+  // matrix instruction: a request of a kilobyte keeps the CU's one address unit busy for 16
+  // cycles, and the four waves ask at the same time.  The barrier stands in front of the last
+  // quarter: this wave's part of K step kt + 1 has landed when at most the loads of NBUF - 2
+  // steps are outstanding; after it everybody's has, and nobody reads this step's buffer any more.
+  auto read_one = [&](int buf, int ks, bf16x8* af, bf16x8* bf, int r) {      // in the order in which the products need them
+    const char* tile = lds_bytes + buf * BUF + rd[ks];
+    const int j = r - 1, i = r - TN;
+    if (r == 0) af[0] = *reinterpret_cast<const bf16x8*>(tile + a_rd);
+    else if (r <= TN) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * EROW);
+    else af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 32 * EROW);
+  };
+  constexpr int READ_SPAN = MF < RD ? MF : RD;
+  auto quarter = [&](const bf16x8* af, const bf16x8* bf, int rbuf, int rks, bf16x8* raf, bf16x8* rbf, int kt_load, int lbuf,
+                     int l0, int l1) {
+#pragma unroll
+    for (int g = 0; g < MF; ++g) {
+      const int i = g / TN, j = g % TN;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);   // transposed
+      if (g < READ_SPAN) {
+#pragma unroll
+        for (int r = (RD * g) / READ_SPAN; r < (RD * (g + 1)) / READ_SPAN; ++r) read_one(rbuf, rks, raf, rbf, r);
+      }
+#pragma unroll
+      for (int l = l0 + ((l1 - l0) * g) / MF; l < l0 + ((l1 - l0) * (g + 1)) / MF; ++l) load_one(kt_load, lbuf, l);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
   int rb = 0;                                   // kt % NBUF
   for (int kt = 0; kt < ktiles; ++kt) {
     const int lb = rb == 0 ? NBUF - 1 : rb - 1, nb = rb == NBUF - 1 ? 0 : rb + 1;
-    read_operands(rb, 1, a[1], b[1]);
-    multiply(a[0], b[0], 0, MF);
-    load_step(kt + NBUF - 1, lb);
-    Interleave<0x100, HALF, RD>::emit();
-    __builtin_amdgcn_sched_group_barrier(0x008, MF - HALF, 0);
-    // (the loads follow the reads in program order; the scheduler places them between the
-    // products of the next quarter)
-    read_operands(rb, 2, a[0], b[0]);
-    multiply(a[1], b[1], 0, MF);
-    Interleave<0x020, MF, LD>::emit();
-    __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);
-    read_operands(rb, 3, a[1], b[1]);
-    multiply(a[0], b[0], 0, MF);
-    Interleave<0x100, MF, RD>::emit();
-    multiply(a[1], b[1], 0, HALF);
-    __builtin_amdgcn_sched_group_barrier(0x008, HALF, 0);
+    quarter(a[0], b[0], rb, 1, a[1], b[1], kt + NBUF - 1, lb, 0, LD / 3);
+    quarter(a[1], b[1], rb, 2, a[0], b[0], kt + NBUF - 1, lb, LD / 3, 2 * LD / 3);
+    quarter(a[0], b[0], rb, 3, a[1], b[1], kt + NBUF - 1, lb, 2 * LD / 3, LD);
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NBUF - 2) * LD) : "memory");
     barrier_no_fence();
-    read_operands(nb, 0, a[0], b[0]);
-    multiply(a[1], b[1], HALF, MF);
-    Interleave<0x100, MF - HALF, RD>::emit();
+    quarter(a[1], b[1], nb, 0, a[0], b[0], 0, 0, 0, 0);
     rb = nb;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
