@@ -5,7 +5,10 @@ and its defaults (/root/reference/internal/llm/model.go:83-100): layer count,
 width, heads, KV heads (default: heads), head size (default: width / heads),
 trained context (default 2048), norm eps (default 1e-5), rope base (default
 10000).  The llama3 rope scaling stands where the reference reads precomputed
-per-dimension divisors (/root/reference/internal/llm/model.go:150-158).
+per-dimension divisors (/root/reference/internal/llm/model.go:150-158).  The gate's
+activation is the SiLU in the reference's code
+(/root/reference/internal/ggml/ops.go:159-165); config.json names it (`hidden_act`), and
+the names that the feed-forward part has kernels for are read.
 """
 from __future__ import annotations
 
@@ -13,6 +16,10 @@ from dataclasses import dataclass, asdict
 from typing import Optional
 
 from .base import KeyReader, ConfigError
+
+
+# config.json's names of a gate activation -> the feed-forward part's
+HIDDEN_ACTS = {"silu": "silu", "gelu": "gelu", "gelu_pytorch_tanh": "gelu_tanh", "relu": "relu"}
 
 
 @dataclass(frozen=True)
@@ -42,6 +49,7 @@ class LlamaConfig:
     bos_token_id: Optional[int]
     eos_token_ids: tuple
     torch_dtype: str
+    hidden_act: str = "silu"
 
     @staticmethod
     def from_dict(data: dict, where: str = "config.json") -> "LlamaConfig":
@@ -63,7 +71,7 @@ class LlamaConfig:
         eos = r.int_or_list("eos_token_id", None)
         dtype = r.str("torch_dtype", r.str("dtype", "bfloat16"))
         act = r.str("hidden_act", "silu")
-        r.require(act == "silu", f"key 'hidden_act': only 'silu' is built, got {act!r}")
+        r.require(act in HIDDEN_ACTS, f"key 'hidden_act': one of {sorted(HIDDEN_ACTS)} expected, got {act!r}")
         for flag in ("attention_bias", "mlp_bias"):
             r.require(not r.bool(flag, False), f"key {flag!r}: biases are not part of this architecture here")
 
@@ -107,7 +115,7 @@ class LlamaConfig:
             num_attention_heads=heads, num_key_value_heads=kv, head_dim=hd, vocab_size=vocab,
             max_position_embeddings=max_pos, rms_norm_eps=eps, rope_theta=theta,
             rope_scaling=scaling, tie_word_embeddings=tie, bos_token_id=bos,
-            eos_token_ids=tuple(eos), torch_dtype=dtype)
+            eos_token_ids=tuple(eos), torch_dtype=dtype, hidden_act=act)
 
     def to_dict(self) -> dict:
         """The config.json that reads back as this configuration."""
@@ -126,7 +134,7 @@ class LlamaConfig:
             "rope_theta": self.rope_theta,
             "rope_scaling": asdict(self.rope_scaling) if self.rope_scaling else None,
             "tie_word_embeddings": self.tie_word_embeddings,
-            "hidden_act": "silu",
+            "hidden_act": self.hidden_act,
             "torch_dtype": self.torch_dtype,
         }
         if self.bos_token_id is not None:
@@ -136,4 +144,4 @@ class LlamaConfig:
         return out
 
 
-__all__ = ["LlamaConfig", "RopeScaling", "ConfigError"]
+__all__ = ["LlamaConfig", "RopeScaling", "ConfigError", "HIDDEN_ACTS"]

@@ -103,6 +103,43 @@ template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return float_to_bf16(v); }
 
+// The activation of a gated feed-forward's gate, as the entry points name it.  The SiLU
+// (/root/reference/internal/ggml/ops.go:159-165) is written out where it is used, in the
+// form that each kernel has been measured with; the others are here, in forms that cost
+// one exponential, as the SiLU does, so that an epilogue which carries them beside it stays
+// small: g/2 (1 + tanh y) = g / (1 + exp(-2y)), and the error function by its rational
+// approximation with exp(-x^2) (Abramowitz and Stegun 7.1.26, absolute error below 1.5e-7;
+// the kernels that use these round the result to bfloat16).
+enum { GATE_SILU = 0, GATE_GELU_TANH = 1, GATE_GELU = 2, GATE_RELU = 3, GATE_KINDS = 4 };
+
+template <int ACT>
+__device__ __forceinline__ float gate_other_as(float g) {
+  if constexpr (ACT == GATE_GELU_TANH) {
+    const float y = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return g * __frcp_rn(1.0f + __expf(-2.0f * y));
+  } else if constexpr (ACT == GATE_GELU) {
+    const float x = fabsf(g) * 0.7071067811865476f, t = __frcp_rn(1.0f + 0.3275911f * x);
+    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+    const float erf_abs = 1.0f - poly * __expf(-x * x);
+    return 0.5f * g * (1.0f + (g < 0.f ? -erf_abs : erf_abs));
+  } else {
+    return fmaxf(g, 0.0f);
+  }
+}
+
+__device__ __forceinline__ float gate_other(float g, int act) {
+  return act == GATE_GELU_TANH ? gate_other_as<GATE_GELU_TANH>(g)
+         : act == GATE_GELU    ? gate_other_as<GATE_GELU>(g)
+                               : gate_other_as<GATE_RELU>(g);
+}
+
+// The same to the last bit of the library's functions, for the 32-bit path.
+__device__ __forceinline__ float gate_other_exact(float g, int act) {
+  if (act == GATE_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  if (act == GATE_GELU) return 0.5f * g * (1.0f + erff(g * 0.7071067811865476f));
+  return fmaxf(g, 0.0f);
+}
+
 // ---- reductions with a fixed order -------------------------------------------
 // Every lane ends with the same value; the tree's shape does not depend on data.
 __device__ __forceinline__ float wave_sum(float v) {

@@ -219,19 +219,20 @@ HFEE_API int hfee_rmsnorm(void* out, int out_dtype, const float* x, const void* 
 // ------------------------------------------------------------------ SiLU gate
 template <typename T>
 __global__ void swiglu_kernel(T* __restrict__ out, int64_t ld_out, const T* __restrict__ gate,
-                              const T* __restrict__ up, int64_t ld_in, int col_stride, int width) {
+                              const T* __restrict__ up, int64_t ld_in, int col_stride, int width, int act) {
   const int row = blockIdx.y;
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= width) return;
   const float g = to_float<T>(gate[(int64_t)row * ld_in + (int64_t)j * col_stride]);
   const float u = to_float<T>(up[(int64_t)row * ld_in + (int64_t)j * col_stride]);
-  out[(int64_t)row * ld_out + j] = from_float<T>(g / (1.0f + expf(-g)) * u);
+  out[(int64_t)row * ld_out + j] = from_float<T>((act == GATE_SILU ? g / (1.0f + expf(-g)) : gate_other_exact(g, act)) * u);
 }
 
 // col_stride: distance between consecutive gate (and up) columns: 1 for two separate
-// blocks, 2 when gate and up alternate.
+// blocks, 2 when gate and up alternate.  act: the gate's activation (GATE_SILU ...).
 HFEE_API int hfee_swiglu(void* out, int64_t ld_out, const void* gate, const void* up, int64_t ld_in,
-                         int col_stride, int dtype, int n, int width, hipStream_t stream) {
+                         int col_stride, int dtype, int n, int width, int act, hipStream_t stream) {
+  HFEE_REQUIRE(act >= 0 && act < GATE_KINDS, "swiglu: unknown activation %d", act);
   HFEE_REQUIRE(n >= 0 && width > 0 && ld_out >= width && col_stride >= 1 &&
                ld_in >= (int64_t)(width - 1) * col_stride + 1, "swiglu: bad sizes");
   HFEE_REQUIRE(n <= 65535 * 16, "swiglu: too many rows (%d)", n);
@@ -243,11 +244,11 @@ HFEE_API int hfee_swiglu(void* out, int64_t ld_out, const void* gate, const void
     if (dtype == DT_F32)
       swiglu_kernel<float><<<grid, 256, 0, stream>>>((float*)out + row0 * ld_out, ld_out,
                                                      (const float*)gate + row0 * ld_in,
-                                                     (const float*)up + row0 * ld_in, ld_in, col_stride, width);
+                                                     (const float*)up + row0 * ld_in, ld_in, col_stride, width, act);
     else if (dtype == DT_BF16)
       swiglu_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out + row0 * ld_out, ld_out,
                                                       (const bf16_t*)gate + row0 * ld_in,
-                                                      (const bf16_t*)up + row0 * ld_in, ld_in, col_stride, width);
+                                                      (const bf16_t*)up + row0 * ld_in, ld_in, col_stride, width, act);
     else
       return fail("swiglu: unknown dtype %d", dtype);
   }

@@ -163,10 +163,29 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(void* __restrict__
 }
 
 
+// The gate's activation of a finished sum.  ACT is known when the epilogue is compiled: an
+// epilogue is unrolled over a wave's 128 gates, and with a choice between the activations at each
+// of them it was 45,000 instructions where the reference's alone has 8,000 (a layer of a
+// 2,048-token prefill took 969 us instead of 885).
+template <int ACT>
+__device__ __forceinline__ float gated(float g) {
+  if constexpr (ACT == GATE_SILU) return g * __frcp_rn(1.0f + __expf(-g));
+  else return gate_other_as<ACT>(g);
+}
+
+// Calls f(std::integral_constant<int, ACT>) for the activation of a gating product (MODE says whether it is one).
+template <int MODE, typename F>
+__device__ __forceinline__ void with_gate_activation(int act, F&& f) {
+  if (MODE != OUT_SWIGLU || act == GATE_SILU) f(std::integral_constant<int, GATE_SILU>{});
+  else if (act == GATE_GELU_TANH) f(std::integral_constant<int, GATE_GELU_TANH>{});
+  else if (act == GATE_GELU) f(std::integral_constant<int, GATE_GELU>{});
+  else f(std::integral_constant<int, GATE_RELU>{});
+}
+
 // Stores a 32 x 32 tile that was formed transposed: register r of lane l holds
 // C[m_base + l % 32][n_base + 8 (r / 4) + 4 (l / 32) + r % 4], so four registers are
 // four consecutive columns.  `vec`: rows of C start 16-byte aligned (8 for bfloat16).
-template <int MODE>
+template <int MODE, int ACT = GATE_SILU>
 __device__ __forceinline__ void store_tile_t(void* C, int64_t ldc, int M, int N, int m, int n_base, int lane,
                                              const f32x16& t, bool vec) {
   if (m >= M) return;
@@ -177,8 +196,8 @@ __device__ __forceinline__ void store_tile_t(void* C, int64_t ldc, int M, int N,
     float v[4] = {t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
     if (MODE == OUT_SWIGLU) {          // columns n, n+1 are gate, up of output column n / 2
       bf16_t* c = (bf16_t*)C + (int64_t)m * ldc + (n >> 1);
-      const bf16_t o0 = float_to_bf16(v[0] * __frcp_rn(1.0f + __expf(-v[0])) * v[1]);
-      const bf16_t o1 = float_to_bf16(v[2] * __frcp_rn(1.0f + __expf(-v[2])) * v[3]);
+      const bf16_t o0 = float_to_bf16(gated<ACT>(v[0]) * v[1]);
+      const bf16_t o1 = float_to_bf16(gated<ACT>(v[2]) * v[3]);
       if (vec && n + 3 < N) {
         *reinterpret_cast<uint32_t*>(c) = (uint32_t)o0 | ((uint32_t)o1 << 16);
       } else {
@@ -228,7 +247,7 @@ struct Stage {
   static constexpr int BYTES = (32 * PITCH + 1023) / 1024 * 1024;
 };
 
-template <int MODE, int TM, int TN>
+template <int MODE, int TM, int TN, int ACT = GATE_SILU>
 __device__ __forceinline__ void store_wave_staged(char* lds, void* C, int64_t ldc, int M, int m_first, int n_first,
                                                   int lane, const f32x16 (&acc)[TM][TN]) {
   using S = Stage<MODE, TN>;
@@ -244,8 +263,8 @@ __device__ __forceinline__ void store_wave_staged(char* lds, void* C, int64_t ld
         const f32x16& t = acc[i][j];
         const float v[4] = {t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
         if constexpr (MODE == OUT_SWIGLU) {
-          const bf16_t o0 = float_to_bf16(v[0] * __frcp_rn(1.0f + __expf(-v[0])) * v[1]);
-          const bf16_t o1 = float_to_bf16(v[2] * __frcp_rn(1.0f + __expf(-v[2])) * v[3]);
+          const bf16_t o0 = float_to_bf16(gated<ACT>(v[0]) * v[1]);
+          const bf16_t o1 = float_to_bf16(gated<ACT>(v[2]) * v[3]);
           *reinterpret_cast<uint32_t*>(mine + (j * 16 + 4 * q + 2 * h) * 2) = (uint32_t)o0 | ((uint32_t)o1 << 16);
         } else if constexpr (MODE == OUT_BF16) {
           u32x2 o;
@@ -367,20 +386,11 @@ struct PStage {
   u32x4 a[2 * TM], w[2 * TN];      // this thread's 16-byte chunks of the A tile and of the W tile
 };
 
-// The second half of a norm whose first half the product before has done (gemm_skinny.hip,
-// ROW SCALE), for products of at most 64 rows: every row of the result is scaled by
-// 1/sqrt(sum of the row's shares / K + eps).  shares null: no scaling.
-struct RowScale {
-  const float* shares;      // [blocks][64]
-  int blocks;
-  float eps;
-};
-
 template <int MODE, int TM, int TN, int STAGES>
 __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restrict__ C, int64_t ldc,
                                                                   const bf16_t* __restrict__ A, int64_t lda,
                                                                   const bf16_t* __restrict__ W, int64_t ldw,
-                                                                  int M, int N, int K, QkvArgs qkv, RowScale rs,
+                                                                  int M, int N, int K, QkvArgs qkv,
                                                                   int k_split, int64_t c_split) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
   extern __shared__ __attribute__((aligned(16))) bf16_t lds_tiles[];
@@ -457,22 +467,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
   PStage<TM, TN> ring[STAGES];
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) load_stage(ring[s], s);
-  // the rows' scales (at most 64 rows, so m0 == 0), behind the first loads of the tiles:
-  // thread -> row tid % 64, every fourth share
-  __shared__ float row_scale[64];
-  __shared__ float row_scale_part[4][64];
-  if (rs.shares != nullptr) {
-    const int row = min(tid & 63, M - 1), q4 = tid >> 6;
-    float t = 0.f;
-#pragma unroll 8
-    for (int b = q4; b < rs.blocks; b += 4) t += rs.shares[(int64_t)b * 64 + row];
-    row_scale_part[q4][tid & 63] = t;
-  }
   store_stage(ring[0], 0, inside(0));
   __syncthreads();
-  if (rs.shares != nullptr && tid < 64)      // (read after the barriers of the loop below, or the one before the stores)
-    row_scale[tid] = 1.0f / sqrtf((((row_scale_part[0][tid] + row_scale_part[1][tid]) + row_scale_part[2][tid]) +
-                                   row_scale_part[3][tid]) / (float)K + rs.eps);
 
   const int lrow = lane & 31, lk = (lane >> 5) * 8;
   auto step = [&](auto slot_c, auto last_c, int kt) {
@@ -523,22 +519,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_pipelined_kernel(void* __restri
   if constexpr (MODE == OUT_QKV) {
     store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
   } else {
-    if (rs.shares != nullptr) {
-      __syncthreads();
+    // (a gating product has a copy of the stores for each activation)
+    with_gate_activation<MODE>(qkv.gate_act, [&](auto act) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const float scale = row_scale[min(wm * 32 * TM + i * 32 + lrow, 63)];
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[i][j][r] *= scale;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+          store_tile_t<MODE, decltype(act)::value>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32,
+                                                   lane, acc[i][j], vec);
+    });
   }
 }
 
@@ -715,7 +704,7 @@ inline bool cuts_by_large_tiles(int M, int N, int K, int splits, int k_split) {
 
 template <int MODE>
 int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                     int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, const RowScale& rs = RowScale{},
+                     int M, int N, int K, const QkvArgs& qkv, hipStream_t stream,
                      const Partial& partial = Partial{}, const NormAfter& norm = NormAfter{}, bool* normed = nullptr) {
   // 128 x 128 tiles, two workgroups per CU.  (128 x 256 tiles halve the LDS reads per
   // matrix instruction but leave one wave per SIMD, and measured 20 % slower; 128 x 64
@@ -731,7 +720,7 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
   if constexpr (MODE == OUT_BF16 || MODE == OUT_F32 || MODE == OUT_ADD_F32) {
     const int splits = pipelined_splits(M, N, K);
     const bool rows_fit = MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0) : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
-    if (splits > 1 && rs.shares == nullptr && rows_fit && partial.at != nullptr && (uintptr_t)partial.at % 16 == 0 &&
+    if (splits > 1 && rows_fit && partial.at != nullptr && (uintptr_t)partial.at % 16 == 0 &&
         partial.floats >= (int64_t)splits * M * N) {
       if (raise_pipelined_lds<OUT_F32>(lds)) return 1;
       const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
@@ -742,7 +731,7 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
       } else {
         grid.y = splits;
         gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
-            partial.at, N, A, lda, W, ldw, M, N, K, qkv, rs, k_split, (int64_t)M * N);
+            partial.at, N, A, lda, W, ldw, M, N, K, qkv, k_split, (int64_t)M * N);
       }
       if constexpr (MODE == OUT_ADD_F32) {
         if (norm.normed != nullptr && launch_finish_norm((float*)C, ldc, partial.at, splits, M, N, norm, stream)) {
@@ -755,7 +744,7 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
       return 0;
     }
   }
-  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv, rs, 0, 0);
+  gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv, 0, 0);
   return 0;
 }
 
@@ -946,15 +935,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
     static_assert(4 * S::BYTES <= 4 * BUF, "the waves' strips fit in the LDS of the buffers");
     __syncthreads();      // nobody reads operands from the LDS any more
     const bool whole_rows = (ldc * S::ES) % 16 == 0 && (uintptr_t)C % 16 == 0 && n0 + wn * 32 * TN + 32 * TN <= N;
-    if (whole_rows) {
-      store_wave_staged<MODE, TM, TN>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
-    } else {
+    // (a gating product has a copy of the stores for each activation)
+    with_gate_activation<MODE>(qkv.gate_act, [&](auto act) {
+      constexpr int ACT = decltype(act)::value;
+      if (whole_rows) {
+        store_wave_staged<MODE, TM, TN, ACT>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
+      } else {
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
-    }
+          for (int j = 0; j < TN; ++j)
+            store_tile_t<MODE, ACT>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+      }
+    });
   }
 #endif
 }
@@ -1131,15 +1124,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
     static_assert(4 * S::BYTES <= NBUF * BUF, "the waves' strips fit in the LDS of the buffers");
     __syncthreads();      // nobody reads operands from the LDS any more
     const bool whole_rows = (ldc * S::ES) % 16 == 0 && (uintptr_t)C % 16 == 0 && n0 + wn * 32 * TN + 32 * TN <= N;
-    if (whole_rows) {
-      store_wave_staged<MODE, TM, TN>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
-    } else {
+    // (a gating product has a copy of the stores for each activation)
+    with_gate_activation<MODE>(qkv.gate_act, [&](auto act) {
+      constexpr int ACT = decltype(act)::value;
+      if (whole_rows) {
+        store_wave_staged<MODE, TM, TN, ACT>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
+      } else {
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          store_tile_t<MODE>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
-    }
+          for (int j = 0; j < TN; ++j)
+            store_tile_t<MODE, ACT>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+      }
+    });
   }
 #endif
 }
@@ -1312,7 +1309,7 @@ int launch_tiled_kernel(int choice, void* C, int64_t ldc, const bf16_t* A, int64
   if (choice == 6) return launch_direct<MODE, 4, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
-  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream, RowScale{}, partial);
+  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream, partial);
 }
 
 template <int MODE>
@@ -1366,33 +1363,6 @@ int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, 
 
 }  // namespace
 
-// The tiled product of at most 64 rows whose result rows are scaled by the second half of
-// a norm (see RowScale): for shapes that are too wide for the streaming kernels.
-// out_mode as hfee_gemm_bf16; operands aligned as for the tiled kernels.
-HFEE_API int hfee_gemm_bf16_scaled(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
-                                   int64_t ldw, int M, int N, int K, const float* shares, int blocks, float eps,
-                                   hipStream_t stream) {
-  HFEE_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_bf16_scaled: 1 to 64 rows, got M=%d N=%d K=%d", M, N, K);
-  HFEE_REQUIRE(out_mode >= 0 && out_mode <= 3, "gemm_bf16_scaled: unknown output mode %d", out_mode);
-  HFEE_REQUIRE(shares != nullptr && blocks > 0 && eps >= 0.f, "gemm_bf16_scaled: no shares");
-  HFEE_REQUIRE((K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) &&
-                   lda >= K && ldw >= K,
-               "gemm_bf16_scaled: K and the leading dimensions must be multiples of 8 and the operands 16-byte aligned");
-  HFEE_REQUIRE(out_mode != 3 || N % 2 == 0, "gemm_bf16_scaled: the SiLU gate needs an even N");
-  HFEE_REQUIRE(ldc >= (out_mode == 3 ? N / 2 : N), "gemm_bf16_scaled: ldc is shorter than a row of the result");
-  const RowScale rs{shares, blocks, eps};
-  const bf16_t* a = (const bf16_t*)A;
-  const bf16_t* w = (const bf16_t*)W;
-  int rc;
-  if (out_mode == OUT_BF16) rc = launch_pipelined<OUT_BF16>(C, ldc, a, lda, w, ldw, M, N, K, QkvArgs{}, stream, rs);
-  else if (out_mode == OUT_F32) rc = launch_pipelined<OUT_F32>(C, ldc, a, lda, w, ldw, M, N, K, QkvArgs{}, stream, rs);
-  else if (out_mode == OUT_ADD_F32) rc = launch_pipelined<OUT_ADD_F32>(C, ldc, a, lda, w, ldw, M, N, K, QkvArgs{}, stream, rs);
-  else rc = launch_pipelined<OUT_SWIGLU>(C, ldc, a, lda, w, ldw, M, N, K, QkvArgs{}, stream, rs);
-  if (rc) return rc;
-  HFEE_CHECK_LAUNCH("gemm_bf16_scaled");
-  return 0;
-}
-
 // How an aligned product of more than 64 rows is laid over the tiled kernels when nothing
 // is forced: kernel of the first n1 columns, n1, kernel of the rest (0: none).  For
 // tests and for reading a profile.
@@ -1414,15 +1384,16 @@ HFEE_API int hfee_gemm_bf16_scratch(int M, int N, int K) {
 }
 
 // C = A W^T for bfloat16 A [M, K] and W [N, K].
-// out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 SiLU gate (the
-// rows of W alternate gate/up; C is [M, N/2] bfloat16; aligned operands only).
+// out_mode: 0 bfloat16 store, 1 float32 store, 2 float32 accumulate, 3 gate (the
+// rows of W alternate gate/up; C is [M, N/2] bfloat16 = activation(gate) * up, the
+// activation being gate_act: GATE_SILU ...; aligned operands only).
 // force_kernel: 0 choose by the sizes, 1 skinny, 2 tiled 128 x 128, 3 the simple tiled
 // kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192 (for tests of each
 // kernel alone; 4 to 6 fall back to 2 where they do not apply).
 // scratch: null, or hfee_gemm_bf16_scratch(M, N, K) float32 words, 16-byte aligned.
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
                             int64_t ldw, int M, int N, int K, int force_kernel, float* scratch,
-                            int64_t scratch_floats, hipStream_t stream) {
+                            int64_t scratch_floats, int gate_act, hipStream_t stream) {
   Partial partial;
   partial.at = scratch;
   partial.floats = scratch != nullptr ? scratch_floats : 0;
@@ -1435,8 +1406,11 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) &&
                    ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
   if (out_mode == 3) {
-    HFEE_REQUIRE(N % 2 == 0 && vec, "gemm_bf16: the SiLU gate needs an even N and aligned operands");
-    if (launch_aligned<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, force_kernel, stream)) return 1;
+    HFEE_REQUIRE(N % 2 == 0 && vec, "gemm_bf16: the gate needs an even N and aligned operands");
+    HFEE_REQUIRE(gate_act >= 0 && gate_act < GATE_KINDS, "gemm_bf16: unknown activation %d", gate_act);
+    QkvArgs gate{};
+    gate.gate_act = gate_act;
+    if (launch_aligned<OUT_SWIGLU>(C, ldc, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, force_kernel, stream, gate)) return 1;
     HFEE_CHECK_LAUNCH("gemm_bf16");
     return 0;
   }
@@ -1483,14 +1457,14 @@ HFEE_API int hfee_gemm_bf16_add_norm(float* C, const void* A, int64_t lda, const
       norm.weight_is_f32 = norm_weight_is_f32 != 0;
       norm.eps = eps;
       if (launch_pipelined<OUT_ADD_F32>(C, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, stream,
-                                        RowScale{}, partial, norm, &done))
+                                        partial, norm, &done))
         return 1;
       HFEE_CHECK_LAUNCH("gemm_bf16_add_norm");
       if (done) return 0;
       return hfee_rmsnorm(normed, DT_BF16, C, norm_weight, norm_weight_is_f32 ? DT_F32 : DT_BF16, nullptr, eps, M, N, stream);
     }
   }
-  if (int rc = hfee_gemm_bf16(C, OUT_ADD_F32, N, A, lda, W, ldw, M, N, K, 0, scratch, scratch_floats, stream)) return rc;
+  if (int rc = hfee_gemm_bf16(C, OUT_ADD_F32, N, A, lda, W, ldw, M, N, K, 0, scratch, scratch_floats, GATE_SILU, stream)) return rc;
   return hfee_rmsnorm(normed, DT_BF16, C, norm_weight, norm_weight_is_f32 ? DT_F32 : DT_BF16, nullptr, eps, M, N, stream);
 }
 
@@ -1516,7 +1490,7 @@ HFEE_API int hfee_gemm_bf16_cuts(const void* A, int64_t lda, const void* W, int6
   dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS), splits);
   const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
   gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
-      scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, RowScale{}, k_split, (int64_t)M * N);
+      scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, k_split, (int64_t)M * N);
   HFEE_CHECK_LAUNCH("gemm_bf16_cuts");
   *cuts = splits;
   return 0;

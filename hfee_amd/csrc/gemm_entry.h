@@ -19,10 +19,6 @@ HFEE_API int hfee_gemm_skinny(void* C, int64_t ldc, const void* A, int a_is_f32,
 HFEE_API int hfee_gemm_bf16_qkv(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int64_t ldw, int M,
                                 int N, int K, const hfee::QkvArgs* qkv, int force_kernel, hipStream_t stream);
 
-HFEE_API int hfee_gemm_bf16_scaled(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
-                                   int64_t ldw, int M, int N, int K, const float* shares, int blocks, float eps,
-                                   hipStream_t stream);
-
 // (elementwise.hip: the norm as a kernel of its own, for the product that is followed by one)
 enum { DT_F32 = 0, DT_BF16 = 1 };      // how the elementwise entry points name a tensor's type
 HFEE_API int hfee_rmsnorm(void* out, int out_dtype, const float* x, const void* w, int w_dtype, const int* rows,

@@ -22,6 +22,8 @@ struct QkvArgs {
   void* cache;                // one cache layer, or null (keys and values are not written)
   CacheLayout lay;
   int num_heads;
+  // (the tiled kernels hand this struct to every epilogue: the gated one finds its activation here)
+  int gate_act;               // GATE_SILU ...
 };
 
 

@@ -26,12 +26,12 @@ _CORE_SIGNATURES = {
     "hfee_embed": [P, P, I, P, I, I, P],
     "hfee_embed_emit": [P, P, P, I, I, P, I, P, L, P, L, P],
     "hfee_rmsnorm": [P, I, P, P, I, P, F, I, I, P],
-    "hfee_swiglu": [P, L, P, P, L, I, I, I, I, P],
+    "hfee_swiglu": [P, L, P, P, L, I, I, I, I, I, P],
     "hfee_residual_add": [P, P, I, L, P],
     "hfee_rope_cache_write": [P, L, P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, P, I, I, I, I, I, I, P],
     "hfee_gemm_f32": [P, L, P, L, P, L, I, I, I, I, P],
     "hfee_attention_ref": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
-    "hfee_gemm_bf16": [P, I, L, P, L, P, L, I, I, I, I, P, L, P],
+    "hfee_gemm_bf16": [P, I, L, P, L, P, L, I, I, I, I, P, L, I, P],
     "hfee_gemm_bf16_add_norm": [P, P, L, P, L, I, I, I, P, L, P, P, I, F, P],
     "hfee_gemm_bf16_cuts": [P, L, P, L, I, I, I, P, L, P, P],
     "hfee_rope_cache_write_cuts": [P, L, P, I, P, P, P, I, P, P, I, I, I, P, I, I, I, I, I, I, P],

@@ -122,16 +122,27 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
                     float(eps), n, d, _stream())
 
 
-def swiglu(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
-    """out = gate / (1 + exp(-gate)) * up.  gate and up are views of one buffer with the
-    same row and column strides (column stride 1: two blocks; 2: alternating columns)."""
+# the activations of a gated feed-forward's gate, as the kernels number them (GATE_SILU ... in csrc/common.h)
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "gelu": 2, "relu": 3}
+
+
+def gate_activation(name: str) -> int:
+    if name not in GATE_ACTIVATIONS:
+        raise KernelError(f"unknown gate activation {name!r}: the kernels have {sorted(GATE_ACTIVATIONS)}")
+    return GATE_ACTIVATIONS[name]
+
+
+def swiglu(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, activation: str = "silu"):
+    """out = activation(gate) * up ("silu": gate / (1 + exp(-gate))).  gate and up are views of one
+    buffer with the same row and column strides (column stride 1: two blocks; 2: alternating columns)."""
+    act = gate_activation(activation)
     _gpu(out, gate, up)
     n, w, ldo = _rows2d(out, "swiglu out")
     _check(gate.dim() == 2 and up.dim() == 2 and tuple(gate.shape) == (n, w) == tuple(up.shape), "swiglu: shape mismatch")
     _check(gate.stride() == up.stride() and gate.stride(1) >= 1, "swiglu: gate and up must share their strides")
     _check(out.dtype == gate.dtype == up.dtype, "swiglu: dtype mismatch")
     ld = gate.stride(0) if n > 1 else max(gate.stride(0), (w - 1) * gate.stride(1) + 1)
-    lib.core().call("hfee_swiglu", _ptr(out), ldo, _ptr(gate), _ptr(up), ld, gate.stride(1), _dt(out), n, w, _stream())
+    lib.core().call("hfee_swiglu", _ptr(out), ldo, _ptr(gate), _ptr(up), ld, gate.stride(1), _dt(out), n, w, act, _stream())
 
 
 def random_fill(out: torch.Tensor, key: int, kind: str, std: float = 1.0, bound: int = 0):
@@ -254,7 +265,7 @@ def linear_add_norm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, no
 
 
 def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate: bool = False, kernel: int = 0,
-           gate: bool = False, scratch=None):
+           gate: bool = False, scratch=None, activation: str = "silu"):
     """out (+)= x @ weight.T, weight stored [out_features, in_features].
     scratch (bfloat16 products): float32, `linear_scratch(M, N, K)` words, or None.
 
@@ -262,7 +273,7 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
     bfloat16 x and weight: matrix cores with float32 accumulation; out bfloat16, or
     float32 (required when accumulating: the residual stream).
     gate (bfloat16, aligned shapes): the rows of weight alternate gate/up and
-    out[m, j] = silu(row 2j) * row 2j+1, out [M, N/2].
+    out[m, j] = activation(row 2j) * row 2j+1, out [M, N/2].
     kernel (bfloat16 only): 0 automatic, 1 skinny, 2 tiled 128x128, 3 the simple tiled
     kernel, 4 tiled 256x256, 5 tiled 256x128."""
     _gpu(out, x, weight)
@@ -275,7 +286,7 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
         _check(x.dtype == weight.dtype == out.dtype == torch.bfloat16 and not accumulate and N % 2 == 0,
                "linear: the gate epilogue takes bfloat16 operands and an even number of weight rows")
         lib.core().call("hfee_gemm_bf16", _ptr(out), 3, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K, kernel,
-                        None, 0, _stream())
+                        None, 0, gate_activation(activation), _stream())
         return
     _check(x.dtype == weight.dtype, "linear: x and weight dtypes differ")
     if x.dtype == torch.float32:
@@ -293,7 +304,7 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
             _gpu(scratch)
             _check(scratch.dtype == torch.float32 and scratch.is_contiguous(), "linear: float32 scratch expected")
         lib.core().call("hfee_gemm_bf16", _ptr(out), mode, ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K,
-                        kernel, _ptr(scratch), 0 if scratch is None else scratch.numel(), _stream())
+                        kernel, _ptr(scratch), 0 if scratch is None else scratch.numel(), 0, _stream())
     else:
         raise KernelError(f"linear: unsupported dtype {x.dtype}")
 
@@ -651,7 +662,8 @@ def linear_fused(out, x, weight, epilogue: str, norm_weight=None, eps: float = 0
     x: bfloat16 [M, K]; or, with norm_weight, the float32 residual stream (at most 16
     rows; `rows` optionally gathers them, then `m` is their number).
     epilogue: "bf16" | "f32" | "add" (out float32 += ...) | "swiglu" (weight rows
-    alternate gate/up; out [M, N/2]) | "qkv" (rotation + cache write; see
+    alternate gate/up; out [M, N/2] = silu(gate) * up: the reference's activation; another one is
+    "bf16" into [M, N] and `swiglu` over its alternating columns) | "qkv" (rotation + cache write; see
     parts/attention.py; qkv = dict(positions, token_segment, block_tables, cos, sin,
     cache_layer, num_heads, kv_heads, head_dim, page_size))."""
     if not isinstance(weight, TiledWeight):

@@ -5,8 +5,9 @@ residual add, then pre-norm gated feed-forward with a residual add
 (/root/reference/internal/llm/forward.go:79-115); the tensors are the
 safetensors counterparts of the names bound at
 /root/reference/internal/llm/model.go:115-141.  Everything numeric comes from the
-configuration; the only facts fixed here are the ones the reference fixes in code:
-SiLU gating (/root/reference/internal/ggml/ops.go:159-165), score scale
+configuration (the gate's activation too: the reference's code has the SiLU,
+/root/reference/internal/ggml/ops.go:159-165, config.json names it); the only facts fixed
+here are the ones the reference fixes in code: score scale
 1/sqrt(head_dim) (/root/reference/internal/llm/forward.go:149), causal reach,
 rotation over the whole head (/root/reference/internal/llm/model.go:100).
 
@@ -17,7 +18,7 @@ rotation under a permutation of each head's rows
 """
 from __future__ import annotations
 
-from ..config.llama import LlamaConfig
+from ..config.llama import HIDDEN_ACTS, LlamaConfig
 from ..config.registry import register_architecture
 from ..config.specs import (FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec,
                             PositionSpec, ScheduleEntry, params)
@@ -37,7 +38,7 @@ def llama_model_spec(cfg: LlamaConfig) -> ModelSpec:
         num_kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim,
         scale=cfg.head_dim ** -0.5, window=0), position=position)
     ffn = FeedForwardSpec("gated_mlp", params(
-        hidden=cfg.hidden_size, intermediate=cfg.intermediate_size, activation="silu"))
+        hidden=cfg.hidden_size, intermediate=cfg.intermediate_size, activation=HIDDEN_ACTS[cfg.hidden_act]))
     norm = NormSpec("rmsnorm", cfg.hidden_size, cfg.rms_norm_eps)
     layers = tuple(
         LayerSpec(arrangement="prenorm", hidden=cfg.hidden_size, mixer=mixer, feed_forward=ffn,

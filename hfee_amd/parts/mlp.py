@@ -1,8 +1,10 @@
 """The gated feed-forward (/root/reference/internal/llm/forward.go:110-114,
-/root/reference/internal/ggml/ops.go:159-165): down(silu(gate(h)) * up(h)), added to
-the residual stream.  gate and up run as one product over a weight whose rows
-alternate gate_j, up_j, so that a step of at most 64 tokens applies the gate in the
-product's epilogue (and folds the norm in front of it into the same launch)."""
+/root/reference/internal/ggml/ops.go:159-165): down(activation(gate(h)) * up(h)), added to
+the residual stream; the reference's activation is the SiLU, and which one it is is a
+parameter of the part (`activation`: one of `ops.GATE_ACTIVATIONS`).  gate and up run as
+one product over a weight whose rows alternate gate_j, up_j, so that the gate is the
+product's epilogue (and a step of at most 64 tokens folds the norm in front of it into
+the same launch)."""
 from __future__ import annotations
 
 import torch
@@ -23,9 +25,10 @@ class GatedMLP(FeedForward):
     def __init__(self, spec: FeedForwardSpec, prefix: str, dtype: torch.dtype):
         self.hidden = spec.get("hidden")
         self.intermediate = spec.get("intermediate")
-        act = spec.get("activation", "silu")
-        if act != "silu":
-            raise ValueError(f"the gated feed-forward is built for 'silu', got {act!r}")
+        self.activation = spec.get("activation", "silu")
+        if self.activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"the gated feed-forward has the activations {sorted(ops.GATE_ACTIVATIONS)}, "
+                             f"not {self.activation!r}")
         self.prefix, self.dtype = prefix, dtype
         self.w_gate_up = self.w_down = None
 
@@ -59,12 +62,19 @@ class GatedMLP(FeedForward):
             norm = None
             if halves is None and lazy and n <= ops.FUSED_NORM_MAX_ROWS and ops.norm_fusion_pays(*w.shape):
                 norm = h.fusable()
+            # the gate as the product's epilogue, where it is the reference's; another activation is a
+            # kernel of its own over the product's alternating columns (the kernels for few rows have
+            # no register to spare for a choice in their loops)
+            silu = self.activation == "silu"
+            out, epilogue = (act, "swiglu") if silu else (ctx.rows("mlp.gate_up", 2 * F), "bf16")
             if halves:        # the norm's first half came with the product before; both projections and the gate
-                ops.linear_fused(act, halves[0], w, "swiglu", row_scale=halves[1], **ctx.workspace.product_scratch(n, w))
+                ops.linear_fused(out, halves[0], w, epilogue, row_scale=halves[1], **ctx.workspace.product_scratch(n, w))
             elif norm:        # norm, both projections and the gate in one launch
-                ops.linear_fused(act, h.x, w, "swiglu", norm_weight=norm[0], eps=norm[1])
+                ops.linear_fused(out, h.x, w, epilogue, norm_weight=norm[0], eps=norm[1])
             else:
-                ops.linear_fused(act, h.tensor() if lazy else h, w, "swiglu", **ctx.workspace.product_scratch(n, w))
+                ops.linear_fused(out, h.tensor() if lazy else h, w, epilogue, **ctx.workspace.product_scratch(n, w))
+            if not silu:
+                ops.swiglu(act, out[:, 0::2], out[:, 1::2], activation=self.activation)
             # the down projection adds into x and, if asked, begins the norm that follows
             emit = then.offer() if then is not None else None
             ops.linear_fused(x, act, self.w_down_tiles, "add", emit=emit,
@@ -72,11 +82,11 @@ class GatedMLP(FeedForward):
             return
         hn = h.tensor() if lazy else h
         if aligned:   # the gate in the product's epilogue
-            ops.linear(act, hn, self.w_gate_up, gate=True)
+            ops.linear(act, hn, self.w_gate_up, gate=True, activation=self.activation)
         else:
             gate_up = ctx.rows("mlp.gate_up", 2 * F)
             ops.linear(gate_up, hn, self.w_gate_up)
-            ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2])
+            ops.swiglu(act, gate_up[:, 0::2], gate_up[:, 1::2], activation=self.activation)
         # the down projection adds into x and, if asked, goes on with the norm that follows
         # (where its K is cut over workgroups: the kernel that adds the cuts up has the row at hand)
         cut = ctx.workspace.split_scratch(n, self.w_down)

@@ -135,10 +135,23 @@ def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: fl
     return out
 
 
-def plain_swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    """/root/reference/internal/ggml/ops.go:159-165: g / (1 + exp(-g)) * up."""
+def plain_swiglu(gate: torch.Tensor, up: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """/root/reference/internal/ggml/ops.go:159-165: g / (1 + exp(-g)) * up.  The other
+    activations (config.json's `hidden_act`; the reference has the SiLU alone, so they are pinned
+    by the library's own functions in test_plain.py): gelu = g/2 (1 + erf(g / sqrt 2)),
+    gelu_pytorch_tanh = g/2 (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), relu = max(g, 0)."""
     g = gate.to(F64)
-    return g / (1 + torch.exp(-g)) * up.to(F64)
+    if activation == "silu":
+        a = g / (1 + torch.exp(-g))
+    elif activation == "gelu":
+        a = 0.5 * g * (1 + torch.erf(g / math.sqrt(2.0)))
+    elif activation == "gelu_pytorch_tanh":
+        a = 0.5 * g * (1 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g ** 3)))
+    elif activation == "relu":
+        a = torch.clamp(g, min=0)
+    else:
+        raise ValueError(f"hidden_act {activation!r}")
+    return a * up.to(F64)
 
 
 # ---------------------------------------------------------------- model -----
@@ -166,6 +179,7 @@ class PlainLlama:
         self.hd = c.get("head_dim") or self.d // self.H
         self.eps = c.get("rms_norm_eps", 1e-5)
         self.tied = bool(c.get("tie_word_embeddings", False))
+        self.act = c.get("hidden_act", "silu")
         scaling = c.get("rope_scaling")
         if scaling is not None and scaling.get("rope_type", scaling.get("type")) != "llama3":
             scaling = None
@@ -205,12 +219,13 @@ class PlainLlama:
 
     def feed_forward_sublayer(self, x, l):
         """/root/reference/internal/llm/forward.go:109-113: what the feed-forward half
-        of layer l adds to the stream: norm first, then down(silu(gate) * up)."""
+        of layer l adds to the stream: norm first, then down(silu(gate) * up) (or the
+        activation that config.json names instead of the SiLU)."""
         w = self.w
         p = f"model.layers.{l}."
         xb = self.r(plain_rmsnorm(x, w[p + "post_attention_layernorm.weight"], self.eps))    # forward.go:109
         h = plain_swiglu(plain_matmul(xb, w[p + "mlp.gate_proj.weight"]),
-                         plain_matmul(xb, w[p + "mlp.up_proj.weight"]))                # forward.go:110-112
+                         plain_matmul(xb, w[p + "mlp.up_proj.weight"]), self.act)      # forward.go:110-112
         return plain_matmul(self.r(h), w[p + "mlp.down_proj.weight"])                  # forward.go:113
 
     def block(self, x, l, pos, kv=None, window=0):

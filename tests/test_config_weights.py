@@ -47,8 +47,8 @@ def test_config_errors_name_everything_that_is_wrong():
         config_from_dict(dict(TINY_B, rope_scaling=dict(TINY_B["rope_scaling"], high_freq_factor=1.0)))
     with pytest.raises(ConfigError, match="metadata is incomplete"):
         config_from_dict(dict(TINY_A, num_hidden_layers=0))
-    with pytest.raises(ConfigError, match="only 'silu'"):
-        config_from_dict(dict(TINY_A, hidden_act="gelu"))
+    with pytest.raises(ConfigError, match="hidden_act.*'silu'.*got 'swoosh'"):
+        config_from_dict(dict(TINY_A, hidden_act="swoosh"))
 
 
 def test_model_spec_carries_no_constant_of_its_own():
@@ -59,6 +59,11 @@ def test_model_spec_carries_no_constant_of_its_own():
     assert abs(m.get("scale") - 32 ** -0.5) < 1e-12 and m.position.get("theta") == 500000.0
     assert spec.layers[0].mixer_norm.eps == 1e-6 and spec.head_name == "lm_head.weight"
     assert model_spec_of(config_from_dict(TINY_A)).head_name is None        # tied
+    # the gate's activation is config.json's to say, under the part's own name for it
+    assert spec.layers[0].feed_forward.get("activation") == "silu"
+    other = config_from_dict(dict(TINY_B, hidden_act="gelu_pytorch_tanh"))
+    assert model_spec_of(other).layers[2].feed_forward.get("activation") == "gelu_tanh"
+    assert config_from_dict(other.to_dict()) == other
 
 
 def test_random_weights_folder_round_trip(tmp_path):

@@ -513,6 +513,46 @@ def test_swiglu_and_add(dtype):
     close(xd, x.double() + out.double().cpu(), 1e-6)
 
 
+def _activation(name, g):
+    f = torch.nn.functional
+    return {"silu": f.silu, "gelu": f.gelu, "gelu_tanh": lambda t: f.gelu(t, approximate="tanh"), "relu": f.relu}[name](g)
+
+
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh", "gelu", "relu"])
+def test_every_gate_kernel_with_every_activation(activation):
+    """The gate's activation is an argument of every kernel that gates: the kernel of its own
+    (both dtypes), the epilogue of each tiled kernel (128 x 128, 256 x 256, 256 x 128, 256 x 192 and
+    the automatic choice), against the library's function in float64.  (The kernels for at most
+    64 rows gate with the reference's activation alone; the feed-forward part sends another one
+    through the kernel of its own.)  An unknown name is refused."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(11)
+    for dtype in (torch.float32, torch.bfloat16):
+        gu = (torch.randn(9, 2 * 173, generator=g) * 3).to(dtype)
+        out = torch.empty(9, 173, dtype=dtype, device=DEV)
+        ops.swiglu(out, gu.to(DEV)[:, 0::2], gu.to(DEV)[:, 1::2], activation=activation)
+        close(out, _activation(activation, gu[:, 0::2].double()) * gu[:, 1::2].double(), 1e-6 if dtype == torch.float32 else 1e-2)
+
+    def check(out, x, w, tol=2e-2):
+        ref = x.double() @ w.double().t()
+        mag = x.abs().double() @ w.abs().double().t()
+        want = _activation(activation, ref[:, 0::2]) * ref[:, 1::2]
+        err = (out.double().cpu() - want).abs()
+        assert (err <= tol * (1 + mag[:, 0::2]) * (1 + mag[:, 1::2])).all(), float(err.max())
+        # (a kernel that took another activation would be far off: the four differ by tenths around 1)
+        assert activation == "silu" or not torch.allclose(want, torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2], atol=1e-2)
+
+    for M, N, K in ((300, 520, 320), (513, 258, 64)):
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(N, K, generator=g) * 2 / math.sqrt(K)).to(torch.bfloat16)
+        for kernel in (0, 2, 4, 5, 6):
+            out = torch.zeros(M, N // 2, dtype=torch.bfloat16, device=DEV)
+            ops.linear(out, x.to(DEV), w.to(DEV), gate=True, kernel=kernel, activation=activation)
+            check(out, x, w)
+    with pytest.raises(ops.KernelError, match="unknown gate activation"):
+        ops.swiglu(out, out, out, activation="swoosh")
+
+
 @pytest.mark.parametrize("d", [97, 104, 2048 + 8, 4096])      # odd; a multiple of 8 (eight elements a thread); several workgroups a row
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_embed(dtype, d):

@@ -3,6 +3,8 @@ that reduce to a library routine, invariants, and the vectors that the reference
 own tests hold.  Each is chosen so that a plausible mistake fails it."""
 import math
 
+import pytest
+
 import torch
 import torch.nn.functional as F
 
@@ -148,6 +150,13 @@ def test_softmax_and_swiglu():
     assert float(plain_swiglu(torch.zeros(1, dtype=F64), torch.ones(1, dtype=F64))) == 0
     assert abs(float(plain_swiglu(torch.tensor([40.0], dtype=F64), torch.tensor([2.0], dtype=F64))) - 80) < 1e-9
     assert abs(float(plain_swiglu(torch.tensor([-40.0], dtype=F64), torch.tensor([2.0], dtype=F64)))) < 1e-12
+    # the other names of config.json's hidden_act, which the reference does not have: the library's functions
+    assert torch.allclose(plain_swiglu(g, u, "gelu"), F.gelu(g) * u, atol=1e-12)
+    assert torch.allclose(plain_swiglu(g, u, "gelu_pytorch_tanh"), F.gelu(g, approximate="tanh") * u, atol=1e-12)
+    assert torch.allclose(plain_swiglu(g, u, "relu"), F.relu(g) * u, atol=0)
+    assert not torch.allclose(plain_swiglu(g, u, "gelu"), plain_swiglu(g, u, "gelu_pytorch_tanh"), atol=1e-6)
+    with pytest.raises(ValueError):
+        plain_swiglu(g, u, "swoosh")
 
 
 def test_sampler_rules():
