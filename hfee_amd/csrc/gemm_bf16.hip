@@ -182,16 +182,30 @@ __device__ __forceinline__ void with_gate_activation(int act, F&& f) {
   else f(std::integral_constant<int, GATE_RELU>{});
 }
 
-// Stores a 32 x 32 tile that was formed transposed: register r of lane l holds
-// C[m_base + l % 32][n_base + 8 (r / 4) + 4 (l / 32) + r % 4], so four registers are
-// four consecutive columns.  `vec`: rows of C start 16-byte aligned (8 for bfloat16).
-template <int MODE, int ACT = GATE_SILU>
+// How a wave holds a tile of a product that was formed transposed (weights as the row
+// operand).  ACC is what the matrix instruction leaves: f32x16 for 32 x 32 x 16 (register r of
+// lane l holds C[m_base + l % 32][n_base + 8 (r / 4) + 4 (l / 32) + r % 4]), f32x4 for
+// 16 x 16 x 32 (C[m_base + l % 16][n_base + 4 (l / 16) + r]).  Either way four registers are four
+// consecutive columns of one row of C: a tile of R x R is Q such groups a lane, group q at
+// columns STEP q + 4 (l / R).
+template <typename ACC>
+struct TileOf {
+  static constexpr int R = sizeof(ACC) == 64 ? 32 : 16;      // rows and columns of a tile
+  static constexpr int STEP = 4 * (64 / R);                  // columns from one of a lane's groups to its next
+  static constexpr int Q = R / STEP;                         // groups a lane and tile
+  static_assert(sizeof(ACC) == 64 || sizeof(ACC) == 16, "f32x16 or f32x4");
+};
+
+// Stores a tile that was formed transposed.  `vec`: rows of C start 16-byte aligned (8 for
+// bfloat16).  m: this lane's row of C (m_base + l % R).
+template <int MODE, int ACT = GATE_SILU, typename ACC>
 __device__ __forceinline__ void store_tile_t(void* C, int64_t ldc, int M, int N, int m, int n_base, int lane,
-                                             const f32x16& t, bool vec) {
+                                             const ACC& t, bool vec) {
+  using T = TileOf<ACC>;
   if (m >= M) return;
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int n = n_base + 8 * q + 4 * (lane >> 5);
+  for (int q = 0; q < T::Q; ++q) {
+    const int n = n_base + T::STEP * q + 4 * (lane / T::R);
     if (n >= N) continue;
     float v[4] = {t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
     if (MODE == OUT_SWIGLU) {          // columns n, n+1 are gate, up of output column n / 2
@@ -238,20 +252,23 @@ __device__ __forceinline__ void store_tile_t(void* C, int64_t ldc, int M, int N,
 // make whole rows of C, 256 bytes and more at a time.  For tiles that lie inside C, with
 // rows of C that start 16-byte aligned; the caller has made sure that nobody reads the
 // LDS any more.  lds: the wave's own STAGE_BYTES.
-template <int MODE, int TN>
+// (TN tiles of R columns a strip row; R rows a strip)
+template <int MODE, int TN, int R = 32>
 struct Stage {
   static constexpr int ES = (MODE == OUT_BF16 || MODE == OUT_SWIGLU) ? 2 : 4;     // bytes of an element of C
-  static constexpr int OC = MODE == OUT_SWIGLU ? 16 * TN : 32 * TN;              // columns of C in a strip row
+  static constexpr int OC = MODE == OUT_SWIGLU ? R / 2 * TN : R * TN;            // columns of C in a strip row
   static constexpr int PITCH = OC * ES + 16;
   static constexpr int CHUNKS = OC * ES / 16;
-  static constexpr int BYTES = (32 * PITCH + 1023) / 1024 * 1024;
+  static constexpr int BYTES = (R * PITCH + 1023) / 1024 * 1024;
 };
 
-template <int MODE, int TM, int TN, int ACT = GATE_SILU>
+template <int MODE, int TM, int TN, int ACT = GATE_SILU, typename ACC>
 __device__ __forceinline__ void store_wave_staged(char* lds, void* C, int64_t ldc, int M, int m_first, int n_first,
-                                                  int lane, const f32x16 (&acc)[TM][TN]) {
-  using S = Stage<MODE, TN>;
-  const int lrow = lane & 31, h = lane >> 5;
+                                                  int lane, const ACC (&acc)[TM][TN]) {
+  using T = TileOf<ACC>;
+  constexpr int R = T::R;
+  using S = Stage<MODE, TN, R>;
+  const int lrow = lane % R, h = lane / R;
   char* crow = (char*)C + ((int64_t)m_first * ldc + (MODE == OUT_SWIGLU ? n_first / 2 : n_first)) * S::ES;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -259,57 +276,61 @@ __device__ __forceinline__ void store_wave_staged(char* lds, void* C, int64_t ld
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const f32x16& t = acc[i][j];
+      for (int q = 0; q < T::Q; ++q) {
+        const ACC& t = acc[i][j];
         const float v[4] = {t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+        const int col = j * R + T::STEP * q + 4 * h;          // this group's first column within the strip
         if constexpr (MODE == OUT_SWIGLU) {
           const bf16_t o0 = float_to_bf16(gated<ACT>(v[0]) * v[1]);
           const bf16_t o1 = float_to_bf16(gated<ACT>(v[2]) * v[3]);
-          *reinterpret_cast<uint32_t*>(mine + (j * 16 + 4 * q + 2 * h) * 2) = (uint32_t)o0 | ((uint32_t)o1 << 16);
+          *reinterpret_cast<uint32_t*>(mine + (col / 2) * 2) = (uint32_t)o0 | ((uint32_t)o1 << 16);
         } else if constexpr (MODE == OUT_BF16) {
           u32x2 o;
           o[0] = (uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16);
           o[1] = (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16);
-          *reinterpret_cast<u32x2*>(mine + (j * 32 + 8 * q + 4 * h) * 2) = o;
+          *reinterpret_cast<u32x2*>(mine + col * 2) = o;
         } else {
-          *reinterpret_cast<f32x4*>(mine + (j * 32 + 8 * q + 4 * h) * 4) = f32x4{v[0], v[1], v[2], v[3]};
+          *reinterpret_cast<f32x4*>(mine + col * 4) = f32x4{v[0], v[1], v[2], v[3]};
         }
       }
     // (the same wave wrote what it reads: its LDS instructions keep their order)
-    constexpr int PIECES = 32 * S::CHUNKS / 64;            // 16-byte pieces of the strip per lane
-    static_assert(32 * S::CHUNKS % 64 == 0, "a strip is a whole number of pieces per lane");
+    constexpr int TOTAL = R * S::CHUNKS, PIECES = (TOTAL + 63) / 64;      // 16-byte pieces of the strip, and per lane
     f32x4* dst[PIECES];
     f32x4 old[PIECES];
 #pragma unroll
     for (int it = 0; it < PIECES; ++it) {
       const int idx = lane + 64 * it, row = idx / S::CHUNKS, c = idx - row * S::CHUNKS;
-      dst[it] = m_first + i * 32 + row < M
-                    ? reinterpret_cast<f32x4*>(crow + (int64_t)(i * 32 + row) * ldc * S::ES + c * 16) : nullptr;
+      dst[it] = idx < TOTAL && m_first + i * R + row < M
+                    ? reinterpret_cast<f32x4*>(crow + (int64_t)(i * R + row) * ldc * S::ES + c * 16) : nullptr;
       // what is added to: every piece asked for before the first is needed
       if (MODE == OUT_ADD_F32 && dst[it]) old[it] = *dst[it];
     }
 #pragma unroll
     for (int it = 0; it < PIECES; ++it) {
       const int idx = lane + 64 * it, row = idx / S::CHUNKS, c = idx - row * S::CHUNKS;
-      const f32x4 piece = *reinterpret_cast<const f32x4*>(lds + row * S::PITCH + c * 16);
-      if (dst[it]) *dst[it] = MODE == OUT_ADD_F32 ? old[it] + piece : piece;
+      if (dst[it]) {
+        const f32x4 piece = *reinterpret_cast<const f32x4*>(lds + row * S::PITCH + c * 16);
+        *dst[it] = MODE == OUT_ADD_F32 ? old[it] + piece : piece;
+      }
     }
   }
 }
 
-// The q/k/v epilogue for a wave's TM x TN tiles of transposed 32 x 32 products: what
+// The q/k/v epilogue for a wave's TM x TN tiles of transposed products: what
 // belongs to a row (position, page, slot) is fetched once per row, what belongs to four
 // columns (head, place in the head, q or k or v) once per four columns.
-template <int TM, int TN>
+template <int TM, int TN, typename ACC>
 __device__ __forceinline__ void store_wave_qkv(void* C, int64_t ldc, int M, int N, int m_first, int n_first, int lane,
-                                               const f32x16 (&acc)[TM][TN], const QkvArgs& qkv) {
-  const int lrow = lane & 31, hd = qkv.lay.head_dim;
+                                               const ACC (&acc)[TM][TN], const QkvArgs& qkv) {
+  using T = TileOf<ACC>;
+  constexpr int R = T::R;
+  const int lrow = lane % R, hd = qkv.lay.head_dim;
   int pos[TM], slot[TM];
   int64_t page_base[TM];
   bool row_ok[TM];
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int m = m_first + i * 32 + lrow;
+    const int m = m_first + i * R + lrow;
     row_ok[i] = m < M;
     const int mm = row_ok[i] ? m : M - 1;
     pos[i] = qkv.positions[mm];
@@ -323,8 +344,8 @@ __device__ __forceinline__ void store_wave_qkv(void* C, int64_t ldc, int M, int 
 #pragma unroll
   for (int j = 0; j < TN; ++j)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = n_first + j * 32 + 8 * q + 4 * (lane >> 5);
+    for (int q = 0; q < T::Q; ++q) {
+      const int n = n_first + j * R + T::STEP * q + 4 * (lane / R);
       if (n >= N) continue;
       const int head = n / hd, d = n - head * hd;
       const bool is_q = head < qkv.num_heads, is_v = head >= qkv.num_heads + qkv.lay.kv_heads;
@@ -353,7 +374,7 @@ __device__ __forceinline__ void store_wave_qkv(void* C, int64_t ldc, int M, int 
         u32x2 o;
         o[0] = (uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16);
         o[1] = (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16);
-        const int m = m_first + i * 32 + lrow;
+        const int m = m_first + i * R + lrow;
         if (is_q) {
           *reinterpret_cast<u32x2*>((bf16_t*)C + (int64_t)m * ldc + n) = o;
         } else if (cache != nullptr) {
@@ -748,6 +769,20 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
   return 0;
 }
 
+// acc += w x for the 16 x 16 x 32 matrix instruction, written as the instruction itself with
+// the accumulator tied to one place in the accumulation registers: given the intrinsic for 48 or
+// 64 accumulators of four registers in a loop of two alternating operand sets, the compiler
+// moved them from place to place (three hundred register moves a K step, and spills).  What
+// the compiler then no longer knows, and the hardware does not check: the result may be read
+// by another kind of instruction only some cycles after the last matrix instruction
+// (accumulators_settle, once behind the loop); between matrix instructions on one accumulator
+// there are 47 others here, and the operands' waits the compiler still counts itself.
+__device__ __forceinline__ void multiply_16x16x32(f32x4& acc, const bf16x8& w, const bf16x8& x) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(x));
+}
+
+__device__ __forceinline__ void accumulators_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+
 // ------------------------------------ tiled, one wave a SIMD, loads into the LDS ---
 // Products with enough tiles of 256 rows to fill the chip.  A 128 x 128 tile at the
 // full matrix rate asks the L1 for 64 bytes a clock, which is all a CU has, and the LDS
@@ -850,77 +885,73 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
     for (int p = 0; p < CA + CW; ++p) load_one(kt, p);
   };
 
-  f32x16 acc[TM][TN];
+  // The matrix instruction is the 16 x 16 x 32 one: with operands as real ones are, the GPU
+  // sustains 2.1 PFLOP/s of it where it sustains 1.76 of the 32 x 32 x 16 one (both 2.5 on zeros):
+  // it passes an accumulator through the matrix pipe half as often for the same products, and the
+  // products of a layer are bound by power.  A wave's tile is TM16 x TN16 tiles of 16 x 16.
+  constexpr int TM16 = 2 * TM, TN16 = 2 * TN;
+  f32x4 acc[TM16][TN16];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TM16; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < TN16; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int lrow = lane & 31, h = lane >> 5;
-  // byte offsets of this lane's operand chunk for columns 0..15 and 16..31 of a step
-  uint32_t rd[2];
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks) rd[ks] = (uint32_t)(lrow * DROW) + (((uint32_t)(ks * 2 + h) ^ swizzle((uint32_t)lrow)) << 4);
+  // An operand of the instruction is 16 tile rows x 32 columns, a whole K step of a 1 KB block:
+  // lane l reads row l % 16, columns 8 (l / 16) .. + 7, which lie at chunk (l / 16) ^ f(row)
+  // (f depends on bits 2 and 3 of the row, which are the lane's own: blocks start at multiples of 16)
+  const int lrow = lane & 15;
+  const uint32_t rd = (uint32_t)(lrow * DROW) + ((((uint32_t)lane >> 4) ^ swizzle((uint32_t)lrow)) << 4);
   const uint32_t a_rd = (uint32_t)(wm * 32 * TM * DROW), w_rd = (uint32_t)(BM * DROW + wn * 32 * TN * DROW);
-  bf16x8 a[2][TM], b[2][TN];
-  auto read_operands = [&](int buf, int ks, bf16x8* af, bf16x8* bf) {
-    const char* tile = lds_bytes + buf * BUF + rd[ks];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 32 * DROW);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * DROW);
-  };
-
-  constexpr int RD = TM + TN, MF = TM * TN, LD = CA + CW;
-  load_step(0);
-  load_step(1);
-  load_step(2);
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LD) : "memory");     // K step 0 has landed
-  barrier_no_fence();
-  read_operands(0, 0, a[0], b[0]);
-
-  // One step in two stretches of MF matrix instructions with the barrier between them: columns
-  // 0..15 with the reads of columns 16..31 under the first matrix instructions of the stretch, so
-  // that the last read is READ_SPAN matrix instructions old when its value is needed; then the
-  // barrier; then columns 16..31 with the first reads of the next step.  The requests for K step
-  // kt + 3 (its buffer was last read in step kt - 1, before that step's barrier) are spread over
-  // the whole step, one for every 32 / LD matrix instructions: a request of a kilobyte keeps the
-  // CU's one address unit busy for 16 cycles, and the four waves ask at the same time.  At the
-  // barrier this wave's part of K step kt + 1 (asked for two steps ago) has landed when at most
-  // the loads of step kt + 2 and the first CA of this step are outstanding; after it everybody's
-  // has, and nobody reads this step's buffer any more.  No fence: it would wait for every load.
-  constexpr int READ_SPAN = MF / 2;
-  // (the order is written out and pinned: every matrix instruction with what follows it stands
-  // between two scheduling barriers)
-  auto read_one = [&](int buf, int ks, bf16x8* af, bf16x8* bf, int r) {      // in the order in which the products need them
-    const char* tile = lds_bytes + buf * BUF + rd[ks];
-    const int j = r - 1, i = r - TN;
+  constexpr int RD = TM16 + TN16, MF = TM16 * TN16, LD = CA + CW;
+  bf16x8 a[2][TM16], b[2][TN16];           // two sets: one is multiplied while the next step's is read
+  auto read_one = [&](int buf, bf16x8* af, bf16x8* bf, int r) {      // in the order in which the products need them
+    const char* tile = lds_bytes + buf * BUF + rd;
+    const int j = r - 1, i = r - TN16;
     if (r == 0) af[0] = *reinterpret_cast<const bf16x8*>(tile + a_rd);
-    else if (r <= TN) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * DROW);
-    else af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 32 * DROW);
+    else if (r <= TN16) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 16 * DROW);
+    else af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 16 * DROW);
   };
-  auto stretch = [&](const bf16x8* af, const bf16x8* bf, int rbuf, int rks, bf16x8* raf, bf16x8* rbf, int kt_load, int l0, int l1) {
+
+#pragma unroll
+  for (int s0 = 0; s0 < 4; ++s0) load_step(s0);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * LD) : "memory");     // K step 0 has landed
+  barrier_no_fence();
+#pragma unroll
+  for (int r = 0; r < RD; ++r) read_one(0, a[0], b[0], r);
+
+  // One K step: the barrier, then MF matrix instructions on the operands that the step before
+  // read, with the reads of the next step's operands under the first half of them and the
+  // requests for K step kt + 4 spread over all of them (a request of a kilobyte keeps the CU's
+  // one address unit busy for 16 cycles, and the four waves ask at the same time).  The order is
+  // written out and pinned: every matrix instruction with what follows it stands between two
+  // scheduling barriers.  In front of the barrier this wave's part of K step kt + 1 has landed
+  // (it was asked for three steps ago: at most the loads of two steps are outstanding) and its
+  // reads of K step kt are done; behind it everybody's, so that step kt + 1 can be read and the
+  // buffer of step kt be asked into.  No fence: it would wait for every load in flight.
+  constexpr int READ_SPAN = MF / 2;
+  auto step = [&](int kt, const bf16x8* af, const bf16x8* bf, bf16x8* raf, bf16x8* rbf) {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * LD) : "memory");
+    barrier_no_fence();
 #pragma unroll
     for (int g = 0; g < MF; ++g) {
-      const int i = g / TN, j = g % TN;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);   // transposed
+      const int i = g / TN16, j = g % TN16;
+      multiply_16x16x32(acc[i][j], bf[j], af[i]);   // transposed
       if (g < READ_SPAN) {
 #pragma unroll
-        for (int r = (RD * g) / READ_SPAN; r < (RD * (g + 1)) / READ_SPAN; ++r) read_one(rbuf, rks, raf, rbf, r);
+        for (int r = (RD * g) / READ_SPAN; r < (RD * (g + 1)) / READ_SPAN; ++r) read_one((kt + 1) & 3, raf, rbf, r);
       }
 #pragma unroll
-      for (int l = l0 + ((l1 - l0) * g) / MF; l < l0 + ((l1 - l0) * (g + 1)) / MF; ++l) load_one(kt_load, l);
+      for (int l = (LD * g) / MF; l < (LD * (g + 1)) / MF; ++l) load_one(kt + 4, l);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  for (int kt = 0; kt < ktiles; ++kt) {
-    stretch(a[0], b[0], kt & 3, 1, a[1], b[1], kt + 3, 0, CA);
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LD + CA) : "memory");
-    barrier_no_fence();
-    stretch(a[1], b[1], (kt + 1) & 3, 0, a[0], b[0], kt + 3, CA, LD);
+  int kt = 0;
+  for (; kt + 1 < ktiles; kt += 2) {
+    step(kt, a[0], b[0], a[1], b[1]);
+    step(kt + 1, a[1], b[1], a[0], b[0]);
   }
+  if (kt < ktiles) step(kt, a[0], b[0], a[1], b[1]);
+  accumulators_settle();
   // the repeats asked for past the end still write into this workgroup's LDS: let them
   // land before the wave can end and the LDS go to another workgroup
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -929,9 +960,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
                  : MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0)
                                     : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
   if constexpr (MODE == OUT_QKV) {
-    store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
+    store_wave_qkv<TM16, TN16>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
   } else {
-    using S = Stage<MODE, TN>;
+    using S = Stage<MODE, TN16, 16>;
     static_assert(4 * S::BYTES <= 4 * BUF, "the waves' strips fit in the LDS of the buffers");
     __syncthreads();      // nobody reads operands from the LDS any more
     const bool whole_rows = (ldc * S::ES) % 16 == 0 && (uintptr_t)C % 16 == 0 && n0 + wn * 32 * TN + 32 * TN <= N;
@@ -939,13 +970,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct_kernel(void* __restrict_
     with_gate_activation<MODE>(qkv.gate_act, [&](auto act) {
       constexpr int ACT = decltype(act)::value;
       if (whole_rows) {
-        store_wave_staged<MODE, TM, TN, ACT>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
+        store_wave_staged<MODE, TM16, TN16, ACT>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
       } else {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM16; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            store_tile_t<MODE, ACT>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+          for (int j = 0; j < TN16; ++j)
+            store_tile_t<MODE, ACT>(C, ldc, M, N, m0 + wm * 32 * TM + i * 16 + lrow, n0 + wn * 32 * TN + j * 16, lane, acc[i][j], vec);
       }
     });
   }
@@ -1040,87 +1071,92 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
     for (int p = 0; p < CA + CW; ++p) load_one(kt, buf, p);
   };
 
-  f32x16 acc[TM][TN];
+  // (the 16 x 16 x 32 matrix instruction, as in the kernel above: TM16 x TN16 tiles of 16 x 16 a wave)
+  constexpr int TM16 = 2 * TM, TN16 = 2 * TN;
+  f32x4 acc[TM16][TN16];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TM16; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < TN16; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int lrow = lane & 31, h = lane >> 5;
-  uint32_t rd[4];       // byte offsets of this lane's operand chunk for each 16 columns of a step
+  // An operand is 16 tile rows x 32 columns, half of the 64 columns of a step: lane l reads row
+  // l % 16, columns 32 kc + 8 (l / 16) .. + 7, which lie at chunk (4 kc + l / 16) ^ f(row); f takes
+  // bit 4 of the row too, which is the parity of the block of 16 rows.
+  const int lrow = lane & 15;
+  uint32_t rd[2][2];       // [half of the step][parity of the block of 16 rows]
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) rd[ks] = (uint32_t)(lrow * EROW) + (((uint32_t)(ks * 2 + h) ^ swizzle8((uint32_t)lrow)) << 4);
+  for (int kc = 0; kc < 2; ++kc)
+#pragma unroll
+    for (int odd = 0; odd < 2; ++odd)
+      rd[kc][odd] = (uint32_t)(lrow * EROW) + (((uint32_t)(kc * 4 + (lane >> 4)) ^ swizzle8((uint32_t)(lrow + 16 * odd))) << 4);
   const uint32_t a_rd = (uint32_t)(wm * 32 * TM * EROW), w_rd = (uint32_t)(BM * EROW + wn * 32 * TN * EROW);
-  bf16x8 a[2][TM], b[2][TN];
-  auto read_operands = [&](int buf, int ks, bf16x8* af, bf16x8* bf) {
-    const char* tile = lds_bytes + buf * BUF + rd[ks];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 32 * EROW);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * EROW);
+  constexpr int RD = TM16 + TN16, MF = TM16 * TN16, LD = CA + CW;
+  static_assert(LD % 2 == 0, "a step's requests go out in two halves");
+  bf16x8 a[2][TM16], b[2][TN16];           // one set a half step: one is multiplied while the next is read
+  auto read_one = [&](int buf, int kc, bf16x8* af, bf16x8* bf, int r) {      // in the order in which the products need them
+    const char* tile = lds_bytes + buf * BUF;
+    const int j = r - 1, i = r - TN16;
+    if (r == 0) af[0] = *reinterpret_cast<const bf16x8*>(tile + a_rd + rd[kc][0]);
+    else if (r <= TN16) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 16 * EROW + rd[kc][j & 1]);
+    else af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 16 * EROW + rd[kc][i & 1]);
   };
 
-  constexpr int RD = TM + TN, MF = TM * TN, LD = CA + CW;
+  // steps 0 and 1 and the first half of step 2 (the rule below: the second half of step kt + 2 goes
+  // out under the first half of step kt)
 #pragma unroll
-  for (int s = 0; s < NBUF - 1; ++s) load_step(s, s);
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 2) * LD) : "memory");     // K step 0 has landed
+  for (int s0 = 0; s0 < 2; ++s0) load_step(s0, s0);
+#pragma unroll
+  for (int p = 0; p < LD / 2; ++p) load_one(2, 2, p);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LD + LD / 2) : "memory");     // K step 0 has landed
   barrier_no_fence();
-  read_operands(0, 0, a[0], b[0]);
+#pragma unroll
+  for (int r = 0; r < RD; ++r) read_one(0, 0, a[0], b[0], r);
 
-  // One step of 64 columns in four quarters of MF matrix instructions; the order is written out
-  // and pinned (every matrix instruction with what follows it stands between two scheduling
-  // barriers).  Under a quarter's first matrix instructions go the reads of the next quarter's
-  // operands.  The requests for K step kt + NBUF - 1 (its buffer was last read in step kt - 1,
-  // before that step's barrier) are spread over the first three quarters, one for every second
-  // matrix instruction: a request of a kilobyte keeps the CU's one address unit busy for 16
-  // cycles, and the four waves ask at the same time.  The barrier stands in front of the last
-  // quarter: this wave's part of K step kt + 1 has landed when at most the loads of NBUF - 2
-  // steps are outstanding; after it everybody's has, and nobody reads this step's buffer any more.
-  auto read_one = [&](int buf, int ks, bf16x8* af, bf16x8* bf, int r) {      // in the order in which the products need them
-    const char* tile = lds_bytes + buf * BUF + rd[ks];
-    const int j = r - 1, i = r - TN;
-    if (r == 0) af[0] = *reinterpret_cast<const bf16x8*>(tile + a_rd);
-    else if (r <= TN) bf[j] = *reinterpret_cast<const bf16x8*>(tile + w_rd + j * 32 * EROW);
-    else af[i] = *reinterpret_cast<const bf16x8*>(tile + a_rd + i * 32 * EROW);
-  };
-  constexpr int READ_SPAN = MF < RD ? MF : RD;
-  auto quarter = [&](const bf16x8* af, const bf16x8* bf, int rbuf, int rks, bf16x8* raf, bf16x8* rbf, int kt_load, int lbuf,
-                     int l0, int l1) {
+  // One step of 64 columns in two halves of MF matrix instructions with the barrier between
+  // them; the order is written out and pinned (every matrix instruction with what follows it
+  // stands between two scheduling barriers).  Under a half's first matrix instructions go the
+  // reads of the next half's operands.  Requests, one for every fifth matrix instruction or so (a
+  // request of a kilobyte keeps the CU's one address unit busy for 16 cycles, and the four waves
+  // ask at the same time): under the first half the second half of K step kt + 2 (its buffer was
+  // last read in step kt - 1, before that step's barrier), under the second half the first half
+  // of K step kt + 3, into this step's buffer, which nobody reads behind the barrier.  In front
+  // of the barrier this wave's part of K step kt + 1 has landed when at most the loads of one
+  // step are outstanding; behind it everybody's has.  No fence: it would wait for every load.
+  static_assert(NBUF == 3, "the requests' order is written for three buffers");
+  constexpr int READ_SPAN = MF / 2;
+  auto half = [&](const bf16x8* af, const bf16x8* bf, int rbuf, int rkc, bf16x8* raf, bf16x8* rbf, int kt_load, int lbuf, int l0) {
 #pragma unroll
     for (int g = 0; g < MF; ++g) {
-      const int i = g / TN, j = g % TN;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);   // transposed
+      const int i = g / TN16, j = g % TN16;
+      multiply_16x16x32(acc[i][j], bf[j], af[i]);   // transposed
       if (g < READ_SPAN) {
 #pragma unroll
-        for (int r = (RD * g) / READ_SPAN; r < (RD * (g + 1)) / READ_SPAN; ++r) read_one(rbuf, rks, raf, rbf, r);
+        for (int r = (RD * g) / READ_SPAN; r < (RD * (g + 1)) / READ_SPAN; ++r) read_one(rbuf, rkc, raf, rbf, r);
       }
 #pragma unroll
-      for (int l = l0 + ((l1 - l0) * g) / MF; l < l0 + ((l1 - l0) * (g + 1)) / MF; ++l) load_one(kt_load, lbuf, l);
+      for (int l = (LD / 2 * g) / MF; l < (LD / 2 * (g + 1)) / MF; ++l) load_one(kt_load, lbuf, l0 + l);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   int rb = 0;                                   // kt % NBUF
   for (int kt = 0; kt < ktiles; ++kt) {
     const int lb = rb == 0 ? NBUF - 1 : rb - 1, nb = rb == NBUF - 1 ? 0 : rb + 1;
-    quarter(a[0], b[0], rb, 1, a[1], b[1], kt + NBUF - 1, lb, 0, LD / 3);
-    quarter(a[1], b[1], rb, 2, a[0], b[0], kt + NBUF - 1, lb, LD / 3, 2 * LD / 3);
-    quarter(a[0], b[0], rb, 3, a[1], b[1], kt + NBUF - 1, lb, 2 * LD / 3, LD);
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NBUF - 2) * LD) : "memory");
+    half(a[0], b[0], rb, 1, a[1], b[1], kt + 2, lb, LD / 2);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LD) : "memory");
     barrier_no_fence();
-    quarter(a[1], b[1], nb, 0, a[0], b[0], 0, 0, 0, 0);
+    half(a[1], b[1], nb, 0, a[0], b[0], kt + 3, rb, 0);
     rb = nb;
   }
+  accumulators_settle();
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   const bool vec = MODE == OUT_SWIGLU ? (ldc % 2 == 0 && (uintptr_t)C % 4 == 0)
                  : MODE == OUT_BF16 ? (ldc % 4 == 0 && (uintptr_t)C % 8 == 0)
                                     : (ldc % 4 == 0 && (uintptr_t)C % 16 == 0);
   if constexpr (MODE == OUT_QKV) {
-    store_wave_qkv<TM, TN>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
+    store_wave_qkv<TM16, TN16>(C, ldc, M, N, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc, qkv);
   } else {
-    using S = Stage<MODE, TN>;
+    using S = Stage<MODE, TN16, 16>;
     static_assert(4 * S::BYTES <= NBUF * BUF, "the waves' strips fit in the LDS of the buffers");
     __syncthreads();      // nobody reads operands from the LDS any more
     const bool whole_rows = (ldc * S::ES) % 16 == 0 && (uintptr_t)C % 16 == 0 && n0 + wn * 32 * TN + 32 * TN <= N;
@@ -1128,13 +1164,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_direct64_kernel(void* __restric
     with_gate_activation<MODE>(qkv.gate_act, [&](auto act) {
       constexpr int ACT = decltype(act)::value;
       if (whole_rows) {
-        store_wave_staged<MODE, TM, TN, ACT>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
+        store_wave_staged<MODE, TM16, TN16, ACT>(lds_bytes + wave * S::BYTES, C, ldc, M, m0 + wm * 32 * TM, n0 + wn * 32 * TN, lane, acc);
       } else {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM16; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            store_tile_t<MODE, ACT>(C, ldc, M, N, m0 + wm * 32 * TM + i * 32 + lrow, n0 + wn * 32 * TN + j * 32, lane, acc[i][j], vec);
+          for (int j = 0; j < TN16; ++j)
+            store_tile_t<MODE, ACT>(C, ldc, M, N, m0 + wm * 32 * TM + i * 16 + lrow, n0 + wn * 32 * TN + j * 16, lane, acc[i][j], vec);
       }
     });
   }
