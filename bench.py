@@ -109,8 +109,8 @@ def yardsticks():
         return min(times)
     read_s = best(lambda: ops.read_stream(buf, 2048, True))
     flops = ops.mfma_loop(1, 1)
-    mfma_s = best(lambda: ops.mfma_loop(2000, 2048))
-    flops = flops * 2000 * 2048
+    mfma_s = best(lambda: ops.mfma_loop(1000, 2048))
+    flops = flops * 1000 * 2048
     del buf
     torch.cuda.empty_cache()
     return (4 << 30) / read_s / 1e9, flops / mfma_s / 1e12

@@ -268,10 +268,32 @@ __device__ __forceinline__ void store_wave_staged(char* lds, void* C, int64_t ld
   using T = TileOf<ACC>;
   constexpr int R = T::R;
   using S = Stage<MODE, TN, R>;
+  constexpr int TOTAL = R * S::CHUNKS, PIECES = (TOTAL + 63) / 64;      // 16-byte pieces of a strip, and per lane
   const int lrow = lane % R, h = lane / R;
   char* crow = (char*)C + ((int64_t)m_first * ldc + (MODE == OUT_SWIGLU ? n_first / 2 : n_first)) * S::ES;
+  // where piece `it` of this lane in strip i goes (null: nowhere)
+  auto place = [&](int i, int it) -> f32x4* {
+    const int idx = lane + 64 * it, row = idx / S::CHUNKS, c = idx - row * S::CHUNKS;
+    return idx < TOTAL && m_first + i * R + row < M
+               ? reinterpret_cast<f32x4*>(crow + (int64_t)(i * R + row) * ldc * S::ES + c * 16) : nullptr;
+  };
+  // What is added to is asked for a strip ahead: with the strips one after the other each would
+  // wait for its own values from memory (eight strips of 16 rows: 78 us against 74.6 for four of 32,
+  // output product of the 8B shape).
+  f32x4 old[2][PIECES];
+  auto ask_old = [&](int i, f32x4* into) {
+    if constexpr (MODE == OUT_ADD_F32) {
+#pragma unroll
+      for (int it = 0; it < PIECES; ++it) {
+        const f32x4* p = place(i, it);
+        if (p) into[it] = *p;
+      }
+    }
+  };
+  ask_old(0, old[0]);
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
+    if (i + 1 < TM) ask_old(i + 1, old[(i + 1) & 1]);
     char* mine = lds + lrow * S::PITCH;
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -294,23 +316,13 @@ __device__ __forceinline__ void store_wave_staged(char* lds, void* C, int64_t ld
         }
       }
     // (the same wave wrote what it reads: its LDS instructions keep their order)
-    constexpr int TOTAL = R * S::CHUNKS, PIECES = (TOTAL + 63) / 64;      // 16-byte pieces of the strip, and per lane
-    f32x4* dst[PIECES];
-    f32x4 old[PIECES];
 #pragma unroll
     for (int it = 0; it < PIECES; ++it) {
       const int idx = lane + 64 * it, row = idx / S::CHUNKS, c = idx - row * S::CHUNKS;
-      dst[it] = idx < TOTAL && m_first + i * R + row < M
-                    ? reinterpret_cast<f32x4*>(crow + (int64_t)(i * R + row) * ldc * S::ES + c * 16) : nullptr;
-      // what is added to: every piece asked for before the first is needed
-      if (MODE == OUT_ADD_F32 && dst[it]) old[it] = *dst[it];
-    }
-#pragma unroll
-    for (int it = 0; it < PIECES; ++it) {
-      const int idx = lane + 64 * it, row = idx / S::CHUNKS, c = idx - row * S::CHUNKS;
-      if (dst[it]) {
+      f32x4* dst = place(i, it);
+      if (dst) {
         const f32x4 piece = *reinterpret_cast<const f32x4*>(lds + row * S::PITCH + c * 16);
-        *dst[it] = MODE == OUT_ADD_F32 ? old[it] + piece : piece;
+        *dst = MODE == OUT_ADD_F32 ? old[i & 1][it] + piece : piece;
       }
     }
   }
@@ -794,12 +806,14 @@ __device__ __forceinline__ void accumulators_settle() { asm volatile("s_nop 15\n
 //    (buffer_load_dwordx4 ... lds: lane l of a wave writes bytes 16 l .. 16 l + 15 of a
 //    1 KB block), so no register stage and no LDS write instruction stands between the
 //    matrix instructions.  Four LDS buffers of one K step each: a step is asked from
-//    memory three steps before it is multiplied.
+//    memory four steps before it is multiplied, and read into registers one step before.
 //  * A 1 KB block is 16 tile rows of 64 bytes, unpadded; the four 16-byte chunks of row
 //    r are stored in the order c ^ f(r), f(r) = bit 3 of r | bit 2 of r << 1: of the
 //    functions whose bits are parities of row bits, the hardware's conflict counter
-//    showed none for this one on a wave's 16-byte operand reads (rows lane % 32, chunks
-//    2 ks + lane / 32), and two-way conflicts for e.g. ((r >> 1) ^ (r >> 3)) & 3.
+//    showed none for this one on a wave's 16-byte operand reads of 32 rows (rows lane % 32,
+//    chunks 2 ks + lane / 32, the operand of the 32 x 32 x 16 instruction), and two-way
+//    conflicts for e.g. ((r >> 1) ^ (r >> 3)) & 3; an operand of the 16 x 16 x 32 instruction
+//    is one such block whole (row lane % 16, chunk lane / 16), every bank once whatever f.
 //  * The one barrier of a step stands where the wave has nothing outstanding in the LDS,
 //    and carries no fence (a fence would wait for every load in flight); what must have
 //    landed is waited for by count.
@@ -807,14 +821,16 @@ __device__ __forceinline__ void accumulators_settle() { asm volatile("s_nop 15\n
 //    it between two scheduling barriers: what does not stand between two matrix
 //    instructions is not overlapped with them, and a burst of requests from four waves in
 //    step queues at the CU's one address unit while the matrix pipes run dry.
-//  * The kernel is bound by power, not by its schedule: by the cycle counter and the
-//    constant-rate counter read around the loop (K = 8,192, all CUs busy), a loop of the
-//    matrix instructions alone takes 32.7 cycles an instruction at 1.82 GHz; with the LDS
-//    reads and the barrier 36.7 at 1.68; with the requests too, all to one address, 37.3 at
-//    1.47; the whole loop 36.0 at 1.39 (38.9 at 1.42 while the requests of a step stood
-//    together under a quarter of its matrix instructions).  After an idle gap the same loop
-//    runs at 1.94 GHz and 54.6 cycles an instruction: the same 0.85 us a step.  Three, four
-//    or five LDS buffers make no difference either.
+//  * The kernel is bound by power, not by its schedule.  With the 32 x 32 x 16 instruction, by
+//    the cycle counter and the constant-rate counter read around the loop (K = 8,192, all CUs
+//    busy): a loop of the matrix instructions alone took 32.7 cycles an instruction at 1.82
+//    GHz; with the LDS reads and the barrier 36.7 at 1.68; with the requests too, all to one
+//    address, 37.3 at 1.47; the whole loop 36.0 at 1.39 (38.9 at 1.42 while the requests of a
+//    step stood together under a quarter of its matrix instructions); after an idle gap the
+//    same loop ran at 1.94 GHz and 54.6 cycles an instruction, the same 0.85 us a step; three,
+//    four or five LDS buffers made no difference.  Hence the 16 x 16 x 32 instruction (see the
+//    kernel): the same loop 18.4 cycles an instruction of half the size at 1.55 GHz, 195 us
+//    where it took 212.
 //  * The products are formed transposed (weights as the row operand): a lane then holds
 //    four consecutive columns of one row of C and stores them with one instruction.
 // K must be a multiple of 32 and every row's byte offset must fit 31 bits.

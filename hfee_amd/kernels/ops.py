@@ -182,7 +182,7 @@ def read_stream(t: torch.Tensor, workgroups: int = 2048, keep_out_of_l2: bool = 
 def mfma_loop(iterations: int, workgroups: int) -> float:
     """Launches a loop of nothing but bfloat16 matrix instructions; returns the flops it does."""
     lib.core().call("hfee_mfma_loop", None, int(iterations), int(workgroups), _stream())
-    return float(workgroups) * 4 * iterations * 8 * 2 * 32 * 32 * 16
+    return float(workgroups) * 4 * iterations * 64 * 2 * 16 * 16 * 32
 
 
 # ---------------------------------------------------------------- matrix product
