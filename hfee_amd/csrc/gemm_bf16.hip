@@ -793,7 +793,10 @@ __device__ __forceinline__ void multiply_16x16x32(f32x4& acc, const bf16x8& w, c
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(x));
 }
 
-__device__ __forceinline__ void accumulators_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+__device__ __forceinline__ void accumulators_settle() {
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);       // (no read of an accumulator is moved up in front of the wait)
+}
 
 // ------------------------------------ tiled, one wave a SIMD, loads into the LDS ---
 // Products with enough tiles of 256 rows to fill the chip.  A 128 x 128 tile at the
