@@ -132,6 +132,27 @@ HFEE_API int hfee_embed(float* out, const void* table, int table_dtype, const in
   return 0;
 }
 
+// ------------------------------------------------------------- rows as they are
+// out[r] = x[rows[r] or r], rounded to the output's type: what stands where a norm would,
+// in a model that has none there.  One block per output row.
+template <typename TOut>
+__global__ void cast_rows_kernel(TOut* __restrict__ out, const float* __restrict__ x, const int* __restrict__ rows, int d) {
+  const int r = blockIdx.x;
+  const float* xr = x + (int64_t)(rows ? rows[r] : r) * d;
+  TOut* o = out + (int64_t)r * d;
+  for (int j = threadIdx.x; j < d; j += blockDim.x) o[j] = from_float<TOut>(xr[j]);
+}
+
+HFEE_API int hfee_cast_rows(void* out, int out_dtype, const float* x, const int* rows, int n, int d, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && d > 0, "cast_rows: bad sizes n=%d d=%d", n, d);
+  if (n == 0) return 0;
+  if (out_dtype == DT_F32) cast_rows_kernel<float><<<n, 256, 0, stream>>>((float*)out, x, rows, d);
+  else if (out_dtype == DT_BF16) cast_rows_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)out, x, rows, d);
+  else return fail("cast_rows: unknown dtype %d", out_dtype);
+  HFEE_CHECK_LAUNCH("cast_rows");
+  return 0;
+}
+
 // -------------------------------------------------------------------- RMSNorm
 // One block per output row.  rows == nullptr: row r of x; else row rows[r] of x.
 template <typename TOut, typename TW>

@@ -26,6 +26,7 @@ _CORE_SIGNATURES = {
     "hfee_embed": [P, P, I, P, I, I, P],
     "hfee_embed_emit": [P, P, P, I, I, P, I, P, L, P, L, P],
     "hfee_rmsnorm": [P, I, P, P, I, P, F, I, I, P],
+    "hfee_cast_rows": [P, I, P, P, I, I, P],
     "hfee_swiglu": [P, L, P, P, L, I, I, I, I, I, P],
     "hfee_residual_add": [P, P, I, L, P],
     "hfee_rope_cache_write": [P, L, P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, P, I, I, I, I, I, I, P],

@@ -122,6 +122,20 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
                     float(eps), n, d, _stream())
 
 
+def cast_rows(out: torch.Tensor, x: torch.Tensor, rows: torch.Tensor | None = None):
+    """out[r] = x[rows[r] or r] in out's type; x float32.  (What a model without a norm at some place
+    has there.)"""
+    _gpu(out, x, rows)
+    n, d, _ = _rows2d(out, "cast_rows out")
+    _check(out.is_contiguous() and x.is_contiguous() and x.dtype == torch.float32, "cast_rows: contiguous float32 x")
+    _check(x.dim() == 2 and x.shape[1] == d, "cast_rows: width mismatch")
+    if rows is None:
+        _check(x.shape[0] >= n, "cast_rows: fewer input rows than output rows")
+    else:
+        _i32(rows, "cast_rows rows", n)
+    lib.core().call("hfee_cast_rows", _ptr(out), _dt(out), _ptr(x), _ptr(rows), n, d, _stream())
+
+
 # the activations of a gated feed-forward's gate, as the kernels number them (GATE_SILU ... in csrc/common.h)
 GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "gelu": 2, "relu": 3}
 

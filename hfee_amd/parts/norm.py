@@ -1,5 +1,6 @@
 """RMSNorm (/root/reference/internal/ggml/ops.go:124-134): y = x / sqrt(mean(x^2) + eps) * w,
-the sum in float32, x the float32 residual stream, y in the engine's dtype."""
+the sum in float32, x the float32 residual stream, y in the engine's dtype; and "none" for a
+place where a model has no norm (the rows as they are, in the engine's dtype)."""
 from __future__ import annotations
 
 from ..config.specs import NormSpec
@@ -27,3 +28,17 @@ class RMSNorm(Norm):
 
     def forward(self, ctx, out, x, rows=None):
         ops.rmsnorm(out, x, self.weight, self.eps, rows)
+
+
+@register_norm("none")
+class NoNorm(Norm):
+    """Stands where an arrangement expects a norm and the model has none (no final norm before
+    the head, a block whose sub-layers read the stream as it is): no tensor, nothing to fold into
+    a product; the rows go to the part behind it rounded to the engine's dtype."""
+    graph_safe = True
+
+    def __init__(self, spec: NormSpec, name: str):
+        self.width = spec.width
+
+    def forward(self, ctx, out, x, rows=None):
+        ops.cast_rows(out, x, rows)

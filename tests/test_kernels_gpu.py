@@ -52,6 +52,21 @@ def test_rmsnorm(n, d, out_dtype):
     close(out2, ref2, 1e-5 if out_dtype == torch.float32 else 1e-2)
 
 
+@pytest.mark.parametrize("n,d", [(1, 7), (5, 1027), (300, 72)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rows_as_they_are(n, d, out_dtype):
+    """What stands where a model has no norm: the rows, all or gathered, rounded once."""
+    from hfee_amd.kernels import ops
+    x = torch.randn(n, d, generator=torch.Generator().manual_seed(n + d)) * 3
+    out = torch.empty(n, d, dtype=out_dtype, device=DEV)
+    ops.cast_rows(out, x.to(DEV))
+    assert torch.equal(out.cpu(), x.to(out_dtype))
+    rows = torch.tensor([n - 1, 0, n // 2], dtype=torch.int32, device=DEV)
+    out2 = torch.full((3, d), 7.0, dtype=out_dtype, device=DEV)
+    ops.cast_rows(out2, x.to(DEV), rows)
+    assert torch.equal(out2.cpu(), x[[n - 1, 0, n // 2]].to(out_dtype))
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (7, 33, 100), (64, 64, 16), (65, 130, 1027), (3, 172, 64), (200, 96, 172)])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_gemm_f32(M, N, K, accumulate):

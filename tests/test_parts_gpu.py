@@ -1015,3 +1015,58 @@ def test_toy_parts_of_every_kind_without_a_change_to_the_framework(tmp_path):
         x = x + (h @ t[w_name].t()) * (1 + at % 2)[:, None] + 0.01 * at[:, None]
     want = plain_rmsnorm(x, t["e.norm.weight"], 1e-5) @ t["e.embed.weight"].t() * 0.5
     assert torch.allclose(got, want, atol=2e-4, rtol=2e-4), float((got - want).abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_model_with_no_norm_at_two_places(tmp_path, dtype):
+    """The norm kind "none" where an arrangement expects a norm: a toy architecture, registered
+    here, that is the dense decoder without its final norm and without the norm in front of the
+    second layer's feed-forward.  A prompt of 70 tokens in one step (the kernels for many rows),
+    then tokens one by one (the streaming kernels, whose fused norms must stand back), against
+    the plain model with the same two norms left out."""
+    import hfee_amd  # noqa: F401
+    from conftest import make_model_folder
+    from hfee_amd.config import NormSpec, register_architecture
+    from hfee_amd.config.llama import LlamaConfig
+    from hfee_amd.engine import Engine, StepEntry, load_model
+    from hfee_amd.models.llama import llama_model_spec
+    from plain_llama import PlainLlama, plain_matmul, plain_swiglu
+
+    def spec_without(cfg):
+        spec = llama_model_spec(cfg)
+        none = NormSpec("none", cfg.hidden_size, 0.0)
+        layers = list(spec.layers)
+        layers[1] = replace(layers[1], feed_forward_norm=none)
+        return replace(spec, layers=tuple(layers), final_norm=none)
+
+    register_architecture("ToyFewerNormsForCausalLM", LlamaConfig, spec_without)
+    cj = dict(TINY_A, architectures=["ToyFewerNormsForCausalLM"], num_hidden_layers=2, hidden_size=72, intermediate_size=104,
+              num_attention_heads=3, num_key_value_heads=1, head_dim=16, vocab_size=211, tie_word_embeddings=False)
+    folder = make_model_folder(tmp_path / "m", cj, seed=8, dtype=dtype, std=0.1, norm_init="one_plus_normal")
+    model, _ = load_model(folder, dtype)
+    names = {s.name for s in model.tensor_specs()}
+    assert "model.norm.weight" not in names and "model.layers.1.post_attention_layernorm.weight" not in names
+    assert "model.layers.0.post_attention_layernorm.weight" in names
+
+    class Plain(PlainLlama):
+        def feed_forward_sublayer(self, x, l):
+            if l != 1:
+                return super().feed_forward_sublayer(x, l)
+            w, p, xb = self.w, f"model.layers.{l}.", self.r(x)
+            h = plain_swiglu(plain_matmul(xb, w[p + "mlp.gate_proj.weight"]), plain_matmul(xb, w[p + "mlp.up_proj.weight"]), self.act)
+            return plain_matmul(self.r(h), w[p + "mlp.down_proj.weight"])
+
+        def head(self, x):
+            return plain_matmul(self.r(x), self.w["lm_head.weight"])
+
+    toks = tu.make_requests(211, [76], seed=5)["r0"]
+    eng = Engine(model, num_pages=8, page_size=16, max_requests=2, max_batch_tokens=128)
+    eng.admit("a")
+    got = [eng.step([StepEntry("a", toks[:70], list(range(70)))]).double().cpu()]
+    for t in range(70, 76):
+        got.append(eng.step([StepEntry("a", toks[t:t + 1], [0])]).double().cpu())
+    got = torch.cat(got)
+    eng.cache.check()
+    want = Plain(folder).forward(toks).double().cpu()
+    worst = float(((got - want).abs().amax(1) / want.abs().amax(1)).max())
+    assert worst < (3e-5 if dtype == "float32" else 5e-2), worst
