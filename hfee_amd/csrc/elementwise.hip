@@ -8,6 +8,8 @@
 //   rotation    internal/llm/forward.go:180-196, cache write forward.go:99-101
 //   SiLU gate   internal/ggml/ops.go:159-165  (g / (1 + exp(-g)) * up)
 //   residual    internal/ggml/ops.go:152-157
+#include <type_traits>
+
 #include "common.h"
 #include "gemm_entry.h"
 
@@ -406,27 +408,34 @@ __global__ void rope_cache_pairs_kernel(bf16_t* __restrict__ q, int64_t ldq, con
       x.u = *reinterpret_cast<const u32x4*>(row);
       return x;
     }
-    constexpr int MOST = 8;
-    const float* p = cuts.at + (int64_t)t * cuts.ld + col;
-    f32x4 lo[MOST], hi[MOST];
+    // (all cuts asked for together, up to 2, 4 or 8 of them; past the last one: a repeat that is not
+    // added.  Always eight, two cuts of a 512-token portion cost the kernel twice the plain one's time.)
+    auto sum_of = [&](auto most) {
+      constexpr int MOST = decltype(most)::value;
+      const float* p = cuts.at + (int64_t)t * cuts.ld + col;
+      f32x4 lo[MOST], hi[MOST];
 #pragma unroll
-    for (int z = 0; z < MOST; ++z) {      // all asked for together; past the last one: a repeat that is not added
-      const float* pz = p + (int64_t)min(z, cuts.count - 1) * cuts.stride;
-      lo[z] = *reinterpret_cast<const f32x4*>(pz);
-      hi[z] = *reinterpret_cast<const f32x4*>(pz + 4);
-    }
-    f32x4 a = lo[0], b = hi[0];
-#pragma unroll
-    for (int z = 1; z < MOST; ++z)
-      if (z < cuts.count) {
-        a += lo[z];
-        b += hi[z];
+      for (int z = 0; z < MOST; ++z) {
+        const float* pz = p + (int64_t)min(z, cuts.count - 1) * cuts.stride;
+        lo[z] = *reinterpret_cast<const f32x4*>(pz);
+        hi[z] = *reinterpret_cast<const f32x4*>(pz + 4);
       }
+      f32x4 a = lo[0], b = hi[0];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      x.e[i] = float_to_bf16(a[i]);
-      x.e[4 + i] = float_to_bf16(b[i]);
-    }
+      for (int z = 1; z < MOST; ++z)
+        if (z < cuts.count) {
+          a += lo[z];
+          b += hi[z];
+        }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        x.e[i] = float_to_bf16(a[i]);
+        x.e[4 + i] = float_to_bf16(b[i]);
+      }
+    };
+    if (cuts.count <= 2) sum_of(std::integral_constant<int, 2>{});
+    else if (cuts.count <= 4) sum_of(std::integral_constant<int, 4>{});
+    else sum_of(std::integral_constant<int, 8>{});
     return x;
   };
   // Some workgroups take the values of 16 consecutive tokens each.  The cache keeps values

@@ -701,9 +701,13 @@ int raise_pipelined_lds(size_t lds) {
 // than 256 tiles (384 where K is long) a part of the chip stands idle while a few workgroups walk the whole of K
 // (the output and down products of a prompt of 128 tokens: 32 tiles); the cut makes up to
 // 512 workgroups of them, each with at least 512 columns.
+inline bool cuts_by_large_tiles(int M, int N, int K, int splits, int k_split);
+
 inline int pipelined_splits(int M, int N, int K) {
   const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
-  const bool long_k = K >= 8192;
+  // (two cuts pay where K is long, and from K = 4,096 on where the kernel of 256 x 128 tiles makes them and
+  // they fill the chip: 512 to 1,024 rows against 4,096 to 6,144 weight rows, half a round of its tiles whole)
+  const bool long_k = K >= 8192 || (K >= 4096 && K % 128 == 0 && cuts_by_large_tiles(M, N, K, 2, K / 2));
   if (M <= 64 || tiles >= (long_k ? 384 : 256) || K < 2048 || N % 4 != 0) return 1;
   // (two workgroups of this kernel fit a CU; measured, a prompt of 128 tokens is faster with one a CU
   // and fewer partial products, one of 512 tokens with two; two cuts only pay where K is long)
@@ -1539,13 +1543,19 @@ HFEE_API int hfee_gemm_bf16_cuts(const void* A, int64_t lda, const void* W, int6
   const int splits = pipelined_splits(M, N, K);
   if (plan.first != 2 || plan.second != 0 || splits < 2 || scratch_floats < (int64_t)splits * M * N) return 0;
   constexpr int TM = 2, TN = 2, STAGES = 3;
-  const size_t lds = (size_t)2 * (64 * TM + 64 * TN) * PPITCH * sizeof(bf16_t);
-  if (raise_pipelined_lds<OUT_F32>(lds)) return 1;
-  const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
-  dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS), splits);
   const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
-  gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
-      scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, k_split, (int64_t)M * N);
+  if (cuts_by_large_tiles(M, N, K, splits, k_split) && large_fits(lda, ldw, M, N, K)) {
+    if (launch_direct64<OUT_F32, 4, 2, 3>(scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, stream,
+                                          k_split, splits, (int64_t)M * N))
+      return 1;
+  } else {
+    const size_t lds = (size_t)2 * (64 * TM + 64 * TN) * PPITCH * sizeof(bf16_t);
+    if (raise_pipelined_lds<OUT_F32>(lds)) return 1;
+    const int64_t tiles = (int64_t)((N + 64 * TN - 1) / (64 * TN)) * ((M + 64 * TM - 1) / (64 * TM));
+    dim3 grid((unsigned)((tiles + XCDS - 1) / XCDS * XCDS), splits);
+    gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
+        scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, k_split, (int64_t)M * N);
+  }
   HFEE_CHECK_LAUNCH("gemm_bf16_cuts");
   *cuts = splits;
   return 0;

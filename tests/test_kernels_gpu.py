@@ -125,14 +125,16 @@ def test_gemm_bf16(M, N, K, kernel, mode):
 
 
 @pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 640, 2112),
-                                   (100, 2048, 2048), (512, 4096, 8192), (1000, 2048, 8256), (2048, 2048, 8192)])
+                                   (100, 2048, 2048), (512, 4096, 8192), (1000, 2048, 8256), (2048, 2048, 8192),
+                                   (1024, 4096, 4096), (768, 4096, 4096), (512, 6144, 4096)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "add"])
 def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
     """Products with too few 128 x 128 tiles for the chip: given scratch, K is cut over up to
     eight times as many workgroups and a second kernel adds the partial products (K that is
     no multiple of the cut, M and N that are no multiples of a tile; the last three sizes: the
     cuts made by the kernel of 256 x 128 tiles, whole tiles of rows and not, a last cut that is
-    shorter); the same numbers as without scratch up to the order of the sums."""
+    shorter; then three more by that kernel: two cuts of K = 4,096, half a round of its tiles each);
+    the same numbers as without scratch up to the order of the sums."""
     from hfee_amd.kernels import ops
     g = torch.Generator().manual_seed(M + 3 * N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -165,7 +167,7 @@ def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
 
 @pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 4096, 2112),
                                    (100, 2052, 2048), (100, 512, 1024), (70, 1001, 2048), (2048, 512, 1024), (40, 512, 2048),
-                                   (90, 260, 2050), (512, 4096, 8192), (1000, 2048, 8256)])
+                                   (90, 260, 2050), (512, 4096, 8192), (1000, 2048, 8256), (1024, 4096, 4096)])
 @pytest.mark.parametrize("weight_dtype", [torch.float32, torch.bfloat16])
 def test_product_that_adds_into_the_stream_and_goes_on_with_the_norm(M, N, K, weight_dtype):
     """The product that adds into the residual stream together with the norm of the new rows:
@@ -895,7 +897,8 @@ def test_rope_cache_write(pairing, dtype):
 
 @pytest.mark.parametrize("H,K,hd,rotary,d,n,portions", [(8, 2, 64, 64, 2048, 100, True), (4, 4, 128, 128, 4096, 65, False),
                                                         (6, 2, 48, 32, 2304, 130, True), (8, 2, 64, 0, 2048, 70, True),
-                                                        (8, 2, 64, 64, 1024, 100, True), (8, 2, 64, 64, 2048, 40, True)])
+                                                        (8, 2, 64, 64, 1024, 100, True), (8, 2, 64, 64, 2048, 40, True),
+                                                        (32, 8, 128, 128, 4096, 512, True)])     # (two cuts by 256 x 128 tiles)
 def test_rotation_that_adds_up_a_cut_product(H, K, hd, rotary, d, n, portions):
     """The q/k/v product of a portion cut along K, its partial products added up by the
     rotation kernel on its way to q and to the cache: bit-equal to the product (with the kernel
@@ -919,7 +922,9 @@ def test_rotation_that_adds_up_a_cut_product(H, K, hd, rotary, d, n, portions):
         first = n // 2
         pos = torch.cat([torch.arange(32, 32 + first), torch.arange(5, 5 + n - first)]).to(torch.int32)
         seg = torch.cat([torch.zeros(first), torch.ones(n - first)]).to(torch.int32)
-        tables = torch.stack([torch.randperm(24, generator=g)[:16], 24 + torch.randperm(24, generator=g)[:16]]).to(torch.int32)
+        per = max(16, (32 + first + ps - 1) // ps)
+        tables = torch.stack([torch.randperm(per + 8, generator=g)[:per],
+                              per + 8 + torch.randperm(per + 8, generator=g)[:per]]).to(torch.int32)
     else:             # one token each of n sequences
         pos = torch.randint(0, 200, (n,), generator=g).to(torch.int32)
         seg = torch.arange(n, dtype=torch.int32)
