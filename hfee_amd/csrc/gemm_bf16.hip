@@ -697,17 +697,42 @@ int raise_pipelined_lds(size_t lds) {
   return 0;
 }
 
-// How many ways K is cut for M x N x K through 128 x 128 tiles (1: not at all): with fewer
-// than 256 tiles (384 where K is long) a part of the chip stands idle while a few workgroups walk the whole of K
-// (the output and down products of a prompt of 128 tokens: 32 tiles); the cut makes up to
-// 512 workgroups of them, each with at least 512 columns.
-inline bool cuts_by_large_tiles(int M, int N, int K, int splits, int k_split);
+// How many cuts the kernel of 256 x 128 tiles makes of such a product (0: it is not one of its
+// cases): its loop runs at 1.2 PFLOP/s where the 128 x 128 kernel's, two workgroups a CU, reaches
+// 0.7 (the down product of the 1B shape at 2,048 rows, N 2,048, K 8,192 in two cuts: 95 us
+// against 70).  Its tiles are half as many: with up to eight cuts they must fill most of the chip
+// and not more than the chip, a cut must be 1,024 columns at least (two cuts: K of 4,096 at
+// least), and the rows may be padded to whole tiles of 256 by a third over their tiles of 128
+// (measured with a tenth, a fifth and a third, and with five, six and eight cuts at most, on the
+// narrow products of the 8B, 13B, 1B and 3B shapes at 160 to 1,280 rows, us with the kernel that adds
+// the cuts: N 4,096, K 14,336 at 160 to 256 rows 57 to 59 -> 47 to 51, at 384 rows 78 -> 69, at 640
+// 110 -> 101, at 896 148 -> 115; N 5,120, K 13,824 at 640 rows 140 -> 106; N 6,144, K 4,096 at 160 to 256
+// rows 38 to 39 -> 33 to 34; one case lost, N 2,048, K 8,192 at 384 rows 38.7 -> 41.4).
+inline int large_tile_cuts(int M, int N, int K) {
+  if (M <= 64 || K % 64 != 0 || N % 4 != 0) return 0;
+  const int64_t rows256 = (int64_t)((M + 255) / 256) * 256, rows128 = (int64_t)((M + 127) / 128) * 128;
+  if (rows256 * 3 > rows128 * 4) return 0;
+  const int64_t tiles = (int64_t)((N + 127) / 128) * (rows256 / 256);
+  if (tiles > 128) return 0;
+  int cuts = (int)(256 / tiles);
+  if (cuts > 8) cuts = 8;
+  while (cuts >= 2 && K / cuts < 1024) --cuts;
+  if (cuts < 2 || tiles * cuts < 192 || (cuts == 2 && K < 4096)) return 0;
+  const int k_split = ((K + cuts - 1) / cuts + 63) / 64 * 64;
+  return (K + k_split - 1) / k_split;
+}
 
+inline bool cuts_by_large_tiles(int M, int N, int K, int splits) { return splits > 1 && large_tile_cuts(M, N, K) == splits; }
+
+// How many ways K is cut for M x N x K (1: not at all): the large tiles' cuts where they apply;
+// else through 128 x 128 tiles: with fewer than 256 of them (384 where K is long) a part of the
+// chip stands idle while a few workgroups walk the whole of K (the output and down products of a
+// prompt of 128 tokens: 32 tiles); the cut makes up to 512 workgroups of them, each with at least
+// 512 columns.
 inline int pipelined_splits(int M, int N, int K) {
+  if (const int cuts = large_tile_cuts(M, N, K); cuts > 1 && K >= 2048) return cuts;
   const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
-  // (two cuts pay where K is long, and from K = 4,096 on where the kernel of 256 x 128 tiles makes them and
-  // they fill the chip: 512 to 1,024 rows against 4,096 to 6,144 weight rows, half a round of its tiles whole)
-  const bool long_k = K >= 8192 || (K >= 4096 && K % 128 == 0 && cuts_by_large_tiles(M, N, K, 2, K / 2));
+  const bool long_k = K >= 8192;
   if (M <= 64 || tiles >= (long_k ? 384 : 256) || K < 2048 || N % 4 != 0) return 1;
   // (two workgroups of this kernel fit a CU; measured, a prompt of 128 tokens is faster with one a CU
   // and fewer partial products, one of 512 tokens with two; two cuts only pay where K is long)
@@ -727,17 +752,6 @@ int launch_direct64(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf
                     int M, int N, int K, const QkvArgs& qkv, hipStream_t stream, int k_split = 0, int splits = 1,
                     int64_t split_stride = 0);
 inline bool large_fits(int64_t lda, int64_t ldw, int M, int N, int K);
-
-// Whether the cuts of a product are better made by the kernel of 256 x 128 tiles: its loop runs
-// at 1.2 PFLOP/s where the 128 x 128 kernel's, two workgroups a CU, reaches 0.7 (the down
-// product of the 1B shape at 2,048 rows, N 2,048, K 8,192 in two cuts: 95 us against 70).  Its
-// tiles are half as many: with the cuts they must still fill most of the chip, and the rows
-// must be whole tiles of 256, or nearly.
-inline bool cuts_by_large_tiles(int M, int N, int K, int splits, int k_split) {
-  const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 255) / 256);
-  return (int64_t)((M + 255) / 256) * 256 * 10 <= (int64_t)((M + 127) / 128) * 128 * 11 && tiles * splits >= 192 &&
-         tiles * splits <= 256 && k_split >= 1024 && k_split % 64 == 0 && K % 64 == 0;
-}
 
 template <int MODE>
 int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
@@ -761,7 +775,7 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
         partial.floats >= (int64_t)splits * M * N) {
       if (raise_pipelined_lds<OUT_F32>(lds)) return 1;
       const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
-      if (cuts_by_large_tiles(M, N, K, splits, k_split) && large_fits(lda, ldw, M, N, K)) {
+      if (cuts_by_large_tiles(M, N, K, splits) && large_fits(lda, ldw, M, N, K)) {
         if (launch_direct64<OUT_F32, 4, 2, 3>(partial.at, N, A, lda, W, ldw, M, N, K, qkv, stream, k_split, splits,
                                               (int64_t)M * N))
           return 1;
@@ -1544,7 +1558,7 @@ HFEE_API int hfee_gemm_bf16_cuts(const void* A, int64_t lda, const void* W, int6
   if (plan.first != 2 || plan.second != 0 || splits < 2 || scratch_floats < (int64_t)splits * M * N) return 0;
   constexpr int TM = 2, TN = 2, STAGES = 3;
   const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
-  if (cuts_by_large_tiles(M, N, K, splits, k_split) && large_fits(lda, ldw, M, N, K)) {
+  if (cuts_by_large_tiles(M, N, K, splits) && large_fits(lda, ldw, M, N, K)) {
     if (launch_direct64<OUT_F32, 4, 2, 3>(scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, stream,
                                           k_split, splits, (int64_t)M * N))
       return 1;
