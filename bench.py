@@ -425,6 +425,9 @@ def run(args):
             dtb, ctx_b = decode_run(b, steps, min(args.warmup, 4))
             points[f"decode_b{b}"] = round(b * steps / dtb, 2)
             points[f"decode_b{b}_hbm_frac"] = round((weight_bytes + b * ctx_b * kv_bytes_per_token) / (dtb / steps) / HBM_PEAK, 4)
+        if not hasattr(args, "point_batches"):        # (the line's own shape: shorter prompts, ms until they are in the cache)
+            for tokens in (128, 512, 1024):
+                points[f"prefill_{tokens}_ms"] = round(prefill_run(tokens) * 1e3, 3)
         line["points"] = points
     return line
 
