@@ -378,10 +378,16 @@ struct GroupShares {
   int parts;
   size_t bytes;
 };
-inline GroupShares group_shares(int kv_heads, int head_dim) {
+inline GroupShares group_shares(int kv_heads, int head_dim, int n) {
   const int most = (int)(48 * 1024 / ((size_t)32 * head_dim));       // heads a workgroup
   if (most < 1) return GroupShares{0, 0};
-  const int parts = (kv_heads + most - 1) / most, heads_a_part = (kv_heads + parts - 1) / parts;
+  int parts = (kv_heads + most - 1) / most;
+  // (few tokens: the groups' workgroups, which run longest, over more of the chip, 128 of them if the
+  // heads allow: a layer of a 256-token prefill at the 8B shape 209 -> 205 us, nothing from 2,048 tokens on)
+  const int groups = (n + 15) / 16;
+  while (parts < kv_heads && groups * parts < 128) ++parts;
+  const int heads_a_part = (kv_heads + parts - 1) / parts;
+  parts = (kv_heads + heads_a_part - 1) / heads_a_part;              // (no workgroup without a head)
   return GroupShares{parts, (size_t)32 * heads_a_part * head_dim};
 }
 
@@ -574,7 +580,7 @@ HFEE_API int hfee_rope_cache_write(void* q, int64_t ldq, const void* k, int64_t 
            (uintptr_t)cos_table % 16 == 0 && (uintptr_t)sin_table % 16 == 0 && (uintptr_t)cache % 16 == 0)
   {
     // (the values of 16 tokens through LDS, if a workgroup's share of it fits and there is more than one group)
-    const GroupShares shares = group_shares(kv_heads, head_dim);
+    const GroupShares shares = group_shares(kv_heads, head_dim, n);
     // (`portions`: the tokens hold runs of consecutive positions of a sequence.  Without them, single
     // tokens of many sequences, a group's workgroup would write 16 tokens' values two bytes at a time
     // on its own, eight workgroups for 128 tokens where every token's own workgroup can do it: 13 us
@@ -626,7 +632,7 @@ HFEE_API int hfee_rope_cache_write_cuts(void* q, int64_t ldq, const float* parti
                    (uintptr_t)sin_table % 16 == 0 && (uintptr_t)cache % 16 == 0,
                "rope_cache_write_cuts: head_dim and the rotary width must be multiples of 8 and the operands 16-byte aligned");
   const QkvCuts c{partial, cuts, (int64_t)n * width, width, num_heads * head_dim, (num_heads + kv_heads) * head_dim};
-  const GroupShares shares = group_shares(kv_heads, head_dim);
+  const GroupShares shares = group_shares(kv_heads, head_dim, n);
   const int by_groups = portions != 0 && n >= 32 ? shares.parts : 0;
   // (k and v: any pointers that are not null; with cuts they are never read.  More threads than
   // the plain kernel has, a piece each where that is at most 768: a thread's eight elements
