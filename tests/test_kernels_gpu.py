@@ -126,14 +126,15 @@ def test_gemm_bf16(M, N, K, kernel, mode):
 
 @pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 640, 2112),
                                    (100, 2048, 2048), (512, 4096, 8192), (1000, 2048, 8256), (2048, 2048, 8192),
-                                   (1024, 4096, 4096), (768, 4096, 4096), (512, 6144, 4096)])
+                                   (1024, 4096, 4096), (768, 4096, 4096), (512, 6144, 4096), (300, 4100, 8192), (200, 3080, 14336)])
 @pytest.mark.parametrize("mode", ["bf16", "f32", "add"])
 def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
     """Products with too few 128 x 128 tiles for the chip: given scratch, K is cut over up to
     eight times as many workgroups and a second kernel adds the partial products (K that is
     no multiple of the cut, M and N that are no multiples of a tile; the last three sizes: the
     cuts made by the kernel of 256 x 128 tiles, whole tiles of rows and not, a last cut that is
-    shorter; then three more by that kernel: two cuts of K = 4,096, half a round of its tiles each);
+    shorter; then more by that kernel: two cuts of K = 4,096, half a round of its tiles each; rows padded
+    by a third to its tiles of 256 and weight rows that are no multiple of a tile, in three and in eight cuts);
     the same numbers as without scratch up to the order of the sums."""
     from hfee_amd.kernels import ops
     g = torch.Generator().manual_seed(M + 3 * N + K)
@@ -167,7 +168,7 @@ def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
 
 @pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 4096, 2112),
                                    (100, 2052, 2048), (100, 512, 1024), (70, 1001, 2048), (2048, 512, 1024), (40, 512, 2048),
-                                   (90, 260, 2050), (512, 4096, 8192), (1000, 2048, 8256), (1024, 4096, 4096)])
+                                   (90, 260, 2050), (512, 4096, 8192), (1000, 2048, 8256), (1024, 4096, 4096), (300, 4100, 8192)])
 @pytest.mark.parametrize("weight_dtype", [torch.float32, torch.bfloat16])
 def test_product_that_adds_into_the_stream_and_goes_on_with_the_norm(M, N, K, weight_dtype):
     """The product that adds into the residual stream together with the norm of the new rows:
