@@ -168,7 +168,7 @@ def test_gemm_bf16_with_k_cut_over_workgroups(M, N, K, mode):
 
 @pytest.mark.parametrize("M,N,K", [(65, 512, 2048), (128, 1024, 4096), (200, 520, 3000), (130, 256, 14336), (384, 4096, 2112),
                                    (100, 2052, 2048), (100, 512, 1024), (70, 1001, 2048), (2048, 512, 1024), (40, 512, 2048),
-                                   (90, 260, 2050), (512, 4096, 8192), (1000, 2048, 8256), (1024, 4096, 4096), (300, 4100, 8192)])
+                                   (90, 260, 2050), (512, 4096, 8192), (1000, 2048, 8256), (1024, 4096, 4096), (300, 4100, 8192), (160, 4096, 14336)])
 @pytest.mark.parametrize("weight_dtype", [torch.float32, torch.bfloat16])
 def test_product_that_adds_into_the_stream_and_goes_on_with_the_norm(M, N, K, weight_dtype):
     """The product that adds into the residual stream together with the norm of the new rows:
