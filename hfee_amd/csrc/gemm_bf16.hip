@@ -734,6 +734,10 @@ inline int pipelined_splits(int M, int N, int K) {
   const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
   const bool long_k = K >= 8192;
   if (M <= 64 || tiles >= (long_k ? 384 : 256) || K < 2048 || N % 4 != 0) return 1;
+  // (a short K in three or four cuts is a few steps between a prologue and an epilogue: with more than 96
+  // tiles the whole product is faster, N 3,072, K 2,048 at 768 rows 31.7 us against 35.9, N 2,048 at 1,024 rows
+  // 35.9 against 38.5; at K = 3,072 the cuts still win, 37.5 against 47)
+  if (K < 3072 && tiles > 96) return 1;
   // (two workgroups of this kernel fit a CU; measured, a prompt of 128 tokens is faster with one a CU
   // and fewer partial products, one of 512 tokens with two; two cuts only pay where K is long)
   // (measured at 128 to 512 rows on the three narrow products of the 8B shape, µs for the pair of
