@@ -787,6 +787,12 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
         if (launch_direct64<OUT_F32, 4, 2, 3>(partial.at, N, A, lda, W, ldw, M, N, K, qkv, stream, k_split, splits,
                                               (int64_t)M * N))
           return 1;
+      } else if (large_fits(lda, ldw, M, N, K)) {
+        // (the kernel that loads straight into LDS, with 128 x 128 tiles: 2 to 4 us less than the one below
+        // for every cut product of 65 to 512 rows of the 8B, 13B, 3B and 1B shapes, 20 to 50 us each)
+        if (launch_direct64<OUT_F32, 2, 2, 3>(partial.at, N, A, lda, W, ldw, M, N, K, qkv, stream, k_split, splits,
+                                              (int64_t)M * N))
+          return 1;
       } else {
         grid.y = splits;
         gemm_bf16_pipelined_kernel<OUT_F32, TM, TN, STAGES><<<grid, 256, lds, stream>>>(
@@ -1321,8 +1327,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(
 }
 
 // Which tiled kernel takes an aligned product: force_kernel 2 the 128 x 128 tiles, 4 the
-// 256 x 256 tiles, 5 the 256 x 128 tiles, 6 the 256 x 192 tiles, anything else the one
-// expected to be fastest:
+// 256 x 256 tiles, 5 the 256 x 128 tiles, 6 the 256 x 192 tiles, 7 the 128 x 128 tiles of the
+// kernel that loads straight into LDS, anything else the one expected to be fastest:
 // rounds of tiles over the chip times the time of a tile, with the share of the matrix
 // peak that each kernel was measured to reach on a busy CU (128 x 128: two workgroups a
 // CU; the large tiles reach more the longer K is, and a tile of empty rows costs as
@@ -1390,6 +1396,7 @@ int launch_tiled_kernel(int choice, void* C, int64_t ldc, const bf16_t* A, int64
   if (choice == 6) return launch_direct<MODE, 4, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  if (choice == 7) return launch_direct64<MODE, 2, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream, partial);
 }
 
@@ -1398,7 +1405,7 @@ int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf1
                    int M, int N, int K, int force_kernel, hipStream_t stream, const QkvArgs& qkv = QkvArgs{},
                    const Partial& partial = Partial{}) {
   const bool large_ok = large_fits(lda, ldw, M, N, K);
-  if (force_kernel == 2 || (force_kernel >= 4 && force_kernel <= 6))
+  if (force_kernel == 2 || (force_kernel >= 4 && force_kernel <= 7))
     return launch_tiled_kernel<MODE>(force_kernel >= 4 && !large_ok ? 2 : force_kernel, C, ldc, A, lda, W, ldw, M, N, K,
                                      stream, qkv, partial);
   // (the q/k/v epilogue finds a column's head by its number: those products stay whole)
@@ -1469,8 +1476,8 @@ HFEE_API int hfee_gemm_bf16_scratch(int M, int N, int K) {
 // rows of W alternate gate/up; C is [M, N/2] bfloat16 = activation(gate) * up, the
 // activation being gate_act: GATE_SILU ...; aligned operands only).
 // force_kernel: 0 choose by the sizes, 1 skinny, 2 tiled 128 x 128, 3 the simple tiled
-// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192 (for tests of each
-// kernel alone; 4 to 6 fall back to 2 where they do not apply).
+// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192, 7 tiled 128 x 128 loaded
+// straight into LDS (for tests of each kernel alone; 4 to 7 fall back to 2 where they do not apply).
 // scratch: null, or hfee_gemm_bf16_scratch(M, N, K) float32 words, 16-byte aligned.
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
                             int64_t ldw, int M, int N, int K, int force_kernel, float* scratch,
@@ -1482,7 +1489,7 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
   HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16: a leading dimension is shorter than its row");
   HFEE_REQUIRE(out_mode >= 0 && out_mode <= 3, "gemm_bf16: unknown output mode %d", out_mode);
   HFEE_REQUIRE(ldc >= (out_mode == 3 ? N / 2 : N), "gemm_bf16: ldc is shorter than a row of the result");
-  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 6, "gemm_bf16: unknown kernel choice %d", force_kernel);
+  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 7, "gemm_bf16: unknown kernel choice %d", force_kernel);
   if (M == 0) return 0;
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) &&
                    ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
@@ -1568,6 +1575,10 @@ HFEE_API int hfee_gemm_bf16_cuts(const void* A, int64_t lda, const void* W, int6
   const int k_split = ((K + splits - 1) / splits + 63) / 64 * 64;
   if (cuts_by_large_tiles(M, N, K, splits) && large_fits(lda, ldw, M, N, K)) {
     if (launch_direct64<OUT_F32, 4, 2, 3>(scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, stream,
+                                          k_split, splits, (int64_t)M * N))
+      return 1;
+  } else if (large_fits(lda, ldw, M, N, K)) {
+    if (launch_direct64<OUT_F32, 2, 2, 3>(scratch, N, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, QkvArgs{}, stream,
                                           k_split, splits, (int64_t)M * N))
       return 1;
   } else {
