@@ -728,14 +728,31 @@ inline int large_tile_cuts(int M, int N, int K) {
 
 inline bool cuts_by_large_tiles(int M, int N, int K, int splits) { return splits > 1 && large_tile_cuts(M, N, K) == splits; }
 
+// One round of at most 256 tiles of 128 x 128 by the kernel that loads straight into LDS is faster
+// whole than in cuts once the tiles are many for the length of K: the cuts' partial products and the kernel
+// that adds them cost more than the idle CUs (us, whole against cut, the cut ones with the norm that their
+// adding kernel does: N 3,072, K 2,048 at 256 / 512 / 1,024 rows 22.5 / 23.2 / 25.0 against 24.6 / 30.6 / 34.0;
+// N 2,048, K 2,048 at 768 / 1,024 rows 30.4 / 31.0 against 33.8 / 40.9; N 6,144, K 4,096 at 384 / 512 rows 35.6 /
+// 36.0 against 42.4 / 43.0; N 4,096, K 4,096 at 768 / 1,024 rows 46.2 / 49.9 against 49.3 / 55.3, but at 512 rows
+// 42.6 against 40.7; N 5,120, K 5,120 at 768 rows 55.9 against 58.4, at 512 rows 50.3 against 48.5; from
+// K = 8,192 on the cuts win at every number of rows).  Inside a prefill only the short K keeps the gain: a
+// layer of the 1B shape at 1,024 / 2,048 rows 226 / 354 -> 214 / 346 us, of the 3B shape at 1,024 rows 299 -> 293,
+// but of the 8B shape at 512 rows 287 -> 290 and of the 13B shape at 768 rows 534 -> 540 (there the kernel
+// that adds the cuts is the rotation or the norm, which run anyway): whole below K = 4,096 only.
+inline bool whole_in_one_round(int M, int N, int K, int64_t tiles) {
+  return M > 64 && K % 64 == 0 && K < 4096 && tiles <= 256 && tiles * 4096 >= (int64_t)144 * K &&
+         (int64_t)M * K < (1ll << 30) && (int64_t)N * K < (1ll << 30);
+}
+
 // How many ways K is cut for M x N x K (1: not at all): the large tiles' cuts where they apply;
 // else through 128 x 128 tiles: with fewer than 256 of them (384 where K is long) a part of the
 // chip stands idle while a few workgroups walk the whole of K (the output and down products of a
 // prompt of 128 tokens: 32 tiles); the cut makes up to 512 workgroups of them, each with at least
 // 512 columns.
 inline int pipelined_splits(int M, int N, int K) {
-  if (const int cuts = large_tile_cuts(M, N, K); cuts > 1 && K >= 2048) return cuts;
   const int64_t tiles = (int64_t)((N + 127) / 128) * ((M + 127) / 128);
+  if (whole_in_one_round(M, N, K, tiles)) return 1;
+  if (const int cuts = large_tile_cuts(M, N, K); cuts > 1 && K >= 2048) return cuts;
   const bool long_k = K >= 8192;
   if (M <= 64 || tiles >= (long_k ? 384 : 256) || K < 2048 || N % 4 != 0) return 1;
   // (a short K in three or four cuts is a few steps between a prologue and an epilogue: with more than 96
@@ -764,7 +781,8 @@ inline bool large_fits(int64_t lda, int64_t ldw, int M, int N, int K);
 template <int MODE>
 int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
                      int M, int N, int K, const QkvArgs& qkv, hipStream_t stream,
-                     const Partial& partial = Partial{}, const NormAfter& norm = NormAfter{}, bool* normed = nullptr) {
+                     const Partial& partial = Partial{}, const NormAfter& norm = NormAfter{}, bool* normed = nullptr,
+                     bool this_kernel_only = false) {
   // 128 x 128 tiles, two workgroups per CU.  (128 x 256 tiles halve the LDS reads per
   // matrix instruction but leave one wave per SIMD, and measured 20 % slower; 128 x 64
   // tiles, which put two workgroups on a CU where 128 x 128 leave one, 15 % slower at 65
@@ -809,6 +827,12 @@ int launch_pipelined(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const b
       return 0;
     }
   }
+  // (one round of tiles, a workgroup a CU: the kernel that loads straight into LDS, a quarter faster
+  // than two workgroups a CU of the one below: N 3,072, K 2,048 at 1,024 rows 25.2 us against 34.5, N 2,048,
+  // K 2,048 at 2,048 rows 31.9 against 41.5, N 4,096, K 4,096 at 1,024 rows 44.1 against 59.8; with more
+  // tiles than CUs it is the slower one, 39.0 against 34.1 and 49.8 against 42.1)
+  if (!this_kernel_only && tiles <= 256 && large_fits(lda, ldw, M, N, K))
+    return launch_direct64<MODE, 2, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   gemm_bf16_pipelined_kernel<MODE, TM, TN, STAGES><<<grid, 256, lds, stream>>>(C, ldc, A, lda, W, ldw, M, N, K, qkv, 0, 0);
   return 0;
 }
@@ -1354,7 +1378,8 @@ inline TiledPlan plan_tiled(int M, int N, int K, bool large_ok, bool may_split) 
   auto cost = [&](int k, int n) {
     const int bm = k == 2 ? 128 : 256, bn = k == 2 ? 128 : k == 4 ? 256 : k == 5 ? 128 : 192;
     const double t = (double)((M + bm - 1) / bm) * ((n + bn - 1) / bn);
-    if (k == 2) return t <= cus ? 128.0 * 128 / 0.22 : rounds(t, 2 * cus) * 2 * 128 * 128 / 0.31;
+    // (up to a tile a CU: the 128 x 128 tiles go to the kernel that loads straight into LDS)
+    if (k == 2) return t <= cus ? 128.0 * 128 / (t <= 256 ? 0.30 : 0.22) : rounds(t, 2 * cus) * 2 * 128 * 128 / 0.31;
     return rounds(t, cus) * bm * bn / ((k == 4 ? 0.46 : k == 5 ? 0.42 : 0.44) * fill);
   };
   TiledPlan best{2, N, 0};
@@ -1392,12 +1417,13 @@ inline TiledPlan plan_tiled(int M, int N, int K, bool large_ok, bool may_split) 
 
 template <int MODE>
 int launch_tiled_kernel(int choice, void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
-                        int M, int N, int K, hipStream_t stream, const QkvArgs& qkv, const Partial& partial = Partial{}) {
+                        int M, int N, int K, hipStream_t stream, const QkvArgs& qkv, const Partial& partial = Partial{},
+                        bool forced = false) {
   if (choice == 6) return launch_direct<MODE, 4, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 7) return launch_direct64<MODE, 2, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
-  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream, partial);
+  return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream, partial, NormAfter{}, nullptr, forced);
 }
 
 template <int MODE>
@@ -1407,7 +1433,7 @@ int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf1
   const bool large_ok = large_fits(lda, ldw, M, N, K);
   if (force_kernel == 2 || (force_kernel >= 4 && force_kernel <= 7))
     return launch_tiled_kernel<MODE>(force_kernel >= 4 && !large_ok ? 2 : force_kernel, C, ldc, A, lda, W, ldw, M, N, K,
-                                     stream, qkv, partial);
+                                     stream, qkv, partial, true);
   // (the q/k/v epilogue finds a column's head by its number: those products stay whole)
   const TiledPlan plan = plan_tiled(M, N, K, large_ok, MODE != OUT_QKV);
   if (int rc = launch_tiled_kernel<MODE>(plan.first, C, ldc, A, lda, W, ldw, M, plan.n1, K, stream, qkv, partial)) return rc;
