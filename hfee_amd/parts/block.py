@@ -25,6 +25,10 @@ class PreNormBlock(Part):
         self.hidden = spec.hidden
 
     def parts(self):
+        # (each with the parts it is made of itself: a mixer lists a step behind its projections)
+        return [q for p in self._own() for q in p.parts()]
+
+    def _own(self):
         return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
 
     # the layer of the paged cache that a run of this block is given belongs to its mixer
@@ -35,10 +39,10 @@ class PreNormBlock(Part):
         return getattr(self.mixer, "key_layout", lambda: None)()
 
     def tensor_specs(self):
-        return [s for p in self.parts() for s in p.tensor_specs()]
+        return [s for p in self._own() for s in p.tensor_specs()]
 
     def bind(self, tensors):
-        for p in self.parts():
+        for p in self._own():
             p.bind(tensors)
 
     # forward takes the normed input that the block before may have begun, and that of
