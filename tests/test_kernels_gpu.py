@@ -1197,3 +1197,96 @@ def test_only_finite_numbers_reach_the_cache(M):
     ops.rope_cache_write(y32[:, :H * hd], y32[:, H * hd:(H + K) * hd], y32[:, (H + K) * hd:], pos, seg, tables, cos, sin,
                          0, layer, H, K, hd, ps, M - 1)
     check(layer, "rotation kernel, 32-bit")
+
+
+def test_a_cache_layer_of_more_than_four_gigabytes():
+    """A pool that the free memory of this GPU suggests makes a cache layer of several gigabytes
+    (128 requests of 8,192 tokens at the 8B sizes: 4.3 GB a layer).  Here a layer of 70,000 pages
+    of 64 KiB (4.6 GB): sequences whose pages lie beyond the 2 GiB and 4 GiB marks, among low
+    ones, in scrambled order.  Keys and values get there through the rotation kernel (portions)
+    and through the decode product's epilogue (the sequences' last tokens); the prefill kernels
+    that take a layer of this size (the ones that address the whole layer through one 32-bit
+    offset are not chosen and refuse it when forced), the decode kernel with and without key
+    splits and the plain kernel read them; all against the formula on the numbers themselves,
+    with a far key scaled up so that a page read from the wrong place shows."""
+    from plain_llama import plain_attention
+    from hfee_amd.kernels import ops
+    H, K, hd, ps, d = 32, 8, 128, 16, 256
+    pages = 70_000
+    free, _ = torch.cuda.mem_get_info()
+    if free < 12 << 30:
+        pytest.skip("needs 12 GB of free device memory")
+    layer = torch.zeros(pages, 2, K, ps * hd, dtype=torch.bfloat16, device=DEV)
+    assert layer.numel() * 2 > 1 << 32
+    g = torch.Generator().manual_seed(70)
+    scale = 1 / math.sqrt(hd)
+    lengths = [701, 301, 91, 34]                 # the last token of each comes through the decode product
+    portions = [(0, 700), (260, 40), (0, 90), (32, 1)]       # (first position, rows) of the prefill kernels' step
+    blocks = [(n + ps - 1) // ps for n in lengths]
+    # pages beyond 4 GiB (from 65,536 on), beyond 2 GiB (from 32,768 on), and low ones
+    pool = torch.cat([65_540 + torch.randperm(4_400, generator=g)[:40], 32_770 + torch.randperm(1_000, generator=g)[:20],
+                      torch.randperm(500, generator=g)[:16]])
+    pool = pool[torch.randperm(pool.numel(), generator=g)].tolist()
+    table = torch.zeros(len(lengths), max(blocks), dtype=torch.int32)
+    w = (torch.randn((H + 2 * K) * hd, d, generator=g) / math.sqrt(d)).to(torch.bfloat16)
+    w_tiles = ops.tile_weight(w.to(DEV))
+    qs, ks, vs, xs = [], [], [], []
+    for s, n in enumerate(lengths):
+        mine, pool = pool[:blocks[s]], pool[blocks[s]:]
+        table[s, :blocks[s]] = torch.tensor(mine, dtype=torch.int32)
+        x_last = torch.randn(1, d, generator=g).to(torch.bfloat16)
+        last = (x_last.double() @ w.double().t()).to(torch.bfloat16)        # what the product makes of the last token
+        q = torch.cat([torch.randn(n - 1, H * hd, generator=g).to(torch.bfloat16), last[:, :H * hd]])
+        k = torch.cat([(torch.randn(n - 1, K * hd, generator=g) * 0.7).to(torch.bfloat16), last[:, H * hd:(H + K) * hd]])
+        v = torch.cat([torch.randn(n - 1, K * hd, generator=g).to(torch.bfloat16), last[:, (H + K) * hd:]])
+        first, rows = portions[s]
+        k[n // 3] = (q[first:first + rows].float().mean(0).view(K, H // K, hd).mean(1) * 5).reshape(K * hd).to(torch.bfloat16)
+        qs.append(q), ks.append(k), vs.append(v), xs.append(x_last)
+    assert int(table.max()) > 65_536
+    table = table.to(DEV)
+    # every token but the last: the rotation kernel without a rotation, one portion a launch and all in one
+    k_all = torch.cat([k[:-1] for k in ks]).to(DEV)
+    v_all = torch.cat([v[:-1] for v in vs]).to(DEV)
+    pos_all = torch.cat([torch.arange(n - 1) for n in lengths]).to(torch.int32).to(DEV)
+    seg_all = torch.cat([torch.full((n - 1,), s) for s, n in enumerate(lengths)]).to(torch.int32).to(DEV)
+    ops.rope_cache_write(None, k_all, v_all, pos_all, seg_all, table, None, None, 1, layer, H, K, hd, ps, max(lengths))
+    # the last tokens: the product of few rows with the cache write in its epilogue
+    q_last = torch.full((len(lengths), H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    last_pos = torch.tensor([n - 1 for n in lengths], dtype=torch.int32, device=DEV)
+    order = torch.arange(len(lengths), dtype=torch.int32, device=DEV)
+    ops.linear_fused(q_last, torch.cat(xs).to(DEV), w_tiles, "qkv",
+                     qkv=dict(positions=last_pos, token_segment=order, block_tables=table, cos=None, sin=None,
+                              cache_layer=layer, num_heads=H, kv_heads=K, head_dim=hd, page_size=ps))
+    close(q_last, torch.stack([q[-1] for q in qs]), 2e-2)
+    # what the formula says for every row of the step and for the last tokens
+    full = [plain_attention(q.view(-1, H, hd), k.view(-1, K, hd), v.view(-1, K, hd), scale) for q, k, v in zip(qs, ks, vs)]
+    ref_step = torch.cat([f[first:first + rows].reshape(rows, H * hd) for f, (first, rows) in zip(full, portions)])
+    ref_last = torch.stack([f[-1].reshape(H * hd) for f in full])
+    q_step = torch.cat([q[first:first + rows] for q, (first, rows) in zip(qs, portions)]).to(DEV)
+    tiles, positions, seg, row = [], [], [], 0
+    for s, (first, rows) in enumerate(portions):
+        for off in range(0, rows, 32):
+            tiles.append((row + off, min(32, rows - off), first + off, s))
+        positions += list(range(first, first + rows))
+        seg += [s] * rows
+        row += rows
+    dev_tiles = torch.tensor(tiles, dtype=torch.int32, device=DEV)
+    for kernel in (0, 1, 2):
+        out = torch.full((row, H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.attention_bf16_prefill(out, q_step, layer, dev_tiles, table, H, K, hd, ps, scale, 0, kernel=kernel)
+        close(out, ref_step, 2e-2)
+    with pytest.raises(Exception, match="two halves"):
+        ops.attention_bf16_prefill(out, q_step, layer, dev_tiles, table, H, K, hd, ps, scale, 0, kernel=3)
+    out = torch.full((row, H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attention_plain(out, q_step, layer, torch.tensor(positions, dtype=torch.int32, device=DEV),
+                        torch.tensor(seg, dtype=torch.int32, device=DEV), table, H, K, hd, ps, scale, 0)
+    close(out, ref_step, 2e-2)
+    counters = torch.zeros(len(lengths) * K, dtype=torch.int32, device=DEV)
+    for splits in (1, 3):
+        out = torch.full((len(lengths), H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+        partial = torch.zeros(len(lengths) * H * splits * (hd + 2), dtype=torch.float32, device=DEV)
+        ops.attention_bf16_decode(out, q_last, layer, None, last_pos, None, table, H, K, hd, ps, scale, 0, partial, splits,
+                                  counters=counters if splits > 1 else None)
+        close(out, ref_last, 2e-2)
+    del layer
+    torch.cuda.empty_cache()
