@@ -1086,6 +1086,10 @@ HFEE_API int hfee_attention_bf16_head_dim() { return HD; }
 // Whether this head size has the prefill kernel with a row tile's keys in two halves (variant 3).
 HFEE_API int hfee_attention_bf16_halves() { return HALVES_FIT ? 1 : 0; }
 
+// log2 of the bytes of a cache layer from which on the kernels that address the whole layer through one
+// 32-bit offset (the ring of key tiles in LDS, the two halves) leave the work to the others.
+HFEE_API int hfee_attention_bf16_layer_limit_log2() { return 32; }
+
 // The most row tiles in a run of `runs` (hfee_attention_bf16_prefill): one wave a row tile.
 HFEE_API int hfee_attention_bf16_run_tiles() { return SHARED_WAVES; }
 

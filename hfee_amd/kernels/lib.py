@@ -53,6 +53,7 @@ _ATTENTION_SIGNATURES = {
     "hfee_attention_bf16_head_dim": [],
     "hfee_attention_bf16_run_tiles": [],
     "hfee_attention_bf16_halves": [],
+    "hfee_attention_bf16_layer_limit_log2": [],
     "hfee_attention_bf16_prefill": [P, L, P, L, P, I, P, I, P, I, P, I, I, I, I, F, I, I, P],
     "hfee_attention_bf16_decode": [P, L, P, L, P, P, P, P, I, P, I, I, I, I, F, I, P, L, I, I, P, I, P],
 }

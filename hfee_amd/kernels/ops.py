@@ -462,9 +462,13 @@ def attention_run_tiles(head_dim: int) -> int:
     return int(lib.attention_bf16(head_dim).raw("hfee_attention_bf16_run_tiles")())
 
 
-def attention_halves_fit(head_dim: int, heads_per_kv_head: int) -> bool:
-    """Whether `attention_bf16_prefill(kernel=3)` takes this shape: a row tile's keys in two halves."""
-    return heads_per_kv_head % 4 == 0 and bool(lib.attention_bf16(head_dim).raw("hfee_attention_bf16_halves")())
+def attention_halves_fit(head_dim: int, heads_per_kv_head: int, cache_layer=None) -> bool:
+    """Whether `attention_bf16_prefill(kernel=3)` takes this shape: a row tile's keys in two halves
+    (and this cache layer, if one is given: that kernel reaches every page through a 32-bit offset)."""
+    dll = lib.attention_bf16(head_dim)
+    if cache_layer is not None and cache_layer.numel() * cache_layer.element_size() >= 1 << int(dll.raw("hfee_attention_bf16_layer_limit_log2")()):
+        return False
+    return heads_per_kv_head % 4 == 0 and bool(dll.raw("hfee_attention_bf16_halves")())
 
 
 def prefill_attention_kernel(tiles, window: int, kv_heads: int, heads_per_kv_head: int, head_dim: int) -> int:

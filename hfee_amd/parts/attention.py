@@ -218,9 +218,12 @@ class Attention(Mixer):
         else:
             tiles = ctx.extra["attention.tiles"]
             if tiles.shape[0]:
+                kernel = ctx.host.get("attention.prefill_kernel", 0)
+                if kernel == 3 and not ops.attention_halves_fit(hd, H // K, cache):
+                    kernel = 0          # (the plan knew the step's row tiles, not the size of the layer)
                 ops.attention_bf16_prefill(att, q, cache, tiles, tables, H, K, hd, ctx.page_size,
                                            self.scale, self.window, runs=ctx.extra["attention.runs"] if H == K else None,
-                                           kernel=ctx.host.get("attention.prefill_kernel", 0))
+                                           kernel=kernel)
             rows = ctx.extra["attention.decode_rows"]
             if rows.numel():
                 nseg = rows.numel()

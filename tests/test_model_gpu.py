@@ -178,3 +178,52 @@ def test_the_cache_pool_follows_the_free_memory(model_folders):
     with pytest.raises(CacheError, match="pages would fit") as e:
         Engine(model, num_pages=free // page + 10, page_size=16, max_requests=4, max_batch_tokens=64)
     assert f"{total:,}" in str(e.value) and torch.cuda.memory_allocated() == before
+
+
+def test_a_pool_whose_layers_are_larger_than_four_gigabytes(tmp_path):
+    """One layer with 8 KV heads of 128 and a pool of 70,000 pages: 4.6 GB a cache layer, as
+    the free memory of this GPU makes them at production sizes.  A request that holds the
+    first 66,000 pages pushes the others' pages beyond the 4 GiB mark.  A prompt of 150 tokens
+    from its start (the step's plan asks for the prefill kernel that walks a row tile's keys in
+    two halves, which does not take such a layer: the mixer falls back at the launch), another
+    in portions beside decoded tokens, then both decode; against the plain model."""
+    from conftest import make_model_folder
+    from plain_llama import PlainLlama
+    from hfee_amd.engine import Engine, StepEntry, load_model
+    from hfee_amd.kernels import ops
+    if torch.cuda.mem_get_info()[0] < 12 << 30:
+        pytest.skip("needs 12 GB of free device memory")
+    cj = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 1, "hidden_size": 64,
+          "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128, "intermediate_size": 96, "vocab_size": 256,
+          "max_position_embeddings": 512, "rope_theta": 10000.0, "rope_scaling": None, "rms_norm_eps": 1e-5,
+          "tie_word_embeddings": True, "hidden_act": "silu"}
+    folder = make_model_folder(tmp_path / "m", cj, seed=5, dtype="bfloat16", std=0.1, norm_init="one_plus_normal")
+    plain = PlainLlama(folder)
+    model, cfg = load_model(folder, "bfloat16")
+    eng = Engine(model, num_pages=70_000, page_size=16, max_requests=4, max_batch_tokens=256)
+    layer = eng.storage.layer(0, (2, 8, 16 * 128))
+    assert layer.numel() * 2 > 1 << 32 and not ops.attention_halves_fit(128, 4, layer) and ops.attention_halves_fit(128, 4)
+    eng.admit("holder")
+    eng.cache.reserve("holder", 66_000 * 16)
+    g = torch.Generator().manual_seed(3)
+    a = torch.randint(0, 256, (170,), generator=g).tolist()
+    b = torch.randint(0, 256, (120,), generator=g).tolist()
+    eng.admit("a")
+    eng.admit("b")
+    got = {}
+    out = eng.step([StepEntry("a", a[:150], [0, 149])])
+    got["a", 0], got["a", 149] = out[0].clone(), out[1].clone()
+    assert min(eng.cache.block_table("a", 0)) >= 66_000
+    out = eng.step([StepEntry("b", b[:70], [69]), StepEntry("a", a[150:151], [0])])
+    got["b", 69], got["a", 150] = out[0].clone(), out[1].clone()
+    out = eng.step([StepEntry("a", a[151:152], [0]), StepEntry("b", b[70:100], [29])])
+    got["a", 151], got["b", 99] = out[0].clone(), out[1].clone()
+    for i in range(18):
+        out = eng.step([StepEntry("a", [a[152 + i]], [0]), StepEntry("b", [b[100 + i]], [0])])
+        got["a", 152 + i], got["b", 100 + i] = out[0].clone(), out[1].clone()
+    eng.cache.check()
+    ref = {"a": plain.forward(a), "b": plain.forward(b[:118])}
+    for (r, p), row in got.items():
+        assert rel_err(row, ref[r][p]) < TOL["bfloat16"], (r, p, rel_err(row, ref[r][p]))
+    del eng, layer
+    torch.cuda.empty_cache()
