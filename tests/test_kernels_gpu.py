@@ -458,6 +458,14 @@ def test_fused_qkv_rotation_and_cache_write(H, K, hd, half, M, norm):
     _check_fused_qkv(H, K, hd, half, M, norm, 96)
 
 
+@pytest.mark.parametrize("H,K,hd,half,M,d", [(4, 2, 16, 8, 100, 128), (2, 2, 128, 64, 300, 256), (6, 3, 48, 8, 130, 192),
+                                             (16, 8, 128, 64, 1100, 512)])
+def test_fused_qkv_through_the_tiled_kernels_with_whole_steps_of_k(H, K, hd, half, M, d):
+    """The same epilogue behind the tiled kernels that take a K of whole steps of 64: one round of
+    128 x 128 tiles loaded straight into LDS (the first three), the large tiles (the last)."""
+    _check_fused_qkv(H, K, hd, half, M, False, d)
+
+
 @pytest.mark.parametrize("kernel", [1, 2])
 @pytest.mark.parametrize("H,K,hd,half,M,d", [(4, 2, 16, 8, 17, 2048), (5, 1, 64, 32, 64, 1024), (6, 3, 48, 8, 40, 3072)])
 def test_fused_qkv_with_the_batch_in_lds(H, K, hd, half, M, d, kernel):
