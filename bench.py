@@ -201,6 +201,9 @@ def main(argv=None) -> int:
         torch.cuda.empty_cache()
         line["points"]["serving_128_generated_tok_s_llama-3.2-1b"] = got["value"]
         line["points"]["serving_128_all_tok_s_llama-3.2-1b"] = got["all_tokens_per_s"]
+        if got.get("gpu_ms_from_first_step_to_last"):
+            line["points"]["serving_128_gpu_inside_steps_frac_llama-3.2-1b"] = round(
+                got["gpu_ms_inside_steps"] / got["gpu_ms_from_first_step_to_last"], 4)
         longer = copy.copy(args)
         longer.context, longer.steps, longer.warmup = 8192, min(args.steps, 16), 2
         got = run(longer)
@@ -314,15 +317,34 @@ def run(args):
         lengths = torch.randint(64, 2049, (count,), generator=gen).tolist()
         for i, n in enumerate(lengths):
             sched.add(Request(("serving", i), torch.randint(0, V, (n,), generator=gen).tolist(), params, seed=i))
+        # an event in front of and behind every step's launches: what lies between a step's two events is
+        # the GPU's time inside steps, whatever it waits for there; the rest of the span it waits for the host
+        marks = []
+        run_step = engine.step
+
+        def marked_step(entries, tokens_from=None):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            out = run_step(entries, tokens_from)
+            b.record()
+            marks.append((a, b))
+            return out
+        engine.step = marked_step
         torch.cuda.synchronize()
         t = time.perf_counter()
         steps = made = 0
-        while sched.has_work():
-            for fin in sched.step():
-                made += len(fin.request.generated)
-            steps += 1
+        try:
+            while sched.has_work():
+                for fin in sched.step():
+                    made += len(fin.request.generated)
+                steps += 1
+        finally:
+            del engine.step
         torch.cuda.synchronize()
-        return time.perf_counter() - t, sum(lengths), made, steps
+        dt = time.perf_counter() - t
+        serving_run.inside_ms = sum(a.elapsed_time(b) for a, b in marks)
+        serving_run.span_ms = marks[0][0].elapsed_time(marks[-1][1]) if marks else 0.0
+        return dt, sum(lengths), made, steps
 
     if args.serving:
         serving_run(min(args.serving, 8))        # (compiles nothing, but captures graphs and sizes buffers)
@@ -331,6 +353,8 @@ def run(args):
             "metric": "continuous batching, generated tok/s (%s bf16)" % SHAPE_NAMES[args.shape],
             "value": round(made / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "seconds": round(dt, 3),
             "all_tokens_per_s": round((prompt_tokens + made) / dt, 1), "dtype": "bf16",
+            "gpu_ms_from_first_step_to_last": round(serving_run.span_ms, 1),
+            "gpu_ms_inside_steps": round(serving_run.inside_ms, 1),
             "data": "synthetic (seeded uniform random token ids, random N(0,0.02) weights)",
             "config": {"model": SHAPE_NAMES[args.shape] + "-shaped", "layers": L, "requests": args.serving,
                        "prompt_tokens_total": prompt_tokens, "generated_total": made, "seq_len": context,
