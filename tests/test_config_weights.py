@@ -237,3 +237,28 @@ def test_second_copies_of_the_weights_only_while_they_leave_room():
     for r, c in ((0, 0), (5, 9), (17, 40), (39, 71)):
         assert t[r // 16, c // 32, ((c % 32) // 8) * 128 + (r % 16) * 8 + c % 8] == w[r, c]
     assert t[2, 2, 511] == 0                             # padding
+
+
+def test_where_a_product_of_a_prompt_is_cut_along_k():
+    """The host's rule for the products of 65 and more rows (asked of the library, which needs no
+    GPU for it): with too few tiles of 128 x 128 for the chip K is cut over more workgroups and the
+    caller brings scratch for the cuts; one round of such tiles runs whole where K is short and the
+    tiles are many for it; nothing is cut up to 64 rows, nor once the tiles fill the chip."""
+    from hfee_amd.kernels import ops
+
+    def cuts(M, N, K):
+        words = ops.linear_scratch(M, N, K)
+        assert words % (M * N) == 0
+        return words // (M * N)
+    # the 8B shape's narrow products at a prompt of 128 tokens: 48 and 32 tiles
+    assert cuts(128, 6144, 4096) == 5 and cuts(128, 4096, 4096) == 8 and cuts(128, 4096, 14336) == 8
+    # two cuts by the tiles of 256 x 128 from K = 4,096 on
+    assert cuts(512, 6144, 4096) == 2 and cuts(1024, 4096, 4096) == 2 and cuts(1024, 4096, 7680) == 2
+    # one round of tiles, a short K: whole (the 1B shape's q/k/v and output products)
+    assert cuts(512, 3072, 2048) == 0 and cuts(1024, 3072, 2048) == 0 and cuts(2048, 2048, 2048) == 0
+    assert cuts(1024, 3072, 3072) == 0
+    # ... but few tiles for the length of K are cut, and a long K always
+    assert cuts(128, 3072, 2048) == 4 and cuts(256, 2048, 2048) == 4 and cuts(1024, 2048, 8192) >= 2
+    # the rows of a decode step, and products that fill the chip
+    assert cuts(64, 4096, 4096) == 0 and cuts(8, 4096, 14336) == 0
+    assert cuts(2048, 4096, 4096) == 0 and cuts(2048, 28672, 4096) == 0 and cuts(512, 28672, 4096) == 0
