@@ -1351,8 +1351,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_bf16_skinny_kernel(
 }
 
 // Which tiled kernel takes an aligned product: force_kernel 2 the 128 x 128 tiles, 4 the
-// 256 x 256 tiles, 5 the 256 x 128 tiles, 6 the 256 x 192 tiles, 7 the 128 x 128 tiles of the
-// kernel that loads straight into LDS, anything else the one expected to be fastest:
+// 256 x 256 tiles, 5 the 256 x 128 tiles, 6 the 256 x 192 tiles, 7 and 8 the 128 x 128 and 128 x 192 tiles
+// of the kernel that loads straight into LDS, anything else the one expected to be fastest:
 // rounds of tiles over the chip times the time of a tile, with the share of the matrix
 // peak that each kernel was measured to reach on a busy CU (128 x 128: two workgroups a
 // CU; the large tiles reach more the longer K is, and a tile of empty rows costs as
@@ -1376,15 +1376,20 @@ inline TiledPlan plan_tiled(int M, int N, int K, bool large_ok, bool may_split) 
   auto rounds = [&](double t, int slots) { return (double)(int64_t)((t + slots - 1) / slots); };
   // time of kernel k on n columns, in tile elements over the share of the peak
   auto cost = [&](int k, int n) {
-    const int bm = k == 2 ? 128 : 256, bn = k == 2 ? 128 : k == 4 ? 256 : k == 5 ? 128 : 192;
+    const int bm = k == 2 || k == 8 ? 128 : 256, bn = k == 2 ? 128 : k == 4 ? 256 : k == 5 ? 128 : 192;
     const double t = (double)((M + bm - 1) / bm) * ((n + bn - 1) / bn);
+    // (128 x 192 tiles, the 256 x 128 kernel compiled for them: where they are at most one a CU.  2,048 rows of
+    // 3,072 columns are 256 of them and 96 of 256 x 128: N 3,072 at K 2,048 / 3,072 / 8,192 33.2 / 48.9 / 97.0 us against
+    // 35.6 / 53.3 / 101.9; 1,024 rows of N 6,144, K 4,096 52.2 against 56.6, of N 5,120, K 5,120 60.6 against 66.8;
+    // in a second round they lose to every other tile)
+    if (k == 8) return t <= cus ? 128.0 * 192 / (0.335 * fill) : 1e30;
     // (up to a tile a CU: the 128 x 128 tiles go to the kernel that loads straight into LDS)
     if (k == 2) return t <= cus ? 128.0 * 128 / (t <= 256 ? 0.30 : 0.22) : rounds(t, 2 * cus) * 2 * 128 * 128 / 0.31;
     return rounds(t, cus) * bm * bn / ((k == 4 ? 0.46 : k == 5 ? 0.42 : 0.44) * fill);
   };
   TiledPlan best{2, N, 0};
   double best_cost = cost(2, N);
-  for (int k : {5, 6, 4})
+  for (int k : {5, 6, 4, 8})
     if (cost(k, N) < best_cost || (k == 4 && cost(k, N) <= best_cost)) {
       best = TiledPlan{k, N, 0};
       best_cost = cost(k, N);
@@ -1423,6 +1428,7 @@ int launch_tiled_kernel(int choice, void* C, int64_t ldc, const bf16_t* A, int64
   if (choice == 4) return launch_direct<MODE, 4, 4>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 5) return launch_direct64<MODE, 4, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   if (choice == 7) return launch_direct64<MODE, 2, 2, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
+  if (choice == 8) return launch_direct64<MODE, 2, 3, 3>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream);
   return launch_pipelined<MODE>(C, ldc, A, lda, W, ldw, M, N, K, qkv, stream, partial, NormAfter{}, nullptr, forced);
 }
 
@@ -1431,7 +1437,7 @@ int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf1
                    int M, int N, int K, int force_kernel, hipStream_t stream, const QkvArgs& qkv = QkvArgs{},
                    const Partial& partial = Partial{}) {
   const bool large_ok = large_fits(lda, ldw, M, N, K);
-  if (force_kernel == 2 || (force_kernel >= 4 && force_kernel <= 7))
+  if (force_kernel == 2 || (force_kernel >= 4 && force_kernel <= 8))
     return launch_tiled_kernel<MODE>(force_kernel >= 4 && !large_ok ? 2 : force_kernel, C, ldc, A, lda, W, ldw, M, N, K,
                                      stream, qkv, partial, true);
   // (the q/k/v epilogue finds a column's head by its number: those products stay whole)
@@ -1502,8 +1508,8 @@ HFEE_API int hfee_gemm_bf16_scratch(int M, int N, int K) {
 // rows of W alternate gate/up; C is [M, N/2] bfloat16 = activation(gate) * up, the
 // activation being gate_act: GATE_SILU ...; aligned operands only).
 // force_kernel: 0 choose by the sizes, 1 skinny, 2 tiled 128 x 128, 3 the simple tiled
-// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192, 7 tiled 128 x 128 loaded
-// straight into LDS (for tests of each kernel alone; 4 to 7 fall back to 2 where they do not apply).
+// kernel, 4 tiled 256 x 256, 5 tiled 256 x 128, 6 tiled 256 x 192, 7 tiled 128 x 128 and 8 tiled 128 x 192 loaded
+// straight into LDS (for tests of each kernel alone; 4 to 8 fall back to 2 where they do not apply).
 // scratch: null, or hfee_gemm_bf16_scratch(M, N, K) float32 words, 16-byte aligned.
 HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, int64_t lda, const void* W,
                             int64_t ldw, int M, int N, int K, int force_kernel, float* scratch,
@@ -1515,7 +1521,7 @@ HFEE_API int hfee_gemm_bf16(void* C, int out_mode, int64_t ldc, const void* A, i
   HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16: a leading dimension is shorter than its row");
   HFEE_REQUIRE(out_mode >= 0 && out_mode <= 3, "gemm_bf16: unknown output mode %d", out_mode);
   HFEE_REQUIRE(ldc >= (out_mode == 3 ? N / 2 : N), "gemm_bf16: ldc is shorter than a row of the result");
-  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 7, "gemm_bf16: unknown kernel choice %d", force_kernel);
+  HFEE_REQUIRE(force_kernel >= 0 && force_kernel <= 8, "gemm_bf16: unknown kernel choice %d", force_kernel);
   if (M == 0) return 0;
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) &&
                    ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);

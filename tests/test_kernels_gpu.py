@@ -201,10 +201,10 @@ def test_product_that_adds_into_the_stream_and_goes_on_with_the_norm(M, N, K, we
 @pytest.mark.parametrize("M,N,K", [(128, 128, 32), (300, 200, 520), (2048, 512, 1024), (129, 258, 72), (65, 130, 200),
                                    (257, 384, 64), (1000, 96, 4096), (600, 520, 192), (256, 512, 64),
                                    (513, 258, 320)])
-@pytest.mark.parametrize("kernel", [0, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("kernel", [0, 2, 3, 4, 5, 6, 7, 8])
 def test_gemm_bf16_tiled_large(M, N, K, kernel):
     """The tiled kernels each alone (2: 128x128 tiles, 3: the simple one, 4: 256x256, 5:
-    256x128, 6: 256x192, 7: 128x128 loaded straight into LDS; 4 to 7 hand a K that is no multiple of 64 to 2) and the automatic
+    256x128, 6: 256x192, 7: 128x128 and 8: 128x192 loaded straight into LDS; 4 to 8 hand a K that is no multiple of 64 to 2) and the automatic
     choice, with every epilogue."""
     from hfee_amd.kernels import ops
     g = torch.Generator().manual_seed(M + N + K)
