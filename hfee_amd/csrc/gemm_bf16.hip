@@ -1408,7 +1408,7 @@ inline TiledPlan plan_tiled(int M, int N, int K, bool large_ok, bool may_split) 
       const int whole = (N / bn) / per_round;
       const int n1 = whole * per_round * bn;
       if (whole < 1 || n1 >= N) continue;
-      for (int b : {2, 5, 6, 4}) {
+      for (int b : {2, 5, 6, 4, 8}) {
         const double c = cost(a, n1) + cost(b, N - n1) + launch;
         if (c < best_cost) {
           best = TiledPlan{a, n1, b};
