@@ -289,7 +289,8 @@ def linear(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, accumulate:
     gate (bfloat16, aligned shapes): the rows of weight alternate gate/up and
     out[m, j] = activation(row 2j) * row 2j+1, out [M, N/2].
     kernel (bfloat16 only): 0 automatic, 1 skinny, 2 tiled 128x128, 3 the simple tiled
-    kernel, 4 tiled 256x256, 5 tiled 256x128."""
+    kernel, 4 tiled 256x256, 5 tiled 256x128, 6 tiled 256x192, 7 and 8 tiled 128x128 and 128x192
+    loaded straight into LDS."""
     _gpu(out, x, weight)
     M, K, lda = _rows2d(x, "linear x")
     N, Kw, ldw = _rows2d(weight, "linear weight")
