@@ -713,7 +713,7 @@ int raise_pipelined_lds(size_t lds) {
 // 110 -> 101, at 896 148 -> 115; N 5,120, K 13,824 at 640 rows 140 -> 106; N 6,144, K 4,096 at 160 to 256
 // rows 38 to 39 -> 33 to 34; one case lost, N 2,048, K 8,192 at 384 rows 38.7 -> 41.4).
 inline int large_tile_cuts(int M, int N, int K) {
-  if (M <= 64 || K % 64 != 0 || N % 4 != 0) return 0;
+  if (M <= 16 || K % 64 != 0 || N % 4 != 0) return 0;
   const int64_t rows256 = (int64_t)((M + 255) / 256) * 256, rows128 = (int64_t)((M + 127) / 128) * 128;
   if (rows256 * 3 > rows128 * 4) return 0;
   const int64_t tiles = (int64_t)((N + 127) / 128) * (rows256 / 256);
@@ -754,7 +754,7 @@ inline int pipelined_splits(int M, int N, int K) {
   if (whole_in_one_round(M, N, K, tiles)) return 1;
   if (const int cuts = large_tile_cuts(M, N, K); cuts > 1 && K >= 2048) return cuts;
   const bool long_k = K >= 8192;
-  if (M <= 64 || tiles >= (long_k ? 384 : 256) || K < 2048 || N % 4 != 0) return 1;
+  if (M <= 16 || tiles >= (long_k ? 384 : 256) || K < 2048 || N % 4 != 0) return 1;
   // (a short K in three or four cuts is a few steps between a prologue and an epilogue: with more than 96
   // tiles the whole product is faster, N 3,072, K 2,048 at 768 rows 31.7 us against 35.9, N 2,048 at 1,024 rows
   // 35.9 against 38.5; at K = 3,072 the cuts still win, 37.5 against 47)
@@ -1452,13 +1452,21 @@ int launch_aligned(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf1
 
 // Up to 16 rows the streaming kernel always wins.  From 17 to 64 rows it re-reads the
 // batch for every 16 weight rows, and the tiled kernel (which wastes matrix
-// instructions but not bandwidth) wins once there are enough tiles to fill the chip.
-inline bool skinny_pays(int M, int N) { return M <= 16 || (M <= 64 && N < 16384); }
+// instructions but not bandwidth) wins once there are enough tiles to fill the chip, or
+// weights enough for its cuts of K to fill it.  (This is the way of weights that lie as rows only:
+// those that also lie in tiles go through hfee_gemm_skinny up to 64 rows.)
+// (weights as rows, us, the streaming kernel against the tiled one with its cuts of K: N 6,144, K 4,096 at 17 /
+// 33 / 64 rows 27.5 / 34.0 / 46.7 against 22.1 / 22.5 / 24.0; N 4,096, K 14,336 48.1 / 59.6 / 75.7 against 33.4 / 34.2 /
+// 36.4; N 8,192, K 28,672 136 / 182 / 271 against 92 / 94 / 102; N 4,096, K 4,096 level up to 24 rows, 28.9 against 22.1
+// at 64; N 3,072, K 2,048 14.7 / 16.6 / 19.6 against 17.4 / 18.2 / 18.8: from sixteen million weights on the tiled one)
+inline bool skinny_pays(int M, int N, int K) {
+  return M <= 16 || (M <= 64 && N < 16384 && (int64_t)N * K < (16ll << 20));
+}
 
 template <int MODE, bool VEC>
 int launch(void* C, int64_t ldc, const bf16_t* A, int64_t lda, const bf16_t* W, int64_t ldw,
            int M, int N, int K, int force_kernel, hipStream_t stream, const Partial& partial) {
-  const bool skinny = force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N));
+  const bool skinny = force_kernel == 1 || (force_kernel == 0 && skinny_pays(M, N, K));
   if (skinny) {
     dim3 grid((N + SK_ROWS - 1) / SK_ROWS);
     for (int m0 = 0; m0 < M; m0 += 64) {   // M > 64 only when the kernel was forced
@@ -1499,6 +1507,7 @@ HFEE_API int hfee_gemm_bf16_plan(int M, int N, int K, int* first, int* n1, int* 
 // too few tiles for the chip are cut along K over more workgroups, which leave their partial
 // products there for a second kernel to add up.
 HFEE_API int hfee_gemm_bf16_scratch(int M, int N, int K) {
+  if (skinny_pays(M, N, K)) return 0;                    // (the streaming kernel cuts nothing)
   const int splits = pipelined_splits(M, N, K);          // (fewer than 256 tiles of 128 x 128, at most 8 cuts: it fits an int)
   return splits > 1 ? splits * M * N : 0;
 }
@@ -1564,7 +1573,7 @@ HFEE_API int hfee_gemm_bf16_add_norm(float* C, const void* A, int64_t lda, const
   if (M == 0) return 0;
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
   bool done = false;
-  if (vec && !skinny_pays(M, N)) {
+  if (vec && !skinny_pays(M, N, K)) {
     const TiledPlan plan = plan_tiled(M, N, K, large_fits(lda, ldw, M, N, K), true);
     if (plan.first == 2 && plan.second == 0) {
       Partial partial;
@@ -1599,7 +1608,7 @@ HFEE_API int hfee_gemm_bf16_cuts(const void* A, int64_t lda, const void* W, int6
   HFEE_REQUIRE(lda >= K && ldw >= K, "gemm_bf16_cuts: a leading dimension is shorter than its row");
   *cuts = 0;
   const bool vec = (K % 8 == 0) && (lda % 8 == 0) && (ldw % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
-  if (!vec || skinny_pays(M, N) || scratch == nullptr || (uintptr_t)scratch % 16 != 0 || N % 4 != 0) return 0;
+  if (!vec || skinny_pays(M, N, K) || scratch == nullptr || (uintptr_t)scratch % 16 != 0 || N % 4 != 0) return 0;
   const TiledPlan plan = plan_tiled(M, N, K, large_fits(lda, ldw, M, N, K), true);
   const int splits = pipelined_splits(M, N, K);
   if (plan.first != 2 || plan.second != 0 || splits < 2 || scratch_floats < (int64_t)splits * M * N) return 0;

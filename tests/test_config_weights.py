@@ -243,7 +243,8 @@ def test_where_a_product_of_a_prompt_is_cut_along_k():
     """The host's rule for the products of 65 and more rows (asked of the library, which needs no
     GPU for it): with too few tiles of 128 x 128 for the chip K is cut over more workgroups and the
     caller brings scratch for the cuts; one round of such tiles runs whole where K is short and the
-    tiles are many for it; nothing is cut up to 64 rows, nor once the tiles fill the chip."""
+    tiles are many for it; nothing is cut up to 16 rows, up to 64 rows of a small weight (they go to the
+    kernel that streams the weight's rows), nor once the tiles fill the chip."""
     from hfee_amd.kernels import ops
 
     def cuts(M, N, K):
@@ -259,6 +260,8 @@ def test_where_a_product_of_a_prompt_is_cut_along_k():
     assert cuts(1024, 3072, 3072) == 0
     # ... but few tiles for the length of K are cut, and a long K always
     assert cuts(128, 3072, 2048) == 4 and cuts(256, 2048, 2048) == 4 and cuts(1024, 2048, 8192) >= 2
-    # the rows of a decode step, and products that fill the chip
-    assert cuts(64, 4096, 4096) == 0 and cuts(8, 4096, 14336) == 0
+    # the rows of a decode step over a weight that lies as rows only: cut from 17 rows on where the weight is large
+    assert cuts(16, 4096, 14336) == 0 and cuts(8, 4096, 14336) == 0 and cuts(64, 3072, 2048) == 0 and cuts(40, 768, 2048) == 0
+    assert cuts(17, 4096, 14336) == 8 and cuts(64, 4096, 4096) == 8 and cuts(64, 6144, 4096) == 5
+    # products that fill the chip
     assert cuts(2048, 4096, 4096) == 0 and cuts(2048, 28672, 4096) == 0 and cuts(512, 28672, 4096) == 0
